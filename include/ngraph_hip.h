@@ -1,0 +1,191 @@
+/*
+ * ngraph_hip.h -- C ABI of libngraph_hip.so, the MI355X (gfx950) execution
+ * library behind the `hipgpu` / `flexhip` transformers.
+ *
+ * The library replaces, for the fused elementwise / reduction / flex16 path,
+ * what the reference GPU transformer obtains from pycuda + NVRTC:
+ *   - device runtime        ngraph/transformers/gputransform.py:912-1000 (GPURuntime)
+ *   - device memory         ngraph/transformers/gputransform.py:525-676  (drv.mem_alloc, views)
+ *   - host <-> device I/O   ngraph/transformers/gputransform.py:710-909  (get / __setitem__)
+ *   - compound kernels      ngraph/transformers/gpu/float_ew2.py:1135-1483
+ *                           (_get_compound_kernel / prepared_async_call)
+ *   - flex scale + maxabs   ngraph/transformers/gpu/float_ew2.py:93-98, 261-281, 1346-1404
+ *                           ngraph/transformers/flexgputransform.py:56-61
+ *   - strided copies        ngraph/transformers/gpu/kernels/cuda/copy_transpose.py:89-282
+ *
+ * Conventions: every entry point returns 0 on success and a negative
+ * NGH_E_* code on failure; the text of the last failure on the calling
+ * thread is available from ngh_last_error().  Nothing aborts.  Pointers
+ * named `dev*` are device addresses obtained from ngh_malloc; all other
+ * pointers are host memory.  All work is issued, in order, on one HIP
+ * stream owned by the context; only ngh_sync, ngh_memcpy_d2h and
+ * ngh_stats_read wait for it.
+ */
+#ifndef NGRAPH_HIP_H
+#define NGRAPH_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NGH_ABI_VERSION 1
+
+/* ---- limits (float_ew2.py:285-286 MAX_AXES = 3) ------------------------ */
+#define NGH_MAX_AXES      3
+#define NGH_MAX_TENSORS   12
+#define NGH_MAX_OPS       96
+#define NGH_MAX_CONSTS    16
+#define NGH_MAX_REGS      32
+#define NGH_MAX_REDUCTIONS 4
+#define NGH_MAX_STAGES    6
+
+/* ---- error codes -------------------------------------------------------- */
+#define NGH_OK             0
+#define NGH_E_INVALID     -1   /* malformed argument or spec               */
+#define NGH_E_RUNTIME     -2   /* a HIP runtime call failed                */
+#define NGH_E_NOMEM       -3   /* device allocation failed                 */
+#define NGH_E_UNSUPPORTED -4   /* valid but outside what the kernels cover */
+#define NGH_E_NODEVICE    -5   /* no usable gfx950 device                  */
+
+/* ---- storage types (float_ew2.py:615-641 _get_register_type) ------------ */
+#define NGH_F32     0          /* float                                     */
+#define NGH_FLEX16  1          /* int16 mantissa, shared per-tensor scale   */
+#define NGH_I32     2          /* int32 (argmax / argmin results, indices)  */
+#define NGH_F16     3          /* IEEE half in memory, float in registers   */
+
+/* ---- opcodes ------------------------------------------------------------
+ * One entry per template of float_ew2.py:31-68 (_op_templates) and
+ * :70-77 (_redop_templates).  Arithmetic follows the NumPy float32 calls the
+ * CPU transformer issues (cputransform.py:512-761) wherever the CUDA template
+ * and NumPy disagree (floor_divide / mod on negative operands, sign of NaN).
+ * All registers are fp32.                                                    */
+enum ngh_opcode {
+    NGH_OP_NOP = 0,
+    /* data movement: LOAD dst=reg a=tensor ; STORE dst=tensor a=reg ;
+     * CONST dst=reg a=const slot ; IOTA dst=reg a=axis (index along axis) */
+    NGH_OP_LOAD, NGH_OP_STORE, NGH_OP_CONST, NGH_OP_IOTA,
+    /* unary: dst=reg a=reg */
+    NGH_OP_ASSIGN, NGH_OP_NEG, NGH_OP_ABS, NGH_OP_SQRT, NGH_OP_SQR, NGH_OP_EXP,
+    NGH_OP_LOG, NGH_OP_RCP, NGH_OP_EXP2, NGH_OP_LOG2, NGH_OP_SIG, NGH_OP_TANH,
+    NGH_OP_SAFELOG, NGH_OP_SGN, NGH_OP_SIN, NGH_OP_COS,
+    /* binary: dst=reg a=reg b=reg */
+    NGH_OP_ADD, NGH_OP_SUB, NGH_OP_MUL, NGH_OP_DIV, NGH_OP_INT_DIV, NGH_OP_MOD,
+    NGH_OP_EQ, NGH_OP_NE, NGH_OP_LT, NGH_OP_LE, NGH_OP_GT, NGH_OP_GE,
+    NGH_OP_POW, NGH_OP_MINIMUM, NGH_OP_MAXIMUM,
+    /* reductions over axis 0 of the stage's view: dst=reduction slot a=reg */
+    NGH_OP_RED_SUM, NGH_OP_RED_PROD, NGH_OP_RED_MAX, NGH_OP_RED_MIN,
+    NGH_OP_RED_ARGMAX, NGH_OP_RED_ARGMIN,
+    NGH_OP_COUNT_
+};
+
+typedef struct ngh_op {
+    uint8_t opcode;            /* enum ngh_opcode                            */
+    uint8_t dst;
+    uint8_t a;
+    uint8_t b;
+} ngh_op;
+
+/* One operand of a fused kernel: the strided view the reference passes as
+ * (pointer, stride_a, stride_b, stride_c [, flex scale [, flex_stats]])
+ * (float_ew2.py:987-1132).  Strides are in ELEMENTS; stride 0 broadcasts. */
+typedef struct ngh_tensor {
+    void*    dev;              /* device address of view element (0,0,0)     */
+    int64_t  strides[NGH_MAX_AXES];
+    int32_t  dtype;            /* NGH_F32 / NGH_FLEX16 / NGH_I32 / NGH_F16   */
+    float    scale;            /* FLEX16 only.  Loaded value = scale * int16;
+                                  stored int16 = rni_sat(value * scale), i.e.
+                                  the caller passes entry.scale for inputs
+                                  and 1/entry.scale for outputs
+                                  (flexgputransform.py:56-61)                */
+    int32_t* dev_stats;        /* FLEX16 outputs: int32 max|mantissa| merged
+                                  with atomic max (float_ew2.py:281,1404);
+                                  NULL = no statistics                       */
+    const float* dev_scale;    /* FLEX16 only, optional: when not NULL the
+                                  kernel reads the scale from this device
+                                  word instead of `scale` (lets an on-device
+                                  exponent update feed the next launch
+                                  without a host round trip)                 */
+} ngh_tensor;
+
+/* One stage = a run of elementwise ops optionally ended by reductions
+ * (float_ew2.py:553-612 _preprocess_ops).  Every stage iterates over the
+ * spec's single view `shape`; reductions run over axis 0 of that view
+ * (gputransform.py:117-122: reductions always pass axis 0), so the tensor
+ * receiving a reduction has stride 0 on axis 0 (the "missing axis" of
+ * float_ew2.py:307-309).  Stages run in order; a later stage reads an
+ * earlier stage's reduction result as a broadcast load.                     */
+typedef struct ngh_stage {
+    int32_t  op_begin, op_end; /* half-open range into ngh_fused_spec.ops    */
+    int32_t  n_reductions;     /* 0 = pure elementwise stage                 */
+    int32_t  red_out[NGH_MAX_REDUCTIONS];  /* tensor index receiving slot k  */
+} ngh_stage;
+
+typedef struct ngh_fused_spec {
+    int32_t     abi_version;   /* NGH_ABI_VERSION                            */
+    int32_t     rank;          /* 1..3; axes beyond rank have length 1       */
+    int64_t     shape[NGH_MAX_AXES];
+    int32_t     n_tensors, n_ops, n_consts, n_stages, n_regs;
+    ngh_tensor  tensors[NGH_MAX_TENSORS];
+    float       consts[NGH_MAX_CONSTS];
+    ngh_op      ops[NGH_MAX_OPS];
+    ngh_stage   stages[NGH_MAX_STAGES];
+} ngh_fused_spec;
+
+typedef struct ngh_context ngh_context;
+
+/* ---- runtime: replaces GPURuntime / drv.init (gputransform.py:912-935) --- */
+int  ngh_abi_version(void);
+const char* ngh_last_error(void);
+int  ngh_device_count(int* count);
+int  ngh_init(int device_id, ngh_context** out_ctx);
+int  ngh_shutdown(ngh_context* ctx);
+int  ngh_sync(ngh_context* ctx);
+/* name (<=255 chars + NUL), compute units, bytes of device memory */
+int  ngh_device_info(ngh_context* ctx, char* name256, int* compute_units,
+                     uint64_t* total_bytes);
+
+/* ---- memory: replaces drv.mem_alloc / free / memcpy / GPUArray.fill
+ *      (gputransform.py:547-569, 710-744, 807-871)                          */
+int  ngh_malloc(ngh_context* ctx, size_t bytes, void** out_dev);
+int  ngh_free(ngh_context* ctx, void* dev);
+int  ngh_memcpy_h2d(ngh_context* ctx, void* dev, const void* host, size_t bytes);
+int  ngh_memcpy_d2h(ngh_context* ctx, void* host, const void* dev, size_t bytes);
+int  ngh_memcpy_d2d(ngh_context* ctx, void* dev_dst, const void* dev_src, size_t bytes);
+int  ngh_memset32(ngh_context* ctx, void* dev, uint32_t value, size_t count);
+int  ngh_memset16(ngh_context* ctx, void* dev, uint16_t value, size_t count);
+
+/* ---- strided copy / dimshuffle: replaces _get_copy_transpose_kernel
+ *      (copy_transpose.py:89-282) and DimShuffleKernel (tensor_ops.py:137-204).
+ *      Copies an N-d view (rank <= 8) element by element; itemsize 2 or 4.   */
+int  ngh_copy_strided(ngh_context* ctx, void* dev_dst, const void* dev_src,
+                      int32_t rank, const int64_t* shape,
+                      const int64_t* dst_strides, const int64_t* src_strides,
+                      int32_t itemsize);
+
+/* ---- compound kernels: replaces CudaSourceFile.add_kernel + compile +
+ *      prepared_async_call (float_ew2.py:1553-1653, gputransform.py:343-345) */
+int  ngh_validate_fused(const ngh_fused_spec* spec);
+int  ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec);
+/* Which pre-built kernel family ngh_launch_fused picks for stage `stage`
+ * of `spec` (diagnostics and tests): writes a NUL-terminated name.          */
+int  ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec,
+                        int32_t stage, char* name128);
+
+/* ---- flex statistics: the int32 device words FlexPtrDescription binds
+ *      (float_ew2.py:363-374); replaces the manager's allocate/readback
+ *      (flexgputransform.py:143-150, 361-366)                                */
+int  ngh_stats_alloc(ngh_context* ctx, int32_t n, int32_t** out_dev);
+int  ngh_stats_reset(ngh_context* ctx, int32_t* dev, int32_t n);
+int  ngh_stats_read(ngh_context* ctx, const int32_t* dev, int32_t n, int32_t* host);
+
+/* ---- timing (HIP events on the context's stream; used by the bench) ----- */
+int  ngh_timer_begin(ngh_context* ctx);
+int  ngh_timer_end(ngh_context* ctx, float* out_ms);   /* waits for the stream */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NGRAPH_HIP_H */

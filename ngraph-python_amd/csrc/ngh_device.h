@@ -1,0 +1,311 @@
+// Device-side building blocks shared by every fused kernel: the per-element
+// arithmetic of each opcode, storage-type conversion on load/store (fp32,
+// flex16, int32, fp16), and the register files the op programs run on.
+//
+// Semantics follow the NumPy float32 calls the CPU transformer issues
+// (ngraph/transformers/cputransform.py:512-761) for the op set the GPU
+// transformer dispatches (ngraph/transformers/gputransform.py:124-275,
+// templates in ngraph/transformers/gpu/float_ew2.py:31-108).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include "ngraph_hip.h"
+
+namespace ngh {
+
+// ---------------------------------------------------------------------------
+// Kernel-side view of one stage of a fused spec.  Axes are already permuted by
+// the host planner so that axis 2 is the one lanes run along.
+// ---------------------------------------------------------------------------
+struct KTensor {
+    char*        p;
+    long long    s[3];       // element strides along kernel axes 0,1,2
+    int          dtype;
+    float        scale;
+    int*         stats;
+    const float* dscale;
+    int          stat_slot;  // which per-thread max|mantissa| accumulator, -1 = none
+    int          pad_;
+};
+
+struct KArgs {
+    long long shape[3];
+    int       n_tensors, op_begin, op_end, n_regs;
+    int       n_red;
+    int       red_out[NGH_MAX_REDUCTIONS];
+    int       red_axis;      // kernel axis the reductions run along (0 or 2), -1 = none
+    int       iota_map[3];   // kernel axis holding spec axis k (for NGH_OP_IOTA)
+    int       n_stat_slots;
+    int*      stat_ptr[4];   // device word of each per-thread accumulator
+    KTensor   t[NGH_MAX_TENSORS];
+    float     consts[NGH_MAX_CONSTS];
+    ngh_op    ops[NGH_MAX_OPS];
+};
+
+// ---------------------------------------------------------------------------
+// Per-element arithmetic.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float np_sign(float x) {
+    // np.sign: -1, 0, +1, NaN for NaN (cputransform.py:727-729)
+    return (x > 0.0f) ? 1.0f : ((x < 0.0f) ? -1.0f : ((x == 0.0f) ? 0.0f : x));
+}
+
+__device__ __forceinline__ float np_maximum(float a, float b) {
+    // np.maximum / np.max propagate NaN (cputransform.py:670-676)
+    return (a >= b || a != a) ? a : b;
+}
+__device__ __forceinline__ float np_minimum(float a, float b) {
+    return (a <= b || a != a) ? a : b;
+}
+
+// NumPy's float divmod (npy_divmod): floor_divide and mod share it
+// (cputransform.py:603-609 emit np.floor_divide / np.mod).
+__device__ __forceinline__ void np_divmod(float a, float b, float& floordiv, float& mod) {
+    if (b == 0.0f) {
+        floordiv = a / b;
+        mod = fmodf(a, b);
+        return;
+    }
+    mod = fmodf(a, b);
+    float div = (a - mod) / b;
+    if (mod != 0.0f) {
+        if ((b < 0.0f) != (mod < 0.0f)) {
+            mod += b;
+            div -= 1.0f;
+        }
+    } else {
+        mod = copysignf(0.0f, b);
+    }
+    if (div != 0.0f) {
+        floordiv = floorf(div);
+        if (div - floordiv > 0.5f) floordiv += 1.0f;
+    } else {
+        floordiv = copysignf(0.0f, a / b);
+    }
+}
+
+__device__ __forceinline__ float op_unary(int opc, float x) {
+    switch (opc) {
+        case NGH_OP_ASSIGN:  return x;
+        case NGH_OP_NEG:     return -x;
+        case NGH_OP_ABS:     return fabsf(x);
+        case NGH_OP_SQRT:    return sqrtf(x);
+        case NGH_OP_SQR:     return x * x;
+        case NGH_OP_EXP:     return expf(x);
+        case NGH_OP_LOG:     return logf(x);
+        case NGH_OP_RCP:     return 1.0f / x;
+        case NGH_OP_EXP2:    return exp2f(x);
+        case NGH_OP_LOG2:    return log2f(x);
+        case NGH_OP_SIG:     return 1.0f / (1.0f + expf(-x));     // float_ew2.py:43
+        case NGH_OP_TANH:    return tanhf(x);
+        case NGH_OP_SAFELOG: return (x > 0.0f) ? logf(x) : -50.0f; // float_ew2.py:48
+        case NGH_OP_SGN:     return np_sign(x);
+        case NGH_OP_SIN:     return sinf(x);
+        case NGH_OP_COS:     return cosf(x);
+        default:             return x;
+    }
+}
+
+__device__ __forceinline__ float op_binary(int opc, float x, float y) {
+    switch (opc) {
+        case NGH_OP_ADD: return x + y;
+        case NGH_OP_SUB: return x - y;
+        case NGH_OP_MUL: return x * y;
+        case NGH_OP_DIV: return x / y;
+        case NGH_OP_INT_DIV: { float q, m; np_divmod(x, y, q, m); return q; }
+        case NGH_OP_MOD:     { float q, m; np_divmod(x, y, q, m); return m; }
+        case NGH_OP_EQ: return (x == y) ? 1.0f : 0.0f;
+        case NGH_OP_NE: return (x != y) ? 1.0f : 0.0f;
+        case NGH_OP_LT: return (x <  y) ? 1.0f : 0.0f;
+        case NGH_OP_LE: return (x <= y) ? 1.0f : 0.0f;
+        case NGH_OP_GT: return (x >  y) ? 1.0f : 0.0f;
+        case NGH_OP_GE: return (x >= y) ? 1.0f : 0.0f;
+        case NGH_OP_POW: return powf(x, y);
+        case NGH_OP_MINIMUM: return np_minimum(x, y);
+        case NGH_OP_MAXIMUM: return np_maximum(x, y);
+        default: return x;
+    }
+}
+
+__host__ __device__ __forceinline__ bool is_unary(int opc)  { return opc >= NGH_OP_ASSIGN && opc <= NGH_OP_COS; }
+__host__ __device__ __forceinline__ bool is_binary(int opc) { return opc >= NGH_OP_ADD && opc <= NGH_OP_MAXIMUM; }
+__host__ __device__ __forceinline__ bool is_reduce(int opc) { return opc >= NGH_OP_RED_SUM && opc <= NGH_OP_RED_ARGMIN; }
+
+// ---------------------------------------------------------------------------
+// flex16 conversion (float_ew2.py:96-97, 261-277): load = scale * mantissa;
+// store = cvt.rni.s16.f32(scale * value): round to nearest even, saturate to
+// [-32768, 32767], NaN -> 0; statistics = max |stored mantissa| as int32.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ int flex_quantize(float v) {
+    float r = rintf(v);                       // round-half-even in the default mode
+    r = fminf(fmaxf(r, -32768.0f), 32767.0f); // saturate (NaN -> -32768 by fmaxf, fixed below)
+    int q = (int)r;
+    return (v != v) ? 0 : q;
+}
+
+__device__ __forceinline__ int iabs(int x) { return x < 0 ? -x : x; }
+
+// ---------------------------------------------------------------------------
+// Element access by storage type.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float tensor_scale(const KTensor& t) {
+    return t.dscale ? *t.dscale : t.scale;
+}
+
+__device__ __forceinline__ float load1(const KTensor& t, long long off, float scale) {
+    switch (t.dtype) {
+        case NGH_F32:    return reinterpret_cast<const float*>(t.p)[off];
+        case NGH_FLEX16: return scale * (float)reinterpret_cast<const short*>(t.p)[off];
+        case NGH_I32:    return (float)reinterpret_cast<const int*>(t.p)[off];
+        case NGH_F16:    return __half2float(reinterpret_cast<const __half*>(t.p)[off]);
+        default:         return 0.0f;
+    }
+}
+
+__device__ __forceinline__ void store1(const KTensor& t, long long off, float v, float scale, int& fmax) {
+    switch (t.dtype) {
+        case NGH_F32: reinterpret_cast<float*>(t.p)[off] = v; break;
+        case NGH_FLEX16: {
+            int q = flex_quantize(scale * v);
+            reinterpret_cast<short*>(t.p)[off] = (short)q;
+            fmax = max(fmax, iabs(q));
+        } break;
+        case NGH_I32: reinterpret_cast<int*>(t.p)[off] = (int)v; break;
+        case NGH_F16: reinterpret_cast<__half*>(t.p)[off] = __float2half(v); break;
+        default: break;
+    }
+}
+
+// 4 consecutive elements; `off` is a multiple of 4 and the base is aligned.
+__device__ __forceinline__ void load4(const KTensor& t, long long off, float scale, float (&v)[4]) {
+    switch (t.dtype) {
+        case NGH_F32: {
+            float4 x = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(t.p) + off);
+            v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+        } break;
+        case NGH_FLEX16: {
+            short4 x = *reinterpret_cast<const short4*>(reinterpret_cast<const short*>(t.p) + off);
+            v[0] = scale * (float)x.x; v[1] = scale * (float)x.y;
+            v[2] = scale * (float)x.z; v[3] = scale * (float)x.w;
+        } break;
+        case NGH_I32: {
+            int4 x = *reinterpret_cast<const int4*>(reinterpret_cast<const int*>(t.p) + off);
+            v[0] = (float)x.x; v[1] = (float)x.y; v[2] = (float)x.z; v[3] = (float)x.w;
+        } break;
+        case NGH_F16: {
+            const __half2* h = reinterpret_cast<const __half2*>(reinterpret_cast<const __half*>(t.p) + off);
+            uint2 raw = *reinterpret_cast<const uint2*>(h);
+            __half2 a = *reinterpret_cast<__half2*>(&raw.x), b = *reinterpret_cast<__half2*>(&raw.y);
+            float2 fa = __half22float2(a), fb = __half22float2(b);
+            v[0] = fa.x; v[1] = fa.y; v[2] = fb.x; v[3] = fb.y;
+        } break;
+        default: v[0] = v[1] = v[2] = v[3] = 0.0f;
+    }
+}
+
+__device__ __forceinline__ void store4(const KTensor& t, long long off, float scale, const float (&v)[4], int& fmax) {
+    switch (t.dtype) {
+        case NGH_F32:
+            *reinterpret_cast<float4*>(reinterpret_cast<float*>(t.p) + off) = make_float4(v[0], v[1], v[2], v[3]);
+            break;
+        case NGH_FLEX16: {
+            int q0 = flex_quantize(scale * v[0]), q1 = flex_quantize(scale * v[1]);
+            int q2 = flex_quantize(scale * v[2]), q3 = flex_quantize(scale * v[3]);
+            short4 x; x.x = (short)q0; x.y = (short)q1; x.z = (short)q2; x.w = (short)q3;
+            *reinterpret_cast<short4*>(reinterpret_cast<short*>(t.p) + off) = x;
+            fmax = max(max(fmax, max(iabs(q0), iabs(q1))), max(iabs(q2), iabs(q3)));
+        } break;
+        case NGH_I32:
+            *reinterpret_cast<int4*>(reinterpret_cast<int*>(t.p) + off) =
+                make_int4((int)v[0], (int)v[1], (int)v[2], (int)v[3]);
+            break;
+        case NGH_F16: {
+            __half2 a = __floats2half2_rn(v[0], v[1]), b = __floats2half2_rn(v[2], v[3]);
+            uint2 raw; raw.x = *reinterpret_cast<unsigned*>(&a); raw.y = *reinterpret_cast<unsigned*>(&b);
+            *reinterpret_cast<uint2*>(reinterpret_cast<__half*>(t.p) + off) = raw;
+        } break;
+        default: break;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Register file of the op interpreter.  The program is only known at run
+// time, so register numbers are run-time values; a per-lane array indexed that
+// way would live in scratch memory.  The file is kept in LDS instead, laid
+// out [register][vector element][thread] so lanes of a wavefront hit
+// consecutive banks.
+// ---------------------------------------------------------------------------
+template <int V>
+struct LdsRegs {
+    float* base;   // &lds[thread]
+    int    nthr;   // threads per workgroup
+    __device__ __forceinline__ float get(int r, int v) const { return base[(r * V + v) * nthr]; }
+    __device__ __forceinline__ void  set(int r, int v, float x) { base[(r * V + v) * nthr] = x; }
+};
+
+// ---------------------------------------------------------------------------
+// Reduction accumulators (float_ew2.py:70-108: inits 0 / 1 / -FLT_MAX /
+// FLT_MAX; argmax/argmin carry (value, index)).  Ties resolve to the lowest
+// index, as np.argmax / np.argmin do (cputransform.py:521-527).
+// ---------------------------------------------------------------------------
+struct Acc {
+    float v;
+    int   i;
+};
+
+__device__ __forceinline__ Acc acc_init(int opc) {
+    Acc a; a.i = 0;
+    switch (opc) {
+        case NGH_OP_RED_SUM:    a.v = 0.0f; break;
+        case NGH_OP_RED_PROD:   a.v = 1.0f; break;
+        case NGH_OP_RED_MAX:    a.v = -__builtin_inff(); break;
+        case NGH_OP_RED_MIN:    a.v =  __builtin_inff(); break;
+        case NGH_OP_RED_ARGMAX: a.v = -__builtin_inff(); a.i = 0x7fffffff; break;
+        case NGH_OP_RED_ARGMIN: a.v =  __builtin_inff(); a.i = 0x7fffffff; break;
+        default: a.v = 0.0f;
+    }
+    return a;
+}
+
+__device__ __forceinline__ Acc acc_merge(int opc, Acc a, Acc b) {
+    switch (opc) {
+        case NGH_OP_RED_SUM:  a.v = a.v + b.v; break;
+        case NGH_OP_RED_PROD: a.v = a.v * b.v; break;
+        case NGH_OP_RED_MAX:  a.v = np_maximum(a.v, b.v); break;
+        case NGH_OP_RED_MIN:  a.v = np_minimum(a.v, b.v); break;
+        case NGH_OP_RED_ARGMAX: {
+            bool a_nan = a.v != a.v, b_nan = b.v != b.v;
+            bool take_b = (a_nan || b_nan) ? (b_nan && (!a_nan || b.i < a.i))
+                                           : (b.v > a.v || (b.v == a.v && b.i < a.i));
+            if (take_b) a = b;
+        } break;
+        case NGH_OP_RED_ARGMIN: {
+            bool a_nan = a.v != a.v, b_nan = b.v != b.v;
+            bool take_b = (a_nan || b_nan) ? (b_nan && (!a_nan || b.i < a.i))
+                                           : (b.v < a.v || (b.v == a.v && b.i < a.i));
+            if (take_b) a = b;
+        } break;
+        default: break;
+    }
+    return a;
+}
+
+__device__ __forceinline__ float acc_result(int opc, Acc a) {
+    return (opc == NGH_OP_RED_ARGMAX || opc == NGH_OP_RED_ARGMIN) ? (float)a.i : a.v;
+}
+
+__device__ __forceinline__ Acc acc_shfl_xor(Acc a, int mask) {
+    Acc b;
+    b.v = __shfl_xor(a.v, mask, 64);
+    b.i = __shfl_xor(a.i, mask, 64);
+    return b;
+}
+
+__device__ __forceinline__ int wave_max_int(int x) {
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) x = max(x, __shfl_xor(x, m, 64));
+    return x;
+}
+
+}  // namespace ngh

@@ -1,0 +1,679 @@
+// libngraph_hip.so -- C ABI implementation: context, device memory, the
+// planner that maps one stage of a fused spec onto a kernel skeleton, and the
+// launches.  See include/ngraph_hip.h for the contract of every entry point.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "ngraph_hip.h"
+#include "ngh_device.h"
+#include "ngh_interp.h"
+#include "ngh_copy.h"
+#include "ngh_special.h"
+
+using namespace ngh;
+
+// ---------------------------------------------------------------------------
+// errors
+// ---------------------------------------------------------------------------
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                    \
+    do {                                                                                 \
+        hipError_t e_ = (expr);                                                          \
+        if (e_ != hipSuccess)                                                            \
+            return fail(e_ == hipErrorOutOfMemory ? NGH_E_NOMEM : NGH_E_RUNTIME,         \
+                        "%s failed: %s", #expr, hipGetErrorString(e_));                  \
+    } while (0)
+
+#define NGH_TRY(expr)                \
+    do {                             \
+        int rc_ = (expr);            \
+        if (rc_ != NGH_OK) return rc_; \
+    } while (0)
+
+int itemsize_of(int dtype) {
+    switch (dtype) {
+        case NGH_F32: case NGH_I32: return 4;
+        case NGH_FLEX16: case NGH_F16: return 2;
+        default: return 0;
+    }
+}
+
+int env_int(const char* name, int dflt) {
+    const char* s = getenv(name);
+    return (s && *s) ? atoi(s) : dflt;
+}
+
+}  // namespace
+
+struct ngh_context {
+    int         device = 0;
+    int         cus = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t  ev0 = nullptr, ev1 = nullptr;
+    void*       ws = nullptr;        // partial results of split reductions
+    size_t      ws_bytes = 0;
+    int         ew_blocks_per_cu = 8;
+    int         force_interp = 0;    // never pick a specialised kernel
+    char        name[256] = "";
+    uint64_t    total_bytes = 0;
+};
+
+// ---------------------------------------------------------------------------
+// spec validation (host only; also run before every launch so a malformed
+// spec can never reach a kernel)
+// ---------------------------------------------------------------------------
+namespace {
+
+int validate(const ngh_fused_spec* sp) {
+    if (!sp) return fail(NGH_E_INVALID, "spec is NULL");
+    if (sp->abi_version != NGH_ABI_VERSION)
+        return fail(NGH_E_INVALID, "spec abi_version %d, library %d", sp->abi_version, NGH_ABI_VERSION);
+    if (sp->rank < 1 || sp->rank > NGH_MAX_AXES) return fail(NGH_E_INVALID, "rank %d out of 1..3", sp->rank);
+    long long total = 1;
+    for (int a = 0; a < NGH_MAX_AXES; ++a) {
+        if (sp->shape[a] < 0) return fail(NGH_E_INVALID, "negative shape on axis %d", a);
+        if (a >= sp->rank && sp->shape[a] != 1) return fail(NGH_E_INVALID, "axis %d beyond rank must have length 1", a);
+        total *= sp->shape[a];
+    }
+    if (sp->n_tensors < 0 || sp->n_tensors > NGH_MAX_TENSORS) return fail(NGH_E_INVALID, "n_tensors %d", sp->n_tensors);
+    if (sp->n_ops < 0 || sp->n_ops > NGH_MAX_OPS) return fail(NGH_E_INVALID, "n_ops %d", sp->n_ops);
+    if (sp->n_consts < 0 || sp->n_consts > NGH_MAX_CONSTS) return fail(NGH_E_INVALID, "n_consts %d", sp->n_consts);
+    if (sp->n_regs < 0 || sp->n_regs > NGH_MAX_REGS) return fail(NGH_E_INVALID, "n_regs %d", sp->n_regs);
+    if (sp->n_stages < 1 || sp->n_stages > NGH_MAX_STAGES) return fail(NGH_E_INVALID, "n_stages %d", sp->n_stages);
+    for (int t = 0; t < sp->n_tensors; ++t) {
+        const ngh_tensor& T = sp->tensors[t];
+        if (itemsize_of(T.dtype) == 0) return fail(NGH_E_INVALID, "tensor %d: unknown dtype %d", t, T.dtype);
+        if (total > 0 && T.dev == nullptr) return fail(NGH_E_INVALID, "tensor %d: NULL device pointer", t);
+        if (((uintptr_t)T.dev) % itemsize_of(T.dtype)) return fail(NGH_E_INVALID, "tensor %d: misaligned pointer", t);
+        for (int a = 0; a < NGH_MAX_AXES; ++a)
+            if (T.strides[a] < 0) return fail(NGH_E_UNSUPPORTED, "tensor %d: negative stride", t);
+    }
+    int next = 0;
+    for (int s = 0; s < sp->n_stages; ++s) {
+        const ngh_stage& S = sp->stages[s];
+        if (S.op_begin != next || S.op_end < S.op_begin || S.op_end > sp->n_ops)
+            return fail(NGH_E_INVALID, "stage %d: op range [%d,%d) does not follow %d", s, S.op_begin, S.op_end, next);
+        next = S.op_end;
+        if (S.n_reductions < 0 || S.n_reductions > NGH_MAX_REDUCTIONS)
+            return fail(NGH_E_INVALID, "stage %d: n_reductions %d", s, S.n_reductions);
+        bool defined[NGH_MAX_REGS] = {false};
+        int n_red_seen = 0;
+        for (int pc = S.op_begin; pc < S.op_end; ++pc) {
+            const ngh_op& o = sp->ops[pc];
+            const int opc = o.opcode;
+            auto reg_ok = [&](int r) { return r < sp->n_regs; };
+            auto need = [&](int r) { return reg_ok(r) && defined[r]; };
+            if (n_red_seen && !is_reduce(opc))
+                return fail(NGH_E_INVALID, "stage %d: op %d follows a reduction inside the stage", s, pc);
+            if (opc == NGH_OP_LOAD) {
+                if (o.a >= sp->n_tensors || !reg_ok(o.dst)) return fail(NGH_E_INVALID, "op %d: bad LOAD", pc);
+                defined[o.dst] = true;
+            } else if (opc == NGH_OP_STORE) {
+                if (o.dst >= sp->n_tensors || !need(o.a)) return fail(NGH_E_INVALID, "op %d: bad STORE", pc);
+                const ngh_tensor& T = sp->tensors[o.dst];
+                for (int a = 0; a < NGH_MAX_AXES; ++a)
+                    if (sp->shape[a] > 1 && T.strides[a] == 0)
+                        return fail(NGH_E_INVALID, "op %d: STORE to a tensor broadcast along axis %d", pc, a);
+            } else if (opc == NGH_OP_CONST) {
+                if (o.a >= sp->n_consts || !reg_ok(o.dst)) return fail(NGH_E_INVALID, "op %d: bad CONST", pc);
+                defined[o.dst] = true;
+            } else if (opc == NGH_OP_IOTA) {
+                if (o.a >= NGH_MAX_AXES || !reg_ok(o.dst)) return fail(NGH_E_INVALID, "op %d: bad IOTA", pc);
+                defined[o.dst] = true;
+            } else if (is_unary(opc)) {
+                if (!need(o.a) || !reg_ok(o.dst)) return fail(NGH_E_INVALID, "op %d: unary operand undefined", pc);
+                defined[o.dst] = true;
+            } else if (is_binary(opc)) {
+                if (!need(o.a) || !need(o.b) || !reg_ok(o.dst))
+                    return fail(NGH_E_INVALID, "op %d: binary operand undefined", pc);
+                defined[o.dst] = true;
+            } else if (is_reduce(opc)) {
+                if (!need(o.a) || o.dst != n_red_seen || n_red_seen >= S.n_reductions)
+                    return fail(NGH_E_INVALID, "op %d: reduction slot %d out of order", pc, o.dst);
+                const int ot = S.red_out[n_red_seen];
+                if (ot < 0 || ot >= sp->n_tensors) return fail(NGH_E_INVALID, "stage %d: red_out[%d]", s, n_red_seen);
+                const ngh_tensor& T = sp->tensors[ot];
+                if (T.strides[0] != 0 && sp->shape[0] > 1)
+                    return fail(NGH_E_INVALID, "stage %d: reduction output %d must have stride 0 on axis 0", s, ot);
+                for (int a = 1; a < NGH_MAX_AXES; ++a)
+                    if (sp->shape[a] > 1 && T.strides[a] == 0)
+                        return fail(NGH_E_INVALID, "stage %d: reduction output broadcast along axis %d", s, a);
+                ++n_red_seen;
+            } else if (opc != NGH_OP_NOP) {
+                return fail(NGH_E_INVALID, "op %d: unknown opcode %d", pc, opc);
+            }
+        }
+        if (n_red_seen != S.n_reductions)
+            return fail(NGH_E_INVALID, "stage %d: %d reduction ops for n_reductions %d", s, n_red_seen, S.n_reductions);
+    }
+    if (next != sp->n_ops) return fail(NGH_E_INVALID, "stages cover %d of %d ops", next, sp->n_ops);
+    return NGH_OK;
+}
+
+// ---------------------------------------------------------------------------
+// planner
+// ---------------------------------------------------------------------------
+enum Family { F_EW = 0, F_RED_ROW, F_RED_COL };
+
+struct Plan {
+    Family   family = F_EW;
+    int      V = 1;
+    KArgs    k;
+    unsigned n_chunks = 0, chunks_per_row = 0;   // EW
+    unsigned n_out = 0, n_seg = 1, seg_len = 0;  // reductions
+    unsigned n_bx = 0;
+    int      special = -1;                        // index into the specialised-kernel table
+    long long tail = 0;                           // 1-D contiguous stage: elements left to a scalar launch
+};
+
+// Which tensors does the stage touch (load or store or reduce into)?
+void stage_tensors(const ngh_fused_spec& sp, const ngh_stage& S, bool* loads, bool* stores) {
+    for (int t = 0; t < NGH_MAX_TENSORS; ++t) loads[t] = stores[t] = false;
+    for (int pc = S.op_begin; pc < S.op_end; ++pc) {
+        const ngh_op& o = sp.ops[pc];
+        if (o.opcode == NGH_OP_LOAD) loads[o.a] = true;
+        if (o.opcode == NGH_OP_STORE) stores[o.dst] = true;
+    }
+}
+
+void fill_kargs(const ngh_fused_spec& sp, const ngh_stage& S, const int perm[3], KArgs& k) {
+    // kernel axis j holds spec axis perm[j]
+    memset(&k, 0, sizeof(k));
+    for (int j = 0; j < 3; ++j) {
+        k.shape[j] = sp.shape[perm[j]];
+        k.iota_map[perm[j]] = j;
+    }
+    k.n_tensors = sp.n_tensors;
+    k.op_begin = S.op_begin;
+    k.op_end = S.op_end;
+    k.n_regs = sp.n_regs;
+    k.n_red = S.n_reductions;
+    k.red_axis = -1;
+    for (int r = 0; r < S.n_reductions; ++r) k.red_out[r] = S.red_out[r];
+    if (S.n_reductions) k.red_axis = k.iota_map[0];
+    bool loads[NGH_MAX_TENSORS], stores[NGH_MAX_TENSORS];
+    stage_tensors(sp, S, loads, stores);
+    for (int t = 0; t < sp.n_tensors; ++t) {
+        const ngh_tensor& T = sp.tensors[t];
+        KTensor& K = k.t[t];
+        K.p = (char*)T.dev;
+        for (int j = 0; j < 3; ++j) K.s[j] = T.strides[perm[j]];
+        K.dtype = T.dtype;
+        K.scale = T.scale;
+        K.stats = T.dev_stats;
+        K.dscale = T.dev_scale;
+        K.stat_slot = -1;
+        if (stores[t] && T.dtype == NGH_FLEX16 && T.dev_stats && k.n_stat_slots < 4) {
+            K.stat_slot = k.n_stat_slots;
+            k.stat_ptr[k.n_stat_slots++] = T.dev_stats;
+        }
+    }
+    memcpy(k.consts, sp.consts, sizeof(k.consts));
+    memcpy(k.ops, sp.ops, sizeof(k.ops));
+}
+
+bool vec4_ok(const KArgs& k, const bool* used) {
+    if (k.shape[2] % 4) return false;
+    for (int t = 0; t < k.n_tensors; ++t) {
+        if (!used[t]) continue;
+        const KTensor& K = k.t[t];
+        if (K.s[2] == 0) continue;
+        if (K.s[2] != 1) return false;
+        if (((uintptr_t)K.p) % (4 * itemsize_of(K.dtype))) return false;
+        for (int j = 0; j < 2; ++j)
+            if (k.shape[j] > 1 && K.s[j] % 4) return false;
+    }
+    return true;
+}
+
+int plan_stage(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan& P) {
+    const ngh_stage& S = sp.stages[stage];
+    bool loads[NGH_MAX_TENSORS], stores[NGH_MAX_TENSORS], used[NGH_MAX_TENSORS];
+    stage_tensors(sp, S, loads, stores);
+    for (int t = 0; t < NGH_MAX_TENSORS; ++t) used[t] = loads[t] || stores[t];
+    long long total = sp.shape[0] * sp.shape[1] * sp.shape[2];
+    if (total >= (1LL << 31) * 4LL) return fail(NGH_E_UNSUPPORTED, "stage view of %lld elements exceeds 2^33", total);
+
+    if (S.n_reductions == 0) {
+        // fast axis = the one most operands are contiguous along; stores count double
+        int best = -1, best_score = -1;
+        for (int a = NGH_MAX_AXES - 1; a >= 0; --a) {
+            if (sp.shape[a] <= 1) continue;
+            int score = 0;
+            for (int t = 0; t < sp.n_tensors; ++t)
+                if (used[t] && sp.tensors[t].strides[a] == 1) score += stores[t] ? 2 : 1;
+            if (score > best_score) { best_score = score; best = a; }
+        }
+        if (best < 0) best = 2;
+        int perm[3], j = 0;
+        for (int a = 0; a < 3; ++a) if (a != best) perm[j++] = a;
+        perm[2] = best;
+        fill_kargs(sp, S, perm, P.k);
+        P.family = F_EW;
+        P.V = vec4_ok(P.k, used) ? 4 : 1;
+        P.tail = 0;
+        if (P.V == 1 && P.k.shape[0] == 1 && P.k.shape[1] == 1 && P.k.shape[2] >= 8) {
+            // contiguous 1-D view whose length is not a multiple of 4: vector body + scalar tail
+            const long long n = P.k.shape[2];
+            P.k.shape[2] = n - n % 4;
+            if (vec4_ok(P.k, used)) { P.V = 4; P.tail = n % 4; }
+            else P.k.shape[2] = n;
+        }
+        const long long rows = P.k.shape[0] * P.k.shape[1];
+        const long long cpr = P.k.shape[2] / P.V;
+        if (rows * cpr >= (1LL << 32) || rows >= (1LL << 32))
+            return fail(NGH_E_UNSUPPORTED, "stage has %lld chunks; split the launch", rows * cpr);
+        P.chunks_per_row = (unsigned)cpr;
+        P.n_chunks = (unsigned)(rows * cpr);
+        return NGH_OK;
+    }
+
+    // ---- reduction stage: spec axis 0 is reduced, (1,2) index the outputs ----
+    const long long R = sp.shape[0];
+    bool r_contig = true, any_main = false;
+    int out_contig_axis = -1;
+    for (int t = 0; t < sp.n_tensors; ++t) {
+        if (!loads[t]) continue;
+        const ngh_tensor& T = sp.tensors[t];
+        if (T.strides[0] == 0) continue;   // broadcast along the reduced axis
+        any_main = true;
+        if (T.strides[0] != 1) r_contig = false;
+    }
+    if (!any_main) r_contig = false;
+    if (!r_contig) {
+        for (int a = 2; a >= 1; --a) {
+            if (sp.shape[a] <= 1) continue;
+            bool ok = true, any = false;
+            for (int t = 0; t < sp.n_tensors; ++t) {
+                if (!loads[t] || sp.tensors[t].strides[0] == 0) continue;
+                any = true;
+                if (sp.tensors[t].strides[a] != 1) ok = false;
+            }
+            if (ok && any) { out_contig_axis = a; break; }
+        }
+    }
+    const long long n_out = sp.shape[1] * sp.shape[2];
+    if (n_out >= (1LL << 31) || R >= (1LL << 31)) return fail(NGH_E_UNSUPPORTED, "reduction extents exceed 2^31");
+    const int target_wgs = ctx->cus * 8;
+    if (out_contig_axis >= 0) {
+        const int other = (out_contig_axis == 2) ? 1 : 2;
+        const int perm[3] = {0, other, out_contig_axis};
+        fill_kargs(sp, S, perm, P.k);
+        P.family = F_RED_COL;
+        P.V = 1;
+        P.n_out = (unsigned)n_out;
+        P.n_bx = (unsigned)((P.k.shape[2] + kColTx - 1) / kColTx);
+        const long long base_wgs = (long long)P.n_bx * P.k.shape[1];
+        long long seg = std::max<long long>(1, target_wgs / std::max<long long>(1, base_wgs));
+        seg = std::min<long long>(seg, std::max<long long>(1, R / 64));
+        seg = std::min<long long>(seg, 1024);
+        P.seg_len = (unsigned)((R + seg - 1) / seg);
+        P.n_seg = (unsigned)((R + P.seg_len - 1) / std::max(1u, P.seg_len));
+        if (P.n_seg == 0) P.n_seg = 1;
+    } else {
+        const int perm[3] = {1, 2, 0};
+        fill_kargs(sp, S, perm, P.k);
+        P.family = F_RED_ROW;
+        P.V = (r_contig && vec4_ok(P.k, used)) ? 4 : 1;
+        P.n_out = (unsigned)n_out;
+        const long long chunks = R / P.V;
+        long long seg = std::max<long long>(1, target_wgs / std::max<long long>(1, n_out));
+        seg = std::min<long long>(seg, std::max<long long>(1, chunks / (kBlock * 4)));
+        seg = std::min<long long>(seg, 1024);
+        P.seg_len = (unsigned)((chunks + seg - 1) / seg);
+        P.n_seg = (unsigned)((chunks + P.seg_len - 1) / std::max(1u, P.seg_len));
+        if (P.n_seg == 0) P.n_seg = 1;
+    }
+    if ((long long)P.n_out * P.n_seg >= (1LL << 31)) return fail(NGH_E_UNSUPPORTED, "reduction grid too large");
+    return NGH_OK;
+}
+
+size_t interp_lds_bytes(const KArgs& k, int V) {
+    return ((size_t)k.n_regs * V + k.n_stat_slots + 2 * k.n_red) * kBlock * sizeof(float);
+}
+
+int ensure_ws(ngh_context* ctx, size_t bytes) {
+    if (bytes <= ctx->ws_bytes) return NGH_OK;
+    if (ctx->ws) {
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+        HIP_TRY(hipFree(ctx->ws));
+        ctx->ws = nullptr;
+        ctx->ws_bytes = 0;
+    }
+    size_t want = std::max(bytes, (size_t)4 << 20);
+    HIP_TRY(hipMalloc(&ctx->ws, want));
+    ctx->ws_bytes = want;
+    return NGH_OK;
+}
+
+int launch_interp(ngh_context* ctx, Plan& P) {
+    const KArgs& k = P.k;
+    int V = P.V;
+    size_t lds = interp_lds_bytes(k, V);
+    if (lds > 64 * 1024 && V == 4 && P.family == F_EW && P.tail == 0) {
+        // too many live registers for a 4-wide file: fall back to one element per lane
+        V = 1;
+        P.V = 1;
+        P.chunks_per_row *= 4;
+        P.n_chunks *= 4;
+        lds = interp_lds_bytes(k, 1);
+    }
+    if (lds > 64 * 1024) return fail(NGH_E_UNSUPPORTED, "program needs %zu bytes of LDS registers", lds);
+    if (P.family == F_EW) {
+        if (P.n_chunks == 0 && P.tail == 0) return NGH_OK;
+        if (P.n_chunks) {
+            unsigned blocks = (P.n_chunks + kBlock - 1) / kBlock;
+            blocks = std::min<unsigned>(blocks, (unsigned)(ctx->cus * ctx->ew_blocks_per_cu));
+            if (V == 4)
+                hipLaunchKernelGGL(ew_interp_kernel<4>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, P.n_chunks, P.chunks_per_row);
+            else
+                hipLaunchKernelGGL(ew_interp_kernel<1>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, P.n_chunks, P.chunks_per_row);
+            HIP_TRY(hipGetLastError());
+        }
+        if (P.tail) {
+            KArgs kt = k;
+            const long long body = k.shape[2];
+            kt.shape[2] = P.tail;
+            for (int t = 0; t < kt.n_tensors; ++t) kt.t[t].p += body * kt.t[t].s[2] * itemsize_of(kt.t[t].dtype);
+            // IOTA along the split axis would restart at 0 in the tail
+            for (int pc = kt.op_begin; pc < kt.op_end; ++pc)
+                if (kt.ops[pc].opcode == NGH_OP_IOTA && kt.iota_map[kt.ops[pc].a] == 2)
+                    return fail(NGH_E_UNSUPPORTED, "IOTA along a split 1-D axis");
+            hipLaunchKernelGGL(ew_interp_kernel<1>, dim3(1), dim3(kBlock), interp_lds_bytes(kt, 1), ctx->stream, kt,
+                               (unsigned)P.tail, (unsigned)P.tail);
+            HIP_TRY(hipGetLastError());
+        }
+        return NGH_OK;
+    }
+    if (P.n_out == 0) return NGH_OK;
+    RedWs ws{nullptr, nullptr};
+    if (P.n_seg > 1) {
+        const size_t n = (size_t)k.n_red * P.n_seg * P.n_out;
+        NGH_TRY(ensure_ws(ctx, n * 8));
+        ws.val = (float*)ctx->ws;
+        ws.idx = (int*)ctx->ws + n;
+    }
+    if (P.family == F_RED_ROW) {
+        const unsigned blocks = P.n_out * P.n_seg;
+        if (V == 4)
+            hipLaunchKernelGGL(red_row_interp_kernel<4>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, P.n_out, P.n_seg, P.seg_len, ws);
+        else
+            hipLaunchKernelGGL(red_row_interp_kernel<1>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, P.n_out, P.n_seg, P.seg_len, ws);
+    } else {
+        const unsigned long long blocks = (unsigned long long)P.n_bx * (unsigned)k.shape[1] * P.n_seg;
+        if (blocks >= (1ULL << 31)) return fail(NGH_E_UNSUPPORTED, "reduction grid too large");
+        hipLaunchKernelGGL(red_col_interp_kernel, dim3((unsigned)blocks), dim3(kBlock), lds, ctx->stream, k, P.n_bx, P.n_seg, P.seg_len, ws);
+    }
+    HIP_TRY(hipGetLastError());
+    if (P.n_seg > 1) {
+        const unsigned blocks = (P.n_out + kBlock - 1) / kBlock;
+        hipLaunchKernelGGL(red_finish_kernel, dim3(blocks), dim3(kBlock), 0, ctx->stream, k, P.n_out, P.n_seg,
+                           P.family == F_RED_ROW ? 1 : 0, ws);
+        HIP_TRY(hipGetLastError());
+    }
+    return NGH_OK;
+}
+
+void describe(const Plan& P, char* out, size_t n) {
+    if (P.special >= 0) {
+        snprintf(out, n, "special:%s", special_name(P.special));
+        return;
+    }
+    switch (P.family) {
+        case F_EW: snprintf(out, n, "ew_interp_v%d%s", P.V, P.tail ? "+tail" : ""); break;
+        case F_RED_ROW: snprintf(out, n, "red_row_interp_v%d_s%u", P.V, P.n_seg); break;
+        case F_RED_COL: snprintf(out, n, "red_col_interp_v1_s%u", P.n_seg); break;
+    }
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------
+extern "C" {
+
+int ngh_abi_version(void) { return NGH_ABI_VERSION; }
+
+const char* ngh_last_error(void) { return g_err; }
+
+int ngh_device_count(int* count) {
+    if (!count) return fail(NGH_E_INVALID, "count is NULL");
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) { *count = 0; return fail(NGH_E_NODEVICE, "hipGetDeviceCount: %s", hipGetErrorString(e)); }
+    *count = n;
+    return NGH_OK;
+}
+
+int ngh_init(int device_id, ngh_context** out_ctx) {
+    if (!out_ctx) return fail(NGH_E_INVALID, "out_ctx is NULL");
+    *out_ctx = nullptr;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) return fail(NGH_E_NODEVICE, "no HIP device visible");
+    if (device_id < 0 || device_id >= n) return fail(NGH_E_INVALID, "device %d not in 0..%d", device_id, n - 1);
+    HIP_TRY(hipSetDevice(device_id));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device_id));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0 && !env_int("NGH_ALLOW_ANY_ARCH", 0))
+        return fail(NGH_E_NODEVICE, "device %d is %s; this library is built for gfx950 only", device_id, prop.gcnArchName);
+    ngh_context* ctx = new ngh_context();
+    ctx->device = device_id;
+    ctx->cus = prop.multiProcessorCount;
+    ctx->total_bytes = prop.totalGlobalMem;
+    snprintf(ctx->name, sizeof(ctx->name), "%s (%s)", prop.name, prop.gcnArchName);
+    ctx->ew_blocks_per_cu = std::max(1, env_int("NGH_EW_BLOCKS_PER_CU", 8));
+    ctx->force_interp = env_int("NGH_FORCE_INTERP", 0);
+    hipError_t e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreate(&ctx->ev0);
+    if (e == hipSuccess) e = hipEventCreate(&ctx->ev1);
+    if (e != hipSuccess) {
+        delete ctx;
+        return fail(NGH_E_RUNTIME, "stream/event creation: %s", hipGetErrorString(e));
+    }
+    *out_ctx = ctx;
+    return NGH_OK;
+}
+
+int ngh_shutdown(ngh_context* ctx) {
+    if (!ctx) return NGH_OK;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->ws) (void)hipFree(ctx->ws);
+    if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
+    if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
+    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return NGH_OK;
+}
+
+int ngh_sync(ngh_context* ctx) {
+    if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return NGH_OK;
+}
+
+int ngh_device_info(ngh_context* ctx, char* name256, int* compute_units, uint64_t* total_bytes) {
+    if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
+    if (name256) { strncpy(name256, ctx->name, 255); name256[255] = 0; }
+    if (compute_units) *compute_units = ctx->cus;
+    if (total_bytes) *total_bytes = ctx->total_bytes;
+    return NGH_OK;
+}
+
+int ngh_malloc(ngh_context* ctx, size_t bytes, void** out_dev) {
+    if (!ctx || !out_dev) return fail(NGH_E_INVALID, "ngh_malloc: NULL argument");
+    *out_dev = nullptr;
+    HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(hipMalloc(out_dev, std::max<size_t>(bytes, 16)));
+    return NGH_OK;
+}
+
+int ngh_free(ngh_context* ctx, void* dev) {
+    if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
+    if (!dev) return NGH_OK;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    HIP_TRY(hipFree(dev));
+    return NGH_OK;
+}
+
+int ngh_memcpy_h2d(ngh_context* ctx, void* dev, const void* host, size_t bytes) {
+    if (!ctx || (bytes && (!dev || !host))) return fail(NGH_E_INVALID, "ngh_memcpy_h2d: NULL argument");
+    if (!bytes) return NGH_OK;
+    HIP_TRY(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, ctx->stream));
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return NGH_OK;
+}
+
+int ngh_memcpy_d2h(ngh_context* ctx, void* host, const void* dev, size_t bytes) {
+    if (!ctx || (bytes && (!dev || !host))) return fail(NGH_E_INVALID, "ngh_memcpy_d2h: NULL argument");
+    if (!bytes) return NGH_OK;
+    HIP_TRY(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return NGH_OK;
+}
+
+int ngh_memcpy_d2d(ngh_context* ctx, void* dev_dst, const void* dev_src, size_t bytes) {
+    if (!ctx || (bytes && (!dev_dst || !dev_src))) return fail(NGH_E_INVALID, "ngh_memcpy_d2d: NULL argument");
+    if (!bytes) return NGH_OK;
+    HIP_TRY(hipMemcpyAsync(dev_dst, dev_src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return NGH_OK;
+}
+
+int ngh_memset32(ngh_context* ctx, void* dev, uint32_t value, size_t count) {
+    if (!ctx || (count && !dev)) return fail(NGH_E_INVALID, "ngh_memset32: NULL argument");
+    if (!count) return NGH_OK;
+    const unsigned blocks = (unsigned)std::min<size_t>((count + kBlock - 1) / kBlock, (size_t)ctx->cus * 16);
+    hipLaunchKernelGGL(fill_kernel<uint32_t>, dim3(blocks), dim3(kBlock), 0, ctx->stream, (uint32_t*)dev, value, count);
+    HIP_TRY(hipGetLastError());
+    return NGH_OK;
+}
+
+int ngh_memset16(ngh_context* ctx, void* dev, uint16_t value, size_t count) {
+    if (!ctx || (count && !dev)) return fail(NGH_E_INVALID, "ngh_memset16: NULL argument");
+    if (!count) return NGH_OK;
+    const unsigned blocks = (unsigned)std::min<size_t>((count + kBlock - 1) / kBlock, (size_t)ctx->cus * 16);
+    hipLaunchKernelGGL(fill_kernel<uint16_t>, dim3(blocks), dim3(kBlock), 0, ctx->stream, (uint16_t*)dev, value, count);
+    HIP_TRY(hipGetLastError());
+    return NGH_OK;
+}
+
+int ngh_copy_strided(ngh_context* ctx, void* dev_dst, const void* dev_src, int32_t rank,
+                     const int64_t* shape, const int64_t* dst_strides, const int64_t* src_strides,
+                     int32_t itemsize) {
+    if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
+    if (rank < 0 || rank > kCopyMaxRank) return fail(NGH_E_INVALID, "rank %d not in 0..%d", rank, kCopyMaxRank);
+    if (itemsize != 2 && itemsize != 4) return fail(NGH_E_INVALID, "itemsize %d (2 or 4)", itemsize);
+    if (rank && (!shape || !dst_strides || !src_strides)) return fail(NGH_E_INVALID, "NULL shape/strides");
+    CopyArgs a;
+    memset(&a, 0, sizeof(a));
+    long long total = 1;
+    // drop length-1 axes, merge axes that are contiguous in both views
+    int r = 0;
+    for (int i = 0; i < rank; ++i) {
+        if (shape[i] < 0) return fail(NGH_E_INVALID, "negative shape");
+        total *= shape[i];
+        if (shape[i] == 1) continue;
+        if (r > 0 && a.ds[r - 1] == dst_strides[i] * shape[i] && a.ss[r - 1] == src_strides[i] * shape[i]) {
+            a.shape[r - 1] *= shape[i];
+            a.ds[r - 1] = dst_strides[i];
+            a.ss[r - 1] = src_strides[i];
+        } else {
+            a.shape[r] = shape[i]; a.ds[r] = dst_strides[i]; a.ss[r] = src_strides[i];
+            ++r;
+        }
+    }
+    if (total == 0) return NGH_OK;
+    if (!dev_dst || !dev_src) return fail(NGH_E_INVALID, "NULL device pointer");
+    if (total >= (1LL << 32)) return fail(NGH_E_UNSUPPORTED, "copy of %lld elements; split it", total);
+    a.rank = r;
+    a.total = (unsigned)total;
+    return launch_copy(ctx->stream, ctx->cus, dev_dst, dev_src, a, itemsize) == hipSuccess
+               ? NGH_OK
+               : fail(NGH_E_RUNTIME, "copy launch: %s", hipGetErrorString(hipGetLastError()));
+}
+
+int ngh_validate_fused(const ngh_fused_spec* spec) { return validate(spec); }
+
+int ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec) {
+    if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
+    NGH_TRY(validate(spec));
+    for (int s = 0; s < spec->n_stages; ++s) {
+        if (spec->stages[s].op_end == spec->stages[s].op_begin) continue;
+        Plan P;
+        NGH_TRY(plan_stage(ctx, *spec, s, P));
+        if (!ctx->force_interp) {
+            P.special = match_special(P.family, P.V, P.k, P.tail);
+            if (P.special >= 0) {
+                hipError_t e = launch_special(P.special, ctx->stream, ctx->cus, P.k, P.n_chunks, P.chunks_per_row);
+                if (e != hipSuccess) return fail(NGH_E_RUNTIME, "special launch: %s", hipGetErrorString(e));
+                continue;
+            }
+        }
+        NGH_TRY(launch_interp(ctx, P));
+    }
+    return NGH_OK;
+}
+
+int ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec, int32_t stage, char* name128) {
+    if (!ctx || !name128) return fail(NGH_E_INVALID, "NULL argument");
+    NGH_TRY(validate(spec));
+    if (stage < 0 || stage >= spec->n_stages) return fail(NGH_E_INVALID, "stage %d", stage);
+    Plan P;
+    NGH_TRY(plan_stage(ctx, *spec, stage, P));
+    if (!ctx->force_interp) P.special = match_special(P.family, P.V, P.k, P.tail);
+    describe(P, name128, 128);
+    return NGH_OK;
+}
+
+int ngh_stats_alloc(ngh_context* ctx, int32_t n, int32_t** out_dev) {
+    if (!ctx || !out_dev || n <= 0) return fail(NGH_E_INVALID, "ngh_stats_alloc: bad argument");
+    void* p = nullptr;
+    NGH_TRY(ngh_malloc(ctx, (size_t)n * 4, &p));
+    *out_dev = (int32_t*)p;
+    return ngh_memset32(ctx, p, 0, (size_t)n);
+}
+
+int ngh_stats_reset(ngh_context* ctx, int32_t* dev, int32_t n) {
+    if (n <= 0) return NGH_OK;
+    return ngh_memset32(ctx, dev, 0, (size_t)n);
+}
+
+int ngh_stats_read(ngh_context* ctx, const int32_t* dev, int32_t n, int32_t* host) {
+    if (n <= 0) return NGH_OK;
+    return ngh_memcpy_d2h(ctx, host, dev, (size_t)n * 4);
+}
+
+int ngh_timer_begin(ngh_context* ctx) {
+    if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
+    HIP_TRY(hipEventRecord(ctx->ev0, ctx->stream));
+    return NGH_OK;
+}
+
+int ngh_timer_end(ngh_context* ctx, float* out_ms) {
+    if (!ctx || !out_ms) return fail(NGH_E_INVALID, "NULL argument");
+    HIP_TRY(hipEventRecord(ctx->ev1, ctx->stream));
+    HIP_TRY(hipEventSynchronize(ctx->ev1));
+    HIP_TRY(hipEventElapsedTime(out_ms, ctx->ev0, ctx->ev1));
+    return NGH_OK;
+}
+
+}  // extern "C"

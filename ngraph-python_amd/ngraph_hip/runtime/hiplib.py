@@ -1,0 +1,437 @@
+"""ctypes binding of libngraph_hip.so (declared in include/ngraph_hip.h).
+
+This is the layer that stands where pycuda stands in the reference GPU
+transformer: device runtime, memory, and kernel launches
+(ngraph/transformers/gputransform.py:912-1000, 525-676, 343-345).  It holds
+no arithmetic of its own: every result comes from the HIP library, and a
+missing library is an error, never a fallback.
+"""
+from __future__ import division
+import ctypes
+import os
+
+import numpy as np
+
+NGH_ABI_VERSION = 1
+NGH_MAX_AXES = 3
+NGH_MAX_TENSORS = 12
+NGH_MAX_OPS = 96
+NGH_MAX_CONSTS = 16
+NGH_MAX_REGS = 32
+NGH_MAX_REDUCTIONS = 4
+NGH_MAX_STAGES = 6
+
+NGH_F32, NGH_FLEX16, NGH_I32, NGH_F16 = 0, 1, 2, 3
+
+_OPCODE_NAMES = [
+    "nop", "load", "store", "const", "iota",
+    "assign", "neg", "abs", "sqrt", "sqr", "exp", "log", "rcp", "exp2", "log2", "sig", "tanh",
+    "safelog", "sgn", "sin", "cos",
+    "add", "sub", "mul", "div", "int_div", "mod", "eq", "ne", "lt", "le", "gt", "ge",
+    "pow", "minimum", "maximum",
+    "sum", "prod", "max", "min", "argmax", "argmin",
+]
+#: op name (the reference's template names, float_ew2.py:31-77) -> opcode
+OPCODES = {name: i for i, name in enumerate(_OPCODE_NAMES)}
+UNARY_OPS = _OPCODE_NAMES[OPCODES["assign"]:OPCODES["cos"] + 1]
+BINARY_OPS = _OPCODE_NAMES[OPCODES["add"]:OPCODES["maximum"] + 1]
+REDUCTION_OPS = _OPCODE_NAMES[OPCODES["sum"]:OPCODES["argmin"] + 1]
+
+
+class ngh_op(ctypes.Structure):
+    _fields_ = [("opcode", ctypes.c_uint8), ("dst", ctypes.c_uint8),
+                ("a", ctypes.c_uint8), ("b", ctypes.c_uint8)]
+
+
+class ngh_tensor(ctypes.Structure):
+    _fields_ = [("dev", ctypes.c_void_p),
+                ("strides", ctypes.c_int64 * NGH_MAX_AXES),
+                ("dtype", ctypes.c_int32),
+                ("scale", ctypes.c_float),
+                ("dev_stats", ctypes.c_void_p),
+                ("dev_scale", ctypes.c_void_p)]
+
+
+class ngh_stage(ctypes.Structure):
+    _fields_ = [("op_begin", ctypes.c_int32), ("op_end", ctypes.c_int32),
+                ("n_reductions", ctypes.c_int32),
+                ("red_out", ctypes.c_int32 * NGH_MAX_REDUCTIONS)]
+
+
+class ngh_fused_spec(ctypes.Structure):
+    _fields_ = [("abi_version", ctypes.c_int32),
+                ("rank", ctypes.c_int32),
+                ("shape", ctypes.c_int64 * NGH_MAX_AXES),
+                ("n_tensors", ctypes.c_int32), ("n_ops", ctypes.c_int32),
+                ("n_consts", ctypes.c_int32), ("n_stages", ctypes.c_int32),
+                ("n_regs", ctypes.c_int32),
+                ("tensors", ngh_tensor * NGH_MAX_TENSORS),
+                ("consts", ctypes.c_float * NGH_MAX_CONSTS),
+                ("ops", ngh_op * NGH_MAX_OPS),
+                ("stages", ngh_stage * NGH_MAX_STAGES)]
+
+
+class HipLibraryError(RuntimeError):
+    """A call into libngraph_hip.so failed; carries the library's message."""
+
+    def __init__(self, code, message):
+        super(HipLibraryError, self).__init__("libngraph_hip error %d: %s" % (code, message))
+        self.code = code
+
+
+#: every symbol include/ngraph_hip.h declares: name -> (argtypes)
+_vp, _i32, _i64p = ctypes.c_void_p, ctypes.c_int32, ctypes.POINTER(ctypes.c_int64)
+_SYMBOLS = {
+    "ngh_abi_version": [],
+    "ngh_last_error": [],
+    "ngh_device_count": [ctypes.POINTER(ctypes.c_int)],
+    "ngh_init": [ctypes.c_int, ctypes.POINTER(_vp)],
+    "ngh_shutdown": [_vp],
+    "ngh_sync": [_vp],
+    "ngh_device_info": [_vp, ctypes.c_char_p, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_uint64)],
+    "ngh_malloc": [_vp, ctypes.c_size_t, ctypes.POINTER(_vp)],
+    "ngh_free": [_vp, _vp],
+    "ngh_memcpy_h2d": [_vp, _vp, _vp, ctypes.c_size_t],
+    "ngh_memcpy_d2h": [_vp, _vp, _vp, ctypes.c_size_t],
+    "ngh_memcpy_d2d": [_vp, _vp, _vp, ctypes.c_size_t],
+    "ngh_memset32": [_vp, _vp, ctypes.c_uint32, ctypes.c_size_t],
+    "ngh_memset16": [_vp, _vp, ctypes.c_uint16, ctypes.c_size_t],
+    "ngh_copy_strided": [_vp, _vp, _vp, _i32, _i64p, _i64p, _i64p, _i32],
+    "ngh_validate_fused": [ctypes.POINTER(ngh_fused_spec)],
+    "ngh_launch_fused": [_vp, ctypes.POINTER(ngh_fused_spec)],
+    "ngh_describe_fused": [_vp, ctypes.POINTER(ngh_fused_spec), _i32, ctypes.c_char_p],
+    "ngh_stats_alloc": [_vp, _i32, ctypes.POINTER(_vp)],
+    "ngh_stats_reset": [_vp, _vp, _i32],
+    "ngh_stats_read": [_vp, _vp, _i32, _vp],
+    "ngh_timer_begin": [_vp],
+    "ngh_timer_end": [_vp, ctypes.POINTER(ctypes.c_float)],
+}
+
+_lib = None
+
+
+def library_path():
+    return os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                        "lib", "libngraph_hip.so")
+
+
+def load_library():
+    """Open libngraph_hip.so and type every entry point.  Raises if absent."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = library_path()
+    if not os.path.exists(path):
+        raise HipLibraryError(-5, "%s is not built (run ngraph-python_amd/build_ext.py)" % path)
+    lib = ctypes.CDLL(path)
+    for name, argtypes in _SYMBOLS.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = ctypes.c_char_p if name == "ngh_last_error" else ctypes.c_int
+    if lib.ngh_abi_version() != NGH_ABI_VERSION:
+        raise HipLibraryError(-1, "ABI version mismatch: library %d, binding %d"
+                              % (lib.ngh_abi_version(), NGH_ABI_VERSION))
+    _lib = lib
+    return lib
+
+
+def exported_symbols():
+    return sorted(_SYMBOLS)
+
+
+def _check(lib, rc):
+    if rc != 0:
+        msg = lib.ngh_last_error()
+        raise HipLibraryError(rc, msg.decode("utf-8", "replace") if msg else "")
+
+
+_NP_DTYPES = {NGH_F32: np.float32, NGH_FLEX16: np.int16, NGH_I32: np.int32, NGH_F16: np.float16}
+
+
+class DeviceArray(object):
+    """A contiguous device allocation with a shape and a storage type."""
+
+    def __init__(self, runtime, shape, ngh_dtype=NGH_F32):
+        self.runtime = runtime
+        self.shape = tuple(int(s) for s in shape)
+        self.ngh_dtype = ngh_dtype
+        self.np_dtype = np.dtype(_NP_DTYPES[ngh_dtype])
+        self.size = int(np.prod(self.shape, dtype=np.int64)) if self.shape else 1
+        self.nbytes = self.size * self.np_dtype.itemsize
+        self.ptr = runtime.malloc(self.nbytes)
+
+    def set(self, host):
+        host = np.ascontiguousarray(host, dtype=self.np_dtype)
+        if host.size != self.size:
+            raise ValueError("size mismatch: %d vs %d" % (host.size, self.size))
+        self.runtime.memcpy_h2d(self.ptr, host)
+        return self
+
+    def get(self):
+        out = np.empty(self.shape, dtype=self.np_dtype)
+        self.runtime.memcpy_d2h(out, self.ptr)
+        return out
+
+    def free(self):
+        if self.ptr:
+            self.runtime.free(self.ptr)
+            self.ptr = None
+
+
+class HipRuntime(object):
+    """One device context: stream, allocations, launches."""
+
+    def __init__(self, device_id=0):
+        self.lib = load_library()
+        ctx = ctypes.c_void_p()
+        _check(self.lib, self.lib.ngh_init(int(device_id), ctypes.byref(ctx)))
+        self.ctx = ctx
+        self._allocs = set()
+
+    # -- lifetime --------------------------------------------------------
+    def close(self):
+        if getattr(self, "ctx", None):
+            for ptr in list(self._allocs):
+                self.lib.ngh_free(self.ctx, ctypes.c_void_p(ptr))
+            self._allocs.clear()
+            self.lib.ngh_shutdown(self.ctx)
+            self.ctx = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def device_info(self):
+        name = ctypes.create_string_buffer(256)
+        cus = ctypes.c_int()
+        total = ctypes.c_uint64()
+        _check(self.lib, self.lib.ngh_device_info(self.ctx, name, ctypes.byref(cus), ctypes.byref(total)))
+        return name.value.decode(), cus.value, total.value
+
+    def sync(self):
+        _check(self.lib, self.lib.ngh_sync(self.ctx))
+
+    # -- memory ----------------------------------------------------------
+    def malloc(self, nbytes):
+        ptr = ctypes.c_void_p()
+        _check(self.lib, self.lib.ngh_malloc(self.ctx, int(nbytes), ctypes.byref(ptr)))
+        self._allocs.add(ptr.value)
+        return ptr.value
+
+    def free(self, ptr):
+        if ptr in self._allocs:
+            self._allocs.discard(ptr)
+            _check(self.lib, self.lib.ngh_free(self.ctx, ctypes.c_void_p(ptr)))
+
+    def memcpy_h2d(self, dev, host):
+        host = np.ascontiguousarray(host)
+        _check(self.lib, self.lib.ngh_memcpy_h2d(self.ctx, ctypes.c_void_p(dev),
+                                                 host.ctypes.data_as(ctypes.c_void_p), host.nbytes))
+
+    def memcpy_d2h(self, host, dev):
+        assert host.flags.c_contiguous
+        _check(self.lib, self.lib.ngh_memcpy_d2h(self.ctx, host.ctypes.data_as(ctypes.c_void_p),
+                                                 ctypes.c_void_p(dev), host.nbytes))
+
+    def memcpy_d2d(self, dst, src, nbytes):
+        _check(self.lib, self.lib.ngh_memcpy_d2d(self.ctx, ctypes.c_void_p(dst), ctypes.c_void_p(src), int(nbytes)))
+
+    def memset32(self, dev, value, count):
+        _check(self.lib, self.lib.ngh_memset32(self.ctx, ctypes.c_void_p(dev), int(value) & 0xffffffff, int(count)))
+
+    def memset16(self, dev, value, count):
+        _check(self.lib, self.lib.ngh_memset16(self.ctx, ctypes.c_void_p(dev), int(value) & 0xffff, int(count)))
+
+    def fill_f32(self, dev, value, count):
+        self.memset32(dev, int(np.float32(value).view(np.uint32)), count)
+
+    def empty(self, shape, ngh_dtype=NGH_F32):
+        return DeviceArray(self, shape, ngh_dtype)
+
+    def array(self, host, ngh_dtype=None):
+        host = np.asarray(host)
+        if ngh_dtype is None:
+            ngh_dtype = {np.dtype(np.float32): NGH_F32, np.dtype(np.int16): NGH_FLEX16,
+                         np.dtype(np.int32): NGH_I32, np.dtype(np.float16): NGH_F16}[host.dtype]
+        return DeviceArray(self, host.shape, ngh_dtype).set(host)
+
+    def copy_strided(self, dst, src, shape, dst_strides, src_strides, itemsize):
+        n = len(shape)
+        arr = ctypes.c_int64 * max(n, 1)
+        _check(self.lib, self.lib.ngh_copy_strided(
+            self.ctx, ctypes.c_void_p(dst), ctypes.c_void_p(src), n,
+            arr(*[int(s) for s in shape]), arr(*[int(s) for s in dst_strides]),
+            arr(*[int(s) for s in src_strides]), int(itemsize)))
+
+    # -- fused kernels ---------------------------------------------------
+    def validate_fused(self, spec):
+        _check(self.lib, self.lib.ngh_validate_fused(ctypes.byref(spec)))
+
+    def launch_fused(self, spec):
+        _check(self.lib, self.lib.ngh_launch_fused(self.ctx, ctypes.byref(spec)))
+
+    def describe_fused(self, spec, stage=0):
+        name = ctypes.create_string_buffer(128)
+        _check(self.lib, self.lib.ngh_describe_fused(self.ctx, ctypes.byref(spec), int(stage), name))
+        return name.value.decode()
+
+    # -- flex statistics ---------------------------------------------------
+    def stats_alloc(self, n):
+        ptr = ctypes.c_void_p()
+        _check(self.lib, self.lib.ngh_stats_alloc(self.ctx, int(n), ctypes.byref(ptr)))
+        self._allocs.add(ptr.value)
+        return ptr.value
+
+    def stats_reset(self, dev, n=1):
+        _check(self.lib, self.lib.ngh_stats_reset(self.ctx, ctypes.c_void_p(dev), int(n)))
+
+    def stats_read(self, dev, n=1):
+        out = np.zeros(n, dtype=np.int32)
+        _check(self.lib, self.lib.ngh_stats_read(self.ctx, ctypes.c_void_p(dev), int(n),
+                                                 out.ctypes.data_as(ctypes.c_void_p)))
+        return out
+
+    # -- timing ------------------------------------------------------------
+    def timer_begin(self):
+        _check(self.lib, self.lib.ngh_timer_begin(self.ctx))
+
+    def timer_end(self):
+        ms = ctypes.c_float()
+        _check(self.lib, self.lib.ngh_timer_end(self.ctx, ctypes.byref(ms)))
+        return ms.value
+
+
+class FusedSpecBuilder(object):
+    """Assembles an ngh_fused_spec: tensors, constants, ops, stages.
+
+    The op vocabulary is the reference's (name, x, y, out, axis) tuples
+    (gputransform.py:277-289) flattened into explicit load / compute /
+    store steps on numbered registers.
+    """
+
+    def __init__(self, shape):
+        shape = [int(s) for s in shape]
+        if not 1 <= len(shape) <= NGH_MAX_AXES:
+            raise ValueError("fused kernels take 1..3 axes, got %d" % len(shape))
+        self.rank = len(shape)
+        self.shape = shape + [1] * (NGH_MAX_AXES - len(shape))
+        self.tensors = []
+        self.consts = []
+        self.ops = []
+        self.stages = []
+        self._stage_begin = 0
+        self._stage_reds = []
+        self.n_regs = 0
+
+    def _pad_strides(self, strides):
+        strides = [int(s) for s in strides]
+        if len(strides) != self.rank:
+            raise ValueError("strides %r do not match rank %d" % (strides, self.rank))
+        return strides + [0] * (NGH_MAX_AXES - len(strides))
+
+    def tensor(self, dev, strides, dtype=NGH_F32, scale=1.0, dev_stats=None, dev_scale=None):
+        if len(self.tensors) >= NGH_MAX_TENSORS:
+            raise ValueError("too many tensors in one fused kernel")
+        self.tensors.append((int(dev), self._pad_strides(strides), int(dtype), float(scale),
+                             dev_stats, dev_scale))
+        return len(self.tensors) - 1
+
+    def const(self, value):
+        value = float(np.float32(value))
+        for i, c in enumerate(self.consts):
+            if c == value and (c != 0 or np.signbit(c) == np.signbit(value)):
+                return i
+        if len(self.consts) >= NGH_MAX_CONSTS:
+            raise ValueError("too many constants in one fused kernel")
+        self.consts.append(value)
+        return len(self.consts) - 1
+
+    def reg(self):
+        self.n_regs += 1
+        if self.n_regs > NGH_MAX_REGS:
+            raise ValueError("too many registers in one fused kernel")
+        return self.n_regs - 1
+
+    def emit(self, name, dst=0, a=0, b=0):
+        if len(self.ops) >= NGH_MAX_OPS:
+            raise ValueError("too many ops in one fused kernel")
+        self.ops.append((OPCODES[name], int(dst), int(a), int(b)))
+
+    # convenience wrappers returning the destination register
+    def load(self, t, dst=None):
+        dst = self.reg() if dst is None else dst
+        self.emit("load", dst, t)
+        return dst
+
+    def store(self, t, r):
+        self.emit("store", t, r)
+
+    def constant(self, value, dst=None):
+        dst = self.reg() if dst is None else dst
+        self.emit("const", dst, self.const(value))
+        return dst
+
+    def iota(self, axis, dst=None):
+        dst = self.reg() if dst is None else dst
+        self.emit("iota", dst, axis)
+        return dst
+
+    def unary(self, name, a, dst=None):
+        dst = self.reg() if dst is None else dst
+        self.emit(name, dst, a)
+        return dst
+
+    def binary(self, name, a, b, dst=None):
+        dst = self.reg() if dst is None else dst
+        self.emit(name, dst, a, b)
+        return dst
+
+    def reduce(self, name, a, out_tensor):
+        slot = len(self._stage_reds)
+        if slot >= NGH_MAX_REDUCTIONS:
+            raise ValueError("too many reductions in one stage")
+        self.emit(name, slot, a)
+        self._stage_reds.append(out_tensor)
+
+    def end_stage(self):
+        self.stages.append((self._stage_begin, len(self.ops), list(self._stage_reds)))
+        self._stage_begin = len(self.ops)
+        self._stage_reds = []
+
+    def build(self):
+        if self._stage_begin != len(self.ops) or not self.stages:
+            self.end_stage()
+        if len(self.stages) > NGH_MAX_STAGES:
+            raise ValueError("too many stages in one fused kernel")
+        spec = ngh_fused_spec()
+        spec.abi_version = NGH_ABI_VERSION
+        spec.rank = self.rank
+        for i in range(NGH_MAX_AXES):
+            spec.shape[i] = self.shape[i]
+        spec.n_tensors = len(self.tensors)
+        spec.n_ops = len(self.ops)
+        spec.n_consts = len(self.consts)
+        spec.n_stages = len(self.stages)
+        spec.n_regs = self.n_regs
+        for i, (dev, strides, dtype, scale, stats, dscale) in enumerate(self.tensors):
+            t = spec.tensors[i]
+            t.dev = dev
+            for j in range(NGH_MAX_AXES):
+                t.strides[j] = strides[j]
+            t.dtype = dtype
+            t.scale = scale
+            t.dev_stats = stats
+            t.dev_scale = dscale
+        for i, c in enumerate(self.consts):
+            spec.consts[i] = c
+        for i, (opc, dst, a, b) in enumerate(self.ops):
+            o = spec.ops[i]
+            o.opcode, o.dst, o.a, o.b = opc, dst, a, b
+        for i, (b, e, reds) in enumerate(self.stages):
+            s = spec.stages[i]
+            s.op_begin, s.op_end, s.n_reductions = b, e, len(reds)
+            for j, t in enumerate(reds):
+                s.red_out[j] = t
+        return spec

@@ -1,0 +1,326 @@
+"""Parity of the fused kernels, driven through the C ABI with hand-built specs.
+
+Each case builds an ngh_fused_spec the way the transformer's lowering does,
+launches it with ngh_launch_fused and compares with the CPU oracle
+(oracle/configs.py, oracle/numpy_ops.py) on the same seeded inputs.
+Tolerance: fp32 rtol 1e-5 / atol 1e-6 (the bar BASELINE.json states).
+"""
+import numpy as np
+import pytest
+
+from oracle import configs, numpy_ops
+from ngraph_hip.runtime import FusedSpecBuilder, NGH_F32, NGH_I32
+from ngraph_hip.runtime.hiplib import UNARY_OPS, BINARY_OPS
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-5, 1e-6
+f32 = np.float32
+
+
+def contiguous_strides(shape):
+    strides, acc = [], 1
+    for s in reversed(shape):
+        strides.insert(0, acc)
+        acc *= s
+    return strides
+
+
+def c1_spec(rt, x_d, a_d, b_d, y_d, shape):
+    st = contiguous_strides(shape)
+    z = [0] * len(shape)
+    sb = FusedSpecBuilder(shape)
+    tx, ta, tb, ty = (sb.tensor(x_d.ptr, st), sb.tensor(a_d.ptr, z), sb.tensor(b_d.ptr, z),
+                      sb.tensor(y_d.ptr, st))
+    x = sb.load(tx)
+    a = sb.load(ta)
+    b = sb.load(tb)
+    t = sb.binary("mul", a, x)
+    t = sb.binary("add", t, b)
+    t = sb.unary("tanh", t)
+    u = sb.unary("neg", x)
+    u = sb.unary("exp", u)
+    one = sb.constant(1.0)
+    u = sb.binary("add", u, one)
+    u = sb.unary("rcp", u)
+    y = sb.binary("mul", t, u)
+    sb.store(ty, y)
+    return sb.build()
+
+
+@pytest.mark.parametrize("shape", [(1024, 1024), (7, 33), (1, 5), (3, 4, 5), (1000003,)])
+def test_c1_tanh_sigmoid_chain(hip_runtime, shape):
+    rt = hip_runtime
+    x, a, b = configs.c1_inputs(shape, seed=0)
+    want = configs.c1_cpu(x, a, b)
+    x_d, a_d, b_d = rt.array(x), rt.array(np.array([a])), rt.array(np.array([b]))
+    y_d = rt.empty(shape)
+    spec = c1_spec(rt, x_d, a_d, b_d, y_d, shape)
+    rt.launch_fused(spec)
+    got = y_d.get()
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+    for d in (x_d, a_d, b_d, y_d):
+        d.free()
+
+
+def bn_specs(rt, x_d, g_d, b_d, y_d, mean_d, var_d, C, R, eps):
+    """Reference-faithful staging: sum -> mean, sum((x-mean)^2) -> var, normalise.
+
+    View is [R, C] with the reduced axis first (gputransform.py:117-122);
+    memory is [C, R] so strides are (1, R).
+    """
+    xs, cs = [1, R], [0, 1]
+    sb = FusedSpecBuilder([R, C])
+    tx = sb.tensor(x_d.ptr, xs)
+    tmean = sb.tensor(mean_d.ptr, cs)
+    x = sb.load(tx)
+    sb.reduce("sum", x, tmean)
+    s1 = sb.build()
+
+    sb = FusedSpecBuilder([C])
+    tmean = sb.tensor(mean_d.ptr, [1])
+    m = sb.load(tmean)
+    n = sb.constant(R)
+    m = sb.binary("div", m, n)
+    sb.store(tmean, m)
+    s2 = sb.build()
+
+    sb = FusedSpecBuilder([R, C])
+    tx = sb.tensor(x_d.ptr, xs)
+    tmean = sb.tensor(mean_d.ptr, cs)
+    tvar = sb.tensor(var_d.ptr, cs)
+    x = sb.load(tx)
+    m = sb.load(tmean)
+    d = sb.binary("sub", x, m)
+    d = sb.unary("sqr", d)
+    sb.reduce("sum", d, tvar)
+    s3 = sb.build()
+
+    sb = FusedSpecBuilder([C])
+    tvar = sb.tensor(var_d.ptr, [1])
+    v = sb.load(tvar)
+    n = sb.constant(R)
+    v = sb.binary("div", v, n)
+    sb.store(tvar, v)
+    s4 = sb.build()
+
+    sb = FusedSpecBuilder([R, C])
+    tx = sb.tensor(x_d.ptr, xs)
+    tmean = sb.tensor(mean_d.ptr, cs)
+    tvar = sb.tensor(var_d.ptr, cs)
+    tg = sb.tensor(g_d.ptr, cs)
+    tb = sb.tensor(b_d.ptr, cs)
+    ty = sb.tensor(y_d.ptr, xs)
+    x = sb.load(tx)
+    m = sb.load(tmean)
+    v = sb.load(tvar)
+    d = sb.binary("sub", x, m)
+    e = sb.constant(eps)
+    r = sb.binary("add", v, e)
+    r = sb.unary("sqrt", r)
+    r = sb.unary("rcp", r)
+    d = sb.binary("mul", d, r)
+    g = sb.load(tg)
+    d = sb.binary("mul", g, d)
+    bb = sb.load(tb)
+    d = sb.binary("add", d, bb)
+    sb.store(ty, d)
+    s5 = sb.build()
+    return [s1, s2, s3, s4, s5]
+
+
+@pytest.mark.parametrize("C,R", [(16, 4096), (3, 1000), (256, 56 * 56), (5, 17)])
+def test_c2_batchnorm_staged(hip_runtime, C, R):
+    rt = hip_runtime
+    x, gamma, beta = configs.c2_inputs(C, R, seed=1)
+    y_w, mean_w, var_w = configs.c2_cpu(x, gamma, beta)
+    x_d, g_d, b_d = rt.array(x), rt.array(gamma), rt.array(beta)
+    y_d, mean_d, var_d = rt.empty((C, R)), rt.empty((C,)), rt.empty((C,))
+    for spec in bn_specs(rt, x_d, g_d, b_d, y_d, mean_d, var_d, C, R, 1e-5):
+        rt.launch_fused(spec)
+    np.testing.assert_allclose(mean_d.get(), mean_w, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(var_d.get(), var_w, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(y_d.get(), y_w, rtol=RTOL, atol=1e-5)
+    for d in (x_d, g_d, b_d, y_d, mean_d, var_d):
+        d.free()
+
+
+def adam_spec(rt, p_d, g_d, m_d, v_d, n, ell, beta1, beta2, eps):
+    sb = FusedSpecBuilder([n])
+    tp, tg, tm, tv = (sb.tensor(d.ptr, [1]) for d in (p_d, g_d, m_d, v_d))
+    b1, b2 = f32(beta1), f32(beta2)
+    g = sb.load(tg)
+    m = sb.load(tm)
+    a = sb.binary("mul", m, sb.constant(b1))
+    b = sb.binary("mul", sb.constant(f32(1) - b1), g)
+    m = sb.binary("add", a, b)
+    sb.store(tm, m)
+    v = sb.load(tv)
+    a = sb.binary("mul", v, sb.constant(b2))
+    b = sb.binary("mul", sb.constant(f32(1) - b2), g)
+    b = sb.binary("mul", b, g)
+    v = sb.binary("add", a, b)
+    sb.store(tv, v)
+    a = sb.binary("mul", sb.constant(ell), m)
+    b = sb.unary("sqrt", v)
+    b = sb.binary("add", b, sb.constant(eps))
+    a = sb.binary("div", a, b)
+    p = sb.load(tp)
+    p = sb.binary("sub", p, a)
+    sb.store(tp, p)
+    return sb.build()
+
+
+@pytest.mark.parametrize("n", [1 << 20, 1000003, 13])
+def test_c3_adam_in_place(hip_runtime, n):
+    rt = hip_runtime
+    p, g, m, v = configs.c3_inputs(n, seed=2)
+    p_d, g_d, m_d, v_d = rt.array(p), rt.array(g), rt.array(m), rt.array(v)
+    for t in (1, 2):
+        configs.c3_cpu(p, g, m, v, t)
+        rt.launch_fused(adam_spec(rt, p_d, g_d, m_d, v_d, n, configs.adam_ell(t), 0.9, 0.999, 1e-8))
+    np.testing.assert_allclose(m_d.get(), m, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(v_d.get(), v, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(p_d.get(), p, rtol=RTOL, atol=ATOL)
+    for d in (p_d, g_d, m_d, v_d):
+        d.free()
+
+
+def lstm_specs(rt, gates_d, cprev_d, c_d, h_d, db_d, H, N):
+    # logical [H, N] views of the transposed storage: strides (1, 4H) / (1, H)
+    gs, cs, os_ = [1, 4 * H], [1, H], [N, 1]
+    sb = FusedSpecBuilder([H, N])
+    itemsize = 4
+    tg = [sb.tensor(gates_d.ptr + k * H * itemsize, gs) for k in range(4)]
+    tc_prev = sb.tensor(cprev_d.ptr, cs)
+    tc = sb.tensor(c_d.ptr, os_)
+    th = sb.tensor(h_d.ptr, os_)
+
+    def sigmoid(r):
+        r = sb.unary("neg", r)
+        r = sb.unary("exp", r)
+        r = sb.binary("add", r, sb.constant(1.0))
+        return sb.unary("rcp", r)
+
+    i = sigmoid(sb.load(tg[0]))
+    f = sigmoid(sb.load(tg[1]))
+    o = sigmoid(sb.load(tg[2]))
+    g = sb.unary("tanh", sb.load(tg[3]))
+    c = sb.binary("mul", f, sb.load(tc_prev))
+    ig = sb.binary("mul", i, g)
+    c = sb.binary("add", c, ig)
+    sb.store(tc, c)
+    tc_act = sb.unary("tanh", c)
+    h = sb.binary("mul", o, tc_act)
+    sb.store(th, h)
+    s1 = sb.build()
+
+    # db = sum over N of gates: view [N, 4H] with the reduced axis first
+    sb = FusedSpecBuilder([N, 4 * H])
+    tg_all = sb.tensor(gates_d.ptr, [4 * H, 1])
+    tdb = sb.tensor(db_d.ptr, [0, 1])
+    sb.reduce("sum", sb.load(tg_all), tdb)
+    s2 = sb.build()
+    return [s1, s2]
+
+
+@pytest.mark.parametrize("H,N", [(1024, 64), (96, 7), (64, 64)])
+def test_c4_lstm_cell_transposed(hip_runtime, H, N):
+    rt = hip_runtime
+    gates, cprev = configs.c4_inputs(H, N, seed=3)
+    c_w, h_w, db_w = configs.c4_cpu(gates, cprev)
+    gates_d, cprev_d = rt.array(gates), rt.array(cprev)
+    c_d, h_d, db_d = rt.empty((H, N)), rt.empty((H, N)), rt.empty((4 * H,))
+    for spec in lstm_specs(rt, gates_d, cprev_d, c_d, h_d, db_d, H, N):
+        rt.launch_fused(spec)
+    np.testing.assert_allclose(c_d.get(), c_w, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(h_d.get(), h_w, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(db_d.get(), db_w, rtol=RTOL, atol=1e-5)
+    for d in (gates_d, cprev_d, c_d, h_d, db_d):
+        d.free()
+
+
+@pytest.mark.parametrize("name", [n for n in UNARY_OPS])
+def test_every_unary_op(hip_runtime, name):
+    rt = hip_runtime
+    rs = np.random.RandomState(11)
+    x = rs.normal(0, 2, 4099).astype(f32)
+    if name in ("sqrt", "log", "log2", "safelog"):
+        x = np.abs(x) + f32(1e-3)
+        if name == "safelog":
+            x[::7] = 0
+            x[1::7] = -1
+    x[:3] = [0.0, 1.0, -1.0] if name not in ("sqrt", "log", "log2") else [1.0, 2.0, 0.5]
+    want = numpy_ops.unary(name, x)
+    x_d, y_d = rt.array(x), rt.empty(x.shape)
+    sb = FusedSpecBuilder(x.shape)
+    tx, ty = sb.tensor(x_d.ptr, [1]), sb.tensor(y_d.ptr, [1])
+    sb.store(ty, sb.unary(name, sb.load(tx)))
+    rt.launch_fused(sb.build())
+    got = y_d.get()
+    # transcendental results may differ from NumPy's by a couple of ulp
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL)
+    x_d.free()
+    y_d.free()
+
+
+@pytest.mark.parametrize("name", [n for n in BINARY_OPS])
+def test_every_binary_op(hip_runtime, name):
+    rt = hip_runtime
+    rs = np.random.RandomState(12)
+    x = rs.normal(0, 3, (37, 129)).astype(f32)
+    y = rs.normal(0, 3, (37, 129)).astype(f32)
+    if name in ("eq", "ne", "le", "ge"):
+        y[::3] = x[::3]
+    if name in ("int_div", "mod"):
+        x = np.round(x * 3).astype(f32)
+        y = np.round(y).astype(f32)
+        y[y == 0] = 2
+    if name == "pow":
+        x = np.abs(x) + f32(0.1)
+    want = numpy_ops.binary(name, x, y)
+    x_d, y_d, z_d = rt.array(x), rt.array(y), rt.empty(x.shape)
+    sb = FusedSpecBuilder(x.shape)
+    st = contiguous_strides(x.shape)
+    tx, ty, tz = sb.tensor(x_d.ptr, st), sb.tensor(y_d.ptr, st), sb.tensor(z_d.ptr, st)
+    sb.store(tz, sb.binary(name, sb.load(tx), sb.load(ty)))
+    rt.launch_fused(sb.build())
+    np.testing.assert_allclose(z_d.get(), want, rtol=RTOL, atol=ATOL)
+    for d in (x_d, y_d, z_d):
+        d.free()
+
+
+@pytest.mark.parametrize("name", ["sum", "prod", "max", "min", "argmax", "argmin"])
+@pytest.mark.parametrize("shape,layout", [((64, 10), "row"), ((64, 10), "col"), ((5000, 3), "row"),
+                                          ((300, 700), "col"), ((1, 9), "row"), ((40000, 2), "col")])
+def test_every_reduction(hip_runtime, name, shape, layout):
+    """Reduce axis 0 of an [R, A] view; 'row' = R contiguous in memory, 'col' = A contiguous."""
+    rt = hip_runtime
+    R, A = shape
+    rs = np.random.RandomState(13)
+    scale = 0.05 if name == "prod" else 1.0
+    logical = (1.0 + rs.normal(0, scale, (R, A))).astype(f32) if name == "prod" else \
+        rs.normal(0, 1, (R, A)).astype(f32)
+    if name in ("argmax", "argmin", "max", "min") and R > 3:
+        logical[R // 2] = logical[R // 3]           # ties: lowest index must win
+    want = numpy_ops.reduce(name, logical, 0)
+    if layout == "row":
+        store, strides = np.ascontiguousarray(logical.T), [1, R]
+    else:
+        store, strides = logical, [A, 1]
+    x_d = rt.array(store)
+    is_arg = name.startswith("arg")
+    out_d = rt.empty((A,), NGH_I32 if is_arg else NGH_F32)
+    sb = FusedSpecBuilder([R, A])
+    tx = sb.tensor(x_d.ptr, strides)
+    to = sb.tensor(out_d.ptr, [0, 1], NGH_I32 if is_arg else NGH_F32)
+    sb.reduce(name, sb.load(tx), to)
+    spec = sb.build()
+    rt.launch_fused(spec)
+    got = out_d.get()
+    if is_arg:
+        np.testing.assert_array_equal(got, want)
+    else:
+        np.testing.assert_allclose(got, want, rtol=1e-5 if name != "prod" else 1e-4, atol=1e-5)
+    x_d.free()
+    out_d.free()
