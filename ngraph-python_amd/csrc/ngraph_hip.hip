@@ -253,13 +253,20 @@ int plan_stage(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan
     if (total >= (1LL << 31) * 4LL) return fail(NGH_E_UNSUPPORTED, "stage view of %lld elements exceeds 2^33", total);
 
     if (S.n_reductions == 0) {
-        // fast axis = the one most operands are contiguous along; stores count double
-        int best = -1, best_score = -1;
+        // fast axis = the one along which most memory traffic is contiguous: every
+        // operand votes with the number of distinct elements it touches (stores twice)
+        int best = -1;
+        double best_score = -1.0;
         for (int a = NGH_MAX_AXES - 1; a >= 0; --a) {
             if (sp.shape[a] <= 1) continue;
-            int score = 0;
-            for (int t = 0; t < sp.n_tensors; ++t)
-                if (used[t] && sp.tensors[t].strides[a] == 1) score += stores[t] ? 2 : 1;
+            double score = 0.0;
+            for (int t = 0; t < sp.n_tensors; ++t) {
+                if (!used[t] || sp.tensors[t].strides[a] != 1) continue;
+                double elems = 1.0;
+                for (int b = 0; b < NGH_MAX_AXES; ++b)
+                    if (sp.tensors[t].strides[b] != 0) elems *= (double)sp.shape[b];
+                score += elems * itemsize_of(sp.tensors[t].dtype) * ((loads[t] ? 1 : 0) + (stores[t] ? 1 : 0));
+            }
             if (score > best_score) { best_score = score; best = a; }
         }
         if (best < 0) best = 2;
@@ -346,6 +353,9 @@ int plan_stage(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan
     return NGH_OK;
 }
 
+constexpr size_t kInterpLdsPreferred = 64 * 1024;   // keeps >= 2 workgroups per CU
+constexpr size_t kInterpLdsMax = 128 * 1024;
+
 size_t interp_lds_bytes(const KArgs& k, int V) {
     return ((size_t)k.n_regs * V + k.n_stat_slots + 2 * k.n_red) * kBlock * sizeof(float);
 }
@@ -365,18 +375,25 @@ int ensure_ws(ngh_context* ctx, size_t bytes) {
 }
 
 int launch_interp(ngh_context* ctx, Plan& P) {
-    const KArgs& k = P.k;
     int V = P.V;
-    size_t lds = interp_lds_bytes(k, V);
-    if (lds > 64 * 1024 && V == 4 && P.family == F_EW && P.tail == 0) {
+    size_t lds = interp_lds_bytes(P.k, V);
+    if (lds > kInterpLdsPreferred && V == 4 && P.family == F_EW) {
         // too many live registers for a 4-wide file: fall back to one element per lane
-        V = 1;
-        P.V = 1;
-        P.chunks_per_row *= 4;
-        P.n_chunks *= 4;
-        lds = interp_lds_bytes(k, 1);
+        Plan Q = P;
+        Q.V = 1;
+        Q.k.shape[2] += Q.tail;
+        Q.tail = 0;
+        Q.chunks_per_row = (unsigned)Q.k.shape[2];
+        const long long chunks = Q.k.shape[0] * Q.k.shape[1] * Q.k.shape[2];
+        if (chunks < (1LL << 32)) {
+            Q.n_chunks = (unsigned)chunks;
+            P = Q;
+            V = 1;
+            lds = interp_lds_bytes(P.k, 1);
+        }
     }
-    if (lds > 64 * 1024) return fail(NGH_E_UNSUPPORTED, "program needs %zu bytes of LDS registers", lds);
+    if (lds > kInterpLdsMax) return fail(NGH_E_UNSUPPORTED, "program needs %zu bytes of LDS registers", lds);
+    const KArgs& k = P.k;
     if (P.family == F_EW) {
         if (P.n_chunks == 0 && P.tail == 0) return NGH_OK;
         if (P.n_chunks) {
@@ -488,6 +505,17 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     if (e != hipSuccess) {
         delete ctx;
         return fail(NGH_E_RUNTIME, "stream/event creation: %s", hipGetErrorString(e));
+    }
+    // the interpreter's register file is dynamic LDS and may exceed the 64 KiB default
+    const void* interp_kernels[] = {(const void*)ew_interp_kernel<4>, (const void*)ew_interp_kernel<1>,
+                                    (const void*)red_row_interp_kernel<4>, (const void*)red_row_interp_kernel<1>,
+                                    (const void*)red_col_interp_kernel};
+    for (const void* fn : interp_kernels) {
+        e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kInterpLdsMax);
+        if (e != hipSuccess) {
+            ngh_shutdown(ctx);
+            return fail(NGH_E_RUNTIME, "hipFuncSetAttribute(max dynamic LDS): %s", hipGetErrorString(e));
+        }
     }
     *out_ctx = ctx;
     return NGH_OK;

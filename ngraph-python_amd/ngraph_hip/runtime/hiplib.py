@@ -400,9 +400,58 @@ class FusedSpecBuilder(object):
         self._stage_begin = len(self.ops)
         self._stage_reds = []
 
-    def build(self):
+    def _compact_registers(self):
+        """Renumber registers stage by stage so a register is reused once its
+        value is dead; keeps the interpreter's LDS register file small."""
+        src_fields = {}
+        for name in UNARY_OPS:
+            src_fields[OPCODES[name]] = (2,)
+        for name in BINARY_OPS:
+            src_fields[OPCODES[name]] = (2, 3)
+        for name in REDUCTION_OPS:
+            src_fields[OPCODES[name]] = (2,)
+        src_fields[OPCODES["store"]] = (2,)
+        writes = set(OPCODES[n] for n in UNARY_OPS + BINARY_OPS + ["load", "const", "iota"])
+        n_regs = 0
+        for begin, end, _ in self.stages:
+            last_use = {}
+            for pc in range(begin, end):
+                op = self.ops[pc]
+                for f in src_fields.get(op[0], ()):
+                    last_use[op[f]] = pc
+            mapping, free, next_reg = {}, [], 0
+            for pc in range(begin, end):
+                op = list(self.ops[pc])
+                srcs = [op[f] for f in src_fields.get(op[0], ())]
+                for f in src_fields.get(op[0], ()):
+                    op[f] = mapping[op[f]]
+                # sources that die here may be reused by this op's destination
+                for r in set(srcs):
+                    if last_use.get(r) == pc and r in mapping:
+                        free.append(mapping.pop(r))
+                if op[0] in writes:
+                    old = op[1]
+                    if old in mapping:
+                        new = mapping[old]
+                    elif free:
+                        new = free.pop()
+                    else:
+                        new = next_reg
+                        next_reg += 1
+                    if old not in last_use:      # never read: release straight away
+                        free.append(new)
+                    else:
+                        mapping[old] = new
+                    op[1] = new
+                self.ops[pc] = tuple(op)
+            n_regs = max(n_regs, next_reg)
+        self.n_regs = max(n_regs, 1)
+
+    def build(self, compact=True):
         if self._stage_begin != len(self.ops) or not self.stages:
             self.end_stage()
+        if compact:
+            self._compact_registers()
         if len(self.stages) > NGH_MAX_STAGES:
             raise ValueError("too many stages in one fused kernel")
         spec = ngh_fused_spec()

@@ -1,0 +1,818 @@
+"""`hipgpu`: the MI355X transformer for fused elementwise / reduction graphs.
+
+Plays the part of ngraph/transformers/gputransform.py for this path:
+
+* `kernel_op_name` maps each op class to a kernel op name the way
+  `ElementWiseKernel.add_op` does (gputransform.py:124-275);
+* `FusionPlanner` groups consecutive elementwise ops (optionally ended by
+  reductions) that share an iteration space into one kernel spec.  The
+  reference generator supports such compounds (float_ew2.py:553-612,
+  1135-1429) but its transformer hands it one op at a time
+  (gputransform.py:381-391); `fusion=False` reproduces that;
+* operands become (pointer, element strides) views over at most three merged
+  axes (float_ew2.py:289-338, MAX_AXES = 3), reductions see the reduced axes
+  first (gputransform.py:117-122);
+* `HipKernelGroup.__call__` is the executor loop (gputransform.py:508-522);
+* `HipDeviceBufferStorage` / `HipDeviceTensor` own device memory and do host
+  I/O, strided views going through the device copy kernel
+  (gputransform.py:525-909).
+
+All arithmetic runs in libngraph_hip.so; if the library or a GPU is missing,
+constructing the transformer raises.
+"""
+from __future__ import division
+from collections import OrderedDict
+
+import numpy as np
+
+from ngraph_hip.op_graph import op_graph as og
+from ngraph_hip.op_graph.op_graph import Op, OrderedSet
+from ngraph_hip.runtime.hiplib import (HipRuntime, HipLibraryError, FusedSpecBuilder, NGH_F32,
+                                       NGH_FLEX16, NGH_I32, NGH_F16, NGH_MAX_TENSORS,
+                                       NGH_MAX_OPS, NGH_MAX_CONSTS, NGH_MAX_REGS,
+                                       NGH_MAX_REDUCTIONS)
+from ngraph_hip.transformers.base import (ComputationGraphTransformer, DeviceBufferStorage,
+                                          DeviceTensor, UnsupportedTransformerException)
+from ngraph_hip.transformers.passes.passes import SimplePrune, TensorSizeFold
+
+# op class -> kernel op name (gputransform.py:129-275)
+_UNARY_NAMES = OrderedDict([
+    (og.AbsoluteOp, "abs"), (og.CosOp, "cos"), (og.ExpOp, "exp"), (og.LogOp, "log"),
+    (og.NegativeOp, "neg"), (og.ReciprocalOp, "rcp"), (og.SignOp, "sgn"),
+    (og.SigmoidAtomicOp, "sig"), (og.SinOp, "sin"), (og.SqrtOp, "sqrt"), (og.SquareOp, "sqr"),
+    (og.TanhOp, "tanh"),
+])
+_BINARY_NAMES = OrderedDict([
+    (og.Add, "add"), (og.Divide, "div"), (og.FloorDivide, "int_div"), (og.Mod, "mod"),
+    (og.Equal, "eq"), (og.Greater, "gt"), (og.GreaterEqual, "ge"), (og.Less, "lt"),
+    (og.LessEqual, "le"), (og.Maximum, "maximum"), (og.Minimum, "minimum"),
+    (og.Multiply, "mul"), (og.NotEqual, "ne"), (og.Power, "pow"), (og.Subtract, "sub"),
+])
+_REDUCTION_NAMES = OrderedDict([
+    (og.Sum, "sum"), (og.Prod, "prod"), (og.Max, "max"), (og.Min, "min"),
+    (og.Argmax, "argmax"), (og.Argmin, "argmin"),
+])
+
+
+def _lookup(table, op):
+    for cls, name in table.items():
+        if isinstance(op, cls):
+            return name
+    return None
+
+
+def kernel_op_name(op):
+    """Kernel op name of a graph op, or None when it is not an elementwise/reduction op."""
+    return _lookup(_UNARY_NAMES, op) or _lookup(_BINARY_NAMES, op) or _lookup(_REDUCTION_NAMES, op)
+
+
+def is_fusable(op):
+    return (kernel_op_name(op) is not None or
+            isinstance(op, (og.AssignOp, og.OneHotOp, og.Fill)))
+
+
+def iteration_axes(op):
+    """Named axes a kernel running `op` loops over."""
+    if isinstance(op, og.ReductionOp):
+        return op.args[0].forwarded.axes
+    if isinstance(op, (og.AssignOp, og.Fill)):
+        return op.args[0].forwarded.axes
+    return op.axes
+
+
+def _scalar_constant_value(op):
+    """Python float of a scalar constant reached only through views, else None."""
+    cur = op.forwarded
+    while True:
+        if isinstance(cur, og.AssignableTensorOp):
+            if cur.is_constant and cur.is_scalar:
+                return float(np.asarray(cur.const).reshape(()))
+            return None
+        if isinstance(cur, og.TensorValueOp):
+            cur = cur.value_tensor.forwarded
+        elif isinstance(cur, og.IndexOp):
+            cur = cur.args[0].forwarded
+        else:
+            return None
+
+
+def _producer(op):
+    """The device op (or state tensor) whose buffer `op` is a view of."""
+    cur = op.forwarded
+    while True:
+        if isinstance(cur, og.TensorValueOp):
+            cur = cur.value_tensor.forwarded
+        elif isinstance(cur, og.IndexOp):
+            cur = cur.args[0].forwarded
+        elif isinstance(cur, og.SequentialOp):
+            cur = cur.value_tensor.forwarded
+        else:
+            return cur
+
+
+def _view_key(td):
+    return (td.base, td.parameter_key)
+
+
+# =============================================================================== storage
+class HipDeviceBufferStorage(DeviceBufferStorage):
+    """One device allocation per base tensor (gputransform.py:642-676); allocated on first use."""
+
+    def __init__(self, transformer, bytes, dtype, **kwargs):
+        super(HipDeviceBufferStorage, self).__init__(transformer, bytes, dtype, **kwargs)
+        self._ptr = None
+
+    @property
+    def ptr(self):
+        if self._ptr is None:
+            self._ptr = self.transformer.runtime.malloc(max(int(self.bytes), 4))
+        return self._ptr
+
+    def create_device_tensor(self, tensor_description):
+        return HipDeviceTensor(self.transformer, self, tensor_description,
+                               name="v_" + tensor_description.name)
+
+    def free(self):
+        if self._ptr is not None:
+            self.transformer.runtime.free(self._ptr)
+            self._ptr = None
+
+
+class HipDeviceTensor(DeviceTensor):
+    """A strided view of a device buffer with host I/O (gputransform.py:679-909)."""
+
+    storage_np_dtype = None   # None: the logical dtype
+
+    def transform_allocate(self):
+        pass
+
+    @property
+    def np_dtype(self):
+        d = self.tensor_description.dtype
+        return d if isinstance(d, np.dtype) else np.dtype(np.int16)
+
+    @property
+    def ngh_dtype(self):
+        return self.transformer.ngh_dtype(self.tensor_description.dtype)
+
+    @property
+    def itemsize(self):
+        return self.np_dtype.itemsize
+
+    @property
+    def ptr(self):
+        return self.device_buffer.ptr + self.tensor_description.offset * self.itemsize
+
+    @property
+    def shape(self):
+        return self.tensor_description.shape
+
+    @property
+    def element_strides(self):
+        return self.tensor_description.full_strides
+
+    def _read_raw(self):
+        """The view's elements as a C-contiguous host array of the storage dtype."""
+        td, rt = self.tensor_description, self.transformer.runtime
+        out = np.empty(td.shape, dtype=self.np_dtype)
+        if out.size == 0:
+            return out
+        if td.c_contiguous:
+            rt.memcpy_d2h(out, self.ptr)
+            return out
+        # strided or broadcast view: gather on the device, then one contiguous copy out
+        tmp = rt.malloc(out.nbytes)
+        try:
+            contiguous = [int(s) // out.itemsize for s in out.strides]
+            rt.copy_strided(tmp, self.ptr, td.shape, contiguous, td.full_strides, out.itemsize)
+            rt.memcpy_d2h(out, tmp)
+        finally:
+            rt.free(tmp)
+        return out
+
+    def _write_raw(self, host):
+        td, rt = self.tensor_description, self.transformer.runtime
+        host = np.ascontiguousarray(np.broadcast_to(host, td.shape), dtype=self.np_dtype)
+        if host.size == 0:
+            return
+        if td.c_contiguous:
+            rt.memcpy_h2d(self.ptr, host)
+            return
+        if any(s == 0 and n > 1 for s, n in zip(td.full_strides, td.shape)):
+            raise ValueError("cannot write through a broadcast view")
+        tmp = rt.malloc(host.nbytes)
+        try:
+            rt.memcpy_h2d(tmp, host)
+            contiguous = [int(s) // host.itemsize for s in host.strides]
+            rt.copy_strided(self.ptr, tmp, td.shape, td.full_strides, contiguous, host.itemsize)
+            rt.sync()
+        finally:
+            rt.free(tmp)
+
+    def get(self, tensor):
+        value = self._read_raw()
+        if tensor is None:
+            return value
+        tensor[...] = value
+        return tensor
+
+    def __getitem__(self, key):
+        return self.get(None)[key]
+
+    def __setitem__(self, key, value):
+        value = np.asarray(value)
+        if key is Ellipsis or key == () or key == slice(None, None, None):
+            self._write_raw(value.astype(self.np_dtype, copy=False))
+        else:
+            whole = self._read_raw()
+            whole[key] = value
+            self._write_raw(whole)
+
+
+# =============================================================================== kernels
+class HipKernel(object):
+    """One launchable unit of a computation (gpu/kernel.py:18-87)."""
+
+    def __init__(self, transformer):
+        self.transformer = transformer
+        self.buffers_bound = False
+
+    def bind_buffers(self):
+        self.buffers_bound = True
+
+    def execute(self):
+        raise NotImplementedError
+
+    # flex hooks (flexgputransform.py:56-61, 347-366)
+    output_flex_ids = ()
+
+    def bind_flex_scales(self):
+        pass
+
+
+class _Dim(object):
+    __slots__ = ("length", "strides", "tag")
+
+    def __init__(self, length, strides, tag=None):
+        self.length, self.strides, self.tag = int(length), list(strides), tag
+
+
+class FusedKernel(HipKernel):
+    """A compound elementwise / reduction kernel = one ngh_fused_spec per outer index.
+
+    `ops` are the graph ops of the group, in execution order.  Lowering
+    happens in bind_buffers, once storage exists.
+    """
+
+    def __init__(self, transformer, ops, store_ops, name):
+        super(FusedKernel, self).__init__(transformer)
+        self.ops = list(ops)
+        self.store_ops = set(store_ops)
+        self.name = name
+        self.specs = []
+        self.flex_bindings = []     # (spec index, tensor slot, flex entry, is_output)
+        self.described = None
+
+    # -- operand bookkeeping ------------------------------------------------------------
+    def bind_buffers(self):
+        if not self.buffers_bound:
+            self._lower()
+        super(FusedKernel, self).bind_buffers()
+
+    def _lower(self):
+        t = self.transformer
+        ops = self.ops
+        first = ops[0]
+        reductions = [op for op in ops if isinstance(op, og.ReductionOp)]
+        it_axes = iteration_axes(first)
+        red_axes = reductions[0].reduction_axes if reductions else og.make_axes(())
+        onehot_axes = [op.axis for op in ops if isinstance(op, og.OneHotOp)]
+
+        # ---- pass 1: collect operands (views) and the program over symbolic registers ----
+        operands = []            # [(td, role)] in slot order
+        slot_of = {}             # view key -> slot
+        program = []             # tuples, see _emit below
+        value_reg = {}           # producing op / view key -> symbolic register
+        n_sym = [0]
+
+        def new_reg():
+            n_sym[0] += 1
+            return n_sym[0] - 1
+
+        def slot(td):
+            key = _view_key(td)
+            if key not in slot_of:
+                slot_of[key] = len(operands)
+                operands.append(td)
+            return slot_of[key]
+
+        def operand_reg(arg):
+            arg = arg.forwarded
+            c = _scalar_constant_value(arg)
+            if c is not None:
+                r = new_reg()
+                program.append(("const", r, c))
+                return r
+            prod = _producer(arg)
+            if prod in value_reg:
+                return value_reg[prod]
+            td = arg.tensor_description()
+            key = _view_key(td)
+            if key in value_reg:
+                return value_reg[key]
+            r = new_reg()
+            program.append(("load", r, slot(td)))
+            value_reg[key] = r
+            return r
+
+        red_slots = []
+        for op in ops:
+            name = kernel_op_name(op)
+            if isinstance(op, og.AssignOp):
+                target, val = op.args[0].forwarded, op.args[1].forwarded
+                r = operand_reg(val)
+                td = target.tensor_description()
+                program.append(("store", slot(td), r))
+                value_reg[_view_key(td)] = r
+                continue
+            if isinstance(op, og.Fill):
+                td = op.args[0].forwarded.tensor_description()
+                r = new_reg()
+                program.append(("const", r, float(op.scalar)))
+                program.append(("store", slot(td), r))
+                value_reg[_view_key(td)] = r
+                continue
+            if isinstance(op, og.OneHotOp):
+                x = operand_reg(op.args[0])
+                i = new_reg()
+                program.append(("iota", i, op.axis))
+                r = new_reg()
+                program.append(("eq", r, i, x))
+            elif isinstance(op, og.ReductionOp):
+                x = operand_reg(op.args[0])
+                if len(op.reduction_axes) == 0 or op.reduction_axes.size == 1:
+                    # nothing to reduce: assign (gputransform.py:117-119, float_ew2.py:582-586)
+                    r = new_reg()
+                    if name in ("argmax", "argmin"):
+                        program.append(("const", r, 0.0))
+                    else:
+                        program.append(("assign", r, x))
+                else:
+                    program.append(("reduce", name, x, slot(op.tensor_description())))
+                    red_slots.append(op)
+                    continue
+            elif name in og_unary_names:
+                x = operand_reg(op.args[0])
+                r = new_reg()
+                program.append((name, r, x))
+            else:
+                x, y = operand_reg(op.args[0]), operand_reg(op.args[1])
+                r = new_reg()
+                program.append((name, r, x, y))
+            value_reg[op] = r
+            if op in self.store_ops:
+                program.append(("store", slot(op.tensor_description()), r))
+
+        # ---- pass 2: dims = iteration axes with every operand's stride -----------------------
+        def strides_over(td, axes):
+            out = []
+            for axis in axes:
+                out.append(td.full_strides[td.axes.index(axis)] if axis in td.axes else 0)
+            return out
+
+        has_reduce = any(p[0] == "reduce" for p in program)
+        if has_reduce:
+            order = list(red_axes) + [a for a in it_axes if a not in red_axes]
+        else:
+            order = list(it_axes)
+        dims = []
+        for axis in order:
+            tag = None
+            if has_reduce and axis in red_axes:
+                tag = "red"
+            if axis in onehot_axes:
+                tag = ("iota", axis.name)
+            dims.append(_Dim(axis.length, [strides_over(td, [axis])[0] for td in operands], tag))
+
+        dims = self._coalesce(dims, has_reduce)
+        outer, inner = self._split_outer(dims, has_reduce)
+
+        # ---- pass 3: one spec per outer index -------------------------------------------------
+        self.specs = []
+        self.flex_bindings = []
+        outer_shape = [d.length for d in outer]
+        n_outer = int(np.prod(outer_shape, dtype=np.int64)) if outer else 1
+        if any(d.length == 0 for d in dims):
+            return
+        for flat in range(n_outer):
+            idx, rem = [], flat
+            for n in reversed(outer_shape):
+                idx.insert(0, rem % n)
+                rem //= n
+            offsets = [sum(i * d.strides[s] for i, d in zip(idx, outer)) for s in range(len(operands))]
+            self.specs.append(self._build_spec(operands, program, inner, offsets, has_reduce))
+
+    @staticmethod
+    def _coalesce(dims, has_reduce):
+        """Drop length-1 dims and merge neighbours every operand walks contiguously."""
+        dims = [d for d in dims if d.length != 1 or isinstance(d.tag, tuple)]
+
+        def mergeable(a, b):
+            if a.tag != b.tag or (a.tag is not None and a.tag != "red"):
+                return False
+            return all(sa == sb * b.length for sa, sb in zip(a.strides, b.strides))
+
+        if not has_reduce:
+            # order by the strides of the operands (outermost first) so mergeable dims meet
+            dims.sort(key=lambda d: tuple(-s for s in d.strides))
+        else:
+            red = [d for d in dims if d.tag == "red"]
+            rest = [d for d in dims if d.tag != "red"]
+            red.sort(key=lambda d: tuple(-s for s in d.strides))
+            rest.sort(key=lambda d: tuple(-s for s in d.strides))
+            dims = red + rest
+        out = []
+        for d in dims:
+            if out and mergeable(out[-1], d):
+                prev = out[-1]
+                out[-1] = _Dim(prev.length * d.length, d.strides, prev.tag)
+            else:
+                out.append(d)
+        return out
+
+    @staticmethod
+    def _split_outer(dims, has_reduce):
+        """At most 3 dims go to the kernel (one reduced dim first); the rest loop on the host."""
+        if has_reduce:
+            red = [d for d in dims if d.tag == "red"]
+            rest = [d for d in dims if d.tag != "red"]
+            if len(red) == 0:
+                red = [_Dim(1, [0] * len(dims[0].strides) if dims else [], "red")]
+            if len(red) > 1:
+                raise og_unsupported("reduction axes are not mergeable into one strided axis; "
+                                     "make the operand contiguous in (reduced..., kept...) order")
+            keep = rest[-2:] if len(rest) > 2 else rest
+            outer = rest[:-2] if len(rest) > 2 else []
+            return outer, red + keep
+        keep = dims[-3:] if len(dims) > 3 else dims
+        outer = dims[:-3] if len(dims) > 3 else []
+        return outer, keep
+
+    def _build_spec(self, operands, program, inner, offsets, has_reduce):
+        t = self.transformer
+        shape = [d.length for d in inner] or [1]
+        nd = len(inner)
+        sb = FusedSpecBuilder(shape)
+        for s, td in enumerate(operands):
+            view = t.get_tensor_description_tensor_view(td)
+            strides = [d.strides[s] for d in inner] or [0]
+            dtype = t.ngh_dtype(td.dtype)
+            slot = sb.tensor(view.ptr + offsets[s] * view.itemsize, strides, dtype)
+            assert slot == s
+        reg_map = {}
+
+        def reg(sym):
+            if sym not in reg_map:
+                reg_map[sym] = sb.reg()
+            return reg_map[sym]
+
+        written = set()
+        for ins in program:
+            kind = ins[0]
+            if kind == "const":
+                sb.constant(ins[2], reg(ins[1]))
+            elif kind == "load":
+                sb.load(ins[2], reg(ins[1]))
+            elif kind == "store":
+                sb.store(ins[1], reg(ins[2]))
+                written.add(ins[1])
+            elif kind == "iota":
+                axis = [i for i, d in enumerate(inner) if d.tag == ("iota", ins[2].name)]
+                if not axis:
+                    raise og_unsupported("one-hot axis was merged away")
+                sb.iota(axis[0], reg(ins[1]))
+            elif kind == "reduce":
+                sb.reduce(ins[1], reg(ins[2]), ins[3])
+                written.add(ins[3])
+            elif len(ins) == 3:
+                sb.unary(kind, reg(ins[2]), reg(ins[1]))
+            else:
+                sb.binary(kind, reg(ins[2]), reg(ins[3]), reg(ins[1]))
+        spec = sb.build()
+        index = len(self.specs)
+        for s, td in enumerate(operands):
+            entry = t.flex_entry_of(td)
+            if entry is not None:
+                self.flex_bindings.append((index, s, entry, s in written))
+        t.runtime.validate_fused(spec)
+        return spec
+
+    def execute(self):
+        rt = self.transformer.runtime
+        for spec in self.specs:
+            rt.launch_fused(spec)
+
+    def describe(self):
+        rt = self.transformer.runtime
+        return [[rt.describe_fused(spec, s) for s in range(spec.n_stages)] for spec in self.specs]
+
+
+og_unary_names = set(_UNARY_NAMES.values())
+
+
+def og_unsupported(msg):
+    return NotImplementedError("hipgpu: " + msg)
+
+
+class CopyKernel(HipKernel):
+    """ContiguousOp: strided device copy (tensor_ops.py:137-204 DimShuffleKernel)."""
+
+    def __init__(self, transformer, op):
+        super(CopyKernel, self).__init__(transformer)
+        self.op = op
+
+    def bind_buffers(self):
+        t = self.transformer
+        src_td = self.op.args[0].forwarded.tensor_description()
+        dst_td = self.op.tensor_description()
+        self.src = t.get_tensor_description_tensor_view(src_td)
+        self.dst = t.get_tensor_description_tensor_view(dst_td)
+        self.shape = dst_td.shape
+        order = [src_td.axes.index(a) for a in dst_td.axes]
+        self.src_strides = [src_td.full_strides[i] for i in order]
+        self.dst_strides = list(dst_td.full_strides)
+        super(CopyKernel, self).bind_buffers()
+
+    def execute(self):
+        self.transformer.runtime.copy_strided(self.dst.ptr, self.src.ptr, self.shape,
+                                              self.dst_strides, self.src_strides, self.dst.itemsize)
+
+
+class HipKernelGroup(object):
+    """The kernels of one computation and the loop that runs them (gputransform.py:348-522)."""
+
+    def __init__(self, transformer, name):
+        self.transformer = transformer
+        self.name = name
+        self.kernels = []
+
+    def setup_kernel_execute(self, kernel):
+        pass
+
+    def after_kernel_execute(self, kernel):
+        pass
+
+    def __call__(self):
+        for k in self.kernels:
+            if not k.buffers_bound:
+                k.bind_buffers()
+        for k in self.kernels:
+            self.setup_kernel_execute(k)
+            k.execute()
+            self.after_kernel_execute(k)
+
+
+# =============================================================================== fusion
+class FusionPlanner(object):
+    """Greedy grouping of consecutive fusable ops over one iteration space.
+
+    A group is a run of elementwise ops, optionally ended by reductions that
+    share their reduced axes (the stage rule of float_ew2.py:553-612).  An op
+    starts a new group when its iteration axes differ, when it follows a
+    reduction, when it would read or write memory the group touches through a
+    different view, or when the kernel's operand / op / constant limits are hit.
+    """
+
+    def __init__(self, transformer, fusion=True):
+        self.transformer = transformer
+        self.fusion = fusion
+
+    def plan(self, ordered_ops, readers, returned):
+        groups, cur = [], None
+        for op in ordered_ops:
+            op = op.forwarded
+            if not op.is_device_op:
+                continue
+            if not is_fusable(op):
+                if cur:
+                    groups.append(cur)
+                    cur = None
+                groups.append(_Group(op, fusable=False))
+                continue
+            if cur is not None and self.fusion and cur.accepts(op):
+                cur.add(op)
+            else:
+                if cur:
+                    groups.append(cur)
+                cur = _Group(op)
+        if cur:
+            groups.append(cur)
+        for g in groups:
+            if g.fusable:
+                g.decide_stores(readers, returned)
+        return groups
+
+
+class _Group(object):
+    def __init__(self, op, fusable=True):
+        self.ops = [op]
+        self.fusable = fusable
+        self.store_ops = set()
+        if fusable:
+            self.axes = iteration_axes(op)
+            self.has_reduce = False
+            self.red_axes = None
+            self.read_views = {}     # base -> set(view keys)
+            self.write_views = {}
+            self.n_ops = 0
+            self.n_consts = 0
+            self.n_reds = 0
+            self._account(op)
+
+    def _operand_views(self, op):
+        reads, writes = [], []
+        if isinstance(op, og.AssignOp):
+            writes.append(op.args[0].forwarded.tensor_description())
+            srcs = [op.args[1]]
+        elif isinstance(op, og.Fill):
+            writes.append(op.args[0].forwarded.tensor_description())
+            srcs = []
+        else:
+            writes.append(op.tensor_description())
+            srcs = list(op.args)
+        for a in srcs:
+            a = a.forwarded
+            if _scalar_constant_value(a) is not None:
+                continue
+            reads.append(a.tensor_description())
+        return reads, writes
+
+    def _account(self, op):
+        reads, writes = self._operand_views(op)
+        for td in reads:
+            self.read_views.setdefault(td.base, set()).add(td.parameter_key)
+        for td in writes:
+            self.write_views.setdefault(td.base, set()).add(td.parameter_key)
+        self.n_ops += 4
+        self.n_consts += sum(1 for a in op.args if _scalar_constant_value(a.forwarded) is not None)
+        if isinstance(op, og.ReductionOp) and op.reduction_axes.size > 1:
+            self.has_reduce = True
+            self.red_axes = op.reduction_axes
+            self.n_reds += 1
+
+    def accepts(self, op):
+        if not iteration_axes(op).is_equal_set(self.axes) or \
+                iteration_axes(op).lengths != tuple(self.axes[self.axes.index(a)].length
+                                                    for a in iteration_axes(op)):
+            return False
+        is_red = isinstance(op, og.ReductionOp) and op.reduction_axes.size > 1
+        if self.has_reduce:
+            if not is_red or not op.reduction_axes.is_equal_set(self.red_axes):
+                return False
+            if self.n_reds >= NGH_MAX_REDUCTIONS:
+                return False
+        reads, writes = self._operand_views(op)
+        for td in reads:
+            # reading what the group wrote is fine through the very same view only
+            w = self.write_views.get(td.base)
+            if w is not None and w != {td.parameter_key}:
+                return False
+        for td in writes:
+            r = self.read_views.get(td.base)
+            if r is not None and r != {td.parameter_key}:
+                return False
+            w = self.write_views.get(td.base)
+            if w is not None and w != {td.parameter_key}:
+                return False
+        if is_red:
+            # a reduction reads its argument through registers; its output must not be re-read here
+            pass
+        bases = set(self.read_views) | set(self.write_views) | set(td.base for td in reads + writes)
+        if len(bases) + 2 > NGH_MAX_TENSORS:
+            return False
+        if self.n_ops + 4 > NGH_MAX_OPS or self.n_consts + 2 > NGH_MAX_CONSTS:
+            return False
+        if self.n_ops // 4 + 1 > NGH_MAX_REGS - 4:
+            return False
+        return True
+
+    def add(self, op):
+        self.ops.append(op)
+        self._account(op)
+
+    def decide_stores(self, readers, returned):
+        """A result goes to memory only if something outside the group can see it."""
+        inside = set(self.ops)
+        for op in self.ops:
+            if not op.is_tensor_op or isinstance(op, (og.AssignOp, og.Fill)):
+                continue
+            base = op.tensor_description().base
+            users = readers.get(base, ())
+            if base in returned or any(u not in inside for u in users):
+                self.store_ops.add(op)
+            elif isinstance(op, og.ReductionOp):
+                self.store_ops.add(op)
+
+
+# =============================================================================== transformer
+class HipTransformer(ComputationGraphTransformer):
+    """Transformer for executing graphs on an MI355X through libngraph_hip.so."""
+
+    transformer_name = "hipgpu"
+    default_rtol = 1e-05
+    default_atol = 1e-08
+
+    kernel_group_class = HipKernelGroup
+
+    def __init__(self, device_id=0, fusion=True, **kwargs):
+        try:
+            self.runtime = HipRuntime(device_id)
+        except HipLibraryError as e:
+            raise UnsupportedTransformerException("hipgpu needs libngraph_hip.so and an MI355X: %s" % e)
+        super(HipTransformer, self).__init__(**kwargs)
+        self.fusion = fusion
+        self.kernel_groups = OrderedDict()
+        self.graph_passes = [SimplePrune(), TensorSizeFold()]
+
+    # -- dtype mapping ---------------------------------------------------------------------
+    def ngh_dtype(self, dtype):
+        if not isinstance(dtype, np.dtype):
+            return NGH_FLEX16
+        if dtype == np.float32:
+            return NGH_F32
+        if dtype == np.int32:
+            return NGH_I32
+        if dtype == np.float16:
+            return NGH_F16
+        raise TypeError("hipgpu: unsupported tensor dtype %s" % dtype)
+
+    def flex_entry_of(self, tensor_description):
+        return None
+
+    # -- hooks ---------------------------------------------------------------------------------
+    def device_buffer_storage(self, bytes, dtype, name):
+        return HipDeviceBufferStorage(self, bytes, dtype, name="a_" + name)
+
+    def start_transform_allocate(self):
+        pass
+
+    def finish_transform_allocate(self):
+        pass
+
+    def gpu_kernel_group(self, name):
+        return self.kernel_group_class(self, name)
+
+    def _usage_maps(self):
+        """Which device ops read each buffer, over every computation of this transformer."""
+        readers, returned = {}, set()
+        for op in self.ops:
+            op = op.forwarded
+            if op.is_device_op:
+                srcs = op.args[1:] if isinstance(op, og.AssignOp) else \
+                    (() if isinstance(op, og.Fill) else op.args)
+                for a in srcs:
+                    a = a.forwarded
+                    if a.is_tensor_op:
+                        readers.setdefault(a.tensor_description().base, set()).add(op)
+        for comp in self.computations:
+            for v in comp.computation_op.values:
+                v = v.forwarded
+                if v.is_tensor_op:
+                    returned.add(v.tensor_description().base)
+        return readers, returned
+
+    def transform_ordered_ops(self, computation, ordered_ops, name):
+        group = self.gpu_kernel_group(name)
+        readers, returned = self._usage_maps()
+        planner = FusionPlanner(self, fusion=self.fusion)
+        for i, g in enumerate(planner.plan(ordered_ops, readers, returned)):
+            if g.fusable:
+                group.kernels.append(self.make_fused_kernel(g.ops, g.store_ops, "%s_k%d" % (name, i)))
+            else:
+                op = g.ops[0]
+                if isinstance(op, og.ContiguousOp):
+                    group.kernels.append(CopyKernel(self, op))
+                else:
+                    raise ValueError("Unhandled op: {}".format(op))
+        self.kernel_groups[computation] = group
+        computation.executor = group
+        return name
+
+    def make_fused_kernel(self, ops, store_ops, name):
+        return FusedKernel(self, ops, store_ops, name)
+
+    def finish_transform(self):
+        pass
+
+    def allocate_storage(self):
+        pass
+
+    def close(self):
+        rt = getattr(self, "runtime", None)
+        if rt is not None:
+            try:
+                rt.sync()
+            except Exception:
+                pass
+            rt.close()
+            self.runtime = None

@@ -299,8 +299,14 @@ def test_every_reduction(hip_runtime, name, shape, layout):
     R, A = shape
     rs = np.random.RandomState(13)
     scale = 0.05 if name == "prod" else 1.0
-    logical = (1.0 + rs.normal(0, scale, (R, A))).astype(f32) if name == "prod" else \
-        rs.normal(0, 1, (R, A)).astype(f32)
+    if name == "prod":
+        logical = (1.0 + rs.normal(0, scale, (R, A))).astype(f32)
+    elif name == "sum":
+        # same-sign data: a relative bound on the result is meaningful (a signed sum
+        # cancels and is checked against float64 in test_signed_sum_against_float64)
+        logical = rs.uniform(0.5, 1.5, (R, A)).astype(f32)
+    else:
+        logical = rs.normal(0, 1, (R, A)).astype(f32)
     if name in ("argmax", "argmin", "max", "min") and R > 3:
         logical[R // 2] = logical[R // 3]           # ties: lowest index must win
     want = numpy_ops.reduce(name, logical, 0)
@@ -322,5 +328,28 @@ def test_every_reduction(hip_runtime, name, shape, layout):
         np.testing.assert_array_equal(got, want)
     else:
         np.testing.assert_allclose(got, want, rtol=1e-5 if name != "prod" else 1e-4, atol=1e-5)
+    x_d.free()
+    out_d.free()
+
+
+@pytest.mark.parametrize("shape,layout", [((40000, 2), "col"), ((200704, 4), "row"), ((3000, 300), "col")])
+def test_signed_sum_against_float64(hip_runtime, shape, layout):
+    """A cancelling sum: error must stay within 1e-6 of sum(|x|), checked against float64."""
+    rt = hip_runtime
+    R, A = shape
+    rs = np.random.RandomState(14)
+    logical = rs.normal(0.5, 2, (R, A)).astype(f32)
+    truth = logical.astype(np.float64).sum(axis=0)
+    bound = 1e-6 * np.abs(logical).astype(np.float64).sum(axis=0)
+    if layout == "row":
+        store, strides = np.ascontiguousarray(logical.T), [1, R]
+    else:
+        store, strides = logical, [A, 1]
+    x_d, out_d = rt.array(store), rt.empty((A,))
+    sb = FusedSpecBuilder([R, A])
+    tx, to = sb.tensor(x_d.ptr, strides), sb.tensor(out_d.ptr, [0, 1])
+    sb.reduce("sum", sb.load(tx), to)
+    rt.launch_fused(sb.build())
+    assert np.all(np.abs(out_d.get().astype(np.float64) - truth) <= bound)
     x_d.free()
     out_d.free()

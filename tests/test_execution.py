@@ -1,0 +1,272 @@
+"""Graph-level parity: the same test bodies run on the NumPy oracle transformer
+("cpu", always) and on the HIP transformer ("hipgpu", GPU box) and are checked
+against NumPy expressions written here, the way the reference's
+tests/transformer_dependent/test_execution.py and test_kernel_generator.py do.
+"""
+import numpy as np
+import pytest
+
+import ngraph_hip as ng
+import ngraph_hip.transformers as ngt
+from ngraph_hip.testing import executor, RandomTensorGenerator
+import oracle.cpu_transformer  # noqa: F401  registers "cpu"
+
+rng = RandomTensorGenerator(0, np.float32)
+RTOL, ATOL = 1e-5, 1e-6
+
+BACKENDS = ["cpu", pytest.param("hipgpu", marks=pytest.mark.gpu),
+            pytest.param("hipgpu-nofuse", marks=pytest.mark.gpu)]
+
+
+@pytest.fixture(params=BACKENDS)
+def backend(request):
+    name = request.param
+    if name == "hipgpu-nofuse":
+        factory = ngt.make_transformer_factory("hipgpu", fusion=False)
+    else:
+        factory = ngt.make_transformer_factory(name)
+    ngt.set_transformer_factory(factory)
+    yield name
+    ngt.set_transformer_factory(None)
+
+
+def axes(**kw):
+    return ng.make_axes([ng.make_axis(length=v, name=k) for k, v in kw.items()])
+
+
+def test_transformer_registry():
+    assert "cpu" in ngt.transformer_choices()
+    assert "hipgpu" in ngt.transformer_choices()
+    assert "flexhip" in ngt.transformer_choices()
+    with pytest.raises(ValueError):
+        ngt.allocate_transformer("no-such-backend")
+    f = ngt.make_transformer_factory("cpu")
+    assert f.name == "cpu"
+
+
+def test_scalar_constant_and_placeholder(backend):
+    x = ng.placeholder(())
+    with executor(x * 2 + 1, x) as f:
+        for v in (0.0, 1.5, -3.25):
+            np.testing.assert_allclose(f(v), np.float32(v) * 2 + 1, rtol=RTOL)
+
+
+UNARY = [(ng.negative, np.negative), (ng.absolute, np.abs), (ng.exp, np.exp), (ng.tanh, np.tanh),
+         (ng.square, np.square), (ng.sign, np.sign), (ng.sin, np.sin), (ng.cos, np.cos),
+         (ng.sigmoid, lambda x: 1.0 / (1.0 + np.exp(-x))),
+         (ng.sigmoidAtomic, lambda x: 1.0 / (1.0 + np.exp(-x)))]
+
+
+@pytest.mark.parametrize("ng_fn,np_fn", UNARY)
+def test_unary_elementwise(backend, ng_fn, np_fn):
+    ax = axes(H=17, W=33)
+    x = ng.placeholder(ax)
+    xv = rng.uniform(-2, 2, ax)
+    with executor(ng_fn(x), x) as f:
+        np.testing.assert_allclose(f(xv), np_fn(xv), rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("ng_fn,np_fn", [(ng.sqrt, np.sqrt), (ng.log, np.log),
+                                         (ng.reciprocal, np.reciprocal), (ng.safelog, np.log)])
+def test_unary_positive_domain(backend, ng_fn, np_fn):
+    ax = axes(H=8, W=65)
+    x = ng.placeholder(ax)
+    xv = rng.uniform(0.1, 5, ax)
+    with executor(ng_fn(x), x) as f:
+        np.testing.assert_allclose(f(xv), np_fn(xv), rtol=RTOL, atol=ATOL)
+
+
+BINARY = [(ng.add, np.add), (ng.subtract, np.subtract), (ng.multiply, np.multiply),
+          (ng.divide, np.divide), (ng.maximum, np.maximum), (ng.minimum, np.minimum),
+          (ng.equal, np.equal), (ng.not_equal, np.not_equal), (ng.greater, np.greater),
+          (ng.less, np.less), (ng.greater_equal, np.greater_equal), (ng.less_equal, np.less_equal)]
+
+
+@pytest.mark.parametrize("ng_fn,np_fn", BINARY)
+def test_binary_elementwise_matched_axes(backend, ng_fn, np_fn):
+    ax = axes(C=5, H=12, N=16)
+    x, y = ng.placeholder(ax), ng.placeholder(ax)
+    xv, yv = rng.uniform(-2, 2, ax), rng.uniform(-2, 2, ax)
+    yv[::2] = xv[::2]
+    with executor(ng_fn(x, y), x, y) as f:
+        np.testing.assert_allclose(f(xv, yv), np_fn(xv, yv).astype(np.float32), rtol=RTOL, atol=ATOL)
+
+
+def test_binary_broadcast_unmatched_axes(backend):
+    """x[C,N] + y[N,H]: result axes C,N,H (op_graph.py:3159-3180)."""
+    C, N, H = ng.make_axis(3, name="C"), ng.make_axis(4, name="N"), ng.make_axis(5, name="H")
+    x, y = ng.placeholder([C, N]), ng.placeholder([N, H])
+    z = x + y
+    assert z.axes == ng.make_axes([C, N, H])
+    xv, yv = rng.uniform(-1, 1, x.axes), rng.uniform(-1, 1, y.axes)
+    with executor(z, x, y) as f:
+        np.testing.assert_allclose(f(xv, yv), xv[:, :, None] + yv[None, :, :], rtol=RTOL)
+    # y already has all the axes: result takes y's order
+    w = ng.placeholder([H, N, C])
+    assert (x * w).axes == w.axes
+
+
+def test_power_floordiv_mod(backend):
+    ax = axes(H=9, W=31)
+    x, y = ng.placeholder(ax), ng.placeholder(ax)
+    xv = np.round(rng.uniform(-9, 9, ax))
+    yv = np.round(rng.uniform(1, 4, ax)) * np.where(rng.uniform(0, 1, ax) > 0.5, 1, -1)
+    with executor([x // y, x % y, ng.power(ng.absolute(x) + 0.5, y)], x, y) as f:
+        fd, md, pw = f(xv, yv)
+    np.testing.assert_allclose(fd, np.floor_divide(xv, yv), rtol=RTOL)
+    np.testing.assert_allclose(md, np.mod(xv, yv), rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(pw, np.power(np.abs(xv) + np.float32(0.5), yv), rtol=RTOL)
+
+
+REDUCTIONS = [(ng.sum, np.sum), (ng.max, np.max), (ng.min, np.min), (ng.prod, np.prod)]
+
+
+@pytest.mark.parametrize("ng_fn,np_fn", REDUCTIONS)
+@pytest.mark.parametrize("sub", [slice(0, 1), slice(1, 2), slice(2, 3), slice(0, 2), slice(1, 3),
+                                 slice(0, 3)])
+def test_reduction_axis_slices(backend, ng_fn, np_fn, sub):
+    """Every contiguous subset of reduction axes (test_execution.py:144-181)."""
+    ax = axes(C=4, H=6, W=10)
+    x = ng.placeholder(ax)
+    xv = rng.uniform(0.5, 1.5, ax)
+    red = ax[sub]
+    np_axes = tuple(ax.index(a) for a in red)
+    with executor(ng_fn(x, reduction_axes=red), x) as f:
+        np.testing.assert_allclose(f(xv), np_fn(xv, axis=np_axes), rtol=1e-5, atol=1e-5)
+
+
+def test_reduction_out_axes_and_noncontiguous(backend):
+    ax = axes(C=3, H=5, W=7, N=4)
+    x = ng.placeholder(ax)
+    xv = rng.uniform(-1, 1, ax)
+    # reduce over H and N (not adjacent in memory): needs a host loop or strided reduction
+    with executor(ng.sum(x, out_axes=ax[0:1] + ax[2:3]), x) as f:
+        np.testing.assert_allclose(f(xv), xv.sum(axis=(1, 3)), rtol=1e-5, atol=1e-5)
+
+
+def test_argmax_argmin_first_index_wins(backend):
+    ax = axes(C=7, N=9)
+    x = ng.placeholder(ax)
+    xv = np.round(rng.uniform(-3, 3, ax))          # many ties
+    with executor([ng.argmax(x, out_axes=ax[1:]), ng.argmin(x, out_axes=ax[1:])], x) as f:
+        amax, amin = f(xv)
+    np.testing.assert_array_equal(amax, xv.argmax(axis=0))
+    np.testing.assert_array_equal(amin, xv.argmin(axis=0))
+
+
+def test_mean_variance(backend):
+    ax = axes(C=6, H=20, N=8)
+    x = ng.placeholder(ax)
+    xv = rng.normal(0.5, 2, ax)
+    out = ax[0:1]
+    with executor([ng.mean(x, out_axes=out), ng.variance(x, out_axes=out)], x) as f:
+        m, v = f(xv)
+    np.testing.assert_allclose(m, xv.mean(axis=(1, 2)), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(v, xv.var(axis=(1, 2)), rtol=1e-5, atol=1e-6)
+
+
+def test_4d_elementwise_and_sums(backend):
+    """Shapes of tests/transformer_dependent/test_kernel_generator.py:43-131."""
+    for shape in [(64, 10, 28, 32), (3, 16, 16, 4), (7, 15, 19, 5), (3, 5, 7, 2)]:
+        ax = ng.make_axes([ng.make_axis(n) for n in shape])
+        a, b = ng.placeholder(ax), ng.placeholder(ax)
+        av, bv = rng.uniform(0, 1, ax), rng.uniform(0, 1, ax)
+        with executor([a + b, ng.sum(a, reduction_axes=ax[1:2]), ng.sum(a, reduction_axes=ax[3:4]),
+                       ng.sum(ng.reciprocal(a + 1) + b, reduction_axes=ax[0:1])], a, b) as f:
+            s, r1, r3, chain = f(av, bv)
+        np.testing.assert_allclose(s, av + bv, rtol=RTOL)
+        np.testing.assert_allclose(r1, av.sum(axis=1), rtol=1e-5)
+        np.testing.assert_allclose(r3, av.sum(axis=3), rtol=1e-5)
+        np.testing.assert_allclose(chain, (1 / (av + 1) + bv).sum(axis=0), rtol=1e-5)
+
+
+def test_run_twice_bit_equal(backend):
+    """Partial blocks must not leak state between calls (test_kernel_generator.py:134-160)."""
+    ax = axes(H=7, W=51)
+    x = ng.placeholder(ax)
+    xv = rng.uniform(-1, 1, ax)
+    with executor(ng.tanh(x) * 3, x) as f:
+        a = f(xv).copy()
+        b = f(xv)
+    np.testing.assert_array_equal(a, b)
+
+
+def test_views_reorder_slice_flatten(backend):
+    C, H, N = ng.make_axis(4, name="C"), ng.make_axis(6, name="H"), ng.make_axis(5, name="N")
+    x = ng.placeholder([C, H, N])
+    xv = rng.uniform(-1, 1, x.axes)
+    t = ng.axes_with_order(x, [N, C, H])
+    s = ng.tensor_slice(x, [slice(1, 3), slice(None), 2])
+    fl = ng.flatten(x, ng.make_axes([C, ng.make_axes([H, N]).flatten(force=True)]))
+    with executor([t * 2, s + 1, ng.sum(fl, out_axes=[C])], x) as f:
+        tv, sv, fv = f(xv)
+    np.testing.assert_allclose(tv, xv.transpose(2, 0, 1) * 2, rtol=RTOL)
+    np.testing.assert_allclose(sv, xv[1:3, :, 2] + 1, rtol=RTOL)
+    np.testing.assert_allclose(fv, xv.reshape(4, -1).sum(axis=1), rtol=1e-5)
+
+
+def test_transposed_flatten_needs_copy(backend):
+    C, H = ng.make_axis(6, name="C"), ng.make_axis(10, name="H")
+    x = ng.placeholder([C, H])
+    xv = rng.uniform(-1, 1, x.axes)
+    y = ng.flatten(ng.axes_with_order(x, [H, C]))       # not a view: a device copy is inserted
+    with executor(y * 2, x) as f:
+        np.testing.assert_allclose(f(xv), xv.T.reshape(-1) * 2, rtol=RTOL)
+
+
+def test_assign_and_sequential_state(backend):
+    """State persists across calls; sequential orders reads after writes."""
+    ax = axes(H=5)
+    w = ng.variable(ax, initial_value=np.arange(5, dtype=np.float32))
+    x = ng.placeholder(ax)
+    step = ng.sequential([ng.assign(w, w + x), w * 1.0])
+    with executor(step, x) as f:
+        ones = np.ones(5, dtype=np.float32)
+        np.testing.assert_allclose(f(ones), np.arange(5) + 1)
+        np.testing.assert_allclose(f(ones), np.arange(5) + 2)
+        np.testing.assert_allclose(f(2 * ones), np.arange(5) + 4)
+
+
+def test_onehot(backend):
+    C, N = ng.make_axis(5, name="C"), ng.make_axis(11, name="N")
+    x = ng.placeholder([N])
+    xv = np.array([0, 1, 2, 3, 4, 4, 3, 2, 1, 0, 2], dtype=np.float32)
+    with executor(ng.one_hot(x, axis=C), x) as f:
+        np.testing.assert_array_equal(f(xv), np.eye(5, dtype=np.float32)[:, xv.astype(int)])
+
+
+def test_softmax_and_simple_prune(backend):
+    C, N = ng.make_axis(10, name="C"), ng.make_axis(6, name="N")
+    x = ng.placeholder([C, N])
+    xv = rng.uniform(-3, 3, x.axes)
+    sm = ng.softmax(x, normalization_axes=ng.make_axes([C]))
+    pruned = (x * 1 + 0) * -1 + ng.log(ng.exp(x))       # == 0 after SimplePrune
+    with executor([sm, pruned], x) as f:
+        smv, pv = f(xv)
+    e = np.exp(xv - xv.max(axis=0))
+    np.testing.assert_allclose(smv, e / e.sum(axis=0), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(pv, np.zeros_like(xv), atol=1e-6)
+
+
+def test_computation_return_shapes_and_errors(backend):
+    ax = axes(H=3)
+    x, y = ng.placeholder(ax), ng.placeholder(ax)
+    t = ngt.make_transformer()
+    a, b = x + y, x * y
+    f_seq = t.computation([a, b], x, y)
+    f_set = t.computation({a, b}, x, y)
+    f_one = t.computation(a, x, y)
+    xv, yv = np.array([1, 2, 3], np.float32), np.array([4, 5, 6], np.float32)
+    r = f_seq(xv, yv)
+    assert isinstance(r, tuple) and len(r) == 2
+    d = f_set(xv, yv)
+    assert set(d.keys()) == {a, b}
+    np.testing.assert_allclose(d[b], xv * yv)
+    np.testing.assert_allclose(f_one(feed_dict={x: xv, y: yv}), xv + yv)
+    with pytest.raises(ValueError):
+        f_one(xv)                                # wrong argument count
+    with pytest.raises(ValueError):
+        t.computation(a, x, y)                   # transformer already finalized
+    with pytest.raises(ValueError):
+        ng.computation(a, x)                     # placeholder y not supplied
+    t.close()
