@@ -1,0 +1,73 @@
+"""The four neon formulas that define the fused benchmark graphs.
+
+Only the op sequences are taken over from the reference front end, so the
+graphs the backend fuses are the ones the reference would hand it:
+
+* `batch_norm_train`  ngraph/frontends/neon/layer.py:1242-1257
+* `adam_update`       ngraph/frontends/neon/optimizer.py:446-470
+* `lstm_cell`         ngraph/frontends/neon/layer.py:1630-1647 (gate order i,f,o,g :1615)
+* `rectlin`           ngraph/frontends/neon/activation.py:46
+"""
+import numpy as np
+
+import ngraph_hip as ng
+
+
+def rectlin(x, slope=0):
+    return ng.maximum(x, 0) + slope * ng.minimum(0, x)
+
+
+def batch_norm_train(in_obj, gamma, beta, out_axes, eps=1e-5):
+    """Training-mode normalisation of `in_obj` over every axis not in out_axes.
+
+    Returns (y, xmean, xvar); the caller may also assign running statistics.
+    """
+    out_axes = ng.make_axes(out_axes)
+    red_axes = in_obj.axes - out_axes
+    flat = ng.flatten(ng.axes_with_order(in_obj, out_axes | red_axes),
+                      out_axes | red_axes.flatten(force=True))
+    xmean = ng.mean(flat, out_axes=out_axes)
+    xvar = ng.variance(flat, out_axes=out_axes)
+    y = ng.unflatten(gamma * ((flat - xmean) * ng.reciprocal(ng.sqrt(xvar + eps))) + beta)
+    return y, xmean, xvar
+
+
+class Adam(object):
+    """Adam learning rule; `__call__` advances t, `variable_update` builds one update."""
+
+    def __init__(self, learning_rate=1e-3, beta_1=0.9, beta_2=0.999, epsilon=1e-8):
+        self.lrate = learning_rate
+        self.beta_1 = ng.constant(beta_1, dtype=np.float32)
+        self.beta_2 = ng.constant(beta_2, dtype=np.float32)
+        self.epsilon = epsilon
+        self.t = ng.persistent_tensor(axes=(), initial_value=0)
+        self.step = None
+        self.ell = None
+
+    def __call__(self):
+        self.step = ng.sequential([ng.assign(self.t, self.t + 1), self.t])
+        self.ell = self.lrate * ng.sqrt(1 - self.beta_2 ** self.step) / (1 - self.beta_1 ** self.step)
+        return self.ell
+
+    def variable_update(self, variable, grad, scale_factor=1):
+        m = ng.persistent_tensor(axes=grad.axes, initial_value=0.)
+        v = ng.persistent_tensor(axes=grad.axes, initial_value=0.)
+        updates = ng.sequential([
+            ng.assign(m, m * self.beta_1 + (1 - self.beta_1) * grad),
+            ng.assign(v, v * self.beta_2 + (1 - self.beta_2) * grad * grad),
+            ng.assign(variable,
+                      variable - (scale_factor * self.ell * m) / (ng.sqrt(v) + self.epsilon))
+        ])
+        return updates, m, v
+
+
+def lstm_cell(gates, c_prev, hidden_axis, gate_slices):
+    """Pointwise part of an LSTM step.
+
+    gates: dict k -> pre-activation [H, N] for k in i, f, o, g.
+    Returns (h, c).
+    """
+    act = {k: ng.tanh(gates[k]) if k == "g" else ng.sigmoid(gates[k]) for k in ("i", "f", "o", "g")}
+    c = act["f"] * c_prev + act["i"] * act["g"]
+    h = act["o"] * ng.tanh(c)
+    return h, c

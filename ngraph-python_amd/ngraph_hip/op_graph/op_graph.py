@@ -943,8 +943,9 @@ class AssignableTensorOp(TensorOp):
                 initial_value = initial_value(self.axes)
             if isinstance(initial_value, TensorOp):
                 raise ValueError("initial_value must be a number or array, not an Op")
-            self.initial_value = np.asarray(initial_value, dtype=np.float64 if not isinstance(
-                self.dtype, np.dtype) else self.dtype)
+            # a private copy: later changes to the caller's array must not reach the graph
+            self.initial_value = np.array(initial_value, dtype=np.float64 if not isinstance(
+                self.dtype, np.dtype) else self.dtype, copy=True)
 
     @property
     def is_device_op(self):

@@ -33,7 +33,7 @@ from ngraph_hip.runtime.hiplib import (HipRuntime, HipLibraryError, FusedSpecBui
                                        NGH_MAX_REDUCTIONS)
 from ngraph_hip.transformers.base import (ComputationGraphTransformer, DeviceBufferStorage,
                                           DeviceTensor, UnsupportedTransformerException)
-from ngraph_hip.transformers.passes.passes import SimplePrune, TensorSizeFold
+from ngraph_hip.transformers.passes.passes import SimplePrune, TensorSizeFold, ReductionLayoutPass
 
 # op class -> kernel op name (gputransform.py:129-275)
 _UNARY_NAMES = OrderedDict([
@@ -732,7 +732,7 @@ class HipTransformer(ComputationGraphTransformer):
         super(HipTransformer, self).__init__(**kwargs)
         self.fusion = fusion
         self.kernel_groups = OrderedDict()
-        self.graph_passes = [SimplePrune(), TensorSizeFold()]
+        self.graph_passes = [SimplePrune(), TensorSizeFold(), ReductionLayoutPass()]
 
     # -- dtype mapping ---------------------------------------------------------------------
     def ngh_dtype(self, dtype):

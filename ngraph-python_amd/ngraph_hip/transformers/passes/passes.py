@@ -139,3 +139,34 @@ class TensorSizeFold(PeepholeGraphPass):
     def visit(self, op, *args):
         if isinstance(op, TensorSizeOp):
             self.replace_op(op, constant(float(op.reduction_axes.size)))
+
+
+def axes_merge_to_one(td, axes):
+    """Can `axes` of the view `td` be walked as ONE strided dimension?"""
+    dims = [(a.length, td.full_strides[td.axes.index(a)]) for a in axes if a.length != 1]
+    dims.sort(key=lambda d: -d[1])
+    for (n0, s0), (n1, s1) in zip(dims[:-1], dims[1:]):
+        if s0 != s1 * n1:
+            return False
+    return True
+
+
+class ReductionLayoutPass(PeepholeGraphPass):
+    """Reductions need their reduced axes to form one strided axis.
+
+    When they do not, the operand is first copied into (reduced..., kept...)
+    order; this is the layout conversion the reference inserts as a
+    DimshuffleOp for the same reason (gpulayout.py:861-979,
+    layout_common.py:347-378).
+    """
+
+    def visit(self, op, *args):
+        from ngraph_hip.op_graph.op_graph import ReductionOp
+        if not isinstance(op, ReductionOp) or len(op.reduction_axes) < 2:
+            return
+        x, = args
+        if axes_merge_to_one(x.tensor_description(), op.reduction_axes):
+            return
+        order = op.reduction_axes + (x.axes - op.reduction_axes)
+        new_x = ContiguousOp(axes_with_order(x, order))
+        self.replace_op(op, type(op)(new_x, reduction_axes=op.reduction_axes, dtype=op.dtype))
