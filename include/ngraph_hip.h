@@ -174,6 +174,12 @@ int  ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec);
 int  ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec,
                         int32_t stage, char* name128);
 
+/* How stage `stage` would be launched, without a device (host-side tooling and
+ * tests): out8 = {kernel family (0 streaming, 1 reduce along the contiguous axis,
+ * 2 reduce across it), vector width, spec axis on kernel axes 0,1,2, tail length,
+ * index of the matching pre-built specialisation or -1, reduction segments}.     */
+int  ngh_plan_fused(const ngh_fused_spec* spec, int32_t stage, int32_t* out8);
+
 /* ---- flex statistics: the int32 device words FlexPtrDescription binds
  *      (float_ew2.py:363-374); replaces the manager's allocate/readback
  *      (flexgputransform.py:143-150, 361-366)                                */

@@ -130,7 +130,7 @@ __device__ __forceinline__ void run_ops(const KArgs& k, LdsRegs<V>& rf, Extra& e
 __device__ __forceinline__ void stats_epilogue(const KArgs& k, Extra& ex) {
     for (int s = 0; s < k.n_stat_slots; ++s) {
         int m = wave_max_int(ex.geti(ex_stat(s)));
-        if ((threadIdx.x & 63) == 0 && m > 0) atomicMax(k.stat_ptr[s], m);
+        if ((threadIdx.x & 63) == 0 && m > 0 && k.stat_ptr[s] != nullptr) atomicMax(k.stat_ptr[s], m);
     }
 }
 

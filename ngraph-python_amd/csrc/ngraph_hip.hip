@@ -182,6 +182,7 @@ struct Plan {
     unsigned n_bx = 0;
     int      special = -1;                        // index into the specialised-kernel table
     long long tail = 0;                           // 1-D contiguous stage: elements left to a scalar launch
+    int      perm[3] = {0, 1, 2};                 // kernel axis j holds spec axis perm[j]
 };
 
 // Which tensors does the stage touch (load or store or reduce into)?
@@ -221,7 +222,7 @@ void fill_kargs(const ngh_fused_spec& sp, const ngh_stage& S, const int perm[3],
         K.stats = T.dev_stats;
         K.dscale = T.dev_scale;
         K.stat_slot = -1;
-        if (stores[t] && T.dtype == NGH_FLEX16 && T.dev_stats && k.n_stat_slots < 4) {
+        if (stores[t] && T.dtype == NGH_FLEX16 && k.n_stat_slots < 4) {
             K.stat_slot = k.n_stat_slots;
             k.stat_ptr[k.n_stat_slots++] = T.dev_stats;
         }
@@ -274,6 +275,7 @@ int plan_stage(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan
         for (int a = 0; a < 3; ++a) if (a != best) perm[j++] = a;
         perm[2] = best;
         fill_kargs(sp, S, perm, P.k);
+        for (int a = 0; a < 3; ++a) P.perm[a] = perm[a];
         P.family = F_EW;
         P.V = vec4_ok(P.k, used) ? 4 : 1;
         P.tail = 0;
@@ -319,11 +321,12 @@ int plan_stage(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan
     }
     const long long n_out = sp.shape[1] * sp.shape[2];
     if (n_out >= (1LL << 31) || R >= (1LL << 31)) return fail(NGH_E_UNSUPPORTED, "reduction extents exceed 2^31");
-    const int target_wgs = ctx->cus * 8;
+    const int target_wgs = (ctx ? ctx->cus : 256) * 8;
     if (out_contig_axis >= 0) {
         const int other = (out_contig_axis == 2) ? 1 : 2;
         const int perm[3] = {0, other, out_contig_axis};
         fill_kargs(sp, S, perm, P.k);
+        for (int a = 0; a < 3; ++a) P.perm[a] = perm[a];
         P.family = F_RED_COL;
         P.V = 1;
         P.n_out = (unsigned)n_out;
@@ -338,6 +341,7 @@ int plan_stage(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan
     } else {
         const int perm[3] = {1, 2, 0};
         fill_kargs(sp, S, perm, P.k);
+        for (int a = 0; a < 3; ++a) P.perm[a] = perm[a];
         P.family = F_RED_ROW;
         P.V = (r_contig && vec4_ok(P.k, used)) ? 4 : 1;
         P.n_out = (unsigned)n_out;
@@ -374,6 +378,24 @@ int ensure_ws(ngh_context* ctx, size_t bytes) {
     return NGH_OK;
 }
 
+// The last (length % 4) elements of a contiguous 1-D stage, one element per lane.
+int launch_tail(ngh_context* ctx, const Plan& P) {
+    KArgs kt = P.k;
+    const long long body = P.k.shape[2];
+    kt.shape[2] = P.tail;
+    for (int t = 0; t < kt.n_tensors; ++t) kt.t[t].p += body * kt.t[t].s[2] * itemsize_of(kt.t[t].dtype);
+    // IOTA along the split axis would restart at 0 in the tail
+    for (int pc = kt.op_begin; pc < kt.op_end; ++pc)
+        if (kt.ops[pc].opcode == NGH_OP_IOTA && kt.iota_map[kt.ops[pc].a] == 2)
+            return fail(NGH_E_UNSUPPORTED, "IOTA along a split 1-D axis");
+    const size_t lds = interp_lds_bytes(kt, 1);
+    if (lds > kInterpLdsMax) return fail(NGH_E_UNSUPPORTED, "program needs %zu bytes of LDS registers", lds);
+    hipLaunchKernelGGL(ew_interp_kernel<1>, dim3(1), dim3(kBlock), lds, ctx->stream, kt, (unsigned)P.tail,
+                       (unsigned)P.tail);
+    HIP_TRY(hipGetLastError());
+    return NGH_OK;
+}
+
 int launch_interp(ngh_context* ctx, Plan& P) {
     int V = P.V;
     size_t lds = interp_lds_bytes(P.k, V);
@@ -405,19 +427,7 @@ int launch_interp(ngh_context* ctx, Plan& P) {
                 hipLaunchKernelGGL(ew_interp_kernel<1>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, P.n_chunks, P.chunks_per_row);
             HIP_TRY(hipGetLastError());
         }
-        if (P.tail) {
-            KArgs kt = k;
-            const long long body = k.shape[2];
-            kt.shape[2] = P.tail;
-            for (int t = 0; t < kt.n_tensors; ++t) kt.t[t].p += body * kt.t[t].s[2] * itemsize_of(kt.t[t].dtype);
-            // IOTA along the split axis would restart at 0 in the tail
-            for (int pc = kt.op_begin; pc < kt.op_end; ++pc)
-                if (kt.ops[pc].opcode == NGH_OP_IOTA && kt.iota_map[kt.ops[pc].a] == 2)
-                    return fail(NGH_E_UNSUPPORTED, "IOTA along a split 1-D axis");
-            hipLaunchKernelGGL(ew_interp_kernel<1>, dim3(1), dim3(kBlock), interp_lds_bytes(kt, 1), ctx->stream, kt,
-                               (unsigned)P.tail, (unsigned)P.tail);
-            HIP_TRY(hipGetLastError());
-        }
+        if (P.tail) NGH_TRY(launch_tail(ctx, P));
         return NGH_OK;
     }
     if (P.n_out == 0) return NGH_OK;
@@ -651,8 +661,10 @@ int ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec) {
         if (!ctx->force_interp) {
             P.special = match_special(P.family, P.V, P.k, P.tail);
             if (P.special >= 0) {
-                hipError_t e = launch_special(P.special, ctx->stream, ctx->cus, P.k, P.n_chunks, P.chunks_per_row);
+                hipError_t e = launch_special(P.special, ctx->stream, ctx->cus, ctx->ew_blocks_per_cu, P.k,
+                                              P.n_chunks, P.chunks_per_row);
                 if (e != hipSuccess) return fail(NGH_E_RUNTIME, "special launch: %s", hipGetErrorString(e));
+                if (P.tail) NGH_TRY(launch_tail(ctx, P));
                 continue;
             }
         }
@@ -669,6 +681,20 @@ int ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec, int32_t sta
     NGH_TRY(plan_stage(ctx, *spec, stage, P));
     if (!ctx->force_interp) P.special = match_special(P.family, P.V, P.k, P.tail);
     describe(P, name128, 128);
+    return NGH_OK;
+}
+
+int ngh_plan_fused(const ngh_fused_spec* spec, int32_t stage, int32_t* out8) {
+    if (!out8) return fail(NGH_E_INVALID, "out8 is NULL");
+    NGH_TRY(validate(spec));
+    if (stage < 0 || stage >= spec->n_stages) return fail(NGH_E_INVALID, "stage %d", stage);
+    Plan P;
+    NGH_TRY(plan_stage(nullptr, *spec, stage, P));
+    out8[0] = (int)P.family; out8[1] = P.V;
+    out8[2] = P.perm[0]; out8[3] = P.perm[1]; out8[4] = P.perm[2];
+    out8[5] = (int)P.tail;
+    out8[6] = match_special(P.family, P.V, P.k, P.tail);
+    out8[7] = (int)P.n_seg;
     return NGH_OK;
 }
 

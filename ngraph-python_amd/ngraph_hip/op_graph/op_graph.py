@@ -173,6 +173,10 @@ class Op(object):
     def is_scalar(self):
         return False
 
+    @property
+    def tensor(self):
+        return self
+
     # -- state tracking ----------------------------------------------------------------
     @property
     def states_read(self):
@@ -584,7 +588,9 @@ class ValueOp(TensorOp, ControlBlockOp):
 
     @property
     def dtype(self):
-        return self.tensor.dtype if self._tensor is not None else default_dtype(None)
+        if self._tensor is not None and self.tensor.is_tensor_op:
+            return self.tensor.dtype
+        return default_dtype(None)
 
     @dtype.setter
     def dtype(self, dtype):

@@ -1,3 +1,3 @@
 from ngraph_hip.runtime.hiplib import (  # noqa: F401
-    HipLibraryError, HipRuntime, FusedSpecBuilder, load_library, library_path, OPCODES,
+    HipLibraryError, HipRuntime, DryRunRuntime, FusedSpecBuilder, load_library, library_path, OPCODES,
     NGH_F32, NGH_FLEX16, NGH_I32, NGH_F16)

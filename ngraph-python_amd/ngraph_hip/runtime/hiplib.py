@@ -100,6 +100,7 @@ _SYMBOLS = {
     "ngh_validate_fused": [ctypes.POINTER(ngh_fused_spec)],
     "ngh_launch_fused": [_vp, ctypes.POINTER(ngh_fused_spec)],
     "ngh_describe_fused": [_vp, ctypes.POINTER(ngh_fused_spec), _i32, ctypes.c_char_p],
+    "ngh_plan_fused": [ctypes.POINTER(ngh_fused_spec), _i32, ctypes.POINTER(ctypes.c_int32)],
     "ngh_stats_alloc": [_vp, _i32, ctypes.POINTER(_vp)],
     "ngh_stats_reset": [_vp, _vp, _i32],
     "ngh_stats_read": [_vp, _vp, _i32, _vp],
@@ -133,6 +134,15 @@ def load_library():
                               % (lib.ngh_abi_version(), NGH_ABI_VERSION))
     _lib = lib
     return lib
+
+
+def plan_fused(spec, stage=0):
+    """(family, V, perm, tail, special index, segments) the library would use for a stage."""
+    lib = load_library()
+    out = (ctypes.c_int32 * 8)()
+    _check(lib, lib.ngh_plan_fused(ctypes.byref(spec), int(stage), out))
+    return {"family": out[0], "V": out[1], "perm": (out[2], out[3], out[4]), "tail": out[5],
+            "special": out[6], "segments": out[7]}
 
 
 def exported_symbols():
@@ -301,6 +311,60 @@ class HipRuntime(object):
         ms = ctypes.c_float()
         _check(self.lib, self.lib.ngh_timer_end(self.ctx, ctypes.byref(ms)))
         return ms.value
+
+
+class DryRunRuntime(object):
+    """Stands in for HipRuntime where no device exists: hands out fake, aligned device
+    addresses and records launches.  It lets the host-side lowering (graph -> kernel specs)
+    run and be validated by the library on a machine without a GPU; it computes nothing,
+    and reading results through it raises."""
+
+    def __init__(self):
+        self.lib = load_library()
+        self._next = 1 << 32
+        self.launched = []
+
+    def close(self):
+        pass
+
+    def sync(self):
+        pass
+
+    def malloc(self, nbytes):
+        ptr = self._next
+        self._next += (int(nbytes) + 255) // 256 * 256 + 256
+        return ptr
+
+    def free(self, ptr):
+        pass
+
+    def memcpy_h2d(self, dev, host):
+        pass
+
+    def memcpy_d2h(self, host, dev):
+        raise HipLibraryError(-5, "dry-run runtime holds no data")
+
+    def copy_strided(self, *args):
+        pass
+
+    def validate_fused(self, spec):
+        _check(self.lib, self.lib.ngh_validate_fused(ctypes.byref(spec)))
+
+    def launch_fused(self, spec):
+        self.validate_fused(spec)
+        self.launched.append(spec)
+
+    def describe_fused(self, spec, stage=0):
+        return "dry-run"
+
+    def stats_alloc(self, n):
+        return self.malloc(4 * n)
+
+    def stats_reset(self, dev, n=1):
+        pass
+
+    def stats_read(self, dev, n=1):
+        raise HipLibraryError(-5, "dry-run runtime holds no data")
 
 
 class FusedSpecBuilder(object):

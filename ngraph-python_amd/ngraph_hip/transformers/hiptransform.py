@@ -27,13 +27,14 @@ import numpy as np
 
 from ngraph_hip.op_graph import op_graph as og
 from ngraph_hip.op_graph.op_graph import Op, OrderedSet
-from ngraph_hip.runtime.hiplib import (HipRuntime, HipLibraryError, FusedSpecBuilder, NGH_F32,
+from ngraph_hip.runtime.hiplib import (HipRuntime, DryRunRuntime, HipLibraryError, FusedSpecBuilder, NGH_F32,
                                        NGH_FLEX16, NGH_I32, NGH_F16, NGH_MAX_TENSORS,
                                        NGH_MAX_OPS, NGH_MAX_CONSTS, NGH_MAX_REGS,
                                        NGH_MAX_REDUCTIONS)
 from ngraph_hip.transformers.base import (ComputationGraphTransformer, DeviceBufferStorage,
                                           DeviceTensor, UnsupportedTransformerException)
-from ngraph_hip.transformers.passes.passes import SimplePrune, TensorSizeFold, ReductionLayoutPass
+from ngraph_hip.transformers.passes.passes import (SimplePrune, TensorSizeFold,
+                                                   ReductionLayoutPass, ConstantFoldPass)
 
 # op class -> kernel op name (gputransform.py:129-275)
 _UNARY_NAMES = OrderedDict([
@@ -571,6 +572,24 @@ class HipKernelGroup(object):
             k.execute()
             self.after_kernel_execute(k)
 
+    def profile(self, repeats=1):
+        """Run the group `repeats` times with every kernel bracketed by HIP events on the
+        launch stream; returns [(kernel, [ms per run])].  Serialises the kernels, so use it
+        for per-kernel durations, not for end-to-end time."""
+        rt = self.transformer.runtime
+        for k in self.kernels:
+            if not k.buffers_bound:
+                k.bind_buffers()
+        times = [[] for _ in self.kernels]
+        for _ in range(repeats):
+            for i, k in enumerate(self.kernels):
+                self.setup_kernel_execute(k)
+                rt.timer_begin()
+                k.execute()
+                times[i].append(rt.timer_end())
+                self.after_kernel_execute(k)
+        return list(zip(self.kernels, times))
+
 
 # =============================================================================== fusion
 class FusionPlanner(object):
@@ -583,28 +602,98 @@ class FusionPlanner(object):
     different view, or when the kernel's operand / op / constant limits are hit.
     """
 
+    small_tensor = 65536
+
     def __init__(self, transformer, fusion=True):
         self.transformer = transformer
         self.fusion = fusion
 
     def plan(self, ordered_ops, readers, returned):
+        """List-schedule the ops: any dependency-respecting order is legal, so among the
+        device ops that are ready prefer one the open group accepts.  Views, reads of state
+        and sequencing ops cost nothing and are released as soon as they are ready."""
+        ops = [op.forwarded for op in ordered_ops]
+        position = {op: i for i, op in enumerate(ops)}
+        pending, users = {}, {}
+        for op in ops:
+            deps = [d for d in op.all_deps if d in position]
+            pending[op] = len(deps)
+            for d in deps:
+                users.setdefault(d, []).append(op)
+        # device-op level dependencies, seen through views / reads / sequencing ops
+        dev_deps, dev_users = {}, {}
+        for op in ops:
+            acc = set()
+            for d in op.all_deps:
+                if d not in position:
+                    continue
+                if d.is_device_op:
+                    acc.add(d)
+                else:
+                    acc |= dev_deps.get(d, set())
+            dev_deps[op] = acc
+            if op.is_device_op:
+                for d in acc:
+                    dev_users.setdefault(d, set()).add(op)
+        ready = [op for op in ops if pending[op] == 0]
+        scheduled = set()
         groups, cur = [], None
-        for op in ordered_ops:
-            op = op.forwarded
-            if not op.is_device_op:
+
+        def release(op):
+            scheduled.add(op)
+            for u in users.get(op, ()):
+                pending[u] -= 1
+                if pending[u] == 0:
+                    ready.append(u)
+
+        def timely(op):
+            """True unless every consumer of `op` still waits for something else: running such
+            an op now would only park its result in memory until the consumer can run."""
+            if isinstance(op, (og.ReductionOp, og.AssignOp, og.Fill)) or not op.is_tensor_op:
+                return True
+            if iteration_axes(op).size <= self.small_tensor:
+                return True            # parking a small result costs nothing worth a split
+            consumers = dev_users.get(op, ())
+            if not consumers:
+                return True
+            for y in consumers:
+                if all(d is op or d in scheduled or d in ready for d in dev_deps[y]):
+                    return True
+            return False
+
+        def size(op):
+            return iteration_axes(op).size if is_fusable(op) else 0
+
+        while ready:
+            free = [op for op in ready if not op.is_device_op]
+            if free:
+                for op in free:
+                    ready.remove(op)
+                    release(op)
                 continue
-            if not is_fusable(op):
+            ready.sort(key=lambda op: position[op])
+            pick = None
+            if cur is not None and self.fusion:
+                for op in ready:
+                    if is_fusable(op) and timely(op) and cur.accepts(op, readers, returned):
+                        pick = op
+                        break
+            if pick is None:
+                # seed of the next group: a timely op if there is one, smallest space first
+                # (scalars tend to be what the big kernels are waiting for)
+                seeds = [op for op in ready if timely(op)] or ready
+                pick = min(seeds, key=lambda op: (size(op), position[op])) if self.fusion else ready[0]
                 if cur:
                     groups.append(cur)
                     cur = None
-                groups.append(_Group(op, fusable=False))
-                continue
-            if cur is not None and self.fusion and cur.accepts(op):
-                cur.add(op)
+                if is_fusable(pick):
+                    cur = _Group(pick)
+                else:
+                    groups.append(_Group(pick, fusable=False))
             else:
-                if cur:
-                    groups.append(cur)
-                cur = _Group(op)
+                cur.add(pick)
+            ready.remove(pick)
+            release(pick)
         if cur:
             groups.append(cur)
         for g in groups:
@@ -660,7 +749,31 @@ class _Group(object):
             self.red_axes = op.reduction_axes
             self.n_reds += 1
 
-    def accepts(self, op):
+    def _memory_operands(self, candidate, readers, returned):
+        """Operand slots the kernel would need with `candidate` added: buffers read from
+        outside the group plus results something outside the group can see."""
+        ops = self.ops + [candidate]
+        inside = set(ops)
+        produced = set()
+        for op in ops:
+            if op.is_tensor_op and not isinstance(op, (og.AssignOp, og.Fill)):
+                produced.add(op.tensor_description().base)
+        views = set()
+        for op in ops:
+            reads, writes = self._operand_views(op)
+            for td in reads:
+                if td.base not in produced:
+                    views.add(_view_key(td))
+            if isinstance(op, (og.AssignOp, og.Fill)):
+                views.update(_view_key(td) for td in writes)
+            else:
+                base = op.tensor_description().base
+                if base in returned or isinstance(op, og.ReductionOp) or \
+                        any(u not in inside for u in readers.get(base, ())):
+                    views.add(_view_key(op.tensor_description()))
+        return len(views)
+
+    def accepts(self, op, readers, returned):
         if not iteration_axes(op).is_equal_set(self.axes) or \
                 iteration_axes(op).lengths != tuple(self.axes[self.axes.index(a)].length
                                                     for a in iteration_axes(op)):
@@ -687,8 +800,7 @@ class _Group(object):
         if is_red:
             # a reduction reads its argument through registers; its output must not be re-read here
             pass
-        bases = set(self.read_views) | set(self.write_views) | set(td.base for td in reads + writes)
-        if len(bases) + 2 > NGH_MAX_TENSORS:
+        if self._memory_operands(op, readers, returned) > NGH_MAX_TENSORS:
             return False
         if self.n_ops + 4 > NGH_MAX_OPS or self.n_consts + 2 > NGH_MAX_CONSTS:
             return False
@@ -724,15 +836,18 @@ class HipTransformer(ComputationGraphTransformer):
 
     kernel_group_class = HipKernelGroup
 
-    def __init__(self, device_id=0, fusion=True, **kwargs):
+    def __init__(self, device_id=0, fusion=True, dry_run=False, **kwargs):
+        """dry_run=True lowers graphs to kernel specs without a device (no results can be
+        read back); it exists so the host-side lowering can be inspected and tested."""
         try:
-            self.runtime = HipRuntime(device_id)
+            self.runtime = DryRunRuntime() if dry_run else HipRuntime(device_id)
         except HipLibraryError as e:
             raise UnsupportedTransformerException("hipgpu needs libngraph_hip.so and an MI355X: %s" % e)
         super(HipTransformer, self).__init__(**kwargs)
         self.fusion = fusion
         self.kernel_groups = OrderedDict()
-        self.graph_passes = [SimplePrune(), TensorSizeFold(), ReductionLayoutPass()]
+        self.graph_passes = [SimplePrune(), TensorSizeFold(), ConstantFoldPass(), SimplePrune(),
+                             ReductionLayoutPass()]
 
     # -- dtype mapping ---------------------------------------------------------------------
     def ngh_dtype(self, dtype):

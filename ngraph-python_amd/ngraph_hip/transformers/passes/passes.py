@@ -170,3 +170,38 @@ class ReductionLayoutPass(PeepholeGraphPass):
         order = op.reduction_axes + (x.axes - op.reduction_axes)
         new_x = ContiguousOp(axes_with_order(x, order))
         self.replace_op(op, type(op)(new_x, reduction_axes=op.reduction_axes, dtype=op.dtype))
+
+
+class ConstantFoldPass(PeepholeGraphPass):
+    """Elementwise ops on scalar constants are evaluated at transform time.
+
+    Such subgraphs ((1 - beta_1), lr * 2, ...) would otherwise each cost a kernel launch per
+    call.  The value is computed in float32 with the NumPy ufunc of the same name, which is
+    what the per-op CPU path does with the same operands (cputransform.py:512-761).
+    """
+
+    _UNARY = {"NegativeOp": np.negative, "AbsoluteOp": np.abs, "SqrtOp": np.sqrt, "ExpOp": np.exp,
+              "LogOp": np.log, "ReciprocalOp": np.reciprocal, "SquareOp": np.square,
+              "TanhOp": np.tanh, "SignOp": np.sign, "SinOp": np.sin, "CosOp": np.cos}
+    _BINARY = {"Add": np.add, "Subtract": np.subtract, "Multiply": np.multiply,
+               "Divide": np.divide, "Power": np.power, "Maximum": np.maximum,
+               "Minimum": np.minimum, "FloorDivide": np.floor_divide, "Mod": np.mod}
+
+    def visit(self, op, *args):
+        name = type(op).__name__
+        if name not in self._UNARY and name not in self._BINARY:
+            return
+        if op.dtype != np.dtype(np.float32):
+            return
+        if name in self._UNARY and len(args) == 1:
+            c = _scalar_const(args[0])
+            if c is not None:
+                with np.errstate(all="ignore"):
+                    val = self._UNARY[name](np.float32(c), dtype=np.float32)
+                self.replace_op(op, constant(float(val), op.axes))
+        elif name in self._BINARY and len(args) == 2:
+            cx, cy = _scalar_const(args[0]), _scalar_const(args[1])
+            if cx is not None and cy is not None:
+                with np.errstate(all="ignore"):
+                    val = self._BINARY[name](np.float32(cx), np.float32(cy), dtype=np.float32)
+                self.replace_op(op, constant(float(val), op.axes))
