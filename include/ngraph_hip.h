@@ -174,6 +174,13 @@ int  ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec);
 int  ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec,
                         int32_t stage, char* name128);
 
+/* Per-row mean and (biased) variance of a [rows, R] fp32 matrix with contiguous rows in ONE
+ * read of x: fuses the reductions behind ng.mean + ng.variance
+ * (op_graph.py:4007-4009, 4252-4266), the statistics of batch normalisation
+ * (frontends/neon/layer.py:1242-1245).  row_stride in elements, multiple of 4.  */
+int  ngh_moments_f32(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t R, int64_t row_stride,
+                     float* dev_mean, float* dev_var);
+
 /* How stage `stage` would be launched, without a device (host-side tooling and
  * tests): out8 = {kernel family (0 streaming, 1 reduce along the contiguous axis,
  * 2 reduce across it), vector width, spec axis on kernel axes 0,1,2, tail length,

@@ -16,6 +16,7 @@
 #include "ngh_interp.h"
 #include "ngh_copy.h"
 #include "ngh_special.h"
+#include "ngh_moments.h"
 
 using namespace ngh;
 
@@ -72,6 +73,7 @@ struct ngh_context {
     size_t      ws_bytes = 0;
     int         ew_blocks_per_cu = 8;
     int         force_interp = 0;    // never pick a specialised kernel
+    int         moments_wgs_per_cu = 16;
     char        name[256] = "";
     uint64_t    total_bytes = 0;
 };
@@ -509,6 +511,7 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     snprintf(ctx->name, sizeof(ctx->name), "%s (%s)", prop.name, prop.gcnArchName);
     ctx->ew_blocks_per_cu = std::max(1, env_int("NGH_EW_BLOCKS_PER_CU", 8));
     ctx->force_interp = env_int("NGH_FORCE_INTERP", 0);
+    ctx->moments_wgs_per_cu = std::max(1, env_int("NGH_MOMENTS_WGS_PER_CU", 16));
     hipError_t e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev0);
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev1);
@@ -681,6 +684,34 @@ int ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec, int32_t sta
     NGH_TRY(plan_stage(ctx, *spec, stage, P));
     if (!ctx->force_interp) P.special = match_special(P.family, P.V, P.k, P.tail);
     describe(P, name128, 128);
+    return NGH_OK;
+}
+
+int ngh_moments_f32(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t R, int64_t row_stride,
+                    float* dev_mean, float* dev_var) {
+    if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
+    if (rows < 0 || R <= 0) return fail(NGH_E_INVALID, "rows %lld, R %lld", (long long)rows, (long long)R);
+    if (rows == 0) return NGH_OK;
+    if (!dev_x || !dev_mean || !dev_var) return fail(NGH_E_INVALID, "NULL device pointer");
+    if (((uintptr_t)dev_x) % 16 || row_stride % 4)
+        return fail(NGH_E_UNSUPPORTED, "rows must start on 16-byte boundaries");
+    if (rows >= (1LL << 24) || R >= (1LL << 32)) return fail(NGH_E_UNSUPPORTED, "extent too large");
+    const unsigned R4 = (unsigned)(R / 4);
+    // enough workgroups to fill the chip, but at least 4 unrolled sweeps per segment
+    long long seg = std::max<long long>(1, (long long)ctx->cus * ctx->moments_wgs_per_cu / rows);
+    seg = std::min<long long>(seg, std::max<long long>(1, R4 / (kMomBlock * kMomUnroll * 2)));
+    seg = std::min<long long>(seg, 4096);
+    const unsigned seg_chunks = (unsigned)((R4 + seg - 1) / seg);
+    const unsigned n_seg = seg_chunks ? (unsigned)((R4 + seg_chunks - 1) / seg_chunks) : 1;
+    const unsigned n_seg_eff = std::max(1u, n_seg);
+    NGH_TRY(ensure_ws(ctx, (size_t)rows * n_seg_eff * sizeof(float2)));
+    float2* partial = (float2*)ctx->ws;
+    hipLaunchKernelGGL(moments_partial_kernel, dim3((unsigned)(rows * n_seg_eff)), dim3(kMomBlock), 0, ctx->stream,
+                       dev_x, (long long)row_stride, R4, n_seg_eff, seg_chunks, partial);
+    HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(moments_finish_kernel, dim3((unsigned)rows), dim3(64), 0, ctx->stream, dev_x,
+                       (long long)row_stride, (unsigned)R, R4 * 4, n_seg_eff, partial, dev_mean, dev_var);
+    HIP_TRY(hipGetLastError());
     return NGH_OK;
 }
 

@@ -100,6 +100,7 @@ _SYMBOLS = {
     "ngh_validate_fused": [ctypes.POINTER(ngh_fused_spec)],
     "ngh_launch_fused": [_vp, ctypes.POINTER(ngh_fused_spec)],
     "ngh_describe_fused": [_vp, ctypes.POINTER(ngh_fused_spec), _i32, ctypes.c_char_p],
+    "ngh_moments_f32": [_vp, _vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, _vp, _vp],
     "ngh_plan_fused": [ctypes.POINTER(ngh_fused_spec), _i32, ctypes.POINTER(ctypes.c_int32)],
     "ngh_stats_alloc": [_vp, _i32, ctypes.POINTER(_vp)],
     "ngh_stats_reset": [_vp, _vp, _i32],
@@ -287,6 +288,11 @@ class HipRuntime(object):
         _check(self.lib, self.lib.ngh_describe_fused(self.ctx, ctypes.byref(spec), int(stage), name))
         return name.value.decode()
 
+    def moments_f32(self, x, rows, R, row_stride, mean, var):
+        _check(self.lib, self.lib.ngh_moments_f32(self.ctx, ctypes.c_void_p(x), int(rows), int(R),
+                                                  int(row_stride), ctypes.c_void_p(mean),
+                                                  ctypes.c_void_p(var)))
+
     # -- flex statistics ---------------------------------------------------
     def stats_alloc(self, n):
         ptr = ctypes.c_void_p()
@@ -356,6 +362,9 @@ class DryRunRuntime(object):
 
     def describe_fused(self, spec, stage=0):
         return "dry-run"
+
+    def moments_f32(self, *args):
+        self.launched.append(("moments",) + args)
 
     def stats_alloc(self, n):
         return self.malloc(4 * n)

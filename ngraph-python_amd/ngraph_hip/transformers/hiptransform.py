@@ -33,7 +33,7 @@ from ngraph_hip.runtime.hiplib import (HipRuntime, DryRunRuntime, HipLibraryErro
                                        NGH_MAX_REDUCTIONS)
 from ngraph_hip.transformers.base import (ComputationGraphTransformer, DeviceBufferStorage,
                                           DeviceTensor, UnsupportedTransformerException)
-from ngraph_hip.transformers.passes.passes import (SimplePrune, TensorSizeFold,
+from ngraph_hip.transformers.passes.passes import (SimplePrune, TensorSizeFold, PeepholeGraphPass,
                                                    ReductionLayoutPass, ConstantFoldPass)
 
 # op class -> kernel op name (gputransform.py:129-275)
@@ -549,6 +549,141 @@ class CopyKernel(HipKernel):
                                               self.dst_strides, self.src_strides, self.dst.itemsize)
 
 
+class MomentsOp(og.TensorOp):
+    """mean and variance of x over `reduction_axes` in one read of x.
+
+    Axes = (K,) + kept axes with K of length 2: row 0 holds the mean, row 1 the (biased)
+    variance.  Introduced by MomentsFusionPass in place of ng.mean + ng.variance
+    (op_graph.py:4007-4009, 4252-4266); consumers read the two rows as slices.
+    """
+
+    def __init__(self, x, reduction_axes, **kwargs):
+        x = og.as_op(x)
+        self.reduction_axes = og.make_axes(reduction_axes)
+        self.kept_axes = x.axes - self.reduction_axes
+        self.k_axis = og.make_axis(2, name="NGH_MOMENT")
+        super(MomentsOp, self).__init__(args=(x,), axes=og.make_axes([self.k_axis]) + self.kept_axes,
+                                        **kwargs)
+
+
+def moments_layout(td, reduction_axes):
+    """(rows, R, row_stride) when `td` is rows x R with contiguous rows over the reduced axes,
+    else None."""
+    red = [(a.length, td.full_strides[td.axes.index(a)]) for a in reduction_axes if a.length != 1]
+    kept = [(a.length, td.full_strides[td.axes.index(a)]) for a in td.axes
+            if a not in reduction_axes and a.length != 1]
+    red.sort(key=lambda d: -d[1])
+    kept.sort(key=lambda d: -d[1])
+    for dims in (red, kept):
+        for (n0, s0), (n1, s1) in zip(dims[:-1], dims[1:]):
+            if s0 != s1 * n1:
+                return None
+    if not red or red[-1][1] != 1:
+        return None
+    R = int(np.prod([n for n, _ in red], dtype=np.int64))
+    rows = int(np.prod([n for n, _ in kept], dtype=np.int64)) if kept else 1
+    row_stride = kept[-1][1] if kept else R
+    if row_stride % 4 or td.offset % 4:
+        return None
+    return rows, R, row_stride
+
+
+class MomentsFusionPass(PeepholeGraphPass):
+    """variance(x) and the mean(x) inside it become one MomentsOp.
+
+    Pattern (after TensorSizeFold): Divide(Sum(Square(Subtract(x, M))), n) with
+    M = Divide(Sum(x), n) over the same axes.  Every other Divide(Sum(x), n) over the same x
+    and axes is the same mean and is redirected to it as well.  Only applied when x is fp32
+    with rows contiguous over the reduced axes (the layout the one-pass kernel handles).
+    """
+
+    @staticmethod
+    def _strip(op):
+        op = op.forwarded
+        while isinstance(op, (og.BroadcastOp, og.ReorderAxes)):
+            op = op.args[0].forwarded
+        return op
+
+    @classmethod
+    def _as_mean(cls, op):
+        """(x, reduction_axes) when op is Divide(Sum(x), const == size of the reduced axes)."""
+        op = cls._strip(op)
+        if not isinstance(op, og.Divide):
+            return None
+        num, den = op.args[0].forwarded, op.args[1].forwarded
+        c = _scalar_constant_value(den)
+        if not isinstance(num, og.Sum) or c is None or c != float(num.reduction_axes.size):
+            return None
+        return num.args[0].forwarded, num.reduction_axes
+
+    @staticmethod
+    def _same_tensor(a, b):
+        ta, tb = a.tensor_description(), b.tensor_description()
+        return ta.base is tb.base and ta.parameter_key == tb.parameter_key and ta.axes == tb.axes
+
+    def do_pass(self, ops, **kwargs):
+        self.moments = []          # (x, reduction axes, mean view, var view)
+        super(MomentsFusionPass, self).do_pass(ops, **kwargs)
+
+    def visit(self, op, *args):
+        if not isinstance(op, og.Divide):
+            return
+        outer = self._as_mean(op)
+        if outer is None:
+            return
+        arg, red_axes = outer
+        # a mean over x that an earlier match already covers
+        for x, axes, mean_view, _ in self.moments:
+            if axes.is_equal_set(red_axes) and self._same_tensor(arg, x):
+                self.replace_op(op, mean_view)
+                return
+        if not isinstance(arg, og.SquareOp):
+            return
+        sub = arg.args[0].forwarded
+        if not isinstance(sub, og.Subtract):
+            return
+        x, m = sub.args[0].forwarded, sub.args[1].forwarded
+        inner = self._as_mean(m)
+        if inner is None:
+            return
+        x2, red2 = inner
+        if not red2.is_equal_set(red_axes) or not self._same_tensor(x, x2):
+            return
+        if x.dtype != np.dtype(np.float32) or moments_layout(x.tensor_description(), red_axes) is None:
+            return
+        mom = MomentsOp(x, red_axes)
+        mean_view = og.slice_along_axis(mom, mom.k_axis, 0)
+        var_view = og.slice_along_axis(mom, mom.k_axis, 1)
+        self.moments.append((x, red_axes, mean_view, var_view))
+        self.replace_op(op, var_view)
+        self.replace_op(self._strip(m), mean_view)
+
+
+class MomentsKernel(HipKernel):
+    def __init__(self, transformer, op):
+        super(MomentsKernel, self).__init__(transformer)
+        self.op = op
+
+    def bind_buffers(self):
+        t = self.transformer
+        x_td = self.op.args[0].forwarded.tensor_description()
+        layout = moments_layout(x_td, self.op.reduction_axes)
+        if layout is None:
+            raise og_unsupported("MomentsOp operand lost its row layout")
+        self.rows, self.R, self.row_stride = layout
+        self.x = t.get_tensor_description_tensor_view(x_td)
+        self.out = t.get_tensor_description_tensor_view(self.op.tensor_description())
+        super(MomentsKernel, self).bind_buffers()
+
+    def execute(self):
+        out = self.out.ptr
+        self.transformer.runtime.moments_f32(self.x.ptr, self.rows, self.R, self.row_stride,
+                                             out, out + self.rows * 4)
+
+    def describe(self):
+        return [["moments_f32"]]
+
+
 class HipKernelGroup(object):
     """The kernels of one computation and the loop that runs them (gputransform.py:348-522)."""
 
@@ -836,7 +971,7 @@ class HipTransformer(ComputationGraphTransformer):
 
     kernel_group_class = HipKernelGroup
 
-    def __init__(self, device_id=0, fusion=True, dry_run=False, **kwargs):
+    def __init__(self, device_id=0, fusion=True, dry_run=False, fuse_moments=None, **kwargs):
         """dry_run=True lowers graphs to kernel specs without a device (no results can be
         read back); it exists so the host-side lowering can be inspected and tested."""
         try:
@@ -846,8 +981,10 @@ class HipTransformer(ComputationGraphTransformer):
         super(HipTransformer, self).__init__(**kwargs)
         self.fusion = fusion
         self.kernel_groups = OrderedDict()
-        self.graph_passes = [SimplePrune(), TensorSizeFold(), ConstantFoldPass(), SimplePrune(),
-                             ReductionLayoutPass()]
+        self.graph_passes = [SimplePrune(), TensorSizeFold(), ConstantFoldPass(), SimplePrune()]
+        if fusion if fuse_moments is None else fuse_moments:
+            self.graph_passes.append(MomentsFusionPass())
+        self.graph_passes.append(ReductionLayoutPass())
 
     # -- dtype mapping ---------------------------------------------------------------------
     def ngh_dtype(self, dtype):
@@ -907,6 +1044,8 @@ class HipTransformer(ComputationGraphTransformer):
                 op = g.ops[0]
                 if isinstance(op, og.ContiguousOp):
                     group.kernels.append(CopyKernel(self, op))
+                elif isinstance(op, MomentsOp):
+                    group.kernels.append(MomentsKernel(self, op))
                 else:
                     raise ValueError("Unhandled op: {}".format(op))
         self.kernel_groups[computation] = group
