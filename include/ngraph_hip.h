@@ -56,6 +56,16 @@ extern "C" {
 #define NGH_I32     2          /* int32 (argmax / argmin results, indices)  */
 #define NGH_F16     3          /* IEEE half in memory, float in registers   */
 
+/* ---- spec flags ---------------------------------------------------------
+ * NGH_SPEC_PROBE: run the program but store NOTHING; instead every FLEX16
+ * tensor the program would write gets, in its dev_stats word, the bit pattern
+ * of max |fp32 value| it would have been asked to store (NaN ignored; compare
+ * as int32).  A flex manager uses one probe launch to choose the first
+ * exponent of a fresh output tensor from its true range, the state the
+ * reference's known-answer vectors show after a tensor's first use
+ * (tests/flex_tests/test_flexew/test_complex_math.py:31,47).                */
+#define NGH_SPEC_PROBE  1
+
 /* ---- opcodes ------------------------------------------------------------
  * One entry per template of float_ew2.py:31-68 (_op_templates) and
  * :70-77 (_redop_templates).  Arithmetic follows the NumPy float32 calls the
@@ -95,11 +105,14 @@ typedef struct ngh_tensor {
     void*    dev;              /* device address of view element (0,0,0)     */
     int64_t  strides[NGH_MAX_AXES];
     int32_t  dtype;            /* NGH_F32 / NGH_FLEX16 / NGH_I32 / NGH_F16   */
-    float    scale;            /* FLEX16 only.  Loaded value = scale * int16;
-                                  stored int16 = rni_sat(value * scale), i.e.
-                                  the caller passes entry.scale for inputs
-                                  and 1/entry.scale for outputs
-                                  (flexgputransform.py:56-61)                */
+    float    scale;            /* FLEX16 only: the tensor's scale 2**-dec.
+                                  Loaded value = scale * int16; stored int16 =
+                                  rni_sat(value * (1/scale)).  The reference
+                                  binds entry.scale to inputs and 1/entry.scale
+                                  to outputs (flexgputransform.py:56-61); one
+                                  field serves both here because 1/scale is
+                                  exact for a power of two, and a tensor
+                                  updated in place needs both directions     */
     int32_t* dev_stats;        /* FLEX16 outputs: int32 max|mantissa| merged
                                   with atomic max (float_ew2.py:281,1404);
                                   NULL = no statistics                       */
@@ -128,6 +141,7 @@ typedef struct ngh_fused_spec {
     int32_t     rank;          /* 1..3; axes beyond rank have length 1       */
     int64_t     shape[NGH_MAX_AXES];
     int32_t     n_tensors, n_ops, n_consts, n_stages, n_regs;
+    int32_t     flags;         /* NGH_SPEC_* bits                            */
     ngh_tensor  tensors[NGH_MAX_TENSORS];
     float       consts[NGH_MAX_CONSTS];
     ngh_op      ops[NGH_MAX_OPS];

@@ -37,6 +37,7 @@ struct KArgs {
     int       red_axis;      // kernel axis the reductions run along (0 or 2), -1 = none
     int       iota_map[3];   // kernel axis holding spec axis k (for NGH_OP_IOTA)
     int       n_stat_slots;
+    int       probe;         // NGH_SPEC_PROBE: record max|value| bits instead of storing
     int*      stat_ptr[4];   // device word of each per-thread accumulator
     KTensor   t[NGH_MAX_TENSORS];
     float     consts[NGH_MAX_CONSTS];
@@ -145,6 +146,11 @@ __device__ __forceinline__ int flex_quantize(float v) {
 }
 
 __device__ __forceinline__ int iabs(int x) { return x < 0 ? -x : x; }
+
+// bit pattern of |v| (ordered like the value for non-negative floats); NaN counts as 0
+__device__ __forceinline__ int probe_bits(float v) {
+    return (v != v) ? 0 : (__float_as_int(v) & 0x7fffffff);
+}
 
 // ---------------------------------------------------------------------------
 // Element access by storage type.

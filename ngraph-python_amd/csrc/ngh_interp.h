@@ -61,9 +61,12 @@ __device__ __forceinline__ void run_ops(const KArgs& k, LdsRegs<V>& rf, Extra& e
             case NGH_OP_STORE: {
                 const KTensor& t = k.t[o.dst];
                 const long long off = i0 * t.s[0] + i1 * t.s[1] + i2 * t.s[2];
-                const float sc = (t.dtype == NGH_FLEX16) ? tensor_scale(t) : 1.0f;
+                const float sc = (t.dtype == NGH_FLEX16) ? 1.0f / tensor_scale(t) : 1.0f;
                 int fmax = 0;
-                if (V == 4 && t.s[2] == 1) {
+                if (k.probe) {
+#pragma unroll
+                    for (int v = 0; v < V; ++v) fmax = max(fmax, probe_bits(rf.get(o.a, v)));
+                } else if (V == 4 && t.s[2] == 1) {
                     float x[4];
 #pragma unroll
                     for (int v = 0; v < 4; ++v) x[v] = rf.get(o.a, v);
@@ -171,9 +174,14 @@ __device__ __forceinline__ void red_emit(const KArgs& k, int slot, Acc a, long l
     if (n_seg == 1) {
         const KTensor& t = k.t[k.red_out[slot]];
         const long long off = o0 * t.s[0] + o1 * t.s[1] + o2 * t.s[2];
-        const float sc = (t.dtype == NGH_FLEX16) ? tensor_scale(t) : 1.0f;
+        const float sc = (t.dtype == NGH_FLEX16) ? 1.0f / tensor_scale(t) : 1.0f;
+        const float result = acc_result(k.ops[k.op_end - k.n_red + slot].opcode, a);
         int fmax = 0;
-        store1(t, off, acc_result(k.ops[k.op_end - k.n_red + slot].opcode, a), sc, fmax);
+        if (k.probe) {
+            if (t.dtype == NGH_FLEX16) fmax = probe_bits(result);
+        } else {
+            store1(t, off, result, sc, fmax);
+        }
         if (t.stats != nullptr && fmax > 0) atomicMax(t.stats, fmax);
     } else {
         const size_t w = ((size_t)slot * n_seg + seg) * n_out + out;

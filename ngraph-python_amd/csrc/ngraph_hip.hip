@@ -210,6 +210,7 @@ void fill_kargs(const ngh_fused_spec& sp, const ngh_stage& S, const int perm[3],
     k.n_regs = sp.n_regs;
     k.n_red = S.n_reductions;
     k.red_axis = -1;
+    k.probe = (sp.flags & NGH_SPEC_PROBE) ? 1 : 0;
     for (int r = 0; r < S.n_reductions; ++r) k.red_out[r] = S.red_out[r];
     if (S.n_reductions) k.red_axis = k.iota_map[0];
     bool loads[NGH_MAX_TENSORS], stores[NGH_MAX_TENSORS];
@@ -661,7 +662,7 @@ int ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec) {
         if (spec->stages[s].op_end == spec->stages[s].op_begin) continue;
         Plan P;
         NGH_TRY(plan_stage(ctx, *spec, s, P));
-        if (!ctx->force_interp) {
+        if (!ctx->force_interp && !P.k.probe) {
             P.special = match_special(P.family, P.V, P.k, P.tail);
             if (P.special >= 0) {
                 hipError_t e = launch_special(P.special, ctx->stream, ctx->cus, ctx->ew_blocks_per_cu, P.k,

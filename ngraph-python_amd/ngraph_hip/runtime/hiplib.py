@@ -22,6 +22,7 @@ NGH_MAX_REDUCTIONS = 4
 NGH_MAX_STAGES = 6
 
 NGH_F32, NGH_FLEX16, NGH_I32, NGH_F16 = 0, 1, 2, 3
+NGH_SPEC_PROBE = 1
 
 _OPCODE_NAMES = [
     "nop", "load", "store", "const", "iota",
@@ -65,6 +66,7 @@ class ngh_fused_spec(ctypes.Structure):
                 ("n_tensors", ctypes.c_int32), ("n_ops", ctypes.c_int32),
                 ("n_consts", ctypes.c_int32), ("n_stages", ctypes.c_int32),
                 ("n_regs", ctypes.c_int32),
+                ("flags", ctypes.c_int32),
                 ("tensors", ngh_tensor * NGH_MAX_TENSORS),
                 ("consts", ctypes.c_float * NGH_MAX_CONSTS),
                 ("ops", ngh_op * NGH_MAX_OPS),

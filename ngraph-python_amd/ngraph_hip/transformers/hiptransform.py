@@ -246,8 +246,12 @@ class HipKernel(object):
 
     # flex hooks (flexgputransform.py:56-61, 347-366)
     output_flex_ids = ()
+    output_flex_entries = ()
 
     def bind_flex_scales(self):
+        pass
+
+    def probe(self):
         pass
 
 
@@ -273,6 +277,10 @@ class FusedKernel(HipKernel):
         self.specs = []
         self.flex_bindings = []     # (spec index, tensor slot, flex entry, is_output)
         self.described = None
+
+    def _constant_value(self, value):
+        """The fp32 immediate a scalar constant becomes (a flex kernel quantises it first)."""
+        return value
 
     # -- operand bookkeeping ------------------------------------------------------------
     def bind_buffers(self):
@@ -312,7 +320,7 @@ class FusedKernel(HipKernel):
             c = _scalar_constant_value(arg)
             if c is not None:
                 r = new_reg()
-                program.append(("const", r, c))
+                program.append(("const", r, self._constant_value(c)))
                 return r
             prod = _producer(arg)
             if prod in value_reg:
@@ -1043,7 +1051,7 @@ class HipTransformer(ComputationGraphTransformer):
             else:
                 op = g.ops[0]
                 if isinstance(op, og.ContiguousOp):
-                    group.kernels.append(CopyKernel(self, op))
+                    group.kernels.append(self.make_copy_kernel(op))
                 elif isinstance(op, MomentsOp):
                     group.kernels.append(MomentsKernel(self, op))
                 else:
@@ -1054,6 +1062,9 @@ class HipTransformer(ComputationGraphTransformer):
 
     def make_fused_kernel(self, ops, store_ops, name):
         return FusedKernel(self, ops, store_ops, name)
+
+    def make_copy_kernel(self, op):
+        return CopyKernel(self, op)
 
     def finish_transform(self):
         pass

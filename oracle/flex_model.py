@@ -1,0 +1,223 @@
+"""NumPy model of the reference's flex16 arithmetic and exponent management.
+
+Oracle (test infrastructure).  Two layers:
+
+1. Arithmetic given scales -- fully determined by the reference's device code:
+     load    value = scale * int16                  float_ew2.py:96
+     store   int16 = cvt.rni.s16.f32(value / scale) float_ew2.py:97, 261-267
+             (round to nearest even, saturate to [-32768, 32767], NaN -> 0)
+     stats   max |stored int16| as int32            float_ew2.py:269-281, 1360, 1404
+     host write = value / scale, clip, astype(int16) truncation
+                                                    flexgputransform.py:183-203, gputransform.py:825-829
+     host read  = int16 * scale                     flexgputransform.py:178-181
+     fill       = int(value / scale) clipped        tensor_ops.py:690-707
+   Pinned by brute force over all int16 values and by the single-shot
+   known-answer vectors of tests/flex_tests/test_flexew (exact equality there).
+
+2. Exponent policy (`FlexPolicy`) -- the reference delegates this to the private
+   `autoflex` package (ngraph/flex/__init__.py:1-4), which is not in the tree.
+   PARITY UNPINNED at source level.  The rules below are the simplest ones found
+   that reproduce the reference's multi-iteration known-answer vectors
+   (tests/golden/flex_vectors.json); each rule names the vectors that force it.
+     P1  first host value: tightest fit dec = 14 - floor(log2(max|v|)), clamped to
+         [0, 31]; an all-zero first value gets default_dec = 8
+         (test_flexew_basic_math.py:41-47, 117-121; test_flexew_inequalities.py:58-64).
+     P2  a kernel output's first dec is the tightest fit of its own result
+         (test_flexew_basic_math.py:63; test_complex_math.py:31,47).
+     P3  a stored max|mantissa| >= 32767 is an overflow: dec -= 2 for the next use
+         (test_flexew_basic_math.py:43-47; test_flexew_inequalities.py:58-64).
+     P4  otherwise dec = tightest fit of  max(h) + 3 * std(h)  over the last 16
+         recorded max|value|, an overflow being recorded as twice the saturated value
+         (test_flexew_basic_math.py:68-72, 79-83, 117-143, 175-181).
+"""
+from __future__ import division
+import collections
+import math
+
+import numpy as np
+
+f32 = np.float32
+
+DEFAULT_DEC = 8          # ngraph/flex/base.py:89
+MIN_DEC, MAX_DEC = 0, 31  # 5 exponent bits (ngraph/flex/base.py:24-33)
+PCLIP, NCLIP = 32767, -32768
+WINDOW = 16
+GAMMA = 3.0
+
+
+# ---------------------------------------------------------------------------------- arithmetic
+def scale_of(dec):
+    return 2.0 ** (-dec)
+
+
+def quantize_rni(values, dec):
+    """Kernel store: int16 = rni_sat(float32(value) * float32(2**dec))."""
+    v = np.asarray(values, dtype=f32)
+    with np.errstate(all="ignore"):
+        scaled = v * f32(2.0 ** dec)
+        r = np.rint(scaled)                        # round half to even
+        r = np.where(np.isnan(r), f32(0), r)
+        r = np.clip(r, NCLIP, PCLIP)
+    return r.astype(np.int16)
+
+
+def dequantize(mantissa, dec):
+    """Kernel load / host read: float32(scale) * float32(int16)."""
+    return (f32(scale_of(dec)) * np.asarray(mantissa).astype(f32)).astype(f32)
+
+
+def quantize_host(values, dec):
+    """Host write: value / scale, clip, truncate toward zero."""
+    v = np.asarray(values, dtype=np.float64) / scale_of(dec)
+    v = np.clip(v, NCLIP, PCLIP)
+    return v.astype(np.int16)                      # astype truncates
+
+
+def maxabs(mantissa):
+    m = np.asarray(mantissa).astype(np.int32)
+    return int(np.max(np.abs(m))) if m.size else 0
+
+
+def fit_dec(value):
+    """Largest dec in [MIN_DEC, MAX_DEC] at which |value| still fits 15 bits."""
+    value = abs(float(value))
+    if value == 0.0 or math.isnan(value):
+        return None
+    if math.isinf(value):
+        return MIN_DEC
+    dec = 14 - int(math.floor(math.log2(value)))
+    return max(MIN_DEC, min(MAX_DEC, dec))
+
+
+# ---------------------------------------------------------------------------------- policy
+class FlexPolicy(object):
+    """Exponent state of one tensor."""
+
+    def __init__(self):
+        self.dec = DEFAULT_DEC
+        self.initialized = False
+        self.history = collections.deque(maxlen=WINDOW)
+
+    @property
+    def scale(self):
+        return scale_of(self.dec)
+
+    def init_from_value(self, max_abs_value):
+        """P1 / P2: first use."""
+        d = fit_dec(max_abs_value)
+        self.dec = DEFAULT_DEC if d is None else d
+        self.initialized = True
+
+    def record(self, max_mantissa):
+        """After a write with the current dec: P3 / P4 choose the next dec."""
+        value = max_mantissa * self.scale
+        if max_mantissa >= PCLIP:
+            self.history.append(2.0 * value)
+            self.dec = max(MIN_DEC, self.dec - 2)
+            return
+        self.history.append(value)
+        h = np.asarray(self.history, dtype=np.float64)
+        predicted = float(h.max() + GAMMA * h.std())
+        d = fit_dec(predicted)
+        if d is not None:
+            self.dec = d
+
+
+# ---------------------------------------------------------------------------------- simulator
+class FlexTensor(object):
+    def __init__(self, shape=()):
+        self.policy = FlexPolicy()
+        self.mantissa = np.zeros(shape, dtype=np.int16)
+
+    def host_write(self, value):
+        value = np.asarray(value, dtype=np.float64)
+        if not self.policy.initialized:
+            self.policy.init_from_value(np.max(np.abs(value)) if value.size else 0.0)
+        self.mantissa = quantize_host(np.broadcast_to(value, self.mantissa.shape), self.policy.dec)
+        self.policy.record(maxabs(self.mantissa))
+
+    def kernel_write(self, compute):
+        """`compute()` returns the fp32 result; P2 on first use, then store + record."""
+        result = np.asarray(compute(), dtype=f32)
+        if not self.policy.initialized:
+            finite = np.where(np.isnan(result), f32(0), np.abs(result))
+            self.policy.init_from_value(float(np.max(finite)) if result.size else 0.0)
+        self.mantissa = quantize_rni(result, self.policy.dec)
+        self.policy.record(maxabs(self.mantissa))
+
+    def read(self):
+        return dequantize(self.mantissa, self.policy.dec)
+
+    def value(self):
+        """What a kernel sees when it loads this tensor (uses the dec it was stored with)."""
+        return dequantize(self.mantissa, self._stored_dec)
+
+
+class FlexSim(object):
+    """Op-by-op flex execution of a tiny graph: placeholders -> ops -> result.
+
+    `program` is a list of (op_name, out, in0[, in1]) over tensor names; placeholders are
+    the names passed to `run`.  Every op output is its own flex tensor, as in the reference
+    transformer where nothing is fused (gputransform.py:381-391).
+    """
+
+    def __init__(self, program, shapes):
+        from oracle import numpy_ops
+        self.ops = numpy_ops
+        self.program = program
+        self.tensors = {name: _SimTensor(shape) for name, shape in shapes.items()}
+
+    def run(self, feeds, result):
+        for name, value in feeds.items():
+            self.tensors[name].host_write(value)
+        for ins in self.program:
+            op, out, srcs = ins[0], ins[1], ins[2:]
+            args = [self.tensors[s].load() for s in srcs]
+            self.tensors[out].kernel_write(lambda: self._apply(op, args))
+        return self.tensors[result].host_read()
+
+    def _apply(self, op, args):
+        o = self.ops
+        if op == "assign":
+            return args[0]
+        if op in o.UNARY or op in ("sig", "safelog"):
+            return o.unary(op, args[0])
+        if op in o.BINARY:
+            return o.binary(op, args[0], args[1])
+        if op in ("sum", "prod", "max", "min", "argmax", "argmin"):
+            return o.reduce(op, args[0], 0)
+        raise ValueError(op)
+
+
+class _SimTensor(object):
+    """Mantissas + the dec they were stored with + the policy deciding the next dec."""
+
+    def __init__(self, shape):
+        self.shape = tuple(shape)
+        self.policy = FlexPolicy()
+        self.mantissa = np.zeros(self.shape, dtype=np.int16)
+        self.stored_dec = DEFAULT_DEC
+
+    def host_write(self, value):
+        value = np.asarray(value, dtype=np.float64)
+        if not self.policy.initialized:
+            self.policy.init_from_value(float(np.max(np.abs(value))) if value.size else 0.0)
+        self.stored_dec = self.policy.dec
+        self.mantissa = quantize_host(np.broadcast_to(value, self.shape), self.stored_dec)
+        self.policy.record(maxabs(self.mantissa))
+
+    def kernel_write(self, compute):
+        result = np.asarray(compute(), dtype=f32)
+        if not self.policy.initialized:
+            mag = np.where(np.isnan(result), f32(0), np.abs(result))
+            self.policy.init_from_value(float(np.max(mag)) if result.size else 0.0)
+        self.stored_dec = self.policy.dec
+        self.mantissa = quantize_rni(np.broadcast_to(result, self.shape) if result.shape != self.shape
+                                     else result, self.stored_dec)
+        self.policy.record(maxabs(self.mantissa))
+
+    def load(self):
+        return dequantize(self.mantissa, self.stored_dec)
+
+    def host_read(self):
+        return dequantize(self.mantissa, self.stored_dec)
