@@ -20,6 +20,8 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     # packed-fp32 instruction forms are kept out of every kernel
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # a*b+c must round twice, as the NumPy statements of the CPU transformer do
+    "-ffp-contract=off",
     "-fno-gpu-rdc", "-Wno-unused-command-line-argument",
 ]
 

@@ -71,6 +71,7 @@ class HipFlexEntry(FlexEntry):
         self.ptr = None                 # device int32 word receiving max|mantissa|
         self.last_maxabs = 0
         self.last_count = -1
+        self.next_dec = None
 
     @property
     def dec(self):
@@ -80,17 +81,29 @@ class HipFlexEntry(FlexEntry):
         self.scale = 1.0 / 2 ** int(dec)
 
     # ---- policy -------------------------------------------------------------------------
+    # `scale` always describes the mantissas currently in memory.  The policy's choice for
+    # the NEXT write is kept in `next_dec` and only takes effect in adjust_scale(), which
+    # runs immediately before something overwrites the whole tensor.
     def init_from_value(self, maxabs_value):
         if not self.manager.fixed_point:
             dec = self.dtype.fit_dec(maxabs_value)
             self.set_dec(FlexManager.default_dec if dec is None else dec)
+        self.next_dec = self.dec
         self.initialized = True
 
+    def adjust_scale(self):
+        if self.initialized and self.next_dec is not None:
+            self.set_dec(self.next_dec)
+
     def manage_before_computation(self, value=None):
-        """Host write path: the first value a tensor receives fixes its initial scale."""
-        if not self.initialized and value is not None:
-            value = np.asarray(value, dtype=np.float64)
-            self.init_from_value(float(np.max(np.abs(value))) if value.size else 0.0)
+        """Host write path: the first value a tensor receives fixes its initial scale; later
+        writes use the scale the policy chose after the previous one."""
+        if not self.initialized:
+            if value is not None:
+                value = np.asarray(value, dtype=np.float64)
+                self.init_from_value(float(np.max(np.abs(value))) if value.size else 0.0)
+        else:
+            self.adjust_scale()
 
     def manage_after_computation(self, maxabs, autoflex_count):
         """Record max|mantissa| of what was just stored and choose the next scale."""
@@ -102,17 +115,17 @@ class HipFlexEntry(FlexEntry):
         value = maxabs * self.scale
         if maxabs >= self.dtype.pclip:
             self.history.append(2.0 * value)
-            self.set_dec(max(self.dtype.min_dec, self.dec - self.overflow_dec_step))
+            self.next_dec = max(self.dtype.min_dec, self.dec - self.overflow_dec_step)
             return
         self.history.append(value)
         h = np.asarray(self.history, dtype=np.float64)
         dec = self.dtype.fit_dec(float(h.max() + self.gamma * h.std()))
-        if dec is not None:
-            self.set_dec(dec)
+        self.next_dec = self.dec if dec is None else dec
 
     def reset_entry(self):
         self.history.clear()
         self.initialized = False
+        self.next_dec = None
         self.set_dec(FlexManager.default_dec)
 
 
@@ -149,7 +162,11 @@ class HipFlexManager(FlexManager):
 
     # ---- around kernels (flexgputransform.py:347-366) ------------------------------------
     def manage_before_computation(self, kernel):
+        in_place = getattr(kernel, "in_place_flex_ids", ())
         for entry in kernel.output_flex_entries:
+            if entry.flex_id not in in_place:
+                # a tensor the kernel also reads keeps the scale its data was stored with
+                entry.adjust_scale()
             self.runtime.stats_reset(entry.ptr, 1)
 
     def manage_after_computation(self, kernel):

@@ -113,12 +113,16 @@ class FlexFusedKernel(FusedKernel):
 
     def bind_buffers(self):
         super(FlexFusedKernel, self).bind_buffers()
-        seen, entries = set(), []
-        for _, _, entry, is_output in self.flex_bindings:
+        seen, entries, read_ids = set(), [], set()
+        for index, slot, entry, is_output in self.flex_bindings:
             if is_output and entry.flex_id not in seen:
                 seen.add(entry.flex_id)
                 entries.append(entry)
+            spec = self.specs[index]
+            if any(o.opcode == 1 and o.a == slot for o in spec.ops[:spec.n_ops]):
+                read_ids.add(entry.flex_id)
         self.output_flex_entries = entries
+        self.in_place_flex_ids = set(e.flex_id for e in entries) & read_ids
 
     @property
     def output_flex_ids(self):

@@ -111,7 +111,8 @@ def test_c5_fused_flex_bit_exact_over_8_iterations(n):
             mant = y_view._read_raw()
             assert entry.last_maxabs == maxabs_want, (i, entry.last_maxabs, maxabs_want)
             np.testing.assert_array_equal(mant, m_want, err_msg="iteration %d mantissas" % i)
-            assert entry.dec == next_dec_want, (i, entry.dec, next_dec_want)
+            assert entry.dec == dec_want and entry.next_dec == next_dec_want, \
+                (i, entry.dec, entry.next_dec, dec_want, next_dec_want)
             np.testing.assert_array_equal(got, fm.dequantize(m_want, dec_want))
         assert len(t.kernel_groups[f].kernels) == 1           # one fused kernel
         assert "special:flex_relu_fma" in kernel.describe()[0][0]

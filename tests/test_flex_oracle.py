@@ -125,6 +125,8 @@ def test_product_policy_matches_oracle_policy():
             m = int(rs.choice([0, 1, 7, 300, 5000, 16384, 20000, 32766, 32767, 32768]))
             entry.manage_after_computation(m, step)
             pol.record(m)
-            assert entry.dec == pol.dec, (trial, step, m)
+            assert entry.next_dec == pol.dec, (trial, step, m)
+            entry.adjust_scale()             # the next write happens at the chosen exponent
+            assert entry.dec == pol.dec
     assert hipflex16.fit_dec(0.0) is None and hipflex16.fit_dec(np.inf) == 0
     assert hipflex16.fit_dec(1.0) == 14 and hipflex16.fit_dec(32767) == 0 and hipflex16.fit_dec(2 ** -30) == 31
