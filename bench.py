@@ -63,6 +63,81 @@ def kernel_bytes(kernel):
     return total
 
 
+def other_configs(ng, ngt, neon, configs, steps, warmup):
+    """C1, C3, C4, C5 with inputs resident: ms per step and algorithmic GB/s (for information;
+    the headline line is C2)."""
+    out = {}
+
+    def run(name, t, f, nbytes, elems, per_step=1):
+        group = t.kernel_groups[f]
+        group()
+        t.runtime.sync()
+        ms = time_steps(t.runtime, group, steps, warmup)
+        kern = []
+        for k, times in group.profile(repeats=5):
+            kern.append({"kernel": "+".join(sum(k.describe(), [])), "ms": round(float(np.mean(times)), 5)})
+        out[name] = {"ms_per_step": round(ms, 5), "GB/s": round(nbytes * per_step / (ms * 1e-3) / 1e9, 1),
+                     "frac_of_hbm_peak": round(nbytes * per_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "elements_per_s": round(elems * per_step / (ms * 1e-3), 1), "kernels": kern}
+        t.close()
+
+    # C1
+    t = ngt.make_transformer_factory("hipgpu")()
+    x_np, a, b = configs.c1_inputs((1024, 1024))
+    H, W = ng.make_axis(1024, name="H"), ng.make_axis(1024, name="W")
+    x, pa, pb = ng.placeholder([H, W]), ng.placeholder(()), ng.placeholder(())
+    f = t.computation(ng.tanh(pa * x + pb) * ng.sigmoid(x), x, pa, pb)
+    f(x_np, a, b)
+    run("C1", t, f, 8388608, 1048576)
+    # C3
+    t = ngt.make_transformer_factory("hipgpu")()
+    n = 25600000
+    p_np, g_np, _, _ = configs.c3_inputs(n)
+    P = ng.make_axis(n, name="P")
+    p, grad = ng.variable([P], initial_value=p_np), ng.placeholder([P])
+    opt = neon.Adam()
+    opt()
+    updates, _, _ = opt.variable_update(p, grad)
+    f = t.computation(updates, grad)
+    f(g_np)                                   # the warm step (t = 1); inputs stay resident
+    run("C3", t, f, 716800000, n)
+    # C4
+    t = ngt.make_transformer_factory("hipgpu")()
+    Hn, Nn = 1024, 64
+    gates_np, cprev_np = configs.c4_inputs(Hn, Nn)
+    H, N, G = ng.make_axis(Hn, name="H"), ng.make_axis(Nn, name="N"), ng.make_axis(4 * Hn, name="G")
+    gates_st, cprev_st = ng.placeholder([N, G]), ng.placeholder([N, H])
+    gates, c_prev = ng.axes_with_order(gates_st, [G, N]), ng.axes_with_order(cprev_st, [H, N])
+    parts = {k: ng.cast_axes(ng.tensor_slice(gates, [slice(j * Hn, (j + 1) * Hn), slice(None)]), [H, N])
+             for j, k in enumerate(("i", "f", "o", "g"))}
+    h, c = neon.lstm_cell(parts, c_prev, H, None)
+    f = t.computation([c, h, ng.sum(gates, out_axes=[G])], gates_st, cprev_st)
+    f(gates_np, cprev_np)
+    run("C4", t, f, 1851392, 327680)
+    # C5: 8 iterations of the fused flex kernel, each with stats readback + exponent update
+    t = ngt.make_transformer_factory("flexhip")()
+    n = 16 * 1024 * 1024
+    x_np, w_np, b_np = configs.c5_inputs(n)
+    P = ng.make_axis(n, name="P")
+    x, w, b = ng.placeholder([P]), ng.placeholder([P]), ng.placeholder([P])
+    f = t.computation(neon.rectlin(x * w + b), x, w, b)
+    f(x_np, w_np, b_np)
+    group = t.kernel_groups[f]
+
+    class Eight(object):
+        kernels = group.kernels
+
+        def __call__(self):
+            for _ in range(8):
+                group()
+
+        def profile(self, repeats):
+            return group.profile(repeats)
+    t.kernel_groups[f] = Eight()
+    run("C5", t, f, 134217728, n, per_step=8)
+    return out
+
+
 def cpu_baseline_c2(dims, budget_s=20.0):
     from oracle import configs
     C, R = dims[0], dims[1] * dims[2] * dims[3]
@@ -88,6 +163,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--all", action="store_true", help="also time configs C1, C3, C4, C5")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
+                    help="also issue N device-to-device copies of x (205 520 896 bytes each): a "
+                         "kernel of known traffic to scale rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (--gpus 1); the path shards without "
@@ -117,7 +195,7 @@ def main():
     value = algorithmic_bytes / (ms * 1e-3) / 1e9
 
     # dominant kernel: HIP-event duration of every launch over the same number of steps
-    prof = group.profile(repeats=max(args.steps, 5))
+    prof = group.profile(repeats=max(args.steps // 2, 5), inner=10)
     per_kernel = []
     for k, times in prof:
         per_kernel.append({"kernel": "+".join(sum(k.describe(), [])) if hasattr(k, "describe") else
@@ -129,6 +207,15 @@ def main():
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": None, "algorithmic_bytes_per_launch": dom["bytes"],
                 "avg_launch_ms": round(dom["ms"], 5)}
+
+    if args.copy_calibration:
+        y_view = t.get_op_tensor_view(f.computation_op.values[0])
+        x_view = t.get_op_tensor_view(x)
+        for _ in range(args.copy_calibration):
+            rt.memcpy_d2d(y_view.ptr, x_view.ptr, n_elems * 4)
+        rt.sync()
+        group()                                                # y holds the normalised output again
+        rt.sync()
 
     # parity spot-check at full size through a size-independent property: normalised output
     # has per-channel mean beta and variance gamma^2 * var / (var + eps)
@@ -147,9 +234,11 @@ def main():
                       "elements_per_s": round(n_elems / (ms * 1e-3), 1),
                       "kernels": per_kernel},
            "roofline": roofline}
+    t.close()
+    if args.all:
+        out["other_configs"] = other_configs(ng, ngt, neon, configs, max(5, args.steps // 3), 2)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_c2(dims)
-    t.close()
     print(json.dumps(out))
 
 

@@ -235,6 +235,73 @@ __device__ __forceinline__ void store4(const KTensor& t, long long off, float sc
     }
 }
 
+// V consecutive elements (V = 4 or 8).  Eight 16-bit elements travel as one 16-byte
+// access, which is what keeps enough bytes in flight per lane for 2-byte storage types.
+template <int V>
+__device__ __forceinline__ void loadv(const KTensor& t, long long off, float scale, float (&v)[V]) {
+    if constexpr (V == 4) {
+        load4(t, off, scale, v);
+    } else {
+        static_assert(V == 8, "vector width");
+        if (t.dtype == NGH_FLEX16) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(reinterpret_cast<const short*>(t.p) + off);
+            const unsigned w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[2 * j] = scale * (float)(short)(w[j] & 0xffffu);
+                v[2 * j + 1] = scale * (float)(short)(w[j] >> 16);
+            }
+        } else if (t.dtype == NGH_F16) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(reinterpret_cast<const __half*>(t.p) + off);
+            const unsigned w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                unsigned u = w[j];
+                const float2 f = __half22float2(*reinterpret_cast<__half2*>(&u));
+                v[2 * j] = f.x;
+                v[2 * j + 1] = f.y;
+            }
+        } else {
+            float a[4], b[4];
+            load4(t, off, scale, a);
+            load4(t, off + 4, scale, b);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) { v[j] = a[j]; v[4 + j] = b[j]; }
+        }
+    }
+}
+
+template <int V>
+__device__ __forceinline__ void storev(const KTensor& t, long long off, float scale, const float (&v)[V], int& fmax) {
+    if constexpr (V == 4) {
+        store4(t, off, scale, v, fmax);
+    } else {
+        static_assert(V == 8, "vector width");
+        if (t.dtype == NGH_FLEX16) {
+            unsigned w[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int q0 = flex_quantize(scale * v[2 * j]), q1 = flex_quantize(scale * v[2 * j + 1]);
+                fmax = max(fmax, max(iabs(q0), iabs(q1)));
+                w[j] = ((unsigned)q0 & 0xffffu) | ((unsigned)q1 << 16);
+            }
+            *reinterpret_cast<uint4*>(reinterpret_cast<short*>(t.p) + off) = make_uint4(w[0], w[1], w[2], w[3]);
+        } else if (t.dtype == NGH_F16) {
+            unsigned w[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                __half2 h = __floats2half2_rn(v[2 * j], v[2 * j + 1]);
+                w[j] = *reinterpret_cast<unsigned*>(&h);
+            }
+            *reinterpret_cast<uint4*>(reinterpret_cast<__half*>(t.p) + off) = make_uint4(w[0], w[1], w[2], w[3]);
+        } else {
+            const float a[4] = {v[0], v[1], v[2], v[3]}, b[4] = {v[4], v[5], v[6], v[7]};
+            store4(t, off, scale, a, fmax);
+            store4(t, off + 4, scale, b, fmax);
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Register file of the op interpreter.  The program is only known at run
 // time, so register numbers are run-time values; a per-lane array indexed that
@@ -306,6 +373,23 @@ __device__ __forceinline__ Acc acc_shfl_xor(Acc a, int mask) {
     b.v = __shfl_xor(a.v, mask, 64);
     b.i = __shfl_xor(a.i, mask, 64);
     return b;
+}
+
+// Merge a per-thread max|mantissa| into the tensor's statistics word: wavefront butterfly,
+// LDS across the workgroup's wavefronts, then ONE atomic per workgroup -- and only when it
+// can still raise the word (a plain read first: tens of thousands of workgroups hammering
+// one address with atomics otherwise costs more than the kernel's memory traffic).
+__device__ __forceinline__ void block_stat_max(int m, int* word, int* lds_slot /* [nwaves] */) {
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) m = max(m, __shfl_xor(m, s, 64));
+    const int wave = threadIdx.x >> 6, nwaves = (blockDim.x * blockDim.y + 63) >> 6;
+    if ((threadIdx.x & 63) == 0) lds_slot[wave] = m;
+    __syncthreads();
+    if (threadIdx.x == 0 && word != nullptr) {
+        for (int w = 1; w < nwaves; ++w) m = max(m, lds_slot[w]);
+        if (m > 0 && m > __atomic_load_n(word, __ATOMIC_RELAXED)) atomicMax(word, m);
+    }
+    __syncthreads();
 }
 
 __device__ __forceinline__ int wave_max_int(int x) {

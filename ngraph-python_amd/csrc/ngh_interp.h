@@ -48,11 +48,11 @@ __device__ __forceinline__ void run_ops(const KArgs& k, LdsRegs<V>& rf, Extra& e
                     const float x = load1(t, off, sc);
 #pragma unroll
                     for (int v = 0; v < V; ++v) rf.set(o.dst, v, x);
-                } else if (V == 4 && t.s[2] == 1) {
-                    float x[4];
-                    load4(t, off, sc, x);
+                } else if (V >= 4 && t.s[2] == 1) {
+                    float x[V >= 4 ? V : 4];
+                    if constexpr (V >= 4) loadv<V>(t, off, sc, x);
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) rf.set(o.dst, v, x[v]);
+                    for (int v = 0; v < V; ++v) rf.set(o.dst, v, x[v]);
                 } else {
 #pragma unroll
                     for (int v = 0; v < V; ++v) rf.set(o.dst, v, load1(t, off + v * t.s[2], sc));
@@ -66,11 +66,11 @@ __device__ __forceinline__ void run_ops(const KArgs& k, LdsRegs<V>& rf, Extra& e
                 if (k.probe) {
 #pragma unroll
                     for (int v = 0; v < V; ++v) fmax = max(fmax, probe_bits(rf.get(o.a, v)));
-                } else if (V == 4 && t.s[2] == 1) {
-                    float x[4];
+                } else if (V >= 4 && t.s[2] == 1) {
+                    float x[V >= 4 ? V : 4];
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) x[v] = rf.get(o.a, v);
-                    store4(t, off, sc, x, fmax);
+                    for (int v = 0; v < V; ++v) x[v] = rf.get(o.a, v);
+                    if constexpr (V >= 4) storev<V>(t, off, sc, x, fmax);
                 } else {
 #pragma unroll
                     for (int v = 0; v < V; ++v) store1(t, off + v * t.s[2], rf.get(o.a, v), sc, fmax);
@@ -131,10 +131,8 @@ __device__ __forceinline__ void run_ops(const KArgs& k, LdsRegs<V>& rf, Extra& e
 }
 
 __device__ __forceinline__ void stats_epilogue(const KArgs& k, Extra& ex) {
-    for (int s = 0; s < k.n_stat_slots; ++s) {
-        int m = wave_max_int(ex.geti(ex_stat(s)));
-        if ((threadIdx.x & 63) == 0 && m > 0 && k.stat_ptr[s] != nullptr) atomicMax(k.stat_ptr[s], m);
-    }
+    __shared__ int stat_lds[kWaves];
+    for (int s = 0; s < k.n_stat_slots; ++s) block_stat_max(ex.geti(ex_stat(s)), k.stat_ptr[s], stat_lds);
 }
 
 // ---------------------------------------------------------------------------

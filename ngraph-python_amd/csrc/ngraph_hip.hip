@@ -71,7 +71,7 @@ struct ngh_context {
     hipEvent_t  ev0 = nullptr, ev1 = nullptr;
     void*       ws = nullptr;        // partial results of split reductions
     size_t      ws_bytes = 0;
-    int         ew_blocks_per_cu = 8;
+    int         ew_blocks_per_cu = 64;
     int         force_interp = 0;    // never pick a specialised kernel
     int         moments_wgs_per_cu = 16;
     char        name[256] = "";
@@ -234,19 +234,25 @@ void fill_kargs(const ngh_fused_spec& sp, const ngh_stage& S, const int perm[3],
     memcpy(k.ops, sp.ops, sizeof(k.ops));
 }
 
-bool vec4_ok(const KArgs& k, const bool* used) {
-    if (k.shape[2] % 4) return false;
+// Can the stage move V consecutive elements per lane along kernel axis 2?
+bool vec_ok(const KArgs& k, const bool* used, int V) {
+    if (k.shape[2] % V) return false;
     for (int t = 0; t < k.n_tensors; ++t) {
         if (!used[t]) continue;
         const KTensor& K = k.t[t];
         if (K.s[2] == 0) continue;
         if (K.s[2] != 1) return false;
-        if (((uintptr_t)K.p) % (4 * itemsize_of(K.dtype))) return false;
+        const int isz = itemsize_of(K.dtype);
+        if (V == 8 && isz != 2) return false;              // 8-wide only pays for 16-bit storage
+        const int align = std::min(16, V * isz);
+        if (((uintptr_t)K.p) % align) return false;
         for (int j = 0; j < 2; ++j)
-            if (k.shape[j] > 1 && K.s[j] % 4) return false;
+            if (k.shape[j] > 1 && K.s[j] % V) return false;
     }
     return true;
 }
+
+bool vec4_ok(const KArgs& k, const bool* used) { return vec_ok(k, used, 4); }
 
 int plan_stage(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan& P) {
     const ngh_stage& S = sp.stages[stage];
@@ -280,14 +286,17 @@ int plan_stage(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan
         fill_kargs(sp, S, perm, P.k);
         for (int a = 0; a < 3; ++a) P.perm[a] = perm[a];
         P.family = F_EW;
-        P.V = vec4_ok(P.k, used) ? 4 : 1;
+        P.V = vec_ok(P.k, used, 8) ? 8 : (vec_ok(P.k, used, 4) ? 4 : 1);
         P.tail = 0;
-        if (P.V == 1 && P.k.shape[0] == 1 && P.k.shape[1] == 1 && P.k.shape[2] >= 8) {
-            // contiguous 1-D view whose length is not a multiple of 4: vector body + scalar tail
+        if (P.V == 1 && P.k.shape[0] == 1 && P.k.shape[1] == 1 && P.k.shape[2] >= 16) {
+            // contiguous 1-D view whose length is not a multiple of the vector width:
+            // vector body + scalar tail
             const long long n = P.k.shape[2];
-            P.k.shape[2] = n - n % 4;
-            if (vec4_ok(P.k, used)) { P.V = 4; P.tail = n % 4; }
-            else P.k.shape[2] = n;
+            for (int V : {8, 4}) {
+                P.k.shape[2] = n - n % V;
+                if (vec_ok(P.k, used, V)) { P.V = V; P.tail = n % V; break; }
+                P.k.shape[2] = n;
+            }
         }
         const long long rows = P.k.shape[0] * P.k.shape[1];
         const long long cpr = P.k.shape[2] / P.V;
@@ -402,20 +411,16 @@ int launch_tail(ngh_context* ctx, const Plan& P) {
 int launch_interp(ngh_context* ctx, Plan& P) {
     int V = P.V;
     size_t lds = interp_lds_bytes(P.k, V);
-    if (lds > kInterpLdsPreferred && V == 4 && P.family == F_EW) {
-        // too many live registers for a 4-wide file: fall back to one element per lane
-        Plan Q = P;
-        Q.V = 1;
-        Q.k.shape[2] += Q.tail;
-        Q.tail = 0;
-        Q.chunks_per_row = (unsigned)Q.k.shape[2];
-        const long long chunks = Q.k.shape[0] * Q.k.shape[1] * Q.k.shape[2];
-        if (chunks < (1LL << 32)) {
-            Q.n_chunks = (unsigned)chunks;
-            P = Q;
-            V = 1;
-            lds = interp_lds_bytes(P.k, 1);
-        }
+    while (lds > kInterpLdsPreferred && V > 1 && P.family == F_EW) {
+        // too many live registers for a V-wide file: narrow the vector (the tail, if any, stays)
+        const int narrower = (V == 8) ? 4 : 1;
+        const long long cpr = P.k.shape[2] / narrower;
+        const long long chunks = P.k.shape[0] * P.k.shape[1] * cpr;
+        if (chunks >= (1LL << 32)) break;
+        V = P.V = narrower;
+        P.chunks_per_row = (unsigned)cpr;
+        P.n_chunks = (unsigned)chunks;
+        lds = interp_lds_bytes(P.k, V);
     }
     if (lds > kInterpLdsMax) return fail(NGH_E_UNSUPPORTED, "program needs %zu bytes of LDS registers", lds);
     const KArgs& k = P.k;
@@ -424,7 +429,9 @@ int launch_interp(ngh_context* ctx, Plan& P) {
         if (P.n_chunks) {
             unsigned blocks = (P.n_chunks + kBlock - 1) / kBlock;
             blocks = std::min<unsigned>(blocks, (unsigned)(ctx->cus * ctx->ew_blocks_per_cu));
-            if (V == 4)
+            if (V == 8)
+                hipLaunchKernelGGL(ew_interp_kernel<8>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, P.n_chunks, P.chunks_per_row);
+            else if (V == 4)
                 hipLaunchKernelGGL(ew_interp_kernel<4>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, P.n_chunks, P.chunks_per_row);
             else
                 hipLaunchKernelGGL(ew_interp_kernel<1>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, P.n_chunks, P.chunks_per_row);
@@ -510,7 +517,7 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->cus = prop.multiProcessorCount;
     ctx->total_bytes = prop.totalGlobalMem;
     snprintf(ctx->name, sizeof(ctx->name), "%s (%s)", prop.name, prop.gcnArchName);
-    ctx->ew_blocks_per_cu = std::max(1, env_int("NGH_EW_BLOCKS_PER_CU", 8));
+    ctx->ew_blocks_per_cu = std::max(1, env_int("NGH_EW_BLOCKS_PER_CU", 64));
     ctx->force_interp = env_int("NGH_FORCE_INTERP", 0);
     ctx->moments_wgs_per_cu = std::max(1, env_int("NGH_MOMENTS_WGS_PER_CU", 16));
     hipError_t e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
@@ -521,7 +528,8 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
         return fail(NGH_E_RUNTIME, "stream/event creation: %s", hipGetErrorString(e));
     }
     // the interpreter's register file is dynamic LDS and may exceed the 64 KiB default
-    const void* interp_kernels[] = {(const void*)ew_interp_kernel<4>, (const void*)ew_interp_kernel<1>,
+    const void* interp_kernels[] = {(const void*)ew_interp_kernel<8>, (const void*)ew_interp_kernel<4>,
+                                    (const void*)ew_interp_kernel<1>,
                                     (const void*)red_row_interp_kernel<4>, (const void*)red_row_interp_kernel<1>,
                                     (const void*)red_col_interp_kernel};
     for (const void* fn : interp_kernels) {

@@ -715,10 +715,14 @@ class HipKernelGroup(object):
             k.execute()
             self.after_kernel_execute(k)
 
-    def profile(self, repeats=1):
-        """Run the group `repeats` times with every kernel bracketed by HIP events on the
-        launch stream; returns [(kernel, [ms per run])].  Serialises the kernels, so use it
-        for per-kernel durations, not for end-to-end time."""
+    def profile(self, repeats=1, inner=1):
+        """Per-kernel durations from HIP events on the launch stream.
+
+        Each kernel is launched `inner` times back to back between one pair of events and the
+        elapsed time divided by `inner` (amortises the event and launch overhead, so the
+        figure is comparable with a profiler's kernel duration); this is repeated `repeats`
+        times.  Returns [(kernel, [ms per launch])].  Kernels run out of their normal
+        interleaving, so use it for per-kernel time, not for end-to-end time."""
         rt = self.transformer.runtime
         for k in self.kernels:
             if not k.buffers_bound:
@@ -728,8 +732,9 @@ class HipKernelGroup(object):
             for i, k in enumerate(self.kernels):
                 self.setup_kernel_execute(k)
                 rt.timer_begin()
-                k.execute()
-                times[i].append(rt.timer_end())
+                for _ in range(inner):
+                    k.execute()
+                times[i].append(rt.timer_end() / inner)
                 self.after_kernel_execute(k)
         return list(zip(self.kernels, times))
 
