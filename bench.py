@@ -23,6 +23,9 @@ for _p in (ROOT, os.path.join(ROOT, "ngraph-python_amd")):
 import numpy as np  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes one launch of the C2 normalise kernel moves, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE scaled by a device copy of known size (profiles/c2_batchnorm_pmc_traffic.md)
+MEASURED_TRAFFIC = {"special:batchnorm": 411108350}
 
 
 def build_c2(ng, neon, t, dims):
@@ -205,7 +208,8 @@ def main():
     achieved = dom["bytes"] / (dom["ms"] * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": dom["kernel"], "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": None, "algorithmic_bytes_per_launch": dom["bytes"],
+                "traffic": next((v for k, v in MEASURED_TRAFFIC.items() if dom["kernel"].startswith(k)), None),
+                "algorithmic_bytes_per_launch": dom["bytes"],
                 "avg_launch_ms": round(dom["ms"], 5)}
 
     if args.copy_calibration:
