@@ -379,17 +379,17 @@ __device__ __forceinline__ Acc acc_shfl_xor(Acc a, int mask) {
 // LDS across the workgroup's wavefronts, then ONE atomic per workgroup -- and only when it
 // can still raise the word (a plain read first: tens of thousands of workgroups hammering
 // one address with atomics otherwise costs more than the kernel's memory traffic).
-__device__ __forceinline__ void block_stat_max(int m, int* word, int* lds_slot /* [nwaves] */) {
+__device__ __forceinline__ void block_stat_max(int m, int* word, int* lds_slot /* [nwaves], one per call */) {
 #pragma unroll
     for (int s = 32; s > 0; s >>= 1) m = max(m, __shfl_xor(m, s, 64));
     const int wave = threadIdx.x >> 6, nwaves = (blockDim.x * blockDim.y + 63) >> 6;
     if ((threadIdx.x & 63) == 0) lds_slot[wave] = m;
     __syncthreads();
+    // no barrier after this: the other wavefronts retire while thread 0 finishes
     if (threadIdx.x == 0 && word != nullptr) {
         for (int w = 1; w < nwaves; ++w) m = max(m, lds_slot[w]);
         if (m > 0 && m > __atomic_load_n(word, __ATOMIC_RELAXED)) atomicMax(word, m);
     }
-    __syncthreads();
 }
 
 __device__ __forceinline__ int wave_max_int(int x) {

@@ -292,7 +292,7 @@ class FusedKernel(HipKernel):
         t = self.transformer
         ops = self.ops
         first = ops[0]
-        reductions = [op for op in ops if isinstance(op, og.ReductionOp)]
+        reductions = [op for op in ops if isinstance(op, og.ReductionOp) and op.reduction_axes.size > 1]
         it_axes = iteration_axes(first)
         red_axes = reductions[0].reduction_axes if reductions else og.make_axes(())
         onehot_axes = [op.axis for op in ops if isinstance(op, og.OneHotOp)]
