@@ -208,6 +208,43 @@ int  ngh_stats_alloc(ngh_context* ctx, int32_t n, int32_t** out_dev);
 int  ngh_stats_reset(ngh_context* ctx, int32_t* dev, int32_t n);
 int  ngh_stats_read(ngh_context* ctx, const int32_t* dev, int32_t n, int32_t* host);
 
+/* ---- device-resident flex exponent management -----------------------------
+ * One record per flex tensor.  A fused kernel reads the tensor's scale through
+ * ngh_tensor.dev_scale = &state.scale and merges max|mantissa| into
+ * ngh_tensor.dev_stats = &state.stats; ngh_flex_prepare / ngh_flex_update run the
+ * exponent policy on the device around a kernel, so no statistics travel to the host
+ * between kernels (the reference reads them back after every kernel,
+ * flexgputransform.py:361-366).  Policy: DESIGN.md section 5; the host mirror is
+ * ngraph_hip/flex/hipflex.py.                                                      */
+#define NGH_FLEX_HISTORY 16
+typedef struct ngh_flex_state {
+    int32_t stats;          /* max |mantissa| merged by kernels since ngh_flex_prepare   */
+    int32_t dec;            /* exponent of the data in memory: scale = 2**-dec           */
+    int32_t next_dec;       /* exponent for the next full overwrite, -1 = none chosen    */
+    int32_t initialized;
+    float   scale;
+    int32_t hist_len, hist_pos;
+    int32_t last_maxabs, last_count, pad_;
+    double  history[NGH_FLEX_HISTORY];   /* recent max |value|, ring buffer               */
+} ngh_flex_state;
+
+int  ngh_flex_states_alloc(ngh_context* ctx, int32_t n, ngh_flex_state** out_dev);
+int  ngh_flex_states_write(ngh_context* ctx, ngh_flex_state* dev, int32_t first, int32_t n,
+                           const ngh_flex_state* host);
+int  ngh_flex_states_read(ngh_context* ctx, const ngh_flex_state* dev, int32_t first, int32_t n,
+                          ngh_flex_state* host);     /* waits for the stream */
+/* ids: up to 8 record indices; in_place[i] != 0 keeps record i's exponent (the kernel also
+ * reads that tensor).  count is stored in last_count (the caller's autoflex_count).    */
+int  ngh_flex_prepare(ngh_context* ctx, ngh_flex_state* dev, const int32_t* ids,
+                      const int32_t* in_place, int32_t n_ids);
+int  ngh_flex_update(ngh_context* ctx, ngh_flex_state* dev, const int32_t* ids, int32_t n_ids,
+                     int32_t count);
+
+/* ngh_flex_prepare + ngh_launch_fused + ngh_flex_update in one call (one host transition per
+ * kernel instead of three).                                                            */
+int  ngh_launch_fused_flex(ngh_context* ctx, const ngh_fused_spec* spec, ngh_flex_state* dev,
+                           const int32_t* ids, const int32_t* in_place, int32_t n_ids, int32_t count);
+
 /* ---- timing (HIP events on the context's stream; used by the bench) ----- */
 int  ngh_timer_begin(ngh_context* ctx);
 int  ngh_timer_end(ngh_context* ctx, float* out_ms);   /* waits for the stream */

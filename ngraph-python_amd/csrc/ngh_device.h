@@ -39,6 +39,7 @@ struct KArgs {
     int       n_stat_slots;
     int       probe;         // NGH_SPEC_PROBE: record max|value| bits instead of storing
     int*      stat_ptr[4];   // device word of each per-thread accumulator
+    int*      stat_partial[4];  // per-workgroup scratch the streaming kernels write instead
     KTensor   t[NGH_MAX_TENSORS];
     float     consts[NGH_MAX_CONSTS];
     ngh_op    ops[NGH_MAX_OPS];
@@ -375,20 +376,35 @@ __device__ __forceinline__ Acc acc_shfl_xor(Acc a, int mask) {
     return b;
 }
 
-// Merge a per-thread max|mantissa| into the tensor's statistics word: wavefront butterfly,
-// LDS across the workgroup's wavefronts, then ONE atomic per workgroup -- and only when it
-// can still raise the word (a plain read first: tens of thousands of workgroups hammering
-// one address with atomics otherwise costs more than the kernel's memory traffic).
-__device__ __forceinline__ void block_stat_max(int m, int* word, int* lds_slot /* [nwaves], one per call */) {
+// Reduce a per-thread max|mantissa| over the workgroup and leave it in this workgroup's slot
+// of a scratch array; a one-workgroup fold kernel launched right after merges the slots
+// into the tensor's statistics word.  No atomics in the streaming kernel: thousands of
+// workgroups finishing together and hitting one word with atomicMax cost more than the
+// kernel's memory traffic (measured: 22 us -> 38 us for the 16 M element flex kernel).
+__device__ __forceinline__ void block_stat_max(int m, int* partial, int* lds_slot /* [nwaves], one per call */) {
 #pragma unroll
     for (int s = 32; s > 0; s >>= 1) m = max(m, __shfl_xor(m, s, 64));
     const int wave = threadIdx.x >> 6, nwaves = (blockDim.x * blockDim.y + 63) >> 6;
     if ((threadIdx.x & 63) == 0) lds_slot[wave] = m;
     __syncthreads();
-    // no barrier after this: the other wavefronts retire while thread 0 finishes
-    if (threadIdx.x == 0 && word != nullptr) {
+    if (threadIdx.x == 0 && partial != nullptr) {
         for (int w = 1; w < nwaves; ++w) m = max(m, lds_slot[w]);
-        if (m > 0 && m > __atomic_load_n(word, __ATOMIC_RELAXED)) atomicMax(word, m);
+        partial[blockIdx.x] = m;
+    }
+}
+
+__global__ __launch_bounds__(256) void stats_fold_kernel(const int* __restrict__ partial, unsigned n,
+                                                         int* __restrict__ word) {
+    __shared__ int sh[4];
+    int m = 0;
+    for (unsigned i = threadIdx.x; i < n; i += 256) m = max(m, partial[i]);
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) m = max(m, __shfl_xor(m, s, 64));
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        m = max(max(sh[0], sh[1]), max(sh[2], sh[3]));
+        if (m > 0) atomicMax(word, m);
     }
 }
 

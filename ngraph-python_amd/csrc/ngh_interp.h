@@ -132,7 +132,7 @@ __device__ __forceinline__ void run_ops(const KArgs& k, LdsRegs<V>& rf, Extra& e
 
 __device__ __forceinline__ void stats_epilogue(const KArgs& k, Extra& ex) {
     __shared__ int stat_lds[4][kWaves];
-    for (int s = 0; s < k.n_stat_slots; ++s) block_stat_max(ex.geti(ex_stat(s)), k.stat_ptr[s], stat_lds[s]);
+    for (int s = 0; s < k.n_stat_slots; ++s) block_stat_max(ex.geti(ex_stat(s)), k.stat_partial[s], stat_lds[s]);
 }
 
 // ---------------------------------------------------------------------------

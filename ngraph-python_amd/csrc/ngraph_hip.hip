@@ -17,6 +17,7 @@
 #include "ngh_copy.h"
 #include "ngh_special.h"
 #include "ngh_moments.h"
+#include "ngh_flex.h"
 
 using namespace ngh;
 
@@ -71,6 +72,8 @@ struct ngh_context {
     hipEvent_t  ev0 = nullptr, ev1 = nullptr;
     void*       ws = nullptr;        // partial results of split reductions
     size_t      ws_bytes = 0;
+    int*        stat_ws = nullptr;   // per-workgroup max|mantissa| of streaming kernels
+    unsigned    stat_ws_blocks = 0;  // capacity per statistics slot
     int         ew_blocks_per_cu = 64;
     int         force_interp = 0;    // never pick a specialised kernel
     int         moments_wgs_per_cu = 16;
@@ -391,6 +394,34 @@ int ensure_ws(ngh_context* ctx, size_t bytes) {
 }
 
 // The last (length % 4) elements of a contiguous 1-D stage, one element per lane.
+// Point the stage's statistics slots at per-workgroup scratch for a launch of `blocks`
+// workgroups, and, after the launch, fold the scratch into each tensor's statistics word.
+int stat_scratch(ngh_context* ctx, KArgs& k, unsigned blocks) {
+    if (k.n_stat_slots == 0) return NGH_OK;
+    if (blocks > ctx->stat_ws_blocks) {
+        if (ctx->stat_ws) {
+            HIP_TRY(hipStreamSynchronize(ctx->stream));
+            HIP_TRY(hipFree(ctx->stat_ws));
+            ctx->stat_ws = nullptr;
+        }
+        const unsigned cap = std::max(blocks, 65536u);
+        HIP_TRY(hipMalloc((void**)&ctx->stat_ws, (size_t)cap * 4 * sizeof(int)));
+        ctx->stat_ws_blocks = cap;
+    }
+    for (int s = 0; s < 4; ++s) k.stat_partial[s] = ctx->stat_ws + (size_t)s * ctx->stat_ws_blocks;
+    return NGH_OK;
+}
+
+int stat_fold(ngh_context* ctx, const KArgs& k, unsigned blocks) {
+    for (int s = 0; s < k.n_stat_slots; ++s) {
+        if (k.stat_ptr[s] == nullptr) continue;
+        hipLaunchKernelGGL(stats_fold_kernel, dim3(1), dim3(256), 0, ctx->stream, k.stat_partial[s], blocks,
+                           k.stat_ptr[s]);
+        HIP_TRY(hipGetLastError());
+    }
+    return NGH_OK;
+}
+
 int launch_tail(ngh_context* ctx, const Plan& P) {
     KArgs kt = P.k;
     const long long body = P.k.shape[2];
@@ -402,10 +433,11 @@ int launch_tail(ngh_context* ctx, const Plan& P) {
             return fail(NGH_E_UNSUPPORTED, "IOTA along a split 1-D axis");
     const size_t lds = interp_lds_bytes(kt, 1);
     if (lds > kInterpLdsMax) return fail(NGH_E_UNSUPPORTED, "program needs %zu bytes of LDS registers", lds);
+    NGH_TRY(stat_scratch(ctx, kt, 1));
     hipLaunchKernelGGL(ew_interp_kernel<1>, dim3(1), dim3(kBlock), lds, ctx->stream, kt, (unsigned)P.tail,
                        (unsigned)P.tail);
     HIP_TRY(hipGetLastError());
-    return NGH_OK;
+    return stat_fold(ctx, kt, 1);
 }
 
 int launch_interp(ngh_context* ctx, Plan& P) {
@@ -423,12 +455,13 @@ int launch_interp(ngh_context* ctx, Plan& P) {
         lds = interp_lds_bytes(P.k, V);
     }
     if (lds > kInterpLdsMax) return fail(NGH_E_UNSUPPORTED, "program needs %zu bytes of LDS registers", lds);
-    const KArgs& k = P.k;
+    KArgs& k = P.k;
     if (P.family == F_EW) {
         if (P.n_chunks == 0 && P.tail == 0) return NGH_OK;
         if (P.n_chunks) {
             unsigned blocks = (P.n_chunks + kBlock - 1) / kBlock;
             blocks = std::min<unsigned>(blocks, (unsigned)(ctx->cus * ctx->ew_blocks_per_cu));
+            NGH_TRY(stat_scratch(ctx, k, blocks));
             if (V == 8)
                 hipLaunchKernelGGL(ew_interp_kernel<8>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, P.n_chunks, P.chunks_per_row);
             else if (V == 4)
@@ -436,6 +469,7 @@ int launch_interp(ngh_context* ctx, Plan& P) {
             else
                 hipLaunchKernelGGL(ew_interp_kernel<1>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, P.n_chunks, P.chunks_per_row);
             HIP_TRY(hipGetLastError());
+            NGH_TRY(stat_fold(ctx, k, blocks));
         }
         if (P.tail) NGH_TRY(launch_tail(ctx, P));
         return NGH_OK;
@@ -450,6 +484,7 @@ int launch_interp(ngh_context* ctx, Plan& P) {
     }
     if (P.family == F_RED_ROW) {
         const unsigned blocks = P.n_out * P.n_seg;
+        NGH_TRY(stat_scratch(ctx, k, blocks));
         if (V == 4)
             hipLaunchKernelGGL(red_row_interp_kernel<4>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, P.n_out, P.n_seg, P.seg_len, ws);
         else
@@ -457,9 +492,13 @@ int launch_interp(ngh_context* ctx, Plan& P) {
     } else {
         const unsigned long long blocks = (unsigned long long)P.n_bx * (unsigned)k.shape[1] * P.n_seg;
         if (blocks >= (1ULL << 31)) return fail(NGH_E_UNSUPPORTED, "reduction grid too large");
+        NGH_TRY(stat_scratch(ctx, k, (unsigned)blocks));
         hipLaunchKernelGGL(red_col_interp_kernel, dim3((unsigned)blocks), dim3(kBlock), lds, ctx->stream, k, P.n_bx, P.n_seg, P.seg_len, ws);
     }
     HIP_TRY(hipGetLastError());
+    if (k.n_stat_slots)
+        NGH_TRY(stat_fold(ctx, k, P.family == F_RED_ROW ? P.n_out * P.n_seg
+                                                        : (unsigned)(P.n_bx * (unsigned)k.shape[1] * P.n_seg)));
     if (P.n_seg > 1) {
         const unsigned blocks = (P.n_out + kBlock - 1) / kBlock;
         hipLaunchKernelGGL(red_finish_kernel, dim3(blocks), dim3(kBlock), 0, ctx->stream, k, P.n_out, P.n_seg,
@@ -548,6 +587,7 @@ int ngh_shutdown(ngh_context* ctx) {
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->ws) (void)hipFree(ctx->ws);
+    if (ctx->stat_ws) (void)hipFree(ctx->stat_ws);
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
     if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -673,9 +713,11 @@ int ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec) {
         if (!ctx->force_interp && !P.k.probe) {
             P.special = match_special(P.family, P.V, P.k, P.tail);
             if (P.special >= 0) {
-                hipError_t e = launch_special(P.special, ctx->stream, ctx->cus, ctx->ew_blocks_per_cu, P.k,
-                                              P.n_chunks, P.chunks_per_row);
+                const unsigned blocks = streaming_blocks(ctx->cus, ctx->ew_blocks_per_cu, P.n_chunks);
+                NGH_TRY(stat_scratch(ctx, P.k, blocks));
+                hipError_t e = launch_special(P.special, ctx->stream, blocks, P.k, P.n_chunks, P.chunks_per_row);
                 if (e != hipSuccess) return fail(NGH_E_RUNTIME, "special launch: %s", hipGetErrorString(e));
+                if (P.n_chunks) NGH_TRY(stat_fold(ctx, P.k, blocks));
                 if (P.tail) NGH_TRY(launch_tail(ctx, P));
                 continue;
             }
@@ -754,6 +796,78 @@ int ngh_stats_reset(ngh_context* ctx, int32_t* dev, int32_t n) {
 int ngh_stats_read(ngh_context* ctx, const int32_t* dev, int32_t n, int32_t* host) {
     if (n <= 0) return NGH_OK;
     return ngh_memcpy_d2h(ctx, host, dev, (size_t)n * 4);
+}
+
+int ngh_flex_states_alloc(ngh_context* ctx, int32_t n, ngh_flex_state** out_dev) {
+    if (!ctx || !out_dev || n <= 0) return fail(NGH_E_INVALID, "ngh_flex_states_alloc: bad argument");
+    void* p = nullptr;
+    NGH_TRY(ngh_malloc(ctx, (size_t)n * sizeof(ngh_flex_state), &p));
+    std::vector<ngh_flex_state> init((size_t)n);
+    for (auto& s : init) {
+        memset(&s, 0, sizeof(s));
+        s.dec = 8;
+        s.next_dec = -1;
+        s.scale = 1.0f / 256.0f;
+    }
+    *out_dev = (ngh_flex_state*)p;
+    return ngh_memcpy_h2d(ctx, p, init.data(), init.size() * sizeof(ngh_flex_state));
+}
+
+int ngh_flex_states_write(ngh_context* ctx, ngh_flex_state* dev, int32_t first, int32_t n,
+                          const ngh_flex_state* host) {
+    if (n <= 0) return NGH_OK;
+    if (!dev || !host || first < 0) return fail(NGH_E_INVALID, "ngh_flex_states_write: bad argument");
+    return ngh_memcpy_h2d(ctx, dev + first, host, (size_t)n * sizeof(ngh_flex_state));
+}
+
+int ngh_flex_states_read(ngh_context* ctx, const ngh_flex_state* dev, int32_t first, int32_t n,
+                         ngh_flex_state* host) {
+    if (n <= 0) return NGH_OK;
+    if (!dev || !host || first < 0) return fail(NGH_E_INVALID, "ngh_flex_states_read: bad argument");
+    return ngh_memcpy_d2h(ctx, host, dev + first, (size_t)n * sizeof(ngh_flex_state));
+}
+
+namespace {
+int make_flex_ids(const int32_t* ids, const int32_t* in_place, int32_t n_ids, FlexIds& out) {
+    if (n_ids < 0 || n_ids > kFlexMaxIds) return fail(NGH_E_INVALID, "n_ids %d not in 0..%d", n_ids, kFlexMaxIds);
+    if (n_ids && !ids) return fail(NGH_E_INVALID, "ids is NULL");
+    memset(&out, 0, sizeof(out));
+    out.n = n_ids;
+    for (int i = 0; i < n_ids; ++i) {
+        if (ids[i] < 0) return fail(NGH_E_INVALID, "negative flex id");
+        out.id[i] = ids[i];
+        out.in_place[i] = in_place ? in_place[i] : 0;
+    }
+    return NGH_OK;
+}
+}  // namespace
+
+int ngh_flex_prepare(ngh_context* ctx, ngh_flex_state* dev, const int32_t* ids, const int32_t* in_place,
+                     int32_t n_ids) {
+    if (!ctx || !dev) return fail(NGH_E_INVALID, "ngh_flex_prepare: NULL argument");
+    if (n_ids == 0) return NGH_OK;
+    FlexIds f;
+    NGH_TRY(make_flex_ids(ids, in_place, n_ids, f));
+    hipLaunchKernelGGL(flex_prepare_kernel, dim3(1), dim3(64), 0, ctx->stream, dev, f);
+    HIP_TRY(hipGetLastError());
+    return NGH_OK;
+}
+
+int ngh_flex_update(ngh_context* ctx, ngh_flex_state* dev, const int32_t* ids, int32_t n_ids, int32_t count) {
+    if (!ctx || !dev) return fail(NGH_E_INVALID, "ngh_flex_update: NULL argument");
+    if (n_ids == 0) return NGH_OK;
+    FlexIds f;
+    NGH_TRY(make_flex_ids(ids, nullptr, n_ids, f));
+    hipLaunchKernelGGL(flex_update_kernel, dim3(1), dim3(64), 0, ctx->stream, dev, f, (int)count);
+    HIP_TRY(hipGetLastError());
+    return NGH_OK;
+}
+
+int ngh_launch_fused_flex(ngh_context* ctx, const ngh_fused_spec* spec, ngh_flex_state* dev,
+                          const int32_t* ids, const int32_t* in_place, int32_t n_ids, int32_t count) {
+    NGH_TRY(ngh_flex_prepare(ctx, dev, ids, in_place, n_ids));
+    NGH_TRY(ngh_launch_fused(ctx, spec));
+    return ngh_flex_update(ctx, dev, ids, n_ids, count);
 }
 
 int ngh_timer_begin(ngh_context* ctx) {

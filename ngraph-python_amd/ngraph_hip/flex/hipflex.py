@@ -25,7 +25,7 @@ import math
 
 import numpy as np
 
-from ngraph_hip.flex.base import Flex, FlexEntry, FlexManager
+from ngraph_hip.flex.base import Flex, FlexManager
 
 
 class HipFlex(Flex):
@@ -46,7 +46,8 @@ class HipFlex(Flex):
             return None
         if math.isinf(maxabs):
             return self.min_dec
-        dec = (self.storage_bits - 2) - int(math.floor(math.log2(maxabs)))
+        _, e = math.frexp(maxabs)            # maxabs = m * 2**e, 0.5 <= m < 1: floor(log2) = e - 1
+        dec = (self.storage_bits - 2) - (e - 1)
         return max(self.min_dec, min(self.max_dec, dec))
 
     def get_scale(self, maxabs):
@@ -56,44 +57,135 @@ class HipFlex(Flex):
 
 hipflex16 = HipFlex(storage_bits=16)
 
+HISTORY = 16
+#: host mirror of struct ngh_flex_state (include/ngraph_hip.h)
+STATE_DTYPE = np.dtype([("stats", "<i4"), ("dec", "<i4"), ("next_dec", "<i4"), ("initialized", "<i4"),
+                        ("scale", "<f4"), ("hist_len", "<i4"), ("hist_pos", "<i4"),
+                        ("last_maxabs", "<i4"), ("last_count", "<i4"), ("pad_", "<i4"),
+                        ("history", "<f8", (HISTORY,))])
+assert STATE_DTYPE.itemsize == 168
 
-class HipFlexEntry(FlexEntry):
-    history_length = 16
-    gamma = 3.0
-    overflow_dec_step = 2
+
+def _policy_step(rec, maxabs, count, dtype):
+    """Record max|mantissa| of what was just stored and choose the next exponent.
+
+    Sequential double-precision steps; csrc/ngh_flex.h flex_update_kernel performs the same
+    steps in the same order on the device, and the two must stay equivalent."""
+    maxabs = int(maxabs)
+    rec["last_maxabs"], rec["last_count"], rec["initialized"] = maxabs, count, 1
+    value = float(maxabs) * float(rec["scale"])
+    pos = int(rec["hist_pos"])
+    hist = rec["history"]
+    if maxabs >= dtype.pclip:
+        hist[pos] = 2.0 * value
+        rec["hist_pos"] = (pos + 1) % HISTORY
+        rec["hist_len"] = min(HISTORY, int(rec["hist_len"]) + 1)
+        rec["next_dec"] = max(dtype.min_dec, int(rec["dec"]) - 2)
+        return
+    hist[pos] = value
+    rec["hist_pos"] = (pos + 1) % HISTORY
+    rec["hist_len"] = min(HISTORY, int(rec["hist_len"]) + 1)
+    n = int(rec["hist_len"])
+    mx, total = float(hist[0]), 0.0
+    for j in range(n):
+        h = float(hist[j])
+        mx = h if h > mx else mx
+        total = total + h
+    mean = total / float(n)
+    ss = 0.0
+    for j in range(n):
+        d = float(hist[j]) - mean
+        ss = ss + d * d
+    sd = math.sqrt(ss / float(n))
+    dec = dtype.fit_dec(mx + 3.0 * sd)
+    rec["next_dec"] = int(rec["dec"]) if dec is None else dec
+
+
+class HipFlexEntry(object):
+    """Exponent state of one flex tensor: a view of one record of the manager's state table.
+
+    `scale` always describes the mantissas currently in memory; the policy's choice for the
+    next write is `next_dec`, applied by adjust_scale() right before the whole tensor is
+    overwritten.
+    """
 
     def __init__(self, _id, dtype, init_dec, manager, name=None):
-        super(HipFlexEntry, self).__init__(_id, dtype, init_dec)
+        self._id = _id
+        self.dtype = dtype
         self.manager = manager
         self.name = name
-        self.initialized = False
-        self.history = collections.deque(maxlen=self.history_length)
-        self.ptr = None                 # device int32 word receiving max|mantissa|
-        self.last_maxabs = 0
-        self.last_count = -1
-        self.next_dec = None
+        rec = self._rec(sync=False)
+        rec["dec"], rec["next_dec"], rec["scale"] = init_dec, -1, 1.0 / 2 ** init_dec
+
+    def _rec(self, sync=True):
+        if sync:
+            self.manager.pull()
+        return self.manager.table[self._id]
+
+    def _touch(self):
+        self.manager.host_dirty = True
+
+    @property
+    def flex_id(self):
+        return self._id
+
+    @property
+    def scale(self):
+        return float(self._rec()["scale"])
 
     @property
     def dec(self):
-        return int(round(-math.log2(self.scale)))
+        return int(self._rec()["dec"])
+
+    @property
+    def next_dec(self):
+        v = int(self._rec()["next_dec"])
+        return None if v < 0 else v
+
+    @property
+    def initialized(self):
+        return bool(self._rec()["initialized"])
+
+    @property
+    def last_maxabs(self):
+        return int(self._rec()["last_maxabs"])
+
+    @property
+    def history(self):
+        rec = self._rec()
+        n, pos = int(rec["hist_len"]), int(rec["hist_pos"])
+        h = [float(x) for x in rec["history"][:n]]
+        return h if n < HISTORY else h[pos:] + h[:pos]
+
+    @property
+    def ptr(self):
+        """Device address of this tensor's statistics word."""
+        return self.manager.state_address(self._id, "stats")
+
+    @property
+    def scale_ptr(self):
+        return self.manager.state_address(self._id, "scale")
 
     def set_dec(self, dec):
-        self.scale = 1.0 / 2 ** int(dec)
+        rec = self._rec()
+        rec["dec"], rec["scale"] = int(dec), 1.0 / 2 ** int(dec)
+        self._touch()
 
     # ---- policy -------------------------------------------------------------------------
-    # `scale` always describes the mantissas currently in memory.  The policy's choice for
-    # the NEXT write is kept in `next_dec` and only takes effect in adjust_scale(), which
-    # runs immediately before something overwrites the whole tensor.
     def init_from_value(self, maxabs_value):
+        rec = self._rec()
         if not self.manager.fixed_point:
             dec = self.dtype.fit_dec(maxabs_value)
-            self.set_dec(FlexManager.default_dec if dec is None else dec)
-        self.next_dec = self.dec
-        self.initialized = True
+            dec = FlexManager.default_dec if dec is None else dec
+            rec["dec"], rec["scale"] = dec, 1.0 / 2 ** dec
+        rec["next_dec"], rec["initialized"] = rec["dec"], 1
+        self._touch()
 
     def adjust_scale(self):
-        if self.initialized and self.next_dec is not None:
-            self.set_dec(self.next_dec)
+        rec = self._rec()
+        if rec["initialized"] and rec["next_dec"] >= 0:
+            rec["dec"], rec["scale"] = rec["next_dec"], 1.0 / 2 ** int(rec["next_dec"])
+            self._touch()
 
     def manage_before_computation(self, value=None):
         """Host write path: the first value a tensor receives fixes its initial scale; later
@@ -106,75 +198,118 @@ class HipFlexEntry(FlexEntry):
             self.adjust_scale()
 
     def manage_after_computation(self, maxabs, autoflex_count):
-        """Record max|mantissa| of what was just stored and choose the next scale."""
-        maxabs = int(maxabs)
-        self.last_maxabs, self.last_count = maxabs, autoflex_count
-        self.initialized = True
+        rec = self._rec()
         if self.manager.fixed_point:
-            return
-        value = maxabs * self.scale
-        if maxabs >= self.dtype.pclip:
-            self.history.append(2.0 * value)
-            self.next_dec = max(self.dtype.min_dec, self.dec - self.overflow_dec_step)
-            return
-        self.history.append(value)
-        h = np.asarray(self.history, dtype=np.float64)
-        dec = self.dtype.fit_dec(float(h.max() + self.gamma * h.std()))
-        self.next_dec = self.dec if dec is None else dec
+            rec["last_maxabs"], rec["last_count"], rec["initialized"] = int(maxabs), autoflex_count, 1
+        else:
+            _policy_step(rec, maxabs, autoflex_count, self.dtype)
+        self._touch()
 
     def reset_entry(self):
-        self.history.clear()
-        self.initialized = False
-        self.next_dec = None
-        self.set_dec(FlexManager.default_dec)
+        rec = self._rec()
+        rec["hist_len"] = rec["hist_pos"] = rec["initialized"] = 0
+        rec["next_dec"] = -1
+        rec["dec"], rec["scale"] = FlexManager.default_dec, 1.0 / 2 ** FlexManager.default_dec
+        self._touch()
 
 
 class HipFlexManager(FlexManager):
-    """Creates entries, owns their device statistics words, runs the policy around kernels."""
+    """Creates entries, owns the state table (host mirror + device copy), runs the policy.
 
-    def __init__(self, fixed_point=False, verbose=False):
+    resident=False  statistics come back to the host after every kernel and the policy runs
+                    in Python, as in the reference (flexgputransform.py:347-366).
+    resident=True   kernels read scales from, and the policy runs on, the device copy of the
+                    table; the host mirror is refreshed only when somebody looks at it.
+    """
+
+    def __init__(self, fixed_point=False, verbose=False, resident=False):
         super(HipFlexManager, self).__init__()
         self.fixed_point = fixed_point
         self.verbose = verbose
+        self.resident = resident and not fixed_point
         self.autoflex_count = 0
         self.runtime = None
-        self._stats_base = None
-        self._allocated = 0
+        self.table = np.zeros(64, dtype=STATE_DTYPE)
+        self.dev_table = None          # device address of the table copy
+        self._dev_capacity = 0
+        self.host_dirty = False        # host mirror changed since the last push
+        self.device_dirty = False      # device copy changed since the last pull
 
     def make_flex_entry(self, name=None, dtype=None):
         flex_id = self._num_flex_tensors
+        if flex_id >= len(self.table):
+            self.pull()
+            grown = np.zeros(2 * len(self.table), dtype=STATE_DTYPE)
+            grown[:len(self.table)] = self.table
+            self.table = grown
+        self._num_flex_tensors += 1
         entry = HipFlexEntry(flex_id, dtype or hipflex16, FlexManager.default_dec, self, name=name)
         self.flex_entries[flex_id] = entry
-        self._num_flex_tensors += 1
+        self.host_dirty = True
         return entry
 
+    # ---- device copy ---------------------------------------------------------------------
     def allocate(self, runtime=None):
-        """Device words for every entry created so far (idempotent; grows when entries were added)."""
+        """(Re)create the device copy so it covers every entry made so far."""
         if runtime is not None:
             self.runtime = runtime
         n = self._num_flex_tensors
-        if n == 0 or n <= self._allocated:
+        if n == 0 or n <= self._dev_capacity:
             return
-        base = self.runtime.stats_alloc(n)
-        self._stats_base, self._allocated = base, n
-        for flex_id, entry in self.flex_entries.items():
-            entry.ptr = base + 4 * flex_id
+        self.pull()
+        capacity = len(self.table)
+        self.dev_table = self.runtime.flex_states_alloc(capacity)
+        self._dev_capacity = capacity
+        self.host_dirty = True
+        self.push()
+
+    def state_address(self, flex_id, field):
+        if self.dev_table is None:
+            return None
+        return self.dev_table + flex_id * STATE_DTYPE.itemsize + STATE_DTYPE.fields[field][1]
+
+    def push(self):
+        if self.host_dirty and self.dev_table is not None:
+            self.runtime.flex_states_write(self.dev_table, 0, self.table[:self._dev_capacity])
+        self.host_dirty = False
+
+    def pull(self):
+        if self.device_dirty and self.dev_table is not None:
+            self.device_dirty = False
+            self.runtime.flex_states_read(self.dev_table, 0, self.table[:self._dev_capacity])
 
     # ---- around kernels (flexgputransform.py:347-366) ------------------------------------
     def manage_before_computation(self, kernel):
+        entries = kernel.output_flex_entries
+        if not entries:
+            return
         in_place = getattr(kernel, "in_place_flex_ids", ())
-        for entry in kernel.output_flex_entries:
+        if self.resident:
+            self.push()
+            self.runtime.flex_prepare(self.dev_table, [e.flex_id for e in entries],
+                                      [1 if e.flex_id in in_place else 0 for e in entries])
+            self.device_dirty = True
+            return
+        for entry in entries:
             if entry.flex_id not in in_place:
                 # a tensor the kernel also reads keeps the scale its data was stored with
                 entry.adjust_scale()
+        for entry in entries:
             self.runtime.stats_reset(entry.ptr, 1)
 
     def manage_after_computation(self, kernel):
-        for entry in kernel.output_flex_entries:
+        entries = kernel.output_flex_entries
+        if not entries:
+            return
+        if self.resident:
+            self.runtime.flex_update(self.dev_table, [e.flex_id for e in entries], self.autoflex_count)
+            self.device_dirty = True
+            return
+        for entry in entries:
             maxabs = int(self.runtime.stats_read(entry.ptr, 1)[0])
             entry.manage_after_computation(maxabs, self.autoflex_count)
             if self.verbose:
-                print("flex %s: maxabs %d -> dec %d" % (entry.name, maxabs, entry.dec))
+                print("flex %s: maxabs %d -> next dec %s" % (entry.name, maxabs, entry.next_dec))
 
     def set_h5py_file(self, data_file):
         self.data_file = data_file

@@ -107,6 +107,13 @@ _SYMBOLS = {
     "ngh_stats_alloc": [_vp, _i32, ctypes.POINTER(_vp)],
     "ngh_stats_reset": [_vp, _vp, _i32],
     "ngh_stats_read": [_vp, _vp, _i32, _vp],
+    "ngh_flex_states_alloc": [_vp, _i32, ctypes.POINTER(_vp)],
+    "ngh_flex_states_write": [_vp, _vp, _i32, _i32, _vp],
+    "ngh_flex_states_read": [_vp, _vp, _i32, _i32, _vp],
+    "ngh_flex_prepare": [_vp, _vp, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32), _i32],
+    "ngh_flex_update": [_vp, _vp, ctypes.POINTER(ctypes.c_int32), _i32, _i32],
+    "ngh_launch_fused_flex": [_vp, ctypes.POINTER(ngh_fused_spec), _vp, ctypes.POINTER(ctypes.c_int32),
+                              ctypes.POINTER(ctypes.c_int32), _i32, _i32],
     "ngh_timer_begin": [_vp],
     "ngh_timer_end": [_vp, ctypes.POINTER(ctypes.c_float)],
 }
@@ -311,6 +318,42 @@ class HipRuntime(object):
                                                  out.ctypes.data_as(ctypes.c_void_p)))
         return out
 
+    # -- device-resident flex state ------------------------------------------
+    def flex_states_alloc(self, n):
+        ptr = ctypes.c_void_p()
+        _check(self.lib, self.lib.ngh_flex_states_alloc(self.ctx, int(n), ctypes.byref(ptr)))
+        self._allocs.add(ptr.value)
+        return ptr.value
+
+    def flex_states_write(self, dev, first, records):
+        records = np.ascontiguousarray(records)
+        _check(self.lib, self.lib.ngh_flex_states_write(self.ctx, ctypes.c_void_p(dev), int(first),
+                                                        len(records), records.ctypes.data_as(ctypes.c_void_p)))
+
+    def flex_states_read(self, dev, first, records):
+        assert records.flags.c_contiguous
+        _check(self.lib, self.lib.ngh_flex_states_read(self.ctx, ctypes.c_void_p(dev), int(first),
+                                                       len(records), records.ctypes.data_as(ctypes.c_void_p)))
+
+    def flex_prepare(self, dev, ids, in_place):
+        n = len(ids)
+        arr = ctypes.c_int32 * max(n, 1)
+        _check(self.lib, self.lib.ngh_flex_prepare(self.ctx, ctypes.c_void_p(dev), arr(*ids), arr(*in_place), n))
+
+    def flex_update(self, dev, ids, count):
+        n = len(ids)
+        arr = ctypes.c_int32 * max(n, 1)
+        _check(self.lib, self.lib.ngh_flex_update(self.ctx, ctypes.c_void_p(dev), arr(*ids), n, int(count)))
+
+    def make_id_arrays(self, ids, in_place):
+        arr = ctypes.c_int32 * max(len(ids), 1)
+        return arr(*ids), arr(*in_place), len(ids)
+
+    def launch_fused_flex(self, spec, dev, id_arrays, count):
+        ids, in_place, n = id_arrays
+        _check(self.lib, self.lib.ngh_launch_fused_flex(self.ctx, ctypes.byref(spec), ctypes.c_void_p(dev),
+                                                        ids, in_place, n, int(count)))
+
     # -- timing ------------------------------------------------------------
     def timer_begin(self):
         _check(self.lib, self.lib.ngh_timer_begin(self.ctx))
@@ -376,6 +419,27 @@ class DryRunRuntime(object):
 
     def stats_read(self, dev, n=1):
         raise HipLibraryError(-5, "dry-run runtime holds no data")
+
+    def flex_states_alloc(self, n):
+        return self.malloc(168 * n)
+
+    def flex_states_write(self, dev, first, records):
+        pass
+
+    def flex_states_read(self, dev, first, records):
+        raise HipLibraryError(-5, "dry-run runtime holds no data")
+
+    def flex_prepare(self, dev, ids, in_place):
+        pass
+
+    def flex_update(self, dev, ids, count):
+        pass
+
+    def make_id_arrays(self, ids, in_place):
+        return (ids, in_place, len(ids))
+
+    def launch_fused_flex(self, spec, dev, id_arrays, count):
+        self.launch_fused(spec)
 
 
 class FusedSpecBuilder(object):

@@ -129,10 +129,30 @@ class FlexFusedKernel(FusedKernel):
         return [e.flex_id for e in self.output_flex_entries]
 
     def bind_flex_scales(self):
+        """Host-managed mode: the current scales travel as kernel arguments, rebound before
+        every launch (flexgputransform.py:56-61)."""
         for index, slot, entry, is_output in self.flex_bindings:
             t = self.specs[index].tensors[slot]
             t.scale = entry.scale
+            t.dev_scale = None
             t.dev_stats = entry.ptr if is_output else None
+
+    def bind_flex_state_pointers(self):
+        """Device-resident mode: kernels read scales from the state table; bound once."""
+        if getattr(self, "_state_bound", False):
+            return
+        for index, slot, entry, is_output in self.flex_bindings:
+            t = self.specs[index].tensors[slot]
+            t.dev_scale = entry.scale_ptr
+            t.dev_stats = entry.ptr if is_output else None
+        self._state_bound = True
+
+    def execute_managed(self, rt, dev_table, count):
+        if not hasattr(self, "_id_arrays"):
+            ids = [e.flex_id for e in self.output_flex_entries]
+            self._id_arrays = rt.make_id_arrays(ids, [1 if i in self.in_place_flex_ids else 0 for i in ids])
+        for spec in self.specs:
+            rt.launch_fused_flex(spec, dev_table, self._id_arrays, count)
 
     def probe(self):
         """Measure max|fp32 result| of every not yet initialised output without storing."""
@@ -160,6 +180,12 @@ class FlexCopyKernel(CopyKernel):
 
     output_flex_entries = ()
 
+    def bind_flex_state_pointers(self):
+        pass
+
+    def execute_managed(self, rt, dev_table, count):
+        self.execute()
+
     def bind_buffers(self):
         t = self.transformer
         src_buf = t.op_tensors[self.op.args[0].forwarded.tensor_description().base]
@@ -175,16 +201,38 @@ class FlexHipKernelGroup(HipKernelGroup):
     """Flex management around every kernel (flexgputransform.py:224-371)."""
 
     def setup_kernel_execute(self, kernel):
-        kernel.probe()
-        self.transformer.flex_manager.manage_before_computation(kernel)
-        kernel.bind_flex_scales()
+        manager = self.transformer.flex_manager
+        if manager.resident and not getattr(kernel, "_all_initialized", False):
+            kernel.probe()
+            kernel._all_initialized = all(e.initialized for e in kernel.output_flex_entries)
+        elif not manager.resident:
+            kernel.probe()
+        manager.manage_before_computation(kernel)
+        if manager.resident:
+            kernel.bind_flex_state_pointers()
+        else:
+            kernel.bind_flex_scales()
 
     def after_kernel_execute(self, kernel):
         self.transformer.flex_manager.manage_after_computation(kernel)
 
     def __call__(self):
-        self.transformer.flex_manager.autoflex_count += 1
+        manager = self.transformer.flex_manager
+        manager.autoflex_count += 1
+        if manager.resident and getattr(self, "_steady", False):
+            # steady state of the device-resident mode: every tensor initialised, pointers
+            # bound; one library call per kernel does prepare + launch + policy update
+            manager.push()
+            rt, count = self.transformer.runtime, manager.autoflex_count
+            for k in self.kernels:
+                k.execute_managed(rt, manager.dev_table, count)
+            manager.device_dirty = True
+            return
         super(FlexHipKernelGroup, self).__call__()
+        if manager.resident:
+            self._steady = all(getattr(k, "_all_initialized", False) or not k.output_flex_entries
+                               for k in self.kernels) and \
+                all(isinstance(k, (FlexFusedKernel, FlexCopyKernel)) for k in self.kernels)
 
     @property
     def output_flex_ids(self):
@@ -203,8 +251,12 @@ class FlexHipTransformer(HipTransformer):
     atol_precision_multiplier = 8
     kernel_group_class = FlexHipKernelGroup
 
-    def __init__(self, fixed_point=False, flex_verbose=False, collect_flex_data=False, **kwargs):
-        self.flex_manager = HipFlexManager(fixed_point=fixed_point, verbose=flex_verbose)
+    def __init__(self, fixed_point=False, flex_verbose=False, collect_flex_data=False,
+                 resident=False, **kwargs):
+        """resident=True keeps scales, statistics and the exponent policy on the device (no
+        host round trip per kernel); False follows the reference's per-kernel read-back."""
+        self.flex_manager = HipFlexManager(fixed_point=fixed_point, verbose=flex_verbose,
+                                           resident=resident)
         kwargs.setdefault("fuse_moments", False)
         super(FlexHipTransformer, self).__init__(**kwargs)
         self.flex_manager.runtime = self.runtime

@@ -85,7 +85,7 @@ def fit_dec(value):
         return None
     if math.isinf(value):
         return MIN_DEC
-    dec = 14 - int(math.floor(math.log2(value)))
+    dec = 14 - int(np.floor(np.log2(np.float64(value))))
     return max(MIN_DEC, min(MAX_DEC, dec))
 
 
@@ -124,35 +124,6 @@ class FlexPolicy(object):
 
 
 # ---------------------------------------------------------------------------------- simulator
-class FlexTensor(object):
-    def __init__(self, shape=()):
-        self.policy = FlexPolicy()
-        self.mantissa = np.zeros(shape, dtype=np.int16)
-
-    def host_write(self, value):
-        value = np.asarray(value, dtype=np.float64)
-        if not self.policy.initialized:
-            self.policy.init_from_value(np.max(np.abs(value)) if value.size else 0.0)
-        self.mantissa = quantize_host(np.broadcast_to(value, self.mantissa.shape), self.policy.dec)
-        self.policy.record(maxabs(self.mantissa))
-
-    def kernel_write(self, compute):
-        """`compute()` returns the fp32 result; P2 on first use, then store + record."""
-        result = np.asarray(compute(), dtype=f32)
-        if not self.policy.initialized:
-            finite = np.where(np.isnan(result), f32(0), np.abs(result))
-            self.policy.init_from_value(float(np.max(finite)) if result.size else 0.0)
-        self.mantissa = quantize_rni(result, self.policy.dec)
-        self.policy.record(maxabs(self.mantissa))
-
-    def read(self):
-        return dequantize(self.mantissa, self.policy.dec)
-
-    def value(self):
-        """What a kernel sees when it loads this tensor (uses the dec it was stored with)."""
-        return dequantize(self.mantissa, self._stored_dec)
-
-
 class FlexSim(object):
     """Op-by-op flex execution of a tiny graph: placeholders -> ops -> result.
 

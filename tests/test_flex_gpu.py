@@ -90,8 +90,9 @@ def _model_c5(xs, w, b):
     return out
 
 
+@pytest.mark.parametrize("resident", [False, True], ids=["host-policy", "device-policy"])
 @pytest.mark.parametrize("n", [1 << 16, 100003])
-def test_c5_fused_flex_bit_exact_over_8_iterations(n):
+def test_c5_fused_flex_bit_exact_over_8_iterations(n, resident):
     x0, w, b = configs.c5_inputs(n, seed=4)
     # activations that grow, then collapse: exercises overflow (dec -= 2), the headroom
     # predictor and the slow return to finer exponents
@@ -99,7 +100,7 @@ def test_c5_fused_flex_bit_exact_over_8_iterations(n):
     xs = [(x0 * g).astype(np.float32) for g in gains]
     want = _model_c5(xs, w, b)
 
-    t = ngt.make_transformer_factory("flexhip")()
+    t = ngt.make_transformer_factory("flexhip", resident=resident)()
     f, (x, wp, bp), y = _c5_graph(t, n)
     try:
         for i, xi in enumerate(xs):
@@ -131,3 +132,38 @@ def test_flex_host_io_truncates_and_dequantises():
         np.testing.assert_array_equal(got, np.array([19660, 18022, -21299, 22937]) / 16384.0)
     finally:
         t.close()
+
+
+def test_device_policy_follows_host_policy_state_for_state():
+    """The exponent policy run by flex_update_kernel against the Python mirror, driven with the
+    same max|mantissa| sequences through the C ABI (no fused kernel involved)."""
+    from ngraph_hip.runtime import HipRuntime
+    from ngraph_hip.flex.hipflex import HipFlexManager, STATE_DTYPE
+    rt = HipRuntime(0)
+    try:
+        rs = np.random.RandomState(9)
+        host = HipFlexManager()
+        n = 8
+        entries = [host.make_flex_entry("e%d" % i) for i in range(n)]
+        for i, e in enumerate(entries):
+            e.init_from_value(10.0 ** rs.uniform(-5, 4))
+        dev = rt.flex_states_alloc(n)
+        rt.flex_states_write(dev, 0, host.table[:n])
+        ids = list(range(n))
+        for step in range(60):
+            maxima = rs.choice([0, 3, 900, 16384, 25000, 32766, 32767, 32768], size=n)
+            # device: prepare (adopts next_dec, clears stats), plant the statistics, update
+            rt.flex_prepare(dev, ids, [0] * n)
+            table = np.zeros(n, dtype=STATE_DTYPE)
+            rt.flex_states_read(dev, 0, table)
+            table["stats"] = maxima
+            rt.flex_states_write(dev, 0, table)
+            rt.flex_update(dev, ids, step)
+            rt.flex_states_read(dev, 0, table)
+            for i, e in enumerate(entries):
+                e.adjust_scale()
+                e.manage_after_computation(int(maxima[i]), step)
+            for field in ("dec", "next_dec", "scale", "hist_len", "hist_pos", "last_maxabs", "history"):
+                np.testing.assert_array_equal(table[field], host.table[:n][field], err_msg=field)
+    finally:
+        rt.close()
