@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define NGH_ABI_VERSION 1
+#define NGH_ABI_VERSION 2
 
 /* ---- limits (float_ew2.py:285-286 MAX_AXES = 3) ------------------------ */
 #define NGH_MAX_AXES      3
@@ -91,6 +91,15 @@ enum ngh_opcode {
     NGH_OP_COUNT_
 };
 
+/* ngh_tensor.cache_hint */
+enum {
+    NGH_CACHE_STREAM_LOAD  = 1u,  /* no other kernel of the computation reads the operand:
+                                     load it non-temporally                                */
+    NGH_CACHE_STREAM_STORE = 2u   /* nothing reads the result soon (not an in-place update,
+                                     no later kernel of the computation reads it): store it
+                                     non-temporally so it does not displace operands        */
+};
+
 typedef struct ngh_op {
     uint8_t opcode;            /* enum ngh_opcode                            */
     uint8_t dst;
@@ -121,6 +130,12 @@ typedef struct ngh_tensor {
                                   word instead of `scale` (lets an on-device
                                   exponent update feed the next launch
                                   without a host round trip)                 */
+    uint32_t cache_hint;       /* NGH_CACHE_* bits: what the caller knows of
+                                  this operand's reuse.  Hints only act in
+                                  streaming kernels whose operands exceed the
+                                  last-level cache; no counterpart in the
+                                  reference (PTX loads there carry no hint)   */
+    uint32_t reserved_;
 } ngh_tensor;
 
 /* One stage = a run of elementwise ops optionally ended by reductions
@@ -189,11 +204,11 @@ int  ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec,
                         int32_t stage, char* name128);
 
 /* Per-row mean and (biased) variance of a [rows, R] fp32 matrix with contiguous rows in ONE
- * read of x: fuses the reductions behind ng.mean + ng.variance
+ * read of x (x_cache_hint: NGH_CACHE_* bits for x): fuses the reductions behind ng.mean + ng.variance
  * (op_graph.py:4007-4009, 4252-4266), the statistics of batch normalisation
  * (frontends/neon/layer.py:1242-1245).  row_stride in elements, multiple of 4.  */
 int  ngh_moments_f32(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t R, int64_t row_stride,
-                     float* dev_mean, float* dev_var);
+                     float* dev_mean, float* dev_var, uint32_t x_cache_hint);
 
 /* How stage `stage` would be launched, without a device (host-side tooling and
  * tests): out8 = {kernel family (0 streaming, 1 reduce along the contiguous axis,

@@ -17,6 +17,19 @@ namespace ngh {
 constexpr int kMomBlock = 256;
 constexpr int kMomUnroll = 4;     // float4 loads in flight per lane
 
+typedef float mom_f4 __attribute__((ext_vector_type(4)));
+
+template <bool NT>
+__device__ __forceinline__ float4 mom_load(const float4* p) {
+    if constexpr (NT) {
+        const mom_f4 v = __builtin_nontemporal_load(reinterpret_cast<const mom_f4*>(p));
+        return make_float4(v.x, v.y, v.z, v.w);
+    } else {
+        return *p;
+    }
+}
+
+template <bool NT>
 __global__ __launch_bounds__(kMomBlock) void moments_partial_kernel(
     const float* __restrict__ x, long long row_stride, unsigned R4, unsigned n_seg, unsigned seg_chunks,
     float2* __restrict__ partial) {
@@ -34,7 +47,7 @@ __global__ __launch_bounds__(kMomBlock) void moments_partial_kernel(
     for (; c + (kMomUnroll - 1) * kMomBlock < c_end; c += kMomUnroll * kMomBlock) {
         float4 v[kMomUnroll];
 #pragma unroll
-        for (int u = 0; u < kMomUnroll; ++u) v[u] = x4[c + u * kMomBlock];
+        for (int u = 0; u < kMomUnroll; ++u) v[u] = mom_load<NT>(x4 + c + u * kMomBlock);
 #pragma unroll
         for (int u = 0; u < kMomUnroll; ++u) {
             const float a = v[u].x - pivot, b = v[u].y - pivot, cc = v[u].z - pivot, d = v[u].w - pivot;
@@ -43,7 +56,7 @@ __global__ __launch_bounds__(kMomBlock) void moments_partial_kernel(
         }
     }
     for (; c < c_end; c += kMomBlock) {
-        const float4 v = x4[c];
+        const float4 v = mom_load<NT>(x4 + c);
         const float a = v.x - pivot, b = v.y - pivot, cc = v.z - pivot, d = v.w - pivot;
         s1[0] += (a + b) + (cc + d);
         s2[0] += (a * a + b * b) + (cc * cc + d * d);

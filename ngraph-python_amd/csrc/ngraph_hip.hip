@@ -76,6 +76,9 @@ struct ngh_context {
     unsigned    stat_ws_blocks = 0;  // capacity per statistics slot
     int         ew_blocks_per_cu = 64;
     int         force_interp = 0;    // never pick a specialised kernel
+    int         cache_policy = -1;   // -1: from the operands' cache hints; 0..3 forces bit 0 = non-temporal
+                                     // loads, bit 1 = non-temporal stores in pre-built kernels
+    long long   stream_bytes = 128ll << 20;  // hints act on stages touching at least this much memory
     int         moments_wgs_per_cu = 16;
     char        name[256] = "";
     uint64_t    total_bytes = 0;
@@ -558,6 +561,8 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     snprintf(ctx->name, sizeof(ctx->name), "%s (%s)", prop.name, prop.gcnArchName);
     ctx->ew_blocks_per_cu = std::max(1, env_int("NGH_EW_BLOCKS_PER_CU", 64));
     ctx->force_interp = env_int("NGH_FORCE_INTERP", 0);
+    ctx->cache_policy = env_int("NGH_CACHE_POLICY", -1);
+    ctx->stream_bytes = (long long)env_int("NGH_STREAM_MIB", 128) << 20;
     ctx->moments_wgs_per_cu = std::max(1, env_int("NGH_MOMENTS_WGS_PER_CU", 16));
     hipError_t e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev0);
@@ -703,6 +708,39 @@ int ngh_copy_strided(ngh_context* ctx, void* dev_dst, const void* dev_src, int32
 
 int ngh_validate_fused(const ngh_fused_spec* spec) { return validate(spec); }
 
+// Cache policy of a streaming stage (bit 0 non-temporal loads, bit 1 non-temporal stores).
+// The hints only matter once the operands no longer fit the last-level cache (256 MiB on
+// MI355X): below `stream_bytes` everything is left cacheable.  Above it, loads stream when
+// every full-size operand read is marked as read by this kernel only, and stores stream
+// when every operand written is marked as not read again soon.
+static int stage_cache_policy(const ngh_context* ctx, const ngh_fused_spec& sp, const ngh_stage& S) {
+    if (ctx->cache_policy >= 0) return ctx->cache_policy & 3;
+    bool loads[NGH_MAX_TENSORS], stores[NGH_MAX_TENSORS];
+    stage_tensors(sp, S, loads, stores);
+    long long bytes = 0;
+    bool any_load = false, all_load = true, any_store = false, all_store = true;
+    for (int t = 0; t < sp.n_tensors; ++t) {
+        if (!loads[t] && !stores[t]) continue;
+        long long n = 1;
+        bool full = true;
+        for (int a = 0; a < sp.rank; ++a) {
+            if (sp.tensors[t].strides[a] != 0) n *= sp.shape[a];
+            else if (sp.shape[a] > 1) full = false;
+        }
+        bytes += n * itemsize_of(sp.tensors[t].dtype);
+        if (loads[t] && full) {
+            any_load = true;
+            all_load = all_load && (sp.tensors[t].cache_hint & NGH_CACHE_STREAM_LOAD);
+        }
+        if (stores[t]) {
+            any_store = true;
+            all_store = all_store && (sp.tensors[t].cache_hint & NGH_CACHE_STREAM_STORE);
+        }
+    }
+    if (bytes < ctx->stream_bytes) return 0;
+    return ((any_load && all_load) ? 1 : 0) | ((any_store && all_store) ? 2 : 0);
+}
+
 int ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec) {
     if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
     NGH_TRY(validate(spec));
@@ -715,7 +753,8 @@ int ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec) {
             if (P.special >= 0) {
                 const unsigned blocks = streaming_blocks(ctx->cus, ctx->ew_blocks_per_cu, P.n_chunks);
                 NGH_TRY(stat_scratch(ctx, P.k, blocks));
-                hipError_t e = launch_special(P.special, ctx->stream, blocks, P.k, P.n_chunks, P.chunks_per_row);
+                hipError_t e = launch_special(P.special, ctx->stream, blocks, P.k, P.n_chunks, P.chunks_per_row,
+                                              stage_cache_policy(ctx, *spec, spec->stages[s]));
                 if (e != hipSuccess) return fail(NGH_E_RUNTIME, "special launch: %s", hipGetErrorString(e));
                 if (P.n_chunks) NGH_TRY(stat_fold(ctx, P.k, blocks));
                 if (P.tail) NGH_TRY(launch_tail(ctx, P));
@@ -735,11 +774,16 @@ int ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec, int32_t sta
     NGH_TRY(plan_stage(ctx, *spec, stage, P));
     if (!ctx->force_interp) P.special = match_special(P.family, P.V, P.k, P.tail);
     describe(P, name128, 128);
+    if (P.special >= 0) {
+        static const char* const suffix[4] = {"", "/nt-loads", "/nt-stores", "/nt-loads-stores"};
+        const int cp = stage_cache_policy(ctx, *spec, spec->stages[stage]);
+        strncat(name128, suffix[cp], 127 - strlen(name128));
+    }
     return NGH_OK;
 }
 
 int ngh_moments_f32(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t R, int64_t row_stride,
-                    float* dev_mean, float* dev_var) {
+                    float* dev_mean, float* dev_var, uint32_t x_cache_hint) {
     if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
     if (rows < 0 || R <= 0) return fail(NGH_E_INVALID, "rows %lld, R %lld", (long long)rows, (long long)R);
     if (rows == 0) return NGH_OK;
@@ -757,8 +801,15 @@ int ngh_moments_f32(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t 
     const unsigned n_seg_eff = std::max(1u, n_seg);
     NGH_TRY(ensure_ws(ctx, (size_t)rows * n_seg_eff * sizeof(float2)));
     float2* partial = (float2*)ctx->ws;
-    hipLaunchKernelGGL(moments_partial_kernel, dim3((unsigned)(rows * n_seg_eff)), dim3(kMomBlock), 0, ctx->stream,
-                       dev_x, (long long)row_stride, R4, n_seg_eff, seg_chunks, partial);
+    const bool stream_x = ctx->cache_policy >= 0
+                              ? (ctx->cache_policy & 1)
+                              : ((x_cache_hint & NGH_CACHE_STREAM_LOAD) && rows * R * 4 >= ctx->stream_bytes);
+    if (stream_x)
+        hipLaunchKernelGGL(moments_partial_kernel<true>, dim3((unsigned)(rows * n_seg_eff)), dim3(kMomBlock), 0,
+                           ctx->stream, dev_x, (long long)row_stride, R4, n_seg_eff, seg_chunks, partial);
+    else
+        hipLaunchKernelGGL(moments_partial_kernel<false>, dim3((unsigned)(rows * n_seg_eff)), dim3(kMomBlock), 0,
+                           ctx->stream, dev_x, (long long)row_stride, R4, n_seg_eff, seg_chunks, partial);
     HIP_TRY(hipGetLastError());
     hipLaunchKernelGGL(moments_finish_kernel, dim3((unsigned)rows), dim3(64), 0, ctx->stream, dev_x,
                        (long long)row_stride, (unsigned)R, R4 * 4, n_seg_eff, partial, dev_mean, dev_var);

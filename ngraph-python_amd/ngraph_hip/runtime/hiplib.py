@@ -12,7 +12,7 @@ import os
 
 import numpy as np
 
-NGH_ABI_VERSION = 1
+NGH_ABI_VERSION = 2
 NGH_MAX_AXES = 3
 NGH_MAX_TENSORS = 12
 NGH_MAX_OPS = 96
@@ -23,6 +23,7 @@ NGH_MAX_STAGES = 6
 
 NGH_F32, NGH_FLEX16, NGH_I32, NGH_F16 = 0, 1, 2, 3
 NGH_SPEC_PROBE = 1
+NGH_CACHE_STREAM_LOAD, NGH_CACHE_STREAM_STORE = 1, 2
 
 _OPCODE_NAMES = [
     "nop", "load", "store", "const", "iota",
@@ -50,7 +51,9 @@ class ngh_tensor(ctypes.Structure):
                 ("dtype", ctypes.c_int32),
                 ("scale", ctypes.c_float),
                 ("dev_stats", ctypes.c_void_p),
-                ("dev_scale", ctypes.c_void_p)]
+                ("dev_scale", ctypes.c_void_p),
+                ("cache_hint", ctypes.c_uint32),
+                ("reserved_", ctypes.c_uint32)]
 
 
 class ngh_stage(ctypes.Structure):
@@ -102,7 +105,7 @@ _SYMBOLS = {
     "ngh_validate_fused": [ctypes.POINTER(ngh_fused_spec)],
     "ngh_launch_fused": [_vp, ctypes.POINTER(ngh_fused_spec)],
     "ngh_describe_fused": [_vp, ctypes.POINTER(ngh_fused_spec), _i32, ctypes.c_char_p],
-    "ngh_moments_f32": [_vp, _vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, _vp, _vp],
+    "ngh_moments_f32": [_vp, _vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, _vp, _vp, ctypes.c_uint32],
     "ngh_plan_fused": [ctypes.POINTER(ngh_fused_spec), _i32, ctypes.POINTER(ctypes.c_int32)],
     "ngh_stats_alloc": [_vp, _i32, ctypes.POINTER(_vp)],
     "ngh_stats_reset": [_vp, _vp, _i32],
@@ -297,10 +300,10 @@ class HipRuntime(object):
         _check(self.lib, self.lib.ngh_describe_fused(self.ctx, ctypes.byref(spec), int(stage), name))
         return name.value.decode()
 
-    def moments_f32(self, x, rows, R, row_stride, mean, var):
+    def moments_f32(self, x, rows, R, row_stride, mean, var, x_cache_hint=0):
         _check(self.lib, self.lib.ngh_moments_f32(self.ctx, ctypes.c_void_p(x), int(rows), int(R),
                                                   int(row_stride), ctypes.c_void_p(mean),
-                                                  ctypes.c_void_p(var)))
+                                                  ctypes.c_void_p(var), int(x_cache_hint)))
 
     # -- flex statistics ---------------------------------------------------
     def stats_alloc(self, n):

@@ -30,7 +30,8 @@ from ngraph_hip.op_graph.op_graph import Op, OrderedSet
 from ngraph_hip.runtime.hiplib import (HipRuntime, DryRunRuntime, HipLibraryError, FusedSpecBuilder, NGH_F32,
                                        NGH_FLEX16, NGH_I32, NGH_F16, NGH_MAX_TENSORS,
                                        NGH_MAX_OPS, NGH_MAX_CONSTS, NGH_MAX_REGS,
-                                       NGH_MAX_REDUCTIONS)
+                                       NGH_MAX_REDUCTIONS, NGH_CACHE_STREAM_LOAD,
+                                       NGH_CACHE_STREAM_STORE)
 from ngraph_hip.transformers.base import (ComputationGraphTransformer, DeviceBufferStorage,
                                           DeviceTensor, UnsupportedTransformerException)
 from ngraph_hip.transformers.passes.passes import (SimplePrune, TensorSizeFold, PeepholeGraphPass,
@@ -255,6 +256,18 @@ class HipKernel(object):
         pass
 
 
+def _no_uses(self):
+    return []
+
+
+def _ignore_hints(self, hint_of):
+    pass
+
+
+HipKernel.buffer_uses = _no_uses
+HipKernel.set_cache_hints = _ignore_hints
+
+
 class _Dim(object):
     __slots__ = ("length", "strides", "tag")
 
@@ -276,6 +289,7 @@ class FusedKernel(HipKernel):
         self.name = name
         self.specs = []
         self.flex_bindings = []     # (spec index, tensor slot, flex entry, is_output)
+        self.spec_uses = []         # per spec: [(base tensor description, is read, is written)] per slot
         self.described = None
 
     def _constant_value(self, value):
@@ -485,13 +499,14 @@ class FusedKernel(HipKernel):
                 reg_map[sym] = sb.reg()
             return reg_map[sym]
 
-        written = set()
+        written, read = set(), set()
         for ins in program:
             kind = ins[0]
             if kind == "const":
                 sb.constant(ins[2], reg(ins[1]))
             elif kind == "load":
                 sb.load(ins[2], reg(ins[1]))
+                read.add(ins[2])
             elif kind == "store":
                 sb.store(ins[1], reg(ins[2]))
                 written.add(ins[1])
@@ -513,8 +528,18 @@ class FusedKernel(HipKernel):
             entry = t.flex_entry_of(td)
             if entry is not None:
                 self.flex_bindings.append((index, s, entry, s in written))
+        self.spec_uses.append([(td.base, s in read, s in written) for s, td in enumerate(operands)])
         t.runtime.validate_fused(spec)
         return spec
+
+    def buffer_uses(self):
+        """(base tensor description, is read, is written) of every operand."""
+        return [u for uses in self.spec_uses for u in uses]
+
+    def set_cache_hints(self, hint_of):
+        for spec, uses in zip(self.specs, self.spec_uses):
+            for s, (base, is_read, is_written) in enumerate(uses):
+                spec.tensors[s].cache_hint = hint_of(base, is_read, is_written)
 
     def execute(self):
         rt = self.transformer.runtime
@@ -551,6 +576,10 @@ class CopyKernel(HipKernel):
         self.src_strides = [src_td.full_strides[i] for i in order]
         self.dst_strides = list(dst_td.full_strides)
         super(CopyKernel, self).bind_buffers()
+
+    def buffer_uses(self):
+        return [(self.op.args[0].forwarded.tensor_description().base, True, False),
+                (self.op.tensor_description().base, False, True)]
 
     def execute(self):
         self.transformer.runtime.copy_strided(self.dst.ptr, self.src.ptr, self.shape,
@@ -671,6 +700,7 @@ class MomentsKernel(HipKernel):
     def __init__(self, transformer, op):
         super(MomentsKernel, self).__init__(transformer)
         self.op = op
+        self.x_cache_hint = 0
 
     def bind_buffers(self):
         t = self.transformer
@@ -683,10 +713,17 @@ class MomentsKernel(HipKernel):
         self.out = t.get_tensor_description_tensor_view(self.op.tensor_description())
         super(MomentsKernel, self).bind_buffers()
 
+    def buffer_uses(self):
+        return [(self.op.args[0].forwarded.tensor_description().base, True, False),
+                (self.op.tensor_description().base, False, True)]
+
+    def set_cache_hints(self, hint_of):
+        self.x_cache_hint = hint_of(self.op.args[0].forwarded.tensor_description().base, True, False)
+
     def execute(self):
         out = self.out.ptr
         self.transformer.runtime.moments_f32(self.x.ptr, self.rows, self.R, self.row_stride,
-                                             out, out + self.rows * 4)
+                                             out, out + self.rows * 4, self.x_cache_hint)
 
     def describe(self):
         return [["moments_f32"]]
@@ -699,6 +736,37 @@ class HipKernelGroup(object):
         self.transformer = transformer
         self.name = name
         self.kernels = []
+        self._bound = False
+
+    def bind(self):
+        """Lower every kernel, then tell each operand what the rest of the computation does
+        with its buffer (the cache hints of the C ABI)."""
+        for k in self.kernels:
+            if not k.buffers_bound:
+                k.bind_buffers()
+        self.assign_cache_hints()
+        self._bound = True
+
+    def assign_cache_hints(self):
+        uses = [k.buffer_uses() for k in self.kernels]
+        readers = {}
+        for i, ku in enumerate(uses):
+            for base, is_read, _ in ku:
+                if is_read:
+                    readers.setdefault(base, set()).add(i)
+        for i, k in enumerate(self.kernels):
+            def hint_of(base, is_read, is_written, i=i):
+                hint = 0
+                r = readers.get(base, set())
+                if is_read and r == {i}:
+                    hint |= NGH_CACHE_STREAM_LOAD
+                # a result that nothing here reads again; state updated in place is read by
+                # the next execution and stays cacheable
+                if is_written and not is_read and not any(j > i for j in r) \
+                        and not getattr(base, "is_persistent", False):
+                    hint |= NGH_CACHE_STREAM_STORE
+                return hint
+            k.set_cache_hints(hint_of)
 
     def setup_kernel_execute(self, kernel):
         pass
@@ -707,9 +775,8 @@ class HipKernelGroup(object):
         pass
 
     def __call__(self):
-        for k in self.kernels:
-            if not k.buffers_bound:
-                k.bind_buffers()
+        if not self._bound:
+            self.bind()
         for k in self.kernels:
             self.setup_kernel_execute(k)
             k.execute()
@@ -724,9 +791,8 @@ class HipKernelGroup(object):
         times.  Returns [(kernel, [ms per launch])].  Kernels run out of their normal
         interleaving, so use it for per-kernel time, not for end-to-end time."""
         rt = self.transformer.runtime
-        for k in self.kernels:
-            if not k.buffers_bound:
-                k.bind_buffers()
+        if not self._bound:
+            self.bind()
         times = [[] for _ in self.kernels]
         for _ in range(repeats):
             for i, k in enumerate(self.kernels):

@@ -152,3 +152,46 @@ def test_c4_graph(transformer, Hn, Nn):
     np.testing.assert_allclose(c_g, c_w, rtol=RTOL, atol=ATOL)
     np.testing.assert_allclose(h_g, h_w, rtol=RTOL, atol=ATOL)
     np.testing.assert_allclose(db_g, db_w, rtol=RTOL, atol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("policy", [0, 1, 2, 3])
+def test_cache_policy_does_not_change_results(policy, monkeypatch):
+    """Non-temporal loads / stores are a cache hint only: forcing each of the four variants
+    of the pre-built Adam and batch-norm kernels gives bit-identical results."""
+    def adam_and_bn():
+        out = []
+        t = ngt.make_transformer_factory("hipgpu")()
+        n = 100000
+        p_np, g_np, _, _ = configs.c3_inputs(n)
+        P = ng.make_axis(n, name="P")
+        p, grad = ng.variable([P], initial_value=p_np), ng.placeholder([P])
+        opt = neon.Adam()
+        opt()
+        updates, m, v = opt.variable_update(p, grad)
+        f = t.computation(updates, grad)
+        read = t.computation([p * 1.0, m * 1.0, v * 1.0])
+        f(g_np)
+        f(g_np)
+        out.extend(np.array(a) for a in read())
+        assert any("special:adam" in d for k in t.kernel_groups[f].kernels for ds in k.describe() for d in ds)
+        t.close()
+        t = ngt.make_transformer_factory("hipgpu")()
+        dims = (64, 16, 16, 16)
+        x_np, gamma_np, beta_np = configs.c2_inputs(dims[0], dims[1] * dims[2] * dims[3])
+        C, H, W, N = (ng.make_axis(k, name=s) for s, k in zip("CHWN", dims))
+        x = ng.placeholder([C, H, W, N])
+        gamma, beta = ng.variable([C], initial_value=gamma_np), ng.variable([C], initial_value=beta_np)
+        y, xmean, xvar = neon.batch_norm_train(x, gamma, beta, out_axes=[C])
+        f = t.computation([y, xmean, xvar], x)
+        out.extend(np.array(a) for a in f(x_np.reshape(dims)))
+        assert any("special:batchnorm" in d for k in t.kernel_groups[f].kernels for ds in k.describe() for d in ds)
+        t.close()
+        return out
+
+    monkeypatch.setenv("NGH_CACHE_POLICY", "0")
+    want = adam_and_bn()
+    monkeypatch.setenv("NGH_CACHE_POLICY", str(policy))
+    got = adam_and_bn()
+    for a, b in zip(got, want):
+        np.testing.assert_array_equal(a, b)

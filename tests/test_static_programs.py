@@ -94,3 +94,53 @@ def test_spec_validation_rejects_malformed_programs():
     t0, t1 = sb.tensor(4096, [4, 1]), sb.tensor(8192, [1, 0])
     sb.store(t1, sb.load(t0))                    # store through a broadcast view
     assert lib.ngh_validate_fused(ctypes.byref(sb.build())) != 0
+
+
+def _hints(group):
+    """{operand role string: cache hint} over the large specs of a bound kernel group."""
+    out = []
+    for k in group.kernels:
+        for spec, uses in zip(getattr(k, "specs", []), getattr(k, "spec_uses", [])):
+            for s, (base, is_read, is_written) in enumerate(uses):
+                if int(np.prod(base.shape or (1,))) > 65536:
+                    out.append((is_read, is_written, spec.tensors[s].cache_hint))
+    return out
+
+
+def test_cache_hints_adam_streams_loads_and_keeps_state_stores_cacheable():
+    t = ngt.make_transformer_factory("hipgpu", dry_run=True)()
+    P = ng.make_axis(1 << 20, name="P")
+    p, grad = ng.variable([P], initial_value=0.0), ng.placeholder([P])
+    opt = neon.Adam()
+    opt()
+    updates, _, _ = opt.variable_update(p, grad)
+    f = t.computation(updates, grad)
+    t.initialize()
+    group = t.kernel_groups[f]
+    group.bind()
+    hints = _hints(group)
+    assert len(hints) == 4                                        # p, g, m, v
+    for is_read, is_written, hint in hints:
+        assert is_read and hint & hiplib.NGH_CACHE_STREAM_LOAD    # each is read by this kernel only
+        assert not hint & hiplib.NGH_CACHE_STREAM_STORE           # in-place state is read next step
+    t.close()
+
+
+def test_cache_hints_batchnorm_keeps_x_cacheable_and_streams_y():
+    t = ngt.make_transformer_factory("hipgpu", dry_run=True)()
+    C, H, W, N = (ng.make_axis(n, name=k) for k, n in zip("CHWN", (64, 16, 16, 16)))
+    x = ng.placeholder([C, H, W, N])
+    gamma, beta = ng.variable([C], initial_value=1.0), ng.variable([C], initial_value=0.0)
+    y, xmean, xvar = neon.batch_norm_train(x, gamma, beta, out_axes=[C])
+    f = t.computation([y, xmean, xvar], x)
+    t.initialize()
+    group = t.kernel_groups[f]
+    group.bind()
+    moments = [k for k in group.kernels if type(k).__name__ == "MomentsKernel"]
+    assert len(moments) == 1 and moments[0].x_cache_hint == 0     # x is read again by normalise
+    hints = _hints(group)
+    reads = [h for r, w, h in hints if r and not w]
+    writes = [h for r, w, h in hints if w and not r]
+    assert reads == [0]                                           # x: two readers, stays cacheable
+    assert writes == [hiplib.NGH_CACHE_STREAM_STORE]              # y: a result nobody here reads
+    t.close()
