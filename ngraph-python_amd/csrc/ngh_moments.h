@@ -4,8 +4,11 @@
 // The graph computes mean = sum(x)/R and variance = mean((x - mean)^2)
 // (ngraph/op_graph/op_graph.py:4007-4009, 4252-4266), which reads x twice.
 // Here each workgroup accumulates sum(x - p) and sum((x - p)^2) around a pivot p
-// (the row's first element) over one segment of a row, and a second tiny kernel
-// merges the segments in a fixed order:  mean = p + S1/R,  var = S2/R - (S1/R)^2.
+// (the row's first element) over one segment of a row, and the last workgroup of the
+// row to finish merges the segments in a fixed order:  mean = p + S1/R,
+// var = S2/R - (S1/R)^2.  Optionally it also writes 1/sqrt(var + eps), the factor the
+// normalisation multiplies by (frontends/neon/layer.py:1255), which saves the graph a
+// kernel launch for a few hundred elements.
 // Shifting by p keeps the subtraction in `var` from cancelling when |mean| is
 // large against the spread.  Segments make rows x segments >> 256 workgroups
 // even for a few hundred rows; the fixed merge order keeps results reproducible.
@@ -29,10 +32,14 @@ __device__ __forceinline__ float4 mom_load(const float4* p) {
     }
 }
 
+// The workgroups of one row take a ticket when their partial sums are written; the one that
+// draws the last ticket merges the row (in segment order, so the result does not depend on
+// which workgroup that was) and resets the row's counter for the next launch.
 template <bool NT>
-__global__ __launch_bounds__(kMomBlock) void moments_partial_kernel(
-    const float* __restrict__ x, long long row_stride, unsigned R4, unsigned n_seg, unsigned seg_chunks,
-    float2* __restrict__ partial) {
+__global__ __launch_bounds__(kMomBlock) void moments_kernel(
+    const float* __restrict__ x, long long row_stride, unsigned R, unsigned R4, unsigned n_seg,
+    unsigned seg_chunks, float2* __restrict__ partial, unsigned* __restrict__ row_tickets,
+    float* __restrict__ mean, float* __restrict__ var, float* __restrict__ rstd, float eps) {
     const unsigned row = blockIdx.x / n_seg;
     const unsigned seg = blockIdx.x - row * n_seg;
     const float* xr = x + (long long)row * row_stride;
@@ -69,30 +76,39 @@ __global__ __launch_bounds__(kMomBlock) void moments_partial_kernel(
         t2 += __shfl_xor(t2, m, 64);
     }
     __shared__ float2 sh[kMomBlock / 64];
+    __shared__ unsigned ticket;
     if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = make_float2(t1, t2);
     __syncthreads();
     if (threadIdx.x == 0) {
         float2 a = sh[0];
         for (int w = 1; w < kMomBlock / 64; ++w) { a.x += sh[w].x; a.y += sh[w].y; }
-        partial[blockIdx.x] = a;
+        // Publish the partial and take a ticket with device-scope read-modify-write atomics
+        // only: they are performed at the device's point of coherence, and the ticket is
+        // issued after the exchange has returned (its increment depends on the returned
+        // value), so whoever draws the last ticket can read every partial of the row there.
+        // A release fence instead would write back the whole L2 once per workgroup.
+        const unsigned long long bits =
+            (unsigned long long)__float_as_uint(a.x) | ((unsigned long long)__float_as_uint(a.y) << 32);
+        const unsigned long long old = __hip_atomic_exchange(
+            reinterpret_cast<unsigned long long*>(partial) + blockIdx.x, bits, __ATOMIC_RELAXED,
+            __HIP_MEMORY_SCOPE_AGENT);
+        unsigned one = 1u;
+        asm volatile("" : "+v"(one) : "v"((unsigned)old));   // orders the ticket after the exchange
+        ticket = __hip_atomic_fetch_add(row_tickets + row, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-}
-
-// One wavefront per row: lanes take segments, butterfly, lane 0 writes.
-__global__ __launch_bounds__(64) void moments_finish_kernel(
-    const float* __restrict__ x, long long row_stride, unsigned R, unsigned tail_begin, unsigned n_seg,
-    const float2* __restrict__ partial, float* __restrict__ mean, float* __restrict__ var) {
-    const unsigned row = blockIdx.x;
-    const float* xr = x + (long long)row * row_stride;
-    const float pivot = xr[0];
-    float t1 = 0.0f, t2 = 0.0f;
+    __syncthreads();
+    if (ticket != n_seg - 1 || threadIdx.x >= 64) return;
+    // last workgroup of the row, first wavefront
+    t1 = t2 = 0.0f;
     for (unsigned g = threadIdx.x; g < n_seg; g += 64) {
-        const float2 p = partial[row * n_seg + g];
-        t1 += p.x;
-        t2 += p.y;
+        const unsigned long long p = __hip_atomic_load(
+            reinterpret_cast<unsigned long long*>(partial) + row * n_seg + g, __ATOMIC_RELAXED,
+            __HIP_MEMORY_SCOPE_AGENT);
+        t1 += __uint_as_float((unsigned)p);
+        t2 += __uint_as_float((unsigned)(p >> 32));
     }
     // elements past the last whole float4 (R % 4) are added here
-    for (unsigned i = tail_begin + threadIdx.x; i < R; i += 64) {
+    for (unsigned i = R4 * 4 + threadIdx.x; i < R; i += 64) {
         const float a = xr[i] - pivot;
         t1 += a;
         t2 += a * a;
@@ -105,8 +121,11 @@ __global__ __launch_bounds__(64) void moments_finish_kernel(
     if (threadIdx.x == 0) {
         const float inv = 1.0f / (float)R;
         const float d = t1 * inv;
+        const float v = fmaxf(t2 * inv - d * d, 0.0f);
         mean[row] = pivot + d;
-        var[row] = fmaxf(t2 * inv - d * d, 0.0f);
+        var[row] = v;
+        if (rstd) rstd[row] = 1.0f / sqrtf(v + eps);
+        __hip_atomic_store(row_tickets + row, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 

@@ -72,6 +72,8 @@ struct ngh_context {
     hipEvent_t  ev0 = nullptr, ev1 = nullptr;
     void*       ws = nullptr;        // partial results of split reductions
     size_t      ws_bytes = 0;
+    unsigned*   tickets = nullptr;   // zero between launches: per-row / per-launch arrival counters
+    size_t      n_tickets = 0;
     int*        stat_ws = nullptr;   // per-workgroup max|mantissa| of streaming kernels
     unsigned    stat_ws_blocks = 0;  // capacity per statistics slot
     int         ew_blocks_per_cu = 64;
@@ -396,6 +398,23 @@ int ensure_ws(ngh_context* ctx, size_t bytes) {
     return NGH_OK;
 }
 
+// Arrival counters for kernels whose last workgroup finishes the job.  They are zero whenever
+// no such kernel is running: allocated zeroed, and each kernel resets what it used.
+int ensure_tickets(ngh_context* ctx, size_t n) {
+    if (n <= ctx->n_tickets) return NGH_OK;
+    if (ctx->tickets) {
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+        HIP_TRY(hipFree(ctx->tickets));
+        ctx->tickets = nullptr;
+        ctx->n_tickets = 0;
+    }
+    const size_t want = std::max(n, (size_t)4096);
+    HIP_TRY(hipMalloc((void**)&ctx->tickets, want * sizeof(unsigned)));
+    HIP_TRY(hipMemsetAsync(ctx->tickets, 0, want * sizeof(unsigned), ctx->stream));
+    ctx->n_tickets = want;
+    return NGH_OK;
+}
+
 // The last (length % 4) elements of a contiguous 1-D stage, one element per lane.
 // Point the stage's statistics slots at per-workgroup scratch for a launch of `blocks`
 // workgroups, and, after the launch, fold the scratch into each tensor's statistics word.
@@ -593,6 +612,7 @@ int ngh_shutdown(ngh_context* ctx) {
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->ws) (void)hipFree(ctx->ws);
     if (ctx->stat_ws) (void)hipFree(ctx->stat_ws);
+    if (ctx->tickets) (void)hipFree(ctx->tickets);
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
     if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -783,7 +803,7 @@ int ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec, int32_t sta
 }
 
 int ngh_moments_f32(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t R, int64_t row_stride,
-                    float* dev_mean, float* dev_var, uint32_t x_cache_hint) {
+                    float* dev_mean, float* dev_var, float* dev_rstd, float eps, uint32_t x_cache_hint) {
     if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
     if (rows < 0 || R <= 0) return fail(NGH_E_INVALID, "rows %lld, R %lld", (long long)rows, (long long)R);
     if (rows == 0) return NGH_OK;
@@ -796,23 +816,21 @@ int ngh_moments_f32(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t 
     long long seg = std::max<long long>(1, (long long)ctx->cus * ctx->moments_wgs_per_cu / rows);
     seg = std::min<long long>(seg, std::max<long long>(1, R4 / (kMomBlock * kMomUnroll * 2)));
     seg = std::min<long long>(seg, 4096);
-    const unsigned seg_chunks = (unsigned)((R4 + seg - 1) / seg);
-    const unsigned n_seg = seg_chunks ? (unsigned)((R4 + seg_chunks - 1) / seg_chunks) : 1;
-    const unsigned n_seg_eff = std::max(1u, n_seg);
-    NGH_TRY(ensure_ws(ctx, (size_t)rows * n_seg_eff * sizeof(float2)));
+    const unsigned seg_chunks = std::max(1u, (unsigned)((R4 + seg - 1) / seg));
+    const unsigned n_seg = std::max(1u, (unsigned)((R4 + seg_chunks - 1) / seg_chunks));
+    NGH_TRY(ensure_ws(ctx, (size_t)rows * n_seg * sizeof(float2)));
+    NGH_TRY(ensure_tickets(ctx, (size_t)rows));
     float2* partial = (float2*)ctx->ws;
     const bool stream_x = ctx->cache_policy >= 0
                               ? (ctx->cache_policy & 1)
                               : ((x_cache_hint & NGH_CACHE_STREAM_LOAD) && rows * R * 4 >= ctx->stream_bytes);
+    const dim3 grid((unsigned)(rows * n_seg));
     if (stream_x)
-        hipLaunchKernelGGL(moments_partial_kernel<true>, dim3((unsigned)(rows * n_seg_eff)), dim3(kMomBlock), 0,
-                           ctx->stream, dev_x, (long long)row_stride, R4, n_seg_eff, seg_chunks, partial);
+        hipLaunchKernelGGL(moments_kernel<true>, grid, dim3(kMomBlock), 0, ctx->stream, dev_x, (long long)row_stride,
+                           (unsigned)R, R4, n_seg, seg_chunks, partial, ctx->tickets, dev_mean, dev_var, dev_rstd, eps);
     else
-        hipLaunchKernelGGL(moments_partial_kernel<false>, dim3((unsigned)(rows * n_seg_eff)), dim3(kMomBlock), 0,
-                           ctx->stream, dev_x, (long long)row_stride, R4, n_seg_eff, seg_chunks, partial);
-    HIP_TRY(hipGetLastError());
-    hipLaunchKernelGGL(moments_finish_kernel, dim3((unsigned)rows), dim3(64), 0, ctx->stream, dev_x,
-                       (long long)row_stride, (unsigned)R, R4 * 4, n_seg_eff, partial, dev_mean, dev_var);
+        hipLaunchKernelGGL(moments_kernel<false>, grid, dim3(kMomBlock), 0, ctx->stream, dev_x, (long long)row_stride,
+                           (unsigned)R, R4, n_seg, seg_chunks, partial, ctx->tickets, dev_mean, dev_var, dev_rstd, eps);
     HIP_TRY(hipGetLastError());
     return NGH_OK;
 }

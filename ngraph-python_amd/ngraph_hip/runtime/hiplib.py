@@ -105,7 +105,8 @@ _SYMBOLS = {
     "ngh_validate_fused": [ctypes.POINTER(ngh_fused_spec)],
     "ngh_launch_fused": [_vp, ctypes.POINTER(ngh_fused_spec)],
     "ngh_describe_fused": [_vp, ctypes.POINTER(ngh_fused_spec), _i32, ctypes.c_char_p],
-    "ngh_moments_f32": [_vp, _vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, _vp, _vp, ctypes.c_uint32],
+    "ngh_moments_f32": [_vp, _vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, _vp, _vp, _vp, ctypes.c_float,
+                        ctypes.c_uint32],
     "ngh_plan_fused": [ctypes.POINTER(ngh_fused_spec), _i32, ctypes.POINTER(ctypes.c_int32)],
     "ngh_stats_alloc": [_vp, _i32, ctypes.POINTER(_vp)],
     "ngh_stats_reset": [_vp, _vp, _i32],
@@ -300,10 +301,11 @@ class HipRuntime(object):
         _check(self.lib, self.lib.ngh_describe_fused(self.ctx, ctypes.byref(spec), int(stage), name))
         return name.value.decode()
 
-    def moments_f32(self, x, rows, R, row_stride, mean, var, x_cache_hint=0):
+    def moments_f32(self, x, rows, R, row_stride, mean, var, rstd=None, eps=0.0, x_cache_hint=0):
         _check(self.lib, self.lib.ngh_moments_f32(self.ctx, ctypes.c_void_p(x), int(rows), int(R),
                                                   int(row_stride), ctypes.c_void_p(mean),
-                                                  ctypes.c_void_p(var), int(x_cache_hint)))
+                                                  ctypes.c_void_p(var), ctypes.c_void_p(rstd or None),
+                                                  float(eps), int(x_cache_hint)))
 
     # -- flex statistics ---------------------------------------------------
     def stats_alloc(self, n):

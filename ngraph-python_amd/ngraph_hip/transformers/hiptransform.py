@@ -589,16 +589,19 @@ class CopyKernel(HipKernel):
 class MomentsOp(og.TensorOp):
     """mean and variance of x over `reduction_axes` in one read of x.
 
-    Axes = (K,) + kept axes with K of length 2: row 0 holds the mean, row 1 the (biased)
-    variance.  Introduced by MomentsFusionPass in place of ng.mean + ng.variance
-    (op_graph.py:4007-4009, 4252-4266); consumers read the two rows as slices.
+    Axes = (K,) + kept axes with K of length 3: row 0 holds the mean, row 1 the (biased)
+    variance, row 2 -- once `epsilon` is set -- 1/sqrt(variance + epsilon).  Introduced by
+    MomentsFusionPass in place of ng.mean + ng.variance (op_graph.py:4007-4009, 4252-4266)
+    and of the reciprocal(sqrt(variance + eps)) that batch normalisation takes of it
+    (frontends/neon/layer.py:1255); consumers read the rows as slices.
     """
 
     def __init__(self, x, reduction_axes, **kwargs):
         x = og.as_op(x)
         self.reduction_axes = og.make_axes(reduction_axes)
         self.kept_axes = x.axes - self.reduction_axes
-        self.k_axis = og.make_axis(2, name="NGH_MOMENT")
+        self.k_axis = og.make_axis(3, name="NGH_MOMENT")
+        self.epsilon = None
         super(MomentsOp, self).__init__(args=(x,), axes=og.make_axes([self.k_axis]) + self.kept_axes,
                                         **kwargs)
 
@@ -660,9 +663,30 @@ class MomentsFusionPass(PeepholeGraphPass):
 
     def do_pass(self, ops, **kwargs):
         self.moments = []          # (x, reduction axes, mean view, var view)
+        self.var_views = {}        # var view -> MomentsOp
         super(MomentsFusionPass, self).do_pass(ops, **kwargs)
 
+    def _visit_rstd(self, op):
+        """reciprocal(sqrt(var + c)) of a fused variance becomes row 2 of its MomentsOp."""
+        root = self._strip(op.args[0])
+        if not isinstance(root, og.SqrtOp):
+            return
+        add = self._strip(root.args[0])
+        if not isinstance(add, og.Add):
+            return
+        a, b = self._strip(add.args[0]), self._strip(add.args[1])
+        for v, c in ((a, b), (b, a)):
+            eps = _scalar_constant_value(c)
+            mom = self.var_views.get(v)
+            if eps is None or mom is None or mom.epsilon not in (None, eps):
+                continue
+            mom.epsilon = eps
+            self.replace_op(op, og.slice_along_axis(mom, mom.k_axis, 2))
+            return
+
     def visit(self, op, *args):
+        if isinstance(op, og.ReciprocalOp):
+            return self._visit_rstd(op)
         if not isinstance(op, og.Divide):
             return
         outer = self._as_mean(op)
@@ -692,6 +716,7 @@ class MomentsFusionPass(PeepholeGraphPass):
         mean_view = og.slice_along_axis(mom, mom.k_axis, 0)
         var_view = og.slice_along_axis(mom, mom.k_axis, 1)
         self.moments.append((x, red_axes, mean_view, var_view))
+        self.var_views[var_view] = mom
         self.replace_op(op, var_view)
         self.replace_op(self._strip(m), mean_view)
 
@@ -721,9 +746,11 @@ class MomentsKernel(HipKernel):
         self.x_cache_hint = hint_of(self.op.args[0].forwarded.tensor_description().base, True, False)
 
     def execute(self):
-        out = self.out.ptr
+        out, eps = self.out.ptr, self.op.epsilon
         self.transformer.runtime.moments_f32(self.x.ptr, self.rows, self.R, self.row_stride,
-                                             out, out + self.rows * 4, self.x_cache_hint)
+                                             out, out + self.rows * 4,
+                                             out + self.rows * 8 if eps is not None else None,
+                                             eps or 0.0, self.x_cache_hint)
 
     def describe(self):
         return [["moments_f32"]]

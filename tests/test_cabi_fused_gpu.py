@@ -353,3 +353,35 @@ def test_signed_sum_against_float64(hip_runtime, shape, layout):
     assert np.all(np.abs(out_d.get().astype(np.float64) - truth) <= bound)
     x_d.free()
     out_d.free()
+
+
+# ------------------------------------------------------------------ one-pass moments
+@pytest.mark.parametrize("rows,R,pad", [(1, 1, 3), (3, 2, 2), (5, 7, 1), (4, 1024, 0), (256, 3136, 0),
+                                        (2, 1000003, 1), (700, 260, 0), (1, 4, 0)])
+def test_moments_rows(hip_runtime, rows, R, pad):
+    """ngh_moments_f32 against float64 row statistics; rows of every length class (shorter than
+    a vector, ragged tails, many segments), with a row stride wider than the row.  Launched
+    twice: the second launch checks that the arrival counters were left at zero."""
+    rt = hip_runtime
+    rs = np.random.RandomState(rows * 7 + R)
+    stride = ((R + 3) // 4) * 4 + 4 * pad
+    host = rs.normal(3.0, 2.0, (rows, stride)).astype(f32)
+    x_d = rt.array(host)
+    out_d = rt.empty((3, rows))
+    eps = 1e-5
+    x64 = host[:, :R].astype(np.float64)
+    for _ in range(2):
+        rt.memset32(out_d.ptr, 0, 3 * rows)
+        rt.moments_f32(x_d.ptr, rows, R, stride, out_d.ptr, out_d.ptr + 4 * rows, out_d.ptr + 8 * rows, eps)
+        mean, var, rstd = out_d.get()
+        np.testing.assert_allclose(mean, x64.mean(axis=1), rtol=RTOL, atol=ATOL)
+        np.testing.assert_allclose(var, x64.var(axis=1), rtol=1e-4, atol=1e-5)
+        # rstd is the fp32 statement sequence add, sqrt, reciprocal on the kernel's own variance
+        want = (f32(1) / np.sqrt(var + f32(eps))).astype(f32)
+        np.testing.assert_array_equal(rstd, want)
+    # without rstd the third row stays untouched
+    rt.memset32(out_d.ptr, 0, 3 * rows)
+    rt.moments_f32(x_d.ptr, rows, R, stride, out_d.ptr, out_d.ptr + 4 * rows)
+    assert not out_d.get()[2].any()
+    for d in (x_d, out_d):
+        d.free()
