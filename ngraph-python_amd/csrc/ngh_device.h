@@ -40,6 +40,12 @@ struct KArgs {
     int       probe;         // NGH_SPEC_PROBE: record max|value| bits instead of storing
     int*      stat_ptr[4];   // device word of each per-thread accumulator
     int*      stat_partial[4];  // per-workgroup scratch the streaming kernels write instead
+    // in-kernel exponent management (pre-built streaming kernels only); flex_state[0] == NULL = off
+    ngh_flex_state* flex_state[4];  // per statistics slot: the stored tensor's record
+    int       flex_in_place[4];     // the kernel also reads the tensor
+    int       flex_count;
+    unsigned* tickets;              // arrival counters, zero between launches
+    int*      group_max;            // per slot and group: merged max|mantissa|, zero between launches
     KTensor   t[NGH_MAX_TENSORS];
     float     consts[NGH_MAX_CONSTS];
     ngh_op    ops[NGH_MAX_OPS];

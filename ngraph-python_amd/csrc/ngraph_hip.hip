@@ -78,6 +78,7 @@ struct ngh_context {
     unsigned    stat_ws_blocks = 0;  // capacity per statistics slot
     int         ew_blocks_per_cu = 64;
     int         force_interp = 0;    // never pick a specialised kernel
+    int         flex_self_managed = 1;  // ngh_launch_fused_flex may fold the policy into the kernel
     int         cache_policy = -1;   // -1: from the operands' cache hints; 0..3 forces bit 0 = non-temporal
                                      // loads, bit 1 = non-temporal stores in pre-built kernels
     long long   stream_bytes = 128ll << 20;  // hints act on stages touching at least this much memory
@@ -580,6 +581,7 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     snprintf(ctx->name, sizeof(ctx->name), "%s (%s)", prop.name, prop.gcnArchName);
     ctx->ew_blocks_per_cu = std::max(1, env_int("NGH_EW_BLOCKS_PER_CU", 64));
     ctx->force_interp = env_int("NGH_FORCE_INTERP", 0);
+    ctx->flex_self_managed = env_int("NGH_FLEX_SELF_MANAGED", 1);
     ctx->cache_policy = env_int("NGH_CACHE_POLICY", -1);
     ctx->stream_bytes = (long long)env_int("NGH_STREAM_MIB", 128) << 20;
     ctx->moments_wgs_per_cu = std::max(1, env_int("NGH_MOMENTS_WGS_PER_CU", 16));
@@ -932,8 +934,52 @@ int ngh_flex_update(ngh_context* ctx, ngh_flex_state* dev, const int32_t* ids, i
     return NGH_OK;
 }
 
+// One launch instead of prepare + kernel + fold + update: possible when the spec is a single
+// stage that a pre-built streaming kernel covers whole (no scalar tail) and every
+// statistics slot belongs to one of the managed tensors.
+static int try_self_managed_launch(ngh_context* ctx, const ngh_fused_spec* spec, ngh_flex_state* dev,
+                                   const int32_t* ids, const int32_t* in_place, int32_t n_ids, int32_t count,
+                                   bool* done) {
+    *done = false;
+    if (ctx->force_interp || !ctx->flex_self_managed || spec->n_stages != 1 || (spec->flags & NGH_SPEC_PROBE))
+        return NGH_OK;
+    if (spec->stages[0].op_end == spec->stages[0].op_begin) return NGH_OK;
+    Plan P;
+    NGH_TRY(plan_stage(ctx, *spec, 0, P));
+    P.special = match_special(P.family, P.V, P.k, P.tail);
+    if (P.special < 0 || P.tail || P.n_chunks == 0 || P.k.n_stat_slots != n_ids || n_ids < 1) return NGH_OK;
+    for (int s = 0; s < P.k.n_stat_slots; ++s) {
+        const ptrdiff_t off = (const char*)P.k.stat_ptr[s] - (const char*)dev;
+        if (!P.k.stat_ptr[s] || off < 0 || off % (ptrdiff_t)sizeof(ngh_flex_state)) return NGH_OK;
+        const int32_t id = (int32_t)(off / (ptrdiff_t)sizeof(ngh_flex_state));
+        int j = 0;
+        while (j < n_ids && ids[j] != id) ++j;
+        if (j == n_ids) return NGH_OK;
+        for (int q = 0; q < s; ++q)
+            if (P.k.flex_state[q] == dev + id) return NGH_OK;      // two slots on one tensor
+        P.k.flex_state[s] = dev + id;
+        P.k.flex_in_place[s] = in_place ? in_place[j] : 0;
+    }
+    NGH_TRY(ensure_tickets(ctx, (size_t)kFlexTicketWords + kFlexGroupMaxWords));
+    P.k.flex_count = count;
+    P.k.tickets = ctx->tickets;
+    P.k.group_max = (int*)(ctx->tickets + kFlexTicketWords);
+    const unsigned blocks = streaming_blocks(ctx->cus, ctx->ew_blocks_per_cu, P.n_chunks);
+    hipError_t e = launch_special(P.special, ctx->stream, blocks, P.k, P.n_chunks, P.chunks_per_row,
+                                  stage_cache_policy(ctx, *spec, spec->stages[0]));
+    if (e != hipSuccess) return fail(NGH_E_RUNTIME, "special launch: %s", hipGetErrorString(e));
+    *done = true;
+    return NGH_OK;
+}
+
 int ngh_launch_fused_flex(ngh_context* ctx, const ngh_fused_spec* spec, ngh_flex_state* dev,
                           const int32_t* ids, const int32_t* in_place, int32_t n_ids, int32_t count) {
+    if (!ctx || !dev) return fail(NGH_E_INVALID, "ngh_launch_fused_flex: NULL argument");
+    NGH_TRY(validate(spec));
+    if (n_ids > 0 && !ids) return fail(NGH_E_INVALID, "ngh_launch_fused_flex: ids is NULL");
+    bool done = false;
+    NGH_TRY(try_self_managed_launch(ctx, spec, dev, ids, in_place, n_ids, count, &done));
+    if (done) return NGH_OK;
     NGH_TRY(ngh_flex_prepare(ctx, dev, ids, in_place, n_ids));
     NGH_TRY(ngh_launch_fused(ctx, spec));
     return ngh_flex_update(ctx, dev, ids, n_ids, count);
