@@ -91,7 +91,7 @@ def _model_c5(xs, w, b):
 
 
 @pytest.mark.parametrize("resident", [False, True], ids=["host-policy", "device-policy"])
-@pytest.mark.parametrize("n", [1 << 16, 100003])
+@pytest.mark.parametrize("n", [1 << 16, 100003, 1 << 21])
 def test_c5_fused_flex_bit_exact_over_8_iterations(n, resident):
     x0, w, b = configs.c5_inputs(n, seed=4)
     # activations that grow, then collapse: exercises overflow (dec -= 2), the headroom
