@@ -213,7 +213,7 @@ int  ngh_moments_f32(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t
 
 /* How stage `stage` would be launched, without a device (host-side tooling and
  * tests): out8 = {kernel family (0 streaming, 1 reduce along the contiguous axis,
- * 2 reduce across it), vector width, spec axis on kernel axes 0,1,2, tail length,
+ * 2 reduce across it, 3 streaming through LDS tiles for transposed operands), vector width, spec axis on kernel axes 0,1,2, tail length,
  * index of the matching pre-built specialisation or -1, reduction segments}.     */
 int  ngh_plan_fused(const ngh_fused_spec* spec, int32_t stage, int32_t* out8);
 

@@ -50,12 +50,12 @@ __global__ __launch_bounds__(kCopyBlock) void copy_nd_kernel(T* dst, const T* sr
 // contiguous along `rows` (ss[r-2] == 1) and the destination along `cols`
 // (ds[r-1] == 1).  A 64x64 tile goes through LDS (row padded to 65 words) so
 // both the global read and the global write are coalesced.
-constexpr int kTile = 64;
+constexpr int kCopyTile = 64;
 
 template <typename T>
 __global__ __launch_bounds__(kCopyBlock) void copy_tr_kernel(T* dst, const T* src, const CopyArgs a,
                                                              unsigned tiles_r, unsigned tiles_c) {
-    __shared__ T tile[kTile][kTile + 1];
+    __shared__ T tile[kCopyTile][kCopyTile + 1];
     const int r_ax = a.rank - 2, c_ax = a.rank - 1;
     const unsigned R = (unsigned)a.shape[r_ax], C = (unsigned)a.shape[c_ax];
     unsigned b = blockIdx.x;
@@ -71,14 +71,14 @@ __global__ __launch_bounds__(kCopyBlock) void copy_tr_kernel(T* dst, const T* sr
     }
     const unsigned tx = threadIdx.x & 63, ty = threadIdx.x >> 6;   // 64 x 4
     // read: lanes along rows (source-contiguous)
-    for (unsigned j = ty; j < kTile; j += 4) {
-        const unsigned r = tr * kTile + tx, c = tc * kTile + j;
+    for (unsigned j = ty; j < kCopyTile; j += 4) {
+        const unsigned r = tr * kCopyTile + tx, c = tc * kCopyTile + j;
         if (r < R && c < C) tile[j][tx] = src[so + (long long)r * a.ss[r_ax] + (long long)c * a.ss[c_ax]];
     }
     __syncthreads();
     // write: lanes along cols (destination-contiguous)
-    for (unsigned j = ty; j < kTile; j += 4) {
-        const unsigned r = tr * kTile + j, c = tc * kTile + tx;
+    for (unsigned j = ty; j < kCopyTile; j += 4) {
+        const unsigned r = tr * kCopyTile + j, c = tc * kCopyTile + tx;
         if (r < R && c < C) dst[dof + (long long)r * a.ds[r_ax] + (long long)c * a.ds[c_ax]] = tile[tx][j];
     }
 }
@@ -87,8 +87,8 @@ template <typename T>
 inline hipError_t launch_copy_t(hipStream_t stream, int cus, void* dst, const void* src, const CopyArgs& a) {
     if (a.rank >= 2 && a.ss[a.rank - 2] == 1 && a.ds[a.rank - 1] == 1 && a.ss[a.rank - 1] != 1 &&
         a.shape[a.rank - 2] >= 16 && a.shape[a.rank - 1] >= 16) {
-        const unsigned tiles_r = (unsigned)((a.shape[a.rank - 2] + kTile - 1) / kTile);
-        const unsigned tiles_c = (unsigned)((a.shape[a.rank - 1] + kTile - 1) / kTile);
+        const unsigned tiles_r = (unsigned)((a.shape[a.rank - 2] + kCopyTile - 1) / kCopyTile);
+        const unsigned tiles_c = (unsigned)((a.shape[a.rank - 1] + kCopyTile - 1) / kCopyTile);
         unsigned long long blocks = (unsigned long long)tiles_r * tiles_c;
         for (int ax = 0; ax < a.rank - 2; ++ax) blocks *= (unsigned long long)a.shape[ax];
         if (blocks < (1ULL << 31)) {

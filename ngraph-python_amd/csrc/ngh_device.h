@@ -26,7 +26,7 @@ struct KTensor {
     int*         stats;
     const float* dscale;
     int          stat_slot;  // which per-thread max|mantissa| accumulator, -1 = none
-    int          pad_;
+    int          stage_slot; // tiled skeleton: which LDS tile carries this operand, -1 = direct access
 };
 
 struct KArgs {
@@ -37,6 +37,7 @@ struct KArgs {
     int       red_axis;      // kernel axis the reductions run along (0 or 2), -1 = none
     int       iota_map[3];   // kernel axis holding spec axis k (for NGH_OP_IOTA)
     int       n_stat_slots;
+    int       n_staged;      // tiled skeleton: operands staged through LDS tiles
     int       probe;         // NGH_SPEC_PROBE: record max|value| bits instead of storing
     int*      stat_ptr[4];   // device word of each per-thread accumulator
     int*      stat_partial[4];  // per-workgroup scratch the streaming kernels write instead
@@ -242,69 +243,74 @@ __device__ __forceinline__ void store4(const KTensor& t, long long off, float sc
     }
 }
 
-// V consecutive elements (V = 4 or 8).  Eight 16-bit elements travel as one 16-byte
+// V consecutive elements (V = 4, 8 or 16).  16-bit elements travel eight to a 16-byte
 // access, which is what keeps enough bytes in flight per lane for 2-byte storage types.
 template <int V>
 __device__ __forceinline__ void loadv(const KTensor& t, long long off, float scale, float (&v)[V]) {
+    static_assert(V == 4 || V == 8 || V == 16, "vector width");
     if constexpr (V == 4) {
         load4(t, off, scale, v);
     } else {
-        static_assert(V == 8, "vector width");
-        if (t.dtype == NGH_FLEX16) {
-            const uint4 raw = *reinterpret_cast<const uint4*>(reinterpret_cast<const short*>(t.p) + off);
-            const unsigned w[4] = {raw.x, raw.y, raw.z, raw.w};
+        if (t.dtype == NGH_FLEX16 || t.dtype == NGH_F16) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                v[2 * j] = scale * (float)(short)(w[j] & 0xffffu);
-                v[2 * j + 1] = scale * (float)(short)(w[j] >> 16);
-            }
-        } else if (t.dtype == NGH_F16) {
-            const uint4 raw = *reinterpret_cast<const uint4*>(reinterpret_cast<const __half*>(t.p) + off);
-            const unsigned w[4] = {raw.x, raw.y, raw.z, raw.w};
+            for (int g = 0; g < V / 8; ++g) {
+                const uint4 raw = *reinterpret_cast<const uint4*>(t.p + (off + 8 * g) * 2);
+                const unsigned w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                unsigned u = w[j];
-                const float2 f = __half22float2(*reinterpret_cast<__half2*>(&u));
-                v[2 * j] = f.x;
-                v[2 * j + 1] = f.y;
+                for (int j = 0; j < 4; ++j) {
+                    if (t.dtype == NGH_FLEX16) {
+                        v[8 * g + 2 * j] = scale * (float)(short)(w[j] & 0xffffu);
+                        v[8 * g + 2 * j + 1] = scale * (float)(short)(w[j] >> 16);
+                    } else {
+                        unsigned u = w[j];
+                        const float2 f = __half22float2(*reinterpret_cast<__half2*>(&u));
+                        v[8 * g + 2 * j] = f.x;
+                        v[8 * g + 2 * j + 1] = f.y;
+                    }
+                }
             }
         } else {
-            float a[4], b[4];
-            load4(t, off, scale, a);
-            load4(t, off + 4, scale, b);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) { v[j] = a[j]; v[4 + j] = b[j]; }
+            for (int g = 0; g < V / 4; ++g) {
+                float a[4];
+                load4(t, off + 4 * g, scale, a);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[4 * g + j] = a[j];
+            }
         }
     }
 }
 
 template <int V>
 __device__ __forceinline__ void storev(const KTensor& t, long long off, float scale, const float (&v)[V], int& fmax) {
+    static_assert(V == 4 || V == 8 || V == 16, "vector width");
     if constexpr (V == 4) {
         store4(t, off, scale, v, fmax);
     } else {
-        static_assert(V == 8, "vector width");
-        if (t.dtype == NGH_FLEX16) {
-            unsigned w[4];
+        if (t.dtype == NGH_FLEX16 || t.dtype == NGH_F16) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int q0 = flex_quantize(scale * v[2 * j]), q1 = flex_quantize(scale * v[2 * j + 1]);
-                fmax = max(fmax, max(iabs(q0), iabs(q1)));
-                w[j] = ((unsigned)q0 & 0xffffu) | ((unsigned)q1 << 16);
-            }
-            *reinterpret_cast<uint4*>(reinterpret_cast<short*>(t.p) + off) = make_uint4(w[0], w[1], w[2], w[3]);
-        } else if (t.dtype == NGH_F16) {
-            unsigned w[4];
+            for (int g = 0; g < V / 8; ++g) {
+                unsigned w[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                __half2 h = __floats2half2_rn(v[2 * j], v[2 * j + 1]);
-                w[j] = *reinterpret_cast<unsigned*>(&h);
+                for (int j = 0; j < 4; ++j) {
+                    if (t.dtype == NGH_FLEX16) {
+                        const int q0 = flex_quantize(scale * v[8 * g + 2 * j]);
+                        const int q1 = flex_quantize(scale * v[8 * g + 2 * j + 1]);
+                        fmax = max(fmax, max(iabs(q0), iabs(q1)));
+                        w[j] = ((unsigned)q0 & 0xffffu) | ((unsigned)q1 << 16);
+                    } else {
+                        __half2 h = __floats2half2_rn(v[8 * g + 2 * j], v[8 * g + 2 * j + 1]);
+                        w[j] = *reinterpret_cast<unsigned*>(&h);
+                    }
+                }
+                *reinterpret_cast<uint4*>(t.p + (off + 8 * g) * 2) = make_uint4(w[0], w[1], w[2], w[3]);
             }
-            *reinterpret_cast<uint4*>(reinterpret_cast<__half*>(t.p) + off) = make_uint4(w[0], w[1], w[2], w[3]);
         } else {
-            const float a[4] = {v[0], v[1], v[2], v[3]}, b[4] = {v[4], v[5], v[6], v[7]};
-            store4(t, off, scale, a, fmax);
-            store4(t, off + 4, scale, b, fmax);
+#pragma unroll
+            for (int g = 0; g < V / 4; ++g) {
+                const float a[4] = {v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3]};
+                store4(t, off + 4 * g, scale, a, fmax);
+            }
         }
     }
 }

@@ -31,49 +31,129 @@ struct Extra {
     __device__ __forceinline__ void  setf(int j, float x) { base[j * nthr] = x; }
 };
 
+// LDS tiles of the tiled skeleton: operand `stage_slot` owns tile number stage_slot; `at` is
+// this thread's element inside every tile.
+constexpr int kTile = 32;                       // 16 for problems too small to fill the chip
+__host__ __device__ constexpr int tile_words(int tile) { return tile * (tile + 1); }
+struct Tiles {
+    float* base;
+    int    at;      // this lane's element 0 inside every tile
+    int    vstep;   // distance of the lane's next element
+    int    words;   // floats per tile
+};
+
+// ---------------------------------------------------------------------------
+// Where the V elements a lane works on live.  The interpreter pays a fixed price
+// per op (decode, LDS register traffic) whatever V is, so every skeleton gives
+// a lane several elements per op: consecutive ones where operands allow vector
+// access (VecAt), otherwise V elements a fixed number of lanes apart (GatherAt),
+// which keeps each wavefront access coalesced.
+// ---------------------------------------------------------------------------
+template <int V>
+struct VecAt {   // (i0, i1, i2 .. i2 + V - 1)
+    long long i0, i1, i2;
+    __device__ __forceinline__ bool valid(int) const { return true; }
+    __device__ __forceinline__ float iota(int ka, int v) const {
+        return (float)(ka == 2 ? i2 + v : (ka == 1 ? i1 : i0));
+    }
+    __device__ __forceinline__ int red_index(int rmode, int v) const { return (int)(rmode == 1 ? i2 + v : i0); }
+    __device__ __forceinline__ void load(const KTensor& t, float (&x)[V]) const {
+        const long long off = i0 * t.s[0] + i1 * t.s[1] + i2 * t.s[2];
+        const float sc = (t.dtype == NGH_FLEX16) ? tensor_scale(t) : 1.0f;
+        if (t.s[2] == 0) {
+            const float b = load1(t, off, sc);
+#pragma unroll
+            for (int v = 0; v < V; ++v) x[v] = b;
+        } else if (V >= 4 && t.s[2] == 1) {
+            if constexpr (V >= 4) loadv<V>(t, off, sc, x);
+        } else {
+#pragma unroll
+            for (int v = 0; v < V; ++v) x[v] = load1(t, off + v * t.s[2], sc);
+        }
+    }
+    __device__ __forceinline__ void store(const KTensor& t, const float (&x)[V], int& fmax) const {
+        const long long off = i0 * t.s[0] + i1 * t.s[1] + i2 * t.s[2];
+        const float sc = (t.dtype == NGH_FLEX16) ? 1.0f / tensor_scale(t) : 1.0f;
+        if (V >= 4 && t.s[2] == 1) {
+            if constexpr (V >= 4) storev<V>(t, off, sc, x, fmax);
+        } else {
+#pragma unroll
+            for (int v = 0; v < V; ++v) store1(t, off + v * t.s[2], x[v], sc, fmax);
+        }
+    }
+};
+
+template <int V>
+struct GatherAt {   // element v at (i0[v], i1[v], i2[v]); only the first nv count -- the others must
+                    // still name an element inside the view, because loads are not predicated
+                    // (a branch per element would serialise the memory round trips)
+    unsigned i0[V], i1[V], i2[V];
+    int nv;
+    __device__ __forceinline__ bool valid(int v) const { return v < nv; }
+    __device__ __forceinline__ float iota(int ka, int v) const {
+        return (float)(ka == 2 ? i2[v] : (ka == 1 ? i1[v] : i0[v]));
+    }
+    __device__ __forceinline__ int red_index(int, int) const { return 0; }   // not used with reductions
+    __device__ __forceinline__ void load(const KTensor& t, float (&x)[V]) const {
+        const float sc = (t.dtype == NGH_FLEX16) ? tensor_scale(t) : 1.0f;
+#pragma unroll
+        for (int v = 0; v < V; ++v)
+            x[v] = load1(t, (long long)i0[v] * t.s[0] + (long long)i1[v] * t.s[1] + (long long)i2[v] * t.s[2], sc);
+    }
+    __device__ __forceinline__ void store(const KTensor& t, const float (&x)[V], int& fmax) const {
+        const float sc = (t.dtype == NGH_FLEX16) ? 1.0f / tensor_scale(t) : 1.0f;
+#pragma unroll
+        for (int v = 0; v < V; ++v)
+            if (v < nv)
+                store1(t, (long long)i0[v] * t.s[0] + (long long)i1[v] * t.s[1] + (long long)i2[v] * t.s[2], x[v], sc, fmax);
+    }
+};
+
 // RMODE: 0 = no reductions, 1 = reduction runs along kernel axis 2 (the vector
-// axis), 2 = reduction runs along kernel axis 0.
-template <int V, int RMODE>
-__device__ __forceinline__ void run_ops(const KArgs& k, LdsRegs<V>& rf, Extra& ex,
-                                        long long i0, long long i1, long long i2) {
+// axis), 2 = reduction runs along kernel axis 0.  TILED: operands with a stage slot are
+// read from / written to their LDS tile instead of memory (element v at tiles.at + v * tiles.vstep).
+template <int V, int RMODE, bool TILED = false, class At>
+__device__ __forceinline__ void run_ops(const KArgs& k, LdsRegs<V>& rf, Extra& ex, const At& at,
+                                        Tiles tiles = Tiles{nullptr, 0, 0, 0}) {
     for (int pc = k.op_begin; pc < k.op_end; ++pc) {
         const ngh_op o = k.ops[pc];
         const int opc = o.opcode;
         switch (opc) {
             case NGH_OP_LOAD: {
                 const KTensor& t = k.t[o.a];
-                const long long off = i0 * t.s[0] + i1 * t.s[1] + i2 * t.s[2];
-                const float sc = (t.dtype == NGH_FLEX16) ? tensor_scale(t) : 1.0f;
-                if (t.s[2] == 0) {
-                    const float x = load1(t, off, sc);
+                if constexpr (TILED) {
+                    if (t.stage_slot >= 0) {
+                        const float* tl = tiles.base + t.stage_slot * tiles.words + tiles.at;
 #pragma unroll
-                    for (int v = 0; v < V; ++v) rf.set(o.dst, v, x);
-                } else if (V >= 4 && t.s[2] == 1) {
-                    float x[V >= 4 ? V : 4];
-                    if constexpr (V >= 4) loadv<V>(t, off, sc, x);
-#pragma unroll
-                    for (int v = 0; v < V; ++v) rf.set(o.dst, v, x[v]);
-                } else {
-#pragma unroll
-                    for (int v = 0; v < V; ++v) rf.set(o.dst, v, load1(t, off + v * t.s[2], sc));
+                        for (int v = 0; v < V; ++v) rf.set(o.dst, v, tl[v * tiles.vstep]);
+                        break;
+                    }
                 }
+                float x[V];
+                at.load(t, x);
+#pragma unroll
+                for (int v = 0; v < V; ++v) rf.set(o.dst, v, x[v]);
             } break;
             case NGH_OP_STORE: {
                 const KTensor& t = k.t[o.dst];
-                const long long off = i0 * t.s[0] + i1 * t.s[1] + i2 * t.s[2];
-                const float sc = (t.dtype == NGH_FLEX16) ? 1.0f / tensor_scale(t) : 1.0f;
+                if constexpr (TILED) {
+                    if (t.stage_slot >= 0 && !k.probe) {
+                        float* tl = tiles.base + t.stage_slot * tiles.words + tiles.at;
+#pragma unroll
+                        for (int v = 0; v < V; ++v) tl[v * tiles.vstep] = rf.get(o.a, v);
+                        break;
+                    }
+                }
                 int fmax = 0;
+                float x[V];
+#pragma unroll
+                for (int v = 0; v < V; ++v) x[v] = rf.get(o.a, v);
                 if (k.probe) {
 #pragma unroll
-                    for (int v = 0; v < V; ++v) fmax = max(fmax, probe_bits(rf.get(o.a, v)));
-                } else if (V >= 4 && t.s[2] == 1) {
-                    float x[V >= 4 ? V : 4];
-#pragma unroll
-                    for (int v = 0; v < V; ++v) x[v] = rf.get(o.a, v);
-                    if constexpr (V >= 4) storev<V>(t, off, sc, x, fmax);
+                    for (int v = 0; v < V; ++v)
+                        if (at.valid(v)) fmax = max(fmax, probe_bits(x[v]));
                 } else {
-#pragma unroll
-                    for (int v = 0; v < V; ++v) store1(t, off + v * t.s[2], rf.get(o.a, v), sc, fmax);
+                    at.store(t, x, fmax);
                 }
                 if (t.stat_slot >= 0) ex.seti(ex_stat(t.stat_slot), max(ex.geti(ex_stat(t.stat_slot)), fmax));
             } break;
@@ -85,8 +165,7 @@ __device__ __forceinline__ void run_ops(const KArgs& k, LdsRegs<V>& rf, Extra& e
             case NGH_OP_IOTA: {
                 const int ka = k.iota_map[o.a];
 #pragma unroll
-                for (int v = 0; v < V; ++v)
-                    rf.set(o.dst, v, (float)(ka == 2 ? i2 + v : (ka == 1 ? i1 : i0)));
+                for (int v = 0; v < V; ++v) rf.set(o.dst, v, at.iota(ka, v));
             } break;
 #define NGH_UN(OPC)                                                                   \
     case OPC: {                                                                       \
@@ -118,7 +197,7 @@ __device__ __forceinline__ void run_ops(const KArgs& k, LdsRegs<V>& rf, Extra& e
                     for (int v = 0; v < V; ++v) {
                         Acc b;
                         b.v = rf.get(o.a, v);
-                        b.i = (int)(RMODE == 1 ? i2 + v : i0);
+                        b.i = at.red_index(RMODE, v);
                         a = acc_merge(opc, a, b);
                     }
                     ex.setf(ex_accv(k, o.dst), a.v);
@@ -155,7 +234,126 @@ __global__ __launch_bounds__(kBlock) void ew_interp_kernel(const KArgs k, unsign
         const unsigned c2 = q - row * chunks_per_row;
         const unsigned i0 = row / d1;
         const unsigned i1 = row - i0 * d1;
-        run_ops<V, 0>(k, rf, ex, i0, i1, (long long)c2 * V);
+        run_ops<V, 0>(k, rf, ex, VecAt<V>{i0, i1, (long long)c2 * V});
+    }
+    stats_epilogue(k, ex);
+}
+
+// ---------------------------------------------------------------------------
+// Streaming elementwise stage without vector access (operands strided along
+// kernel axis 2, or lengths that are not a multiple of the vector width).
+// Elements are taken in the view's linear order; a lane works on G of them,
+// 256 elements apart, so each of its accesses is as coalesced as the strides
+// allow and every op is decoded once for G elements.
+// ---------------------------------------------------------------------------
+template <int G>
+__global__ __launch_bounds__(kBlock) void ew_gather_interp_kernel(const KArgs k, unsigned long long total) {
+    extern __shared__ float lds[];
+    LdsRegs<G> rf{lds + threadIdx.x, kBlock};
+    Extra ex{lds + (size_t)k.n_regs * G * kBlock + threadIdx.x, kBlock};
+    for (int s = 0; s < k.n_stat_slots; ++s) ex.seti(ex_stat(s), 0);
+    const unsigned d1 = (unsigned)k.shape[1], d2 = (unsigned)k.shape[2];
+    const unsigned long long span = (unsigned long long)kBlock * G;
+    for (unsigned long long base = blockIdx.x * span; base < total; base += gridDim.x * span) {
+        GatherAt<G> at;
+        at.nv = 0;
+#pragma unroll
+        for (int v = 0; v < G; ++v) {
+            const unsigned long long q = base + (unsigned)v * kBlock + threadIdx.x;
+            at.i0[v] = at.i1[v] = at.i2[v] = 0;
+            if (q < total) {
+                at.nv = v + 1;
+                unsigned row;
+                if (total <= 0xffffffffull) {
+                    row = (unsigned)q / d2;
+                    at.i2[v] = (unsigned)q - row * d2;
+                } else {
+                    row = (unsigned)(q / d2);
+                    at.i2[v] = (unsigned)(q - (unsigned long long)row * d2);
+                }
+                at.i0[v] = row / d1;
+                at.i1[v] = row - at.i0[v] * d1;
+            }
+        }
+        run_ops<G, 0>(k, rf, ex, at);
+    }
+    stats_epilogue(k, ex);
+}
+
+// ---------------------------------------------------------------------------
+// Tiled elementwise stage for operands of mixed contiguity: some contiguous
+// along kernel axis 2 (the axis lanes compute along), others -- transposed
+// views -- contiguous along kernel axis 1.  A workgroup owns a 32 x 32 tile of
+// axes (1, 2).  Operands of the second kind are staged through LDS: read with
+// lanes along axis 1 (coalesced) into a padded tile, used by the program with
+// lanes along axis 2 (pitch 33: conflict-free), and results bound for such
+// operands travel the same way in reverse.  Every access to memory is
+// coalesced whatever the orientation of the view (the reference's kernels
+// index strided views directly, float_ew2.py:987-1132).
+// ---------------------------------------------------------------------------
+template <int TILE>
+__global__ __launch_bounds__(kBlock) void ew_tiled_interp_kernel(const KArgs k, unsigned tiles_a,
+                                                                 unsigned tiles_b, unsigned n_tiles,
+                                                                 unsigned load_mask, unsigned store_mask) {
+    constexpr int V = TILE * TILE / kBlock;        // elements per lane: 4 (32 x 32) or 1 (16 x 16)
+    constexpr int kRowStep = kBlock / TILE;        // tile rows between a lane's elements
+    extern __shared__ float lds[];
+    LdsRegs<V> rf{lds + threadIdx.x, kBlock};
+    Extra ex{lds + (size_t)k.n_regs * V * kBlock + threadIdx.x, kBlock};
+    float* tile_base = lds + (size_t)(k.n_regs * V + k.n_stat_slots) * kBlock;
+    for (int s = 0; s < k.n_stat_slots; ++s) ex.seti(ex_stat(s), 0);
+    const unsigned A = (unsigned)k.shape[1], B = (unsigned)k.shape[2];
+    constexpr int kTile = TILE, kTilePitch = TILE + 1, kTileWords = tile_words(TILE);
+    const unsigned lx = threadIdx.x & (kTile - 1), ly = threadIdx.x / kTile;
+    for (unsigned tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const unsigned tb = tile % tiles_b;
+        const unsigned r = tile / tiles_b;
+        const unsigned ta = r % tiles_a;
+        const unsigned i0 = r / tiles_a;
+        const unsigned a0 = ta * kTile, b0 = tb * kTile;
+        // stage in: lanes along axis 1
+        for (int t = 0; t < k.n_tensors; ++t) {
+            const KTensor& T = k.t[t];
+            if (T.stage_slot < 0 || !(load_mask >> t & 1u)) continue;
+            const float sc = (T.dtype == NGH_FLEX16) ? tensor_scale(T) : 1.0f;
+            float* tl = tile_base + T.stage_slot * kTileWords;
+            if (a0 + lx < A)
+                for (unsigned y = ly; y < kTile && b0 + y < B; y += kBlock / kTile)
+                    tl[y * kTilePitch + lx] =
+                        load1(T, (long long)i0 * T.s[0] + (long long)(a0 + lx) * T.s[1] + (long long)(b0 + y) * T.s[2], sc);
+        }
+        __syncthreads();
+        // compute: lanes along axis 2
+        if (b0 + lx < B && a0 + ly < A) {
+            GatherAt<V> at;
+            at.nv = 0;
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                at.i0[v] = i0;
+                at.i1[v] = a0 + ly + v * kRowStep;
+                at.i2[v] = b0 + lx;
+                if (at.i1[v] < A) at.nv = v + 1;
+                else at.i1[v] = a0 + ly;
+            }
+            run_ops<V, 0, true>(k, rf, ex, at, Tiles{tile_base, (int)(lx * kTilePitch + ly), kRowStep, kTileWords});
+        }
+        __syncthreads();
+        // stage out: lanes along axis 1
+        if (!k.probe) {
+            for (int t = 0; t < k.n_tensors; ++t) {
+                const KTensor& T = k.t[t];
+                if (T.stage_slot < 0 || !(store_mask >> t & 1u)) continue;
+                const float sc = (T.dtype == NGH_FLEX16) ? 1.0f / tensor_scale(T) : 1.0f;
+                const float* tl = tile_base + T.stage_slot * kTileWords;
+                int fmax = 0;
+                if (a0 + lx < A)
+                    for (unsigned y = ly; y < kTile && b0 + y < B; y += kBlock / kTile)
+                        store1(T, (long long)i0 * T.s[0] + (long long)(a0 + lx) * T.s[1] + (long long)(b0 + y) * T.s[2],
+                               tl[y * kTilePitch + lx], sc, fmax);
+                if (T.stat_slot >= 0) ex.seti(ex_stat(T.stat_slot), max(ex.geti(ex_stat(T.stat_slot)), fmax));
+            }
+            __syncthreads();
+        }
     }
     stats_epilogue(k, ex);
 }
@@ -221,7 +419,7 @@ __global__ __launch_bounds__(kBlock) void red_row_interp_kernel(const KArgs k, u
     const unsigned c_begin = seg * seg_chunks;
     const unsigned c_end = min(total_chunks, c_begin + seg_chunks);
     for (unsigned c = c_begin + threadIdx.x; c < c_end; c += kBlock)
-        run_ops<V, 1>(k, rf, ex, i0, i1, (long long)c * V);
+        run_ops<V, 1>(k, rf, ex, VecAt<V>{i0, i1, (long long)c * V});
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int s = 0; s < k.n_red; ++s) {
@@ -275,7 +473,7 @@ __global__ __launch_bounds__(kBlock) void red_col_interp_kernel(const KArgs k, u
     const unsigned r_begin = seg * seg_rows;
     const unsigned r_end = min((unsigned)k.shape[0], r_begin + seg_rows);
     if (i2 < d2)
-        for (unsigned r = r_begin + ty; r < r_end; r += kColTy) run_ops<1, 2>(k, rf, ex, r, i1, i2);
+        for (unsigned r = r_begin + ty; r < r_end; r += kColTy) run_ops<1, 2>(k, rf, ex, VecAt<1>{r, i1, i2});
 
     for (int s = 0; s < k.n_red; ++s) {
         Acc a;

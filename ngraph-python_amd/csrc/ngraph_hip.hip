@@ -78,6 +78,7 @@ struct ngh_context {
     unsigned    stat_ws_blocks = 0;  // capacity per statistics slot
     int         ew_blocks_per_cu = 64;
     int         force_interp = 0;    // never pick a specialised kernel
+    int         no_tiles = 0;        // never use the LDS-tiled elementwise skeleton
     int         flex_self_managed = 1;  // ngh_launch_fused_flex may fold the policy into the kernel
     int         cache_policy = -1;   // -1: from the operands' cache hints; 0..3 forces bit 0 = non-temporal
                                      // loads, bit 1 = non-temporal stores in pre-built kernels
@@ -182,11 +183,12 @@ int validate(const ngh_fused_spec* sp) {
 // ---------------------------------------------------------------------------
 // planner
 // ---------------------------------------------------------------------------
-enum Family { F_EW = 0, F_RED_ROW, F_RED_COL };
+enum Family { F_EW = 0, F_RED_ROW, F_RED_COL, F_EW_TILED };
 
 struct Plan {
     Family   family = F_EW;
-    int      V = 1;
+    int      V = 1;                               // elements per lane (pre-built kernels)
+    int      Vi = 1;                              // elements per lane when the interpreter runs the stage
     KArgs    k;
     unsigned n_chunks = 0, chunks_per_row = 0;   // EW
     unsigned n_out = 0, n_seg = 1, seg_len = 0;  // reductions
@@ -194,6 +196,9 @@ struct Plan {
     int      special = -1;                        // index into the specialised-kernel table
     long long tail = 0;                           // 1-D contiguous stage: elements left to a scalar launch
     int      perm[3] = {0, 1, 2};                 // kernel axis j holds spec axis perm[j]
+    unsigned tiles_a = 0, tiles_b = 0, n_tiles = 0;   // tiled elementwise
+    int      tile = kTile;
+    unsigned load_mask = 0, store_mask = 0;           // tensors the stage loads / stores
 };
 
 // Which tensors does the stage touch (load or store or reduce into)?
@@ -234,6 +239,7 @@ void fill_kargs(const ngh_fused_spec& sp, const ngh_stage& S, const int perm[3],
         K.stats = T.dev_stats;
         K.dscale = T.dev_scale;
         K.stat_slot = -1;
+        K.stage_slot = -1;
         if (stores[t] && T.dtype == NGH_FLEX16 && k.n_stat_slots < 4) {
             K.stat_slot = k.n_stat_slots;
             k.stat_ptr[k.n_stat_slots++] = T.dev_stats;
@@ -244,7 +250,7 @@ void fill_kargs(const ngh_fused_spec& sp, const ngh_stage& S, const int perm[3],
 }
 
 // Can the stage move V consecutive elements per lane along kernel axis 2?
-bool vec_ok(const KArgs& k, const bool* used, int V) {
+bool vec_ok(const KArgs& k, const bool* used, int V, bool any_type = false) {
     if (k.shape[2] % V) return false;
     for (int t = 0; t < k.n_tensors; ++t) {
         if (!used[t]) continue;
@@ -252,7 +258,7 @@ bool vec_ok(const KArgs& k, const bool* used, int V) {
         if (K.s[2] == 0) continue;
         if (K.s[2] != 1) return false;
         const int isz = itemsize_of(K.dtype);
-        if (V == 8 && isz != 2) return false;              // 8-wide only pays for 16-bit storage
+        if (V >= 8 && isz != 2 && !any_type) return false;   // pre-built kernels: 8-wide only pays for 16-bit storage
         const int align = std::min(16, V * isz);
         if (((uintptr_t)K.p) % align) return false;
         for (int j = 0; j < 2; ++j)
@@ -262,6 +268,28 @@ bool vec_ok(const KArgs& k, const bool* used, int V) {
 }
 
 bool vec4_ok(const KArgs& k, const bool* used) { return vec_ok(k, used, 4); }
+
+constexpr size_t kInterpLdsPreferred = 64 * 1024;   // keeps >= 2 workgroups per CU
+constexpr size_t kInterpLdsMax = 128 * 1024;
+constexpr size_t kInterpLdsWide = 40 * 1024;        // budget when widening the interpreter's vectors
+
+size_t interp_lds_bytes(const KArgs& k, int V) {
+    return ((size_t)k.n_regs * V + k.n_stat_slots + 2 * k.n_red) * kBlock * sizeof(float);
+}
+
+size_t tiled_lds_bytes(const KArgs& k, int tile) {
+    return interp_lds_bytes(k, tile * tile / kBlock) + (size_t)k.n_staged * tile_words(tile) * sizeof(float);
+}
+
+// Elements per lane of the gather kernel: 4 when every operand is contiguous (or broadcast)
+// along the lanes and the register file still fits; 1 otherwise -- batching uncoalesced
+// accesses only deepens the queue in front of the texture addresser (measured 1.4x slower).
+int gather_width(const KArgs& k) {
+    if (k.shape[0] * k.shape[1] * k.shape[2] < 256LL * kBlock * 4) return 1;   // too small to fill the chip 4-wide
+    for (int t = 0; t < k.n_tensors; ++t)
+        if (k.t[t].s[2] != 0 && k.t[t].s[2] != 1) return 1;
+    return interp_lds_bytes(k, 4) <= kInterpLdsPreferred ? 4 : 1;
+}
 
 int plan_stage(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan& P) {
     const ngh_stage& S = sp.stages[stage];
@@ -307,6 +335,66 @@ int plan_stage(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan
                 P.k.shape[2] = n;
             }
         }
+        if (P.V == 1 && P.tail == 0 && !(ctx && ctx->no_tiles)) {
+            // Operands of mixed contiguity: if enough of the traffic is contiguous along a
+            // second axis (transposed views), stage those operands through LDS tiles.
+            double total = 0.0, along[NGH_MAX_AXES] = {0.0, 0.0, 0.0};
+            for (int t = 0; t < sp.n_tensors; ++t) {
+                if (!used[t]) continue;
+                const ngh_tensor& T = sp.tensors[t];
+                double elems = 1.0;
+                for (int b = 0; b < NGH_MAX_AXES; ++b)
+                    if (T.strides[b] != 0) elems *= (double)sp.shape[b];
+                const double w = elems * itemsize_of(T.dtype) * ((loads[t] ? 1 : 0) + (stores[t] ? 1 : 0));
+                total += w;
+                if (T.strides[best] == 1 || T.strides[best] == 0) continue;
+                for (int a = 0; a < NGH_MAX_AXES; ++a)
+                    if (a != best && sp.shape[a] > 1 && T.strides[a] == 1) along[a] += w;
+            }
+            int second = -1;
+            for (int a = 0; a < NGH_MAX_AXES; ++a)
+                if (a != best && along[a] > 0.0 && (second < 0 || along[a] > along[second])) second = a;
+            if (second >= 0 && along[second] >= 0.2 * total && sp.shape[second] >= 8 && sp.shape[best] >= 8) {
+                int outer = 0;
+                while (outer == best || outer == second) ++outer;
+                const int tperm[3] = {outer, second, best};
+                KArgs kt;
+                fill_kargs(sp, S, tperm, kt);
+                int n_staged = 0;
+                for (int t = 0; t < sp.n_tensors; ++t) {
+                    kt.t[t].stage_slot = -1;
+                    if (used[t] && kt.t[t].s[1] == 1 && kt.t[t].s[2] != 0 && kt.t[t].s[2] != 1)
+                        kt.t[t].stage_slot = n_staged++;
+                }
+                kt.n_staged = n_staged;
+                // small problems take 16 x 16 tiles: four times the workgroups, one element per lane
+                int tile = kTile;
+                if (kt.shape[0] * ((kt.shape[1] + 31) / 32) * ((kt.shape[2] + 31) / 32) < 4LL * (ctx ? ctx->cus : 256))
+                    tile = 16;
+                const long long ta = (kt.shape[1] + tile - 1) / tile, tb = (kt.shape[2] + tile - 1) / tile;
+                const long long n_tiles = kt.shape[0] * ta * tb;
+                if (n_staged > 0 && n_tiles < (1LL << 31) && tiled_lds_bytes(kt, tile) <= kInterpLdsPreferred - 1024) {
+                    P.tile = tile;
+                    P.k = kt;
+                    for (int a = 0; a < 3; ++a) P.perm[a] = tperm[a];
+                    P.family = F_EW_TILED;
+                    P.tiles_a = (unsigned)ta;
+                    P.tiles_b = (unsigned)tb;
+                    P.n_tiles = (unsigned)n_tiles;
+                    for (int t = 0; t < sp.n_tensors; ++t) {
+                        if (loads[t]) P.load_mask |= 1u << t;
+                        if (stores[t]) P.store_mask |= 1u << t;
+                    }
+                    return NGH_OK;
+                }
+            }
+        }
+        // The interpreter pays a fixed price per op whatever the width, so it takes 8 elements
+        // per lane for every storage type when the register file still leaves several
+        // workgroups per CU (16 per lane measured slower: the file crowds out occupancy).
+        P.Vi = P.V;
+        if (P.tail == 0 && P.V >= 4)
+            if (P.V < 8 && vec_ok(P.k, used, 8, true) && interp_lds_bytes(P.k, 8) <= kInterpLdsWide) P.Vi = 8;
         const long long rows = P.k.shape[0] * P.k.shape[1];
         const long long cpr = P.k.shape[2] / P.V;
         if (rows * cpr >= (1LL << 32) || rows >= (1LL << 32))
@@ -376,13 +464,6 @@ int plan_stage(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan
     }
     if ((long long)P.n_out * P.n_seg >= (1LL << 31)) return fail(NGH_E_UNSUPPORTED, "reduction grid too large");
     return NGH_OK;
-}
-
-constexpr size_t kInterpLdsPreferred = 64 * 1024;   // keeps >= 2 workgroups per CU
-constexpr size_t kInterpLdsMax = 128 * 1024;
-
-size_t interp_lds_bytes(const KArgs& k, int V) {
-    return ((size_t)k.n_regs * V + k.n_stat_slots + 2 * k.n_red) * kBlock * sizeof(float);
 }
 
 int ensure_ws(ngh_context* ctx, size_t bytes) {
@@ -457,40 +538,64 @@ int launch_tail(ngh_context* ctx, const Plan& P) {
     const size_t lds = interp_lds_bytes(kt, 1);
     if (lds > kInterpLdsMax) return fail(NGH_E_UNSUPPORTED, "program needs %zu bytes of LDS registers", lds);
     NGH_TRY(stat_scratch(ctx, kt, 1));
-    hipLaunchKernelGGL(ew_interp_kernel<1>, dim3(1), dim3(kBlock), lds, ctx->stream, kt, (unsigned)P.tail,
-                       (unsigned)P.tail);
+    hipLaunchKernelGGL(ew_gather_interp_kernel<1>, dim3(1), dim3(kBlock), lds, ctx->stream, kt,
+                       (unsigned long long)P.tail);
     HIP_TRY(hipGetLastError());
     return stat_fold(ctx, kt, 1);
 }
 
 int launch_interp(ngh_context* ctx, Plan& P) {
-    int V = P.V;
+    if (P.family == F_EW_TILED) {
+        if (P.n_tiles == 0) return NGH_OK;
+        const unsigned blocks = std::min<unsigned>(P.n_tiles, (unsigned)(ctx->cus * ctx->ew_blocks_per_cu));
+        NGH_TRY(stat_scratch(ctx, P.k, blocks));
+        if (P.tile == 16)
+            hipLaunchKernelGGL(ew_tiled_interp_kernel<16>, dim3(blocks), dim3(kBlock), tiled_lds_bytes(P.k, 16),
+                               ctx->stream, P.k, P.tiles_a, P.tiles_b, P.n_tiles, P.load_mask, P.store_mask);
+        else
+            hipLaunchKernelGGL(ew_tiled_interp_kernel<32>, dim3(blocks), dim3(kBlock), tiled_lds_bytes(P.k, 32),
+                               ctx->stream, P.k, P.tiles_a, P.tiles_b, P.n_tiles, P.load_mask, P.store_mask);
+        HIP_TRY(hipGetLastError());
+        return stat_fold(ctx, P.k, blocks);
+    }
+    int V = (P.family == F_EW) ? P.Vi : P.V;
     size_t lds = interp_lds_bytes(P.k, V);
     while (lds > kInterpLdsPreferred && V > 1 && P.family == F_EW) {
         // too many live registers for a V-wide file: narrow the vector (the tail, if any, stays)
-        const int narrower = (V == 8) ? 4 : 1;
-        const long long cpr = P.k.shape[2] / narrower;
-        const long long chunks = P.k.shape[0] * P.k.shape[1] * cpr;
-        if (chunks >= (1LL << 32)) break;
-        V = P.V = narrower;
-        P.chunks_per_row = (unsigned)cpr;
-        P.n_chunks = (unsigned)chunks;
+        const int narrower = (V > 4) ? V / 2 : 1;
+        if (P.k.shape[0] * P.k.shape[1] * (P.k.shape[2] / narrower) >= (1LL << 32)) break;
+        V = narrower;
         lds = interp_lds_bytes(P.k, V);
+    }
+    if (P.family == F_EW) {
+        P.Vi = V;
+        P.chunks_per_row = (unsigned)(P.k.shape[2] / V);
+        P.n_chunks = (unsigned)(P.k.shape[0] * P.k.shape[1] * (P.k.shape[2] / V));
     }
     if (lds > kInterpLdsMax) return fail(NGH_E_UNSUPPORTED, "program needs %zu bytes of LDS registers", lds);
     KArgs& k = P.k;
     if (P.family == F_EW) {
         if (P.n_chunks == 0 && P.tail == 0) return NGH_OK;
-        if (P.n_chunks) {
+        if (P.n_chunks && V == 1) {
+            const int G = gather_width(k);
+            const unsigned long long total = P.n_chunks;
+            unsigned blocks = (unsigned)((total + (unsigned long long)kBlock * G - 1) / ((unsigned long long)kBlock * G));
+            blocks = std::min<unsigned>(blocks, (unsigned)(ctx->cus * ctx->ew_blocks_per_cu));
+            NGH_TRY(stat_scratch(ctx, k, blocks));
+            if (G == 4)
+                hipLaunchKernelGGL(ew_gather_interp_kernel<4>, dim3(blocks), dim3(kBlock), interp_lds_bytes(k, 4), ctx->stream, k, total);
+            else
+                hipLaunchKernelGGL(ew_gather_interp_kernel<1>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, total);
+            HIP_TRY(hipGetLastError());
+            NGH_TRY(stat_fold(ctx, k, blocks));
+        } else if (P.n_chunks) {
             unsigned blocks = (P.n_chunks + kBlock - 1) / kBlock;
             blocks = std::min<unsigned>(blocks, (unsigned)(ctx->cus * ctx->ew_blocks_per_cu));
             NGH_TRY(stat_scratch(ctx, k, blocks));
             if (V == 8)
                 hipLaunchKernelGGL(ew_interp_kernel<8>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, P.n_chunks, P.chunks_per_row);
-            else if (V == 4)
-                hipLaunchKernelGGL(ew_interp_kernel<4>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, P.n_chunks, P.chunks_per_row);
             else
-                hipLaunchKernelGGL(ew_interp_kernel<1>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, P.n_chunks, P.chunks_per_row);
+                hipLaunchKernelGGL(ew_interp_kernel<4>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, P.n_chunks, P.chunks_per_row);
             HIP_TRY(hipGetLastError());
             NGH_TRY(stat_fold(ctx, k, blocks));
         }
@@ -537,9 +642,13 @@ void describe(const Plan& P, char* out, size_t n) {
         return;
     }
     switch (P.family) {
-        case F_EW: snprintf(out, n, "ew_interp_v%d%s", P.V, P.tail ? "+tail" : ""); break;
+        case F_EW:
+            if (P.Vi == 1) snprintf(out, n, "ew_gather_interp_g%d", gather_width(P.k));
+            else snprintf(out, n, "ew_interp_v%d%s", P.Vi, P.tail ? "+tail" : "");
+            break;
         case F_RED_ROW: snprintf(out, n, "red_row_interp_v%d_s%u", P.V, P.n_seg); break;
         case F_RED_COL: snprintf(out, n, "red_col_interp_v1_s%u", P.n_seg); break;
+        case F_EW_TILED: snprintf(out, n, "ew_tiled_interp_t%d_s%d", P.tile, P.k.n_staged); break;
     }
 }
 
@@ -582,6 +691,7 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->ew_blocks_per_cu = std::max(1, env_int("NGH_EW_BLOCKS_PER_CU", 64));
     ctx->force_interp = env_int("NGH_FORCE_INTERP", 0);
     ctx->flex_self_managed = env_int("NGH_FLEX_SELF_MANAGED", 1);
+    ctx->no_tiles = env_int("NGH_NO_TILES", 0);
     ctx->cache_policy = env_int("NGH_CACHE_POLICY", -1);
     ctx->stream_bytes = (long long)env_int("NGH_STREAM_MIB", 128) << 20;
     ctx->moments_wgs_per_cu = std::max(1, env_int("NGH_MOMENTS_WGS_PER_CU", 16));
@@ -594,9 +704,10 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     }
     // the interpreter's register file is dynamic LDS and may exceed the 64 KiB default
     const void* interp_kernels[] = {(const void*)ew_interp_kernel<8>, (const void*)ew_interp_kernel<4>,
-                                    (const void*)ew_interp_kernel<1>,
+                                    (const void*)ew_gather_interp_kernel<4>, (const void*)ew_gather_interp_kernel<1>,
                                     (const void*)red_row_interp_kernel<4>, (const void*)red_row_interp_kernel<1>,
-                                    (const void*)red_col_interp_kernel};
+                                    (const void*)red_col_interp_kernel, (const void*)ew_tiled_interp_kernel<16>,
+                                    (const void*)ew_tiled_interp_kernel<32>};
     for (const void* fn : interp_kernels) {
         e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kInterpLdsMax);
         if (e != hipSuccess) {

@@ -385,3 +385,75 @@ def test_moments_rows(hip_runtime, rows, R, pad):
     assert not out_d.get()[2].any()
     for d in (x_d, out_d):
         d.free()
+
+
+# ------------------------------------------------------------------ tiled skeleton (transposed views)
+def _transpose_program(rt, shape3, x_d, y_d, z_d, w_d, in_place):
+    """Over logical [O, A, B]:  y[o,a,b] (B-contiguous) = 2*x[o,b,a]^T + z[o,a,b];
+    w[o,b,a] (A-contiguous, i.e. a transposed output) = y - 1; with in_place, x is overwritten
+    by w instead."""
+    O, A, B = shape3
+    sb = FusedSpecBuilder([O, A, B])
+    tx = sb.tensor(x_d.ptr, [A * B, 1, A])        # x stored [O, B, A]: contiguous along A
+    tz = sb.tensor(z_d.ptr, [A * B, B, 1])        # z stored [O, A, B]
+    ty = sb.tensor(y_d.ptr, [A * B, B, 1])
+    tw = tx if in_place else sb.tensor(w_d.ptr, [A * B, 1, A])
+    x = sb.load(tx)
+    z = sb.load(tz)
+    y = sb.binary("add", sb.binary("mul", x, sb.constant(2.0)), z)
+    sb.store(ty, y)
+    sb.store(tw, sb.binary("sub", y, sb.constant(1.0)))
+    return sb.build()
+
+
+@pytest.mark.parametrize("shape3", [(1, 64, 64), (1, 1024, 64), (3, 50, 37), (2, 33, 200), (1, 9, 8), (1, 2048, 2048)])
+@pytest.mark.parametrize("in_place", [False, True])
+def test_tiled_transposed_operands(hip_runtime, shape3, in_place):
+    """Inputs and outputs of both orientations in one stage: the planner picks the LDS-tiled
+    skeleton (family 3) and every element lands where the strided views say."""
+    from ngraph_hip.runtime import hiplib
+    rt = hip_runtime
+    O, A, B = shape3
+    rs = np.random.RandomState(A * 31 + B)
+    x = rs.normal(0, 1, (O, B, A)).astype(f32)
+    z = rs.normal(0, 1, (O, A, B)).astype(f32)
+    x_d, z_d = rt.array(x), rt.array(z)
+    y_d, w_d = rt.empty((O, A, B)), rt.empty((O, B, A))
+    spec = _transpose_program(rt, shape3, x_d, y_d, z_d, w_d, in_place)
+    assert hiplib.plan_fused(spec, 0)["family"] == 3
+    assert rt.describe_fused(spec, 0).startswith("ew_tiled_interp")
+    rt.launch_fused(spec)
+    y_w = (x.transpose(0, 2, 1) * f32(2.0) + z).astype(f32)
+    w_w = (y_w - f32(1.0)).transpose(0, 2, 1)
+    np.testing.assert_array_equal(y_d.get(), y_w)
+    np.testing.assert_array_equal((x_d if in_place else w_d).get(), w_w)
+    for d in (x_d, z_d, y_d, w_d):
+        d.free()
+
+
+def test_tiled_flex_transposed_output_with_statistics(hip_runtime):
+    """A flex16 result written through a transposed view: quantisation and max|mantissa| happen
+    at the staged store."""
+    from ngraph_hip.runtime import NGH_FLEX16
+    from oracle import flex_model as fm
+    rt = hip_runtime
+    A, B = 70, 45
+    rs = np.random.RandomState(5)
+    x = rs.normal(0, 1, (A, B)).astype(f32)
+    x_d = rt.array(x)
+    y_d = rt.empty((B, A), NGH_FLEX16)
+    stats = rt.stats_alloc(1)
+    dec = 12
+    sb = FusedSpecBuilder([A, B])
+    tx = sb.tensor(x_d.ptr, [B, 1])
+    ty = sb.tensor(y_d.ptr, [1, A], NGH_FLEX16, scale=2.0 ** -dec, dev_stats=stats)
+    sb.store(ty, sb.binary("mul", sb.load(tx), sb.constant(3.0)))
+    spec = sb.build()
+    assert rt.describe_fused(spec, 0).startswith("ew_tiled_interp")
+    rt.launch_fused(spec)
+    want = fm.quantize_rni((x * f32(3.0)).T, dec)
+    np.testing.assert_array_equal(y_d.get(), want)
+    assert int(rt.stats_read(stats, 1)[0]) == fm.maxabs(want)
+    for d in (x_d, y_d):
+        d.free()
+    rt.free(stats)
