@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define NGH_ABI_VERSION 2
+#define NGH_ABI_VERSION 3
 
 /* ---- limits (float_ew2.py:285-286 MAX_AXES = 3) ------------------------ */
 #define NGH_MAX_AXES      3
@@ -88,6 +88,12 @@ enum ngh_opcode {
     /* reductions over axis 0 of the stage's view: dst=reduction slot a=reg */
     NGH_OP_RED_SUM, NGH_OP_RED_PROD, NGH_OP_RED_MAX, NGH_OP_RED_MIN,
     NGH_OP_RED_ARGMAX, NGH_OP_RED_ARGMIN,
+    /* lookup ("take", float_ew2.py:65, 122-125, 1242-1258; the fprop of LookupTableOp,
+     * gputransform.py:197-199): dst=reg a=reg holding the index b=tensor | axis << 4.
+     * Loads the tensor's element whose coordinate along `axis` is (int)index instead of the
+     * loop coordinate; the tensor's stride on that axis is the table's stride along its
+     * looked-up axis and take_extent its length there (indices are clamped to it).       */
+    NGH_OP_TAKE,
     NGH_OP_COUNT_
 };
 
@@ -135,7 +141,8 @@ typedef struct ngh_tensor {
                                   streaming kernels whose operands exceed the
                                   last-level cache; no counterpart in the
                                   reference (PTX loads there carry no hint)   */
-    uint32_t reserved_;
+    uint32_t take_extent;      /* operand of NGH_OP_TAKE: length of the looked-up
+                                  axis; 0 otherwise                           */
 } ngh_tensor;
 
 /* One stage = a run of elementwise ops optionally ended by reductions

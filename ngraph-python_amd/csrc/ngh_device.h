@@ -27,6 +27,8 @@ struct KTensor {
     const float* dscale;
     int          stat_slot;  // which per-thread max|mantissa| accumulator, -1 = none
     int          stage_slot; // tiled skeleton: which LDS tile carries this operand, -1 = direct access
+    unsigned     take_extent;  // table operand of NGH_OP_TAKE: length of the looked-up axis
+    int          pad_;
 };
 
 struct KArgs {

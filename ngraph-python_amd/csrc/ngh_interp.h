@@ -57,6 +57,7 @@ struct VecAt {   // (i0, i1, i2 .. i2 + V - 1)
         return (float)(ka == 2 ? i2 + v : (ka == 1 ? i1 : i0));
     }
     __device__ __forceinline__ int red_index(int rmode, int v) const { return (int)(rmode == 1 ? i2 + v : i0); }
+    __device__ __forceinline__ long long coord(int ka, int v) const { return ka == 2 ? i2 + v : (ka == 1 ? i1 : i0); }
     __device__ __forceinline__ void load(const KTensor& t, float (&x)[V]) const {
         const long long off = i0 * t.s[0] + i1 * t.s[1] + i2 * t.s[2];
         const float sc = (t.dtype == NGH_FLEX16) ? tensor_scale(t) : 1.0f;
@@ -94,6 +95,7 @@ struct GatherAt {   // element v at (i0[v], i1[v], i2[v]); only the first nv cou
         return (float)(ka == 2 ? i2[v] : (ka == 1 ? i1[v] : i0[v]));
     }
     __device__ __forceinline__ int red_index(int, int) const { return 0; }   // not used with reductions
+    __device__ __forceinline__ long long coord(int ka, int v) const { return ka == 2 ? i2[v] : (ka == 1 ? i1[v] : i0[v]); }
     __device__ __forceinline__ void load(const KTensor& t, float (&x)[V]) const {
         const float sc = (t.dtype == NGH_FLEX16) ? tensor_scale(t) : 1.0f;
 #pragma unroll
@@ -156,6 +158,22 @@ __device__ __forceinline__ void run_ops(const KArgs& k, LdsRegs<V>& rf, Extra& e
                     at.store(t, x, fmax);
                 }
                 if (t.stat_slot >= 0) ex.seti(ex_stat(t.stat_slot), max(ex.geti(ex_stat(t.stat_slot)), fmax));
+            } break;
+            case NGH_OP_TAKE: {
+                // table lookup: the coordinate along one axis comes from a register
+                const KTensor& t = k.t[o.b & 15];
+                const int ka = k.iota_map[o.b >> 4];
+                const float sc = (t.dtype == NGH_FLEX16) ? tensor_scale(t) : 1.0f;
+#pragma unroll
+                for (int v = 0; v < V; ++v) {
+                    long long idx = (long long)rf.get(o.a, v);            // astype(int): truncation
+                    idx = idx < 0 ? 0 : (idx >= (long long)t.take_extent ? (long long)t.take_extent - 1 : idx);
+                    long long off = idx * t.s[ka];
+#pragma unroll
+                    for (int a = 0; a < 3; ++a)
+                        if (a != ka) off += at.coord(a, v) * t.s[a];
+                    rf.set(o.dst, v, load1(t, off, sc));
+                }
             } break;
             case NGH_OP_CONST: {
                 const float c = k.consts[o.a];

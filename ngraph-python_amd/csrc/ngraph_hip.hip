@@ -147,6 +147,13 @@ int validate(const ngh_fused_spec* sp) {
             } else if (opc == NGH_OP_CONST) {
                 if (o.a >= sp->n_consts || !reg_ok(o.dst)) return fail(NGH_E_INVALID, "op %d: bad CONST", pc);
                 defined[o.dst] = true;
+            } else if (opc == NGH_OP_TAKE) {
+                const int t = o.b & 15, axis = o.b >> 4;
+                if (t >= sp->n_tensors || axis >= sp->rank || !need(o.a) || !reg_ok(o.dst))
+                    return fail(NGH_E_INVALID, "op %d: bad TAKE", pc);
+                if (sp->tensors[t].take_extent == 0)
+                    return fail(NGH_E_INVALID, "op %d: TAKE from tensor %d without take_extent", pc, t);
+                defined[o.dst] = true;
             } else if (opc == NGH_OP_IOTA) {
                 if (o.a >= NGH_MAX_AXES || !reg_ok(o.dst)) return fail(NGH_E_INVALID, "op %d: bad IOTA", pc);
                 defined[o.dst] = true;
@@ -240,6 +247,7 @@ void fill_kargs(const ngh_fused_spec& sp, const ngh_stage& S, const int perm[3],
         K.dscale = T.dev_scale;
         K.stat_slot = -1;
         K.stage_slot = -1;
+        K.take_extent = T.take_extent;
         if (stores[t] && T.dtype == NGH_FLEX16 && k.n_stat_slots < 4) {
             K.stat_slot = k.n_stat_slots;
             k.stat_ptr[k.n_stat_slots++] = T.dev_stats;

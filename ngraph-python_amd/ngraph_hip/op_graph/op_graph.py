@@ -1343,6 +1343,38 @@ def one_hot(x, axis):
     return OneHotOp(x, axis)
 
 
+class LookupTableOp(TensorOp):
+    """Forward lookup: rows (lut_axis 0) or columns (lut_axis 1) of a 2-D table selected by a
+    1-D index tensor (op_graph/lookuptable.py:55-115).  `axes` are the output axes; the one at
+    position lut_axis must be the index axis, the other one the table's remaining axis."""
+
+    def __init__(self, lut, idx, axes, update=True, pad_idx=None, **kwargs):
+        lut, idx = as_op(lut), as_op(idx)
+        axes = make_axes(axes)
+        if len(lut.shape) != 2:
+            raise ValueError("lookup table shape must be length 2, found {}".format(len(lut.shape)))
+        if len(idx.shape) != 1:
+            raise ValueError("index shape must be length 1, found {}".format(len(idx.shape)))
+        if not (lut.axes[0] in axes or lut.axes[1] in axes):
+            raise ValueError("Output axes must indicate which axis to do lookup.  None of the "
+                             "output axes is from lookup table.  Found lut axes: {} Found output "
+                             "axes: {}.".format(lut.axes, axes))
+        if idx.axes[0] not in axes:
+            raise ValueError("Output axes must index axes.  Found index axes: {} Found output "
+                             "axes: {}.".format(idx.axes, axes))
+        self.lut_axis = 0 if lut.axes[1] in axes else 1
+        self.pad_idx = pad_idx
+        self.update = update
+        if axes[self.lut_axis] != idx.axes[0]:
+            raise ValueError("Cannot transpose lut axes implicitly")
+        super(LookupTableOp, self).__init__(args=(lut, idx), axes=axes, **kwargs)
+
+
+def lookuptable(lut, idx, axes, update=True, pad_idx=None):
+    """Look `idx` up in `lut`; `axes` are the output axes (op_graph/lookuptable.py:20-36)."""
+    return LookupTableOp(lut, idx, axes=axes, update=update, pad_idx=pad_idx)
+
+
 class SigmoidOp(ValueOp):
     """sigmoid as the composite reciprocal(exp(-x) + 1) (op_graph.py:4183-4202)."""
 

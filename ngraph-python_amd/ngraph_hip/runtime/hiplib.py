@@ -12,7 +12,7 @@ import os
 
 import numpy as np
 
-NGH_ABI_VERSION = 2
+NGH_ABI_VERSION = 3
 NGH_MAX_AXES = 3
 NGH_MAX_TENSORS = 12
 NGH_MAX_OPS = 96
@@ -32,6 +32,7 @@ _OPCODE_NAMES = [
     "add", "sub", "mul", "div", "int_div", "mod", "eq", "ne", "lt", "le", "gt", "ge",
     "pow", "minimum", "maximum",
     "sum", "prod", "max", "min", "argmax", "argmin",
+    "take",
 ]
 #: op name (the reference's template names, float_ew2.py:31-77) -> opcode
 OPCODES = {name: i for i, name in enumerate(_OPCODE_NAMES)}
@@ -53,7 +54,7 @@ class ngh_tensor(ctypes.Structure):
                 ("dev_stats", ctypes.c_void_p),
                 ("dev_scale", ctypes.c_void_p),
                 ("cache_hint", ctypes.c_uint32),
-                ("reserved_", ctypes.c_uint32)]
+                ("take_extent", ctypes.c_uint32)]
 
 
 class ngh_stage(ctypes.Structure):
@@ -475,11 +476,14 @@ class FusedSpecBuilder(object):
             raise ValueError("strides %r do not match rank %d" % (strides, self.rank))
         return strides + [0] * (NGH_MAX_AXES - len(strides))
 
-    def tensor(self, dev, strides, dtype=NGH_F32, scale=1.0, dev_stats=None, dev_scale=None):
+    def tensor(self, dev, strides, dtype=NGH_F32, scale=1.0, dev_stats=None, dev_scale=None,
+               take_extent=0):
+        """take_extent: for the table operand of `take`, the length of its looked-up axis (its
+        stride on the take axis is then the table's stride along that axis)."""
         if len(self.tensors) >= NGH_MAX_TENSORS:
             raise ValueError("too many tensors in one fused kernel")
         self.tensors.append((int(dev), self._pad_strides(strides), int(dtype), float(scale),
-                             dev_stats, dev_scale))
+                             dev_stats, dev_scale, int(take_extent)))
         return len(self.tensors) - 1
 
     def const(self, value):
@@ -532,6 +536,12 @@ class FusedSpecBuilder(object):
         self.emit(name, dst, a, b)
         return dst
 
+    def take(self, table, index_reg, axis, dst=None):
+        """dst = table[.., (int)index_reg along `axis`, ..] (the other coordinates are the loop's)."""
+        dst = self.reg() if dst is None else dst
+        self.emit("take", dst, index_reg, int(table) | (int(axis) << 4))
+        return dst
+
     def reduce(self, name, a, out_tensor):
         slot = len(self._stage_reds)
         if slot >= NGH_MAX_REDUCTIONS:
@@ -555,7 +565,8 @@ class FusedSpecBuilder(object):
         for name in REDUCTION_OPS:
             src_fields[OPCODES[name]] = (2,)
         src_fields[OPCODES["store"]] = (2,)
-        writes = set(OPCODES[n] for n in UNARY_OPS + BINARY_OPS + ["load", "const", "iota"])
+        src_fields[OPCODES["take"]] = (2,)
+        writes = set(OPCODES[n] for n in UNARY_OPS + BINARY_OPS + ["load", "const", "iota", "take"])
         n_regs = 0
         for begin, end, _ in self.stages:
             last_use = {}
@@ -608,7 +619,7 @@ class FusedSpecBuilder(object):
         spec.n_consts = len(self.consts)
         spec.n_stages = len(self.stages)
         spec.n_regs = self.n_regs
-        for i, (dev, strides, dtype, scale, stats, dscale) in enumerate(self.tensors):
+        for i, (dev, strides, dtype, scale, stats, dscale, take_extent) in enumerate(self.tensors):
             t = spec.tensors[i]
             t.dev = dev
             for j in range(NGH_MAX_AXES):
@@ -617,6 +628,7 @@ class FusedSpecBuilder(object):
             t.scale = scale
             t.dev_stats = stats
             t.dev_scale = dscale
+            t.take_extent = take_extent
         for i, c in enumerate(self.consts):
             spec.consts[i] = c
         for i, (opc, dst, a, b) in enumerate(self.ops):

@@ -70,7 +70,7 @@ def kernel_op_name(op):
 
 def is_fusable(op):
     return (kernel_op_name(op) is not None or
-            isinstance(op, (og.AssignOp, og.OneHotOp, og.Fill)))
+            isinstance(op, (og.AssignOp, og.OneHotOp, og.Fill, og.LookupTableOp)))
 
 
 def iteration_axes(op):
@@ -269,10 +269,12 @@ HipKernel.set_cache_hints = _ignore_hints
 
 
 class _Dim(object):
-    __slots__ = ("length", "strides", "tag")
+    __slots__ = ("length", "strides", "tag", "named")
 
-    def __init__(self, length, strides, tag=None):
-        self.length, self.strides, self.tag = int(length), list(strides), tag
+    def __init__(self, length, strides, tag=None, named=None):
+        # tag "red" marks a reduced axis; `named` keeps the axis name of a dim some op refers
+        # to by coordinate (one-hot, lookup), which therefore must not merge with another
+        self.length, self.strides, self.tag, self.named = int(length), list(strides), tag, named
 
 
 class FusedKernel(HipKernel):
@@ -310,6 +312,9 @@ class FusedKernel(HipKernel):
         it_axes = iteration_axes(first)
         red_axes = reductions[0].reduction_axes if reductions else og.make_axes(())
         onehot_axes = [op.axis for op in ops if isinstance(op, og.OneHotOp)]
+        take_axes = []           # output axes whose coordinate a lookup replaces by an index value
+        take_strides = {}        # (operand slot, axis) -> the table's stride along its looked-up axis
+        self.take_extents = {}   # operand slot -> length of the table's looked-up axis
 
         # ---- pass 1: collect operands (views) and the program over symbolic registers ----
         operands = []            # [(td, role)] in slot order
@@ -371,6 +376,18 @@ class FusedKernel(HipKernel):
                 program.append(("iota", i, op.axis))
                 r = new_reg()
                 program.append(("eq", r, i, x))
+            elif isinstance(op, og.LookupTableOp):
+                # gputransform.py:197-199: ("take", x=idx, y=lut, axis=lut_axis)
+                lut, idx = op.args[0].forwarded, op.args[1].forwarded
+                x = operand_reg(idx)
+                lut_td = lut.tensor_description()
+                table = slot(lut_td)
+                out_axis = op.axes[op.lut_axis]
+                take_axes.append(out_axis)
+                take_strides[(table, out_axis)] = lut_td.full_strides[op.lut_axis]
+                self.take_extents[table] = lut_td.shape[op.lut_axis]
+                r = new_reg()
+                program.append(("take", r, x, table, out_axis))
             elif isinstance(op, og.ReductionOp):
                 x = operand_reg(op.args[0])
                 if len(op.reduction_axes) == 0 or op.reduction_axes.size == 1:
@@ -413,9 +430,9 @@ class FusedKernel(HipKernel):
             tag = None
             if has_reduce and axis in red_axes:
                 tag = "red"
-            if axis in onehot_axes:
-                tag = ("iota", axis.name)
-            dims.append(_Dim(axis.length, [strides_over(td, [axis])[0] for td in operands], tag))
+            named = axis.name if (axis in onehot_axes or axis in take_axes) else None
+            strides = [take_strides.get((s, axis), strides_over(td, [axis])[0]) for s, td in enumerate(operands)]
+            dims.append(_Dim(axis.length, strides, tag, named))
 
         dims = self._coalesce(dims, has_reduce)
         outer, inner = self._split_outer(dims, has_reduce)
@@ -438,10 +455,10 @@ class FusedKernel(HipKernel):
     @staticmethod
     def _coalesce(dims, has_reduce):
         """Drop length-1 dims and merge neighbours every operand walks contiguously."""
-        dims = [d for d in dims if d.length != 1 or isinstance(d.tag, tuple)]
+        dims = [d for d in dims if d.length != 1 or d.named is not None]
 
         def mergeable(a, b):
-            if a.tag != b.tag or (a.tag is not None and a.tag != "red"):
+            if a.tag != b.tag or a.named is not None or b.named is not None:
                 return False
             return all(sa == sb * b.length for sa, sb in zip(a.strides, b.strides))
 
@@ -458,7 +475,7 @@ class FusedKernel(HipKernel):
         for d in dims:
             if out and mergeable(out[-1], d):
                 prev = out[-1]
-                out[-1] = _Dim(prev.length * d.length, d.strides, prev.tag)
+                out[-1] = _Dim(prev.length * d.length, d.strides, prev.tag)   # neither is named
             else:
                 out.append(d)
         return out
@@ -490,7 +507,8 @@ class FusedKernel(HipKernel):
             view = t.get_tensor_description_tensor_view(td)
             strides = [d.strides[s] for d in inner] or [0]
             dtype = t.ngh_dtype(td.dtype)
-            slot = sb.tensor(view.ptr + offsets[s] * view.itemsize, strides, dtype)
+            slot = sb.tensor(view.ptr + offsets[s] * view.itemsize, strides, dtype,
+                             take_extent=self.take_extents.get(s, 0))
             assert slot == s
         reg_map = {}
 
@@ -511,10 +529,16 @@ class FusedKernel(HipKernel):
                 sb.store(ins[1], reg(ins[2]))
                 written.add(ins[1])
             elif kind == "iota":
-                axis = [i for i, d in enumerate(inner) if d.tag == ("iota", ins[2].name)]
+                axis = [i for i, d in enumerate(inner) if d.named == ins[2].name]
                 if not axis:
                     raise og_unsupported("one-hot axis was merged away")
                 sb.iota(axis[0], reg(ins[1]))
+            elif kind == "take":
+                axis = [i for i, d in enumerate(inner) if d.named == ins[4].name]
+                if not axis:
+                    raise og_unsupported("lookup axis was merged away or looped on the host")
+                sb.take(ins[3], reg(ins[2]), axis[0], reg(ins[1]))
+                read.add(ins[3])
             elif kind == "reduce":
                 sb.reduce(ins[1], reg(ins[2]), ins[3])
                 written.add(ins[3])

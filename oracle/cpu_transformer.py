@@ -119,6 +119,10 @@ class NumpyTransformer(ComputationGraphTransformer):
                 o, x = view(op), view(op.args[0])
                 o[:] = np.eye(o.shape[0])[:, x.astype(np.int32)]
             return onehot
+        if isinstance(op, og.LookupTableOp):
+            def lookup():                                            # cpuengine.py:421-422 fprop_lut
+                view(op)[:] = view(op.args[0]).take(view(op.args[1]).astype(int), op.lut_axis)
+            return lookup
         if isinstance(op, og.ReductionOp):
             x_axes = op.args[0].forwarded.axes
             np_axis = tuple(x_axes.index(a) for a in op.reduction_axes)           # :348-370

@@ -457,3 +457,44 @@ def test_tiled_flex_transposed_output_with_statistics(hip_runtime):
     for d in (x_d, y_d):
         d.free()
     rt.free(stats)
+
+
+# ------------------------------------------------------------------ take (table lookup)
+@pytest.mark.parametrize("lut_axis", [0, 1])
+@pytest.mark.parametrize("I,F,V", [(37, 24, 50), (1000, 256, 300), (5, 3, 2)])
+def test_take_lookup(hip_runtime, lut_axis, I, F, V):
+    """NGH_OP_TAKE against ndarray.take; indices outside the table are clamped to it."""
+    rt = hip_runtime
+    rs = np.random.RandomState(I + F)
+    lut = rs.normal(0, 1, (V, F) if lut_axis == 0 else (F, V)).astype(f32)
+    idx = rs.randint(0, V, I).astype(f32)
+    idx[0], idx[-1] = -3.0, V + 7.0                       # out of range on both sides
+    lut_d, idx_d = rt.array(lut), rt.array(idx)
+    if lut_axis == 0:          # out[i, f] = lut[idx[i], f]
+        shape, idx_st, lut_st, out_st, axis = [I, F], [1, 0], [F, 1], [F, 1], 0
+    else:                      # out[f, i] = lut[f, idx[i]]
+        shape, idx_st, lut_st, out_st, axis = [F, I], [0, 1], [V, 1], [I, 1], 1
+    out_d = rt.empty(shape)
+    sb = FusedSpecBuilder(shape)
+    ti = sb.tensor(idx_d.ptr, idx_st)
+    tl = sb.tensor(lut_d.ptr, lut_st, take_extent=V)
+    to = sb.tensor(out_d.ptr, out_st)
+    sb.store(to, sb.take(tl, sb.load(ti), axis))
+    rt.launch_fused(sb.build())
+    want = lut.take(np.clip(idx, 0, V - 1).astype(int), lut_axis)
+    np.testing.assert_array_equal(out_d.get(), want)
+    for d in (lut_d, idx_d, out_d):
+        d.free()
+
+
+def test_take_needs_an_extent(hip_runtime):
+    from ngraph_hip.runtime.hiplib import HipLibraryError
+    rt = hip_runtime
+    lut_d, idx_d, out_d = rt.empty((4, 4)), rt.empty((3,)), rt.empty((3, 4))
+    sb = FusedSpecBuilder([3, 4])
+    ti, tl, to = sb.tensor(idx_d.ptr, [1, 0]), sb.tensor(lut_d.ptr, [4, 1]), sb.tensor(out_d.ptr, [4, 1])
+    sb.store(to, sb.take(tl, sb.load(ti), 0))
+    with pytest.raises(HipLibraryError):
+        rt.launch_fused(sb.build())
+    for d in (lut_d, idx_d, out_d):
+        d.free()

@@ -235,6 +235,41 @@ def test_onehot(backend):
         np.testing.assert_array_equal(f(xv), np.eye(5, dtype=np.float32)[:, xv.astype(int)])
 
 
+@pytest.mark.parametrize("lut_axis", [0, 1])
+def test_lookuptable_forward(backend, lut_axis):
+    """LookupTableOp fprop = the "take" template (gputransform.py:197-199) against
+    ndarray.take (cpuengine.py:421-422), alone and fused into a following chain."""
+    a = axes(V=50, F=24, I=37)
+    V, F, I = a
+    lut_axes = [V, F] if lut_axis == 0 else [F, V]
+    out_axes = [I, F] if lut_axis == 0 else [F, I]
+    lut = ng.placeholder(lut_axes)
+    idx = ng.placeholder([I])
+    looked = ng.lookuptable(lut, idx, out_axes)
+    rs = np.random.RandomState(11)
+    lut_np = rs.normal(0, 1, [x.length for x in lut_axes]).astype(np.float32)
+    idx_np = rs.randint(0, 50, 37).astype(np.float32)
+    want = lut_np.take(idx_np.astype(int), lut_axis)
+    with executor([looked, ng.tanh(looked * 2.0) + 1.0, ng.sum(looked, out_axes=[F])], lut, idx) as f:
+        got, chained, summed = f(lut_np, idx_np)
+        np.testing.assert_array_equal(got, want)
+        np.testing.assert_allclose(chained, np.tanh(want * np.float32(2.0)) + 1.0, rtol=RTOL, atol=ATOL)
+        np.testing.assert_allclose(summed, want.sum(axis=lut_axis), rtol=RTOL, atol=1e-5)
+
+
+def test_lookuptable_argument_checks():
+    a = axes(V=5, F=4, I=3)
+    V, F, I = a
+    lut, idx = ng.placeholder([V, F]), ng.placeholder([I])
+    with pytest.raises(ValueError):
+        ng.lookuptable(ng.placeholder([V]), idx, [I, F])
+    with pytest.raises(ValueError):
+        ng.lookuptable(lut, ng.placeholder([I, F]), [I, F])
+    with pytest.raises(ValueError):
+        ng.lookuptable(lut, idx, [F, I])           # would transpose the table implicitly
+    assert ng.lookuptable(lut, idx, [I, F]).lut_axis == 0
+
+
 def test_softmax_and_simple_prune(backend):
     C, N = ng.make_axis(10, name="C"), ng.make_axis(6, name="N")
     x = ng.placeholder([C, N])
