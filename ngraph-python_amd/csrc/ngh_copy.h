@@ -83,8 +83,95 @@ __global__ __launch_bounds__(kCopyBlock) void copy_tr_kernel(T* dst, const T* sr
     }
 }
 
+// Rows that are contiguous in both views: 16-byte accesses, one chunk per lane.
+template <typename T>
+__global__ __launch_bounds__(kCopyBlock) void copy_vec_kernel(T* dst, const T* src, const CopyArgs a,
+                                                              unsigned n_chunks, unsigned chunks_per_row) {
+    constexpr int V = 16 / (int)sizeof(T);
+    const unsigned step = gridDim.x * kCopyBlock;
+    for (unsigned q = blockIdx.x * kCopyBlock + threadIdx.x; q < n_chunks; q += step) {
+        unsigned rem = q / chunks_per_row;
+        const unsigned c = q - rem * chunks_per_row;
+        long long so = (long long)c * V, dof = (long long)c * V;
+        for (int ax = a.rank - 2; ax >= 0; --ax) {
+            const unsigned d = (unsigned)a.shape[ax];
+            const unsigned i = rem % d;
+            rem /= d;
+            so += (long long)i * a.ss[ax];
+            dof += (long long)i * a.ds[ax];
+        }
+        *reinterpret_cast<uint4*>(dst + dof) = *reinterpret_cast<const uint4*>(src + so);
+    }
+}
+
+// Transpose of 4-byte elements with 16-byte accesses on both sides: a lane reads four
+// consecutive source rows-elements (float4 along the source-contiguous axis), scatters them
+// into the padded tile, and after the barrier gathers four tile elements that are consecutive
+// along the destination-contiguous axis.  Needs R, C and the strides to be multiples of 4.
+__global__ __launch_bounds__(kCopyBlock) void copy_tr4_kernel(uint32_t* dst, const uint32_t* src, const CopyArgs a,
+                                                              unsigned tiles_r, unsigned tiles_c) {
+    __shared__ uint32_t tile[kCopyTile][kCopyTile + 1];     // [c_local][r_local]
+    const int r_ax = a.rank - 2, c_ax = a.rank - 1;
+    const unsigned R = (unsigned)a.shape[r_ax], C = (unsigned)a.shape[c_ax];
+    unsigned b = blockIdx.x;
+    const unsigned tc = b % tiles_c; b /= tiles_c;
+    const unsigned tr = b % tiles_r; b /= tiles_r;
+    long long so = 0, dof = 0;
+    for (int ax = r_ax - 1; ax >= 0; --ax) {
+        const unsigned d = (unsigned)a.shape[ax];
+        const unsigned i = b % d;
+        b /= d;
+        so += (long long)i * a.ss[ax];
+        dof += (long long)i * a.ds[ax];
+    }
+    const unsigned cx = threadIdx.x & 15, j = threadIdx.x >> 4;     // 16 chunks of 4 x 16 lines
+    uint4 v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const unsigned c = tc * kCopyTile + j + 16 * i, r = tr * kCopyTile + cx * 4;
+        v[i] = make_uint4(0, 0, 0, 0);
+        if (r < R && c < C) v[i] = *reinterpret_cast<const uint4*>(src + so + (long long)c * a.ss[c_ax] + r);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        uint32_t* row = tile[j + 16 * i] + cx * 4;
+        row[0] = v[i].x; row[1] = v[i].y; row[2] = v[i].z; row[3] = v[i].w;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const unsigned rl = j + 16 * i;
+        const unsigned r = tr * kCopyTile + rl, c = tc * kCopyTile + cx * 4;
+        if (r < R && c < C) {
+            const uint4 w = make_uint4(tile[cx * 4][rl], tile[cx * 4 + 1][rl], tile[cx * 4 + 2][rl], tile[cx * 4 + 3][rl]);
+            *reinterpret_cast<uint4*>(dst + dof + (long long)r * a.ds[r_ax] + c) = w;
+        }
+    }
+}
+
+inline bool copy_aligned(const void* dst, const void* src, const CopyArgs& a, int skip0, int skip1, int V) {
+    if (((uintptr_t)dst | (uintptr_t)src) & 15) return false;
+    for (int ax = 0; ax < a.rank; ++ax) {
+        if (ax == skip0 || ax == skip1) continue;
+        if (a.ss[ax] % V || a.ds[ax] % V) return false;
+    }
+    return true;
+}
+
 template <typename T>
 inline hipError_t launch_copy_t(hipStream_t stream, int cus, void* dst, const void* src, const CopyArgs& a) {
+    constexpr int V = 16 / (int)sizeof(T);
+    const int last = a.rank - 1;
+    if (a.rank >= 1 && a.ss[last] == 1 && a.ds[last] == 1 && a.shape[last] % V == 0 &&
+        copy_aligned(dst, src, a, last, -1, V)) {
+        const unsigned cpr = (unsigned)(a.shape[last] / V);
+        const unsigned n_chunks = a.total / V;
+        unsigned blocks = (n_chunks + kCopyBlock - 1) / kCopyBlock;
+        blocks = blocks < (unsigned)(cus * 64) ? blocks : (unsigned)(cus * 64);
+        hipLaunchKernelGGL(copy_vec_kernel<T>, dim3(blocks), dim3(kCopyBlock), 0, stream, (T*)dst, (const T*)src, a,
+                           n_chunks, cpr);
+        return hipGetLastError();
+    }
     if (a.rank >= 2 && a.ss[a.rank - 2] == 1 && a.ds[a.rank - 1] == 1 && a.ss[a.rank - 1] != 1 &&
         a.shape[a.rank - 2] >= 16 && a.shape[a.rank - 1] >= 16) {
         const unsigned tiles_r = (unsigned)((a.shape[a.rank - 2] + kCopyTile - 1) / kCopyTile);
@@ -92,6 +179,16 @@ inline hipError_t launch_copy_t(hipStream_t stream, int cus, void* dst, const vo
         unsigned long long blocks = (unsigned long long)tiles_r * tiles_c;
         for (int ax = 0; ax < a.rank - 2; ++ax) blocks *= (unsigned long long)a.shape[ax];
         if (blocks < (1ULL << 31)) {
+            if constexpr (sizeof(T) == 4) {
+                // 16-byte accesses: the source is read along r, the destination written along c
+                if (a.shape[a.rank - 2] % 4 == 0 && a.shape[a.rank - 1] % 4 == 0 &&
+                    a.ss[a.rank - 1] % 4 == 0 && a.ds[a.rank - 2] % 4 == 0 &&
+                    copy_aligned(dst, src, a, a.rank - 2, a.rank - 1, 4)) {
+                    hipLaunchKernelGGL(copy_tr4_kernel, dim3((unsigned)blocks), dim3(kCopyBlock), 0, stream,
+                                       (uint32_t*)dst, (const uint32_t*)src, a, tiles_r, tiles_c);
+                    return hipGetLastError();
+                }
+            }
             hipLaunchKernelGGL(copy_tr_kernel<T>, dim3((unsigned)blocks), dim3(kCopyBlock), 0, stream, (T*)dst,
                                (const T*)src, a, tiles_r, tiles_c);
             return hipGetLastError();

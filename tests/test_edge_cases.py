@@ -134,7 +134,8 @@ def test_misaligned_and_broadcast_operands(hip_runtime):
 
 
 @gpu
-@pytest.mark.parametrize("shape", [(5, 7, 11), (64, 64), (128, 70), (3, 130, 66), (2, 3, 4, 5)])
+@pytest.mark.parametrize("shape", [(5, 7, 11), (64, 64), (128, 70), (3, 130, 66), (2, 3, 4, 5), (256, 192),
+                                   (4, 96, 200), (8, 1024)])
 @pytest.mark.parametrize("itemsize", [4, 2])
 def test_strided_copy_all_permutations(hip_runtime, shape, itemsize):
     """Dimshuffle: every axis permutation against numpy.transpose (tensor_ops.py:137-204)."""
@@ -152,6 +153,28 @@ def test_strided_copy_all_permutations(hip_runtime, shape, itemsize):
         np.testing.assert_array_equal(d_d.get(), want)
         d_d.free()
     s_d.free()
+
+
+@gpu
+@pytest.mark.parametrize("offset", [0, 4, 3])
+def test_strided_copy_of_row_slices(hip_runtime, offset):
+    """Rows contiguous in both views (the 16-byte path when aligned, element-wise otherwise):
+    a column window of a wider matrix, at aligned and unaligned starting columns."""
+    rt = hip_runtime
+    base = np.arange(70 * 200, dtype=np.float32).reshape(70, 200)
+    s_d = rt.array(base)
+    want = np.ascontiguousarray(base[5:65, offset:offset + 128])
+    d_d = rt.empty(want.shape)
+    rt.copy_strided(d_d.ptr, s_d.ptr + (5 * 200 + offset) * 4, want.shape, [128, 1], [200, 1], 4)
+    np.testing.assert_array_equal(d_d.get(), want)
+    # and scattered back into a wider destination
+    w_d = rt.array(np.zeros((60, 200), np.float32))
+    rt.copy_strided(w_d.ptr + offset * 4, d_d.ptr, want.shape, [200, 1], [128, 1], 4)
+    back = w_d.get()
+    np.testing.assert_array_equal(back[:, offset:offset + 128], want)
+    assert not back[:, :offset].any() and not back[:, offset + 128:].any()
+    for d in (s_d, d_d, w_d):
+        d.free()
 
 
 @gpu
