@@ -58,11 +58,32 @@ def pattern_flex_relu(t):
     return t.computation(neon.rectlin(x * w + b), x, w, b)
 
 
+def _reduction_pattern(fn, out_axis):
+    def build(t):
+        A, B = _axes(A=4096, B=4096)
+        x = ng.placeholder([A, B])
+        return t.computation(fn(x, out_axes=[A if out_axis == 0 else B]), x)
+    return build
+
+
+def pattern_lstm_bias_gradient(t):
+    # db = sum over N of gates [4H, N] stored transposed (frontends/neon/layer.py:1630-1647)
+    N, G = _axes(N=64, G=4096)
+    gates_st = ng.placeholder([N, G])
+    gates = ng.axes_with_order(gates_st, [G, N])
+    return t.computation(ng.sum(gates, out_axes=[G]), gates_st)
+
+
 PATTERNS = [
     ("c1_tanh_sigmoid", "hipgpu", pattern_c1),
     ("adam", "hipgpu", pattern_adam),
     ("batchnorm", "hipgpu", pattern_batchnorm),
     ("flex_relu_fma", "flexhip", pattern_flex_relu),
+    ("sum_along", "hipgpu", _reduction_pattern(ng.sum, 0)),
+    ("sum_across", "hipgpu", _reduction_pattern(ng.sum, 1)),
+    ("max_along", "hipgpu", _reduction_pattern(ng.max, 0)),
+    ("max_across", "hipgpu", _reduction_pattern(ng.max, 1)),
+    ("sum_across_small", "hipgpu", pattern_lstm_bias_gradient),
 ]
 
 
@@ -82,13 +103,19 @@ def collect():
                 for stage in range(spec.n_stages):
                     plan = hiplib.plan_fused(spec, stage)
                     st = spec.stages[stage]
-                    if plan["family"] != 0 or plan["V"] < 4 or st.n_reductions:
+                    family = plan["family"]
+                    if family > 2 or (family == 0 and (plan["V"] < 4 or st.n_reductions)):
                         continue
+                    if family == 1 and spec.shape[0] // plan["V"] <= 64:
+                        continue          # short rows run the several-rows-per-workgroup kernel
                     total = spec.shape[0] * spec.shape[1] * spec.shape[2]
                     if total < 4096:
                         continue          # tiny stages are launch-bound; the interpreter is fine
+                    if any(o.opcode >= hiplib.OPCODES["take"] for o in spec.ops[st.op_begin:st.op_end]):
+                        continue          # lookups only run in the interpreter
                     ops = [(o.opcode, o.dst, o.a, o.b) for o in spec.ops[st.op_begin:st.op_end]]
                     fast = plan["perm"][2]
+                    red_out = [st.red_out[r] for r in range(st.n_reductions)]
                     dtypes = [spec.tensors[i].dtype for i in range(spec.n_tensors)]
                     bcast = [1 if spec.tensors[i].strides[fast] == 0 else 0 for i in range(spec.n_tensors)]
                     stored = set(o[1] for o in ops if o[0] == hiplib.OPCODES["store"])
@@ -99,12 +126,12 @@ def collect():
                             n_slots += 1
                         else:
                             stat_slot.append(-1)
-                    key = (tuple(ops), tuple(dtypes), tuple(bcast), plan["V"])
+                    key = (tuple(ops), tuple(dtypes), tuple(bcast), plan["V"], family, tuple(red_out))
                     if key in seen:
                         continue
                     seen.add(key)
                     programs.append(("%s_k%d" % (name, k_index), ops, dtypes, bcast, stat_slot,
-                                     n_slots, spec.n_regs, plan["V"]))
+                                     n_slots, spec.n_regs, plan["V"], family, red_out))
             k_index += 1
         t.close()
     return programs
@@ -113,10 +140,13 @@ def collect():
 def render(programs):
     lines = ["// GENERATED by gen_programs.py from the host lowering -- do not edit.",
              "// One entry per streaming elementwise op program that gets a pre-built kernel."]
-    for i, (name, ops, dtypes, bcast, stat_slot, n_slots, n_regs, V) in enumerate(programs):
+    for i, (name, ops, dtypes, bcast, stat_slot, n_slots, n_regs, V, family, red_out) in enumerate(programs):
         lines.append("struct SP%d {  // %s" % (i, name))
         lines.append("    static constexpr int V = %d, n_ops = %d, n_regs = %d, n_tensors = %d, "
-                     "n_stat_slots = %d;" % (V, len(ops), max(n_regs, 1), len(dtypes), n_slots))
+                     "n_stat_slots = %d, family = %d, n_red = %d;"
+                     % (V, len(ops), max(n_regs, 1), len(dtypes), n_slots, family, len(red_out)))
+        lines.append("    static constexpr int red_out[%d] = {%s};"
+                     % (max(len(red_out), 1), ", ".join(map(str, red_out or [0]))))
         lines.append("    static constexpr ngh_op ops[%d] = {%s};"
                      % (len(ops), ", ".join("{%d,%d,%d,%d}" % o for o in ops)))
         lines.append("    static constexpr int dtypes[%d] = {%s};" % (len(dtypes), ", ".join(map(str, dtypes))))
@@ -125,10 +155,11 @@ def render(programs):
         lines.append("};")
     lines.append("static const StaticEntry kStaticTable[] = {")
     for i, p in enumerate(programs):
-        lines.append('    {"%s", SP%d::V, SP%d::n_ops, SP%d::ops, SP%d::n_tensors, SP%d::dtypes, SP%d::bcast, '
-                     '&launch_static<SP%d>},' % (p[0], i, i, i, i, i, i, i))
+        launch = ("&launch_static<SP%d>, nullptr" % i) if p[8] == 0 else ("nullptr, &launch_static_red<SP%d>" % i)
+        lines.append('    {"%s", SP%d::family, SP%d::V, SP%d::n_ops, SP%d::ops, SP%d::n_tensors, SP%d::dtypes, '
+                     'SP%d::bcast, SP%d::n_red, SP%d::red_out, %s},' % (p[0], i, i, i, i, i, i, i, i, i, launch))
     if not programs:
-        lines.append('    {"none", 4, 0, nullptr, 0, nullptr, nullptr, nullptr},')
+        lines.append('    {"none", 0, 4, 0, nullptr, 0, nullptr, nullptr, 0, nullptr, nullptr, nullptr},')
     lines.append("};")
     lines.append("static const int kStaticCount = %d;" % len(programs))
     return "\n".join(lines) + "\n"

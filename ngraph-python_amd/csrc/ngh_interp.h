@@ -19,8 +19,14 @@ constexpr int kWaves = kBlock / 64;
 // Extra LDS rows behind the register file: per-thread max|mantissa| of each
 // statistics slot, then (value, index) of each reduction slot.
 __device__ __forceinline__ int ex_stat(int slot) { return slot; }
-__device__ __forceinline__ int ex_accv(const KArgs& k, int slot) { return k.n_stat_slots + 2 * slot; }
-__device__ __forceinline__ int ex_acci(const KArgs& k, int slot) { return k.n_stat_slots + 2 * slot + 1; }
+// A reduction slot owns `na` accumulators per thread: one when the lane's V elements belong
+// to the same output (reduction along the vector axis), V when each is an output of its own.
+__device__ __forceinline__ int ex_accv(const KArgs& k, int slot, int na = 1, int v = 0) {
+    return k.n_stat_slots + 2 * (slot * na + v);
+}
+__device__ __forceinline__ int ex_acci(const KArgs& k, int slot, int na = 1, int v = 0) {
+    return k.n_stat_slots + 2 * (slot * na + v) + 1;
+}
 
 struct Extra {
     float* base;  // &extra[thread]
@@ -207,19 +213,34 @@ __device__ __forceinline__ void run_ops(const KArgs& k, LdsRegs<V>& rf, Extra& e
 #undef NGH_BIN
             case NGH_OP_RED_SUM: case NGH_OP_RED_PROD: case NGH_OP_RED_MAX:
             case NGH_OP_RED_MIN: case NGH_OP_RED_ARGMAX: case NGH_OP_RED_ARGMIN: {
-                if (RMODE != 0) {
+                // the index half of an accumulator only matters to argmax / argmin
+                const bool with_index = opc >= NGH_OP_RED_ARGMAX;
+                if constexpr (RMODE == 1) {
                     Acc a;
                     a.v = ex.getf(ex_accv(k, o.dst));
-                    a.i = ex.geti(ex_acci(k, o.dst));
+                    a.i = with_index ? ex.geti(ex_acci(k, o.dst)) : 0;
 #pragma unroll
                     for (int v = 0; v < V; ++v) {
                         Acc b;
                         b.v = rf.get(o.a, v);
                         b.i = at.red_index(RMODE, v);
-                        a = acc_merge(opc, a, b);
+                        if (at.valid(v)) a = acc_merge(opc, a, b);
                     }
                     ex.setf(ex_accv(k, o.dst), a.v);
-                    ex.seti(ex_acci(k, o.dst), a.i);
+                    if (with_index) ex.seti(ex_acci(k, o.dst), a.i);
+                } else if constexpr (RMODE == 2) {
+                    // the lane's V elements are V different outputs
+#pragma unroll
+                    for (int v = 0; v < V; ++v) {
+                        Acc a, b;
+                        a.v = ex.getf(ex_accv(k, o.dst, V, v));
+                        a.i = with_index ? ex.geti(ex_acci(k, o.dst, V, v)) : 0;
+                        b.v = rf.get(o.a, v);
+                        b.i = at.red_index(RMODE, v);
+                        a = acc_merge(opc, a, b);
+                        ex.setf(ex_accv(k, o.dst, V, v), a.v);
+                        if (with_index) ex.seti(ex_acci(k, o.dst, V, v), a.i);
+                    }
                 }
             } break;
             default: break;
@@ -462,65 +483,109 @@ __global__ __launch_bounds__(kBlock) void red_row_interp_kernel(const KArgs k, u
 }
 
 // ---------------------------------------------------------------------------
-// Reduction along kernel axis 0 with outputs contiguous along kernel axis 2:
-// workgroup = 64 consecutive outputs x 4 interleaved rows of the reduced
-// axis; lanes stay coalesced along axis 2 while each walks down axis 0.
+// Reduction along kernel axis 0 with outputs contiguous along kernel axis 2.
+// Lanes run along axis 2 (V consecutive outputs each) so loads stay
+// coalesced while every lane walks down axis 0.  A wavefront spans TX column
+// chunks x 64/TX rows: with few outputs (TX < 64) the spare lanes take more
+// rows instead of idling, and a butterfly over the row lanes folds them.
+// The four wavefronts then meet in LDS.
 // ---------------------------------------------------------------------------
-constexpr int kColTx = 64, kColTy = kBlock / kColTx;
-
-__global__ __launch_bounds__(kBlock) void red_col_interp_kernel(const KArgs k, unsigned n_bx,
-                                                                unsigned n_seg, unsigned seg_rows,
-                                                                RedWs ws) {
+template <int V>
+__global__ __launch_bounds__(kBlock) void red_col_interp_kernel(const KArgs k, unsigned n_bx, unsigned n_seg,
+                                                                unsigned seg_rows, unsigned TX, RedWs ws) {
     extern __shared__ float lds[];
-    __shared__ Acc sh[NGH_MAX_REDUCTIONS][kColTy][kColTx];
-    LdsRegs<1> rf{lds + threadIdx.x, kBlock};
-    Extra ex{lds + (size_t)k.n_regs * kBlock + threadIdx.x, kBlock};
+    __shared__ Acc sh[kWaves][64][V];
+    LdsRegs<V> rf{lds + threadIdx.x, kBlock};
+    Extra ex{lds + (size_t)k.n_regs * V * kBlock + threadIdx.x, kBlock};
     for (int s = 0; s < k.n_stat_slots; ++s) ex.seti(ex_stat(s), 0);
     for (int s = 0; s < k.n_red; ++s) {
-        Acc a = acc_init(red_opcode(k, s));
-        ex.setf(ex_accv(k, s), a.v);
-        ex.seti(ex_acci(k, s), a.i);
+        const Acc a = acc_init(red_opcode(k, s));
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            ex.setf(ex_accv(k, s, V, v), a.v);
+            ex.seti(ex_acci(k, s, V, v), a.i);
+        }
     }
-    const unsigned tx = threadIdx.x & (kColTx - 1), ty = threadIdx.x / kColTx;
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned tx = lane & (TX - 1), ry = lane / TX, rows_per_wave = 64 / TX;
     unsigned b = blockIdx.x;
     const unsigned seg = b % n_seg;  b /= n_seg;
     const unsigned bx = b % n_bx;    b /= n_bx;
     const unsigned i1 = b;
     const unsigned d2 = (unsigned)k.shape[2];
-    const unsigned i2 = bx * kColTx + tx;
+    const unsigned i2 = (bx * TX + tx) * V;
     const unsigned r_begin = seg * seg_rows;
     const unsigned r_end = min((unsigned)k.shape[0], r_begin + seg_rows);
     if (i2 < d2)
-        for (unsigned r = r_begin + ty; r < r_end; r += kColTy) run_ops<1, 2>(k, rf, ex, VecAt<1>{r, i1, i2});
+        for (unsigned r = r_begin + wave * rows_per_wave + ry; r < r_end; r += kWaves * rows_per_wave)
+            run_ops<V, 2>(k, rf, ex, VecAt<V>{r, i1, i2});
 
+    const unsigned n_out = (unsigned)k.shape[1] * d2;
     for (int s = 0; s < k.n_red; ++s) {
-        Acc a;
-        a.v = ex.getf(ex_accv(k, s));
-        a.i = ex.geti(ex_acci(k, s));
-        sh[s][ty][tx] = a;
-    }
-    __syncthreads();
-    if (ty == 0 && i2 < d2) {
-        const unsigned n_out = (unsigned)k.shape[1] * d2;
-        const unsigned out = i1 * d2 + i2;
-        for (int s = 0; s < k.n_red; ++s) {
-            const int opc = red_opcode(k, s);
-            Acc a = sh[s][0][tx];
-            for (int y = 1; y < kColTy; ++y) a = acc_merge(opc, a, sh[s][y][tx]);
-            red_emit(k, s, a, 0, i1, i2, out, n_out, seg, n_seg, ws);
+        const int opc = red_opcode(k, s);
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            Acc a;
+            a.v = ex.getf(ex_accv(k, s, V, v));
+            a.i = ex.geti(ex_acci(k, s, V, v));
+            for (unsigned m = 32; m >= TX; m >>= 1) a = acc_merge(opc, a, acc_shfl_xor(a, (int)m));
+            if (lane < TX) sh[wave][lane][v] = a;
         }
+        __syncthreads();
+        if (wave == 0 && lane < TX && i2 < d2) {
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                Acc a = sh[0][lane][v];
+                for (int w = 1; w < kWaves; ++w) a = acc_merge(opc, a, sh[w][lane][v]);
+                red_emit(k, s, a, 0, i1, i2 + v, i1 * d2 + i2 + v, n_out, seg, n_seg, ws);
+            }
+        }
+        __syncthreads();
     }
     stats_epilogue(k, ex);
 }
 
-// Second pass of a split reduction: one thread per output merges the
-// segments in order and stores through the output's storage type.
-// `row_mode` tells how an output number maps to kernel coordinates.
-__global__ __launch_bounds__(kBlock) void red_finish_kernel(const KArgs k, unsigned n_out,
-                                                            unsigned n_seg, int row_mode, RedWs ws) {
-    const unsigned out = blockIdx.x * kBlock + threadIdx.x;
-    if (out >= n_out) return;
-    long long o0, o1, o2;
+// ---------------------------------------------------------------------------
+// Reduction along kernel axis 2 for short rows (at most 64 chunks of V): a row
+// takes TR lanes (a power of two), a workgroup 256 / TR rows, and a butterfly
+// inside the TR lanes finishes the row -- no LDS, no idle wavefronts where
+// one workgroup per row would leave most of its 256 threads without work.
+// ---------------------------------------------------------------------------
+template <int V>
+__global__ __launch_bounds__(kBlock) void red_rows_small_interp_kernel(const KArgs k, unsigned n_out, unsigned TR) {
+    extern __shared__ float lds[];
+    LdsRegs<V> rf{lds + threadIdx.x, kBlock};
+    Extra ex{lds + (size_t)k.n_regs * V * kBlock + threadIdx.x, kBlock};
+    for (int s = 0; s < k.n_stat_slots; ++s) ex.seti(ex_stat(s), 0);
+    for (int s = 0; s < k.n_red; ++s) {
+        const Acc a = acc_init(red_opcode(k, s));
+        ex.setf(ex_accv(k, s), a.v);
+        ex.seti(ex_acci(k, s), a.i);
+    }
+    const unsigned pos = threadIdx.x & (TR - 1);
+    const unsigned out = blockIdx.x * (kBlock / TR) + threadIdx.x / TR;
+    const unsigned d1 = (unsigned)k.shape[1];
+    const unsigned i0 = out / d1, i1 = out - i0 * d1;
+    const unsigned chunks = (unsigned)(k.shape[2] / V);
+    if (out < n_out && pos < chunks) run_ops<V, 1>(k, rf, ex, VecAt<V>{i0, i1, (long long)pos * V});
+    RedWs none{nullptr, nullptr};
+    for (int s = 0; s < k.n_red; ++s) {
+        const int opc = red_opcode(k, s);
+        Acc a;
+        a.v = ex.getf(ex_accv(k, s));
+        a.i = ex.geti(ex_acci(k, s));
+        for (unsigned m = TR >> 1; m > 0; m >>= 1) a = acc_merge(opc, a, acc_shfl_xor(a, (int)m));
+        if (pos == 0 && out < n_out) red_emit(k, s, a, i0, i1, 0, out, n_out, 0, 1, none);
+    }
+    stats_epilogue(k, ex);
+}
+
+// Second pass of a split reduction: merges an output's segments (in a fixed order) and
+// stores through the output's storage type.  `row_mode` tells how an output number maps to
+// kernel coordinates.  With few segments a thread takes an output; with many, a wavefront
+// does: lanes stride over the segments and a butterfly folds them.
+__device__ __forceinline__ void red_finish_coords(const KArgs& k, unsigned out, int row_mode, long long& o0,
+                                                  long long& o1, long long& o2) {
     if (row_mode) {
         const unsigned d1 = (unsigned)k.shape[1];
         o0 = out / d1; o1 = out - (unsigned)o0 * d1; o2 = 0;
@@ -528,6 +593,14 @@ __global__ __launch_bounds__(kBlock) void red_finish_kernel(const KArgs k, unsig
         const unsigned d2 = (unsigned)k.shape[2];
         o0 = 0; o1 = out / d2; o2 = out - (unsigned)o1 * d2;
     }
+}
+
+__global__ __launch_bounds__(kBlock) void red_finish_kernel(const KArgs k, unsigned n_out,
+                                                            unsigned n_seg, int row_mode, RedWs ws) {
+    const unsigned out = blockIdx.x * kBlock + threadIdx.x;
+    if (out >= n_out) return;
+    long long o0, o1, o2;
+    red_finish_coords(k, out, row_mode, o0, o1, o2);
     for (int s = 0; s < k.n_red; ++s) {
         const int opc = red_opcode(k, s);
         Acc a = acc_init(opc);
@@ -538,6 +611,30 @@ __global__ __launch_bounds__(kBlock) void red_finish_kernel(const KArgs k, unsig
         }
         RedWs none{nullptr, nullptr};
         red_emit(k, s, a, o0, o1, o2, out, n_out, 0, 1, none);
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void red_finish_wave_kernel(const KArgs k, unsigned n_out,
+                                                                 unsigned n_seg, int row_mode, RedWs ws) {
+    const unsigned lane = threadIdx.x & 63;
+    const unsigned out = blockIdx.x * kWaves + (threadIdx.x >> 6);
+    if (out >= n_out) return;
+    long long o0, o1, o2;
+    red_finish_coords(k, out, row_mode, o0, o1, o2);
+    for (int s = 0; s < k.n_red; ++s) {
+        const int opc = red_opcode(k, s);
+        Acc a = acc_init(opc);
+        for (unsigned g = lane; g < n_seg; g += 64) {
+            const size_t w = ((size_t)s * n_seg + g) * n_out + out;
+            Acc b; b.v = ws.val[w]; b.i = ws.idx[w];
+            a = acc_merge(opc, a, b);
+        }
+#pragma unroll
+        for (int m = 32; m > 0; m >>= 1) a = acc_merge(opc, a, acc_shfl_xor(a, m));
+        if (lane == 0) {
+            RedWs none{nullptr, nullptr};
+            red_emit(k, s, a, o0, o1, o2, out, n_out, 0, 1, none);
+        }
     }
 }
 

@@ -78,6 +78,7 @@ struct ngh_context {
     unsigned    stat_ws_blocks = 0;  // capacity per statistics slot
     int         ew_blocks_per_cu = 64;
     int         force_interp = 0;    // never pick a specialised kernel
+    int         red_wgs_per_cu = 8;  // workgroups per CU a split reduction aims for
     int         no_tiles = 0;        // never use the LDS-tiled elementwise skeleton
     int         flex_self_managed = 1;  // ngh_launch_fused_flex may fold the policy into the kernel
     int         cache_policy = -1;   // -1: from the operands' cache hints; 0..3 forces bit 0 = non-temporal
@@ -203,8 +204,12 @@ struct Plan {
     int      special = -1;                        // index into the specialised-kernel table
     long long tail = 0;                           // 1-D contiguous stage: elements left to a scalar launch
     int      perm[3] = {0, 1, 2};                 // kernel axis j holds spec axis perm[j]
+    unsigned tx = 64;                                 // column reduction: column chunks per wavefront;
+                                                      // short-row reduction: lanes per row
+    bool     small_rows = false;                      // row reduction with several rows per workgroup
     unsigned tiles_a = 0, tiles_b = 0, n_tiles = 0;   // tiled elementwise
     int      tile = kTile;
+    int      cache_policy = 0;
     unsigned load_mask = 0, store_mask = 0;           // tensors the stage loads / stores
 };
 
@@ -281,8 +286,9 @@ constexpr size_t kInterpLdsPreferred = 64 * 1024;   // keeps >= 2 workgroups per
 constexpr size_t kInterpLdsMax = 128 * 1024;
 constexpr size_t kInterpLdsWide = 40 * 1024;        // budget when widening the interpreter's vectors
 
-size_t interp_lds_bytes(const KArgs& k, int V) {
-    return ((size_t)k.n_regs * V + k.n_stat_slots + 2 * k.n_red) * kBlock * sizeof(float);
+// registers (V elements each) + statistics slots + reduction accumulators (`na` per slot)
+size_t interp_lds_bytes(const KArgs& k, int V, int na = 1) {
+    return ((size_t)k.n_regs * V + k.n_stat_slots + 2 * k.n_red * na) * kBlock * sizeof(float);
 }
 
 size_t tiled_lds_bytes(const KArgs& k, int tile) {
@@ -438,20 +444,29 @@ int plan_stage(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan
     }
     const long long n_out = sp.shape[1] * sp.shape[2];
     if (n_out >= (1LL << 31) || R >= (1LL << 31)) return fail(NGH_E_UNSUPPORTED, "reduction extents exceed 2^31");
-    const int target_wgs = (ctx ? ctx->cus : 256) * 8;
+    const int target_wgs = (ctx ? ctx->cus * ctx->red_wgs_per_cu : 256 * 8);
     if (out_contig_axis >= 0) {
         const int other = (out_contig_axis == 2) ? 1 : 2;
         const int perm[3] = {0, other, out_contig_axis};
         fill_kargs(sp, S, perm, P.k);
         for (int a = 0; a < 3; ++a) P.perm[a] = perm[a];
         P.family = F_RED_COL;
-        P.V = 1;
+        // 4 consecutive outputs per lane when every operand read allows 16-byte access
+        P.V = (vec_ok(P.k, used, 4, true) && interp_lds_bytes(P.k, 4, 4) <= kInterpLdsPreferred) ? 4 : 1;
+        // ... unless that leaves most of the chip without a workgroup
+        if (P.V == 4 && ((P.k.shape[2] / 4 + 63) / 64) * P.k.shape[1] * std::max<long long>(1, R / 256) <
+                            (ctx ? ctx->cus : 256))
+            P.V = 1;
         P.n_out = (unsigned)n_out;
-        P.n_bx = (unsigned)((P.k.shape[2] + kColTx - 1) / kColTx);
+        const long long col_chunks = (P.k.shape[2] + P.V - 1) / P.V;
+        P.tx = 1;
+        while (P.tx < 64 && (long long)P.tx < col_chunks) P.tx <<= 1;
+        P.n_bx = (unsigned)((col_chunks + P.tx - 1) / P.tx);
+        const long long rows_per_pass = (long long)kWaves * (64 / P.tx);
         const long long base_wgs = (long long)P.n_bx * P.k.shape[1];
         long long seg = std::max<long long>(1, target_wgs / std::max<long long>(1, base_wgs));
-        seg = std::min<long long>(seg, std::max<long long>(1, R / 64));
-        seg = std::min<long long>(seg, 1024);
+        seg = std::min<long long>(seg, std::max<long long>(1, R / (rows_per_pass * 8)));
+        seg = std::min<long long>(seg, 4096);
         P.seg_len = (unsigned)((R + seg - 1) / seg);
         P.n_seg = (unsigned)((R + P.seg_len - 1) / std::max(1u, P.seg_len));
         if (P.n_seg == 0) P.n_seg = 1;
@@ -463,6 +478,15 @@ int plan_stage(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan
         P.V = (r_contig && vec4_ok(P.k, used)) ? 4 : 1;
         P.n_out = (unsigned)n_out;
         const long long chunks = R / P.V;
+        if (chunks <= 64) {
+            // short rows: TR lanes per row, several rows per workgroup, no segments
+            P.small_rows = true;
+            P.tx = 1;
+            while ((long long)P.tx < chunks) P.tx <<= 1;
+            P.n_seg = 1;
+            P.seg_len = (unsigned)chunks;
+            return NGH_OK;
+        }
         long long seg = std::max<long long>(1, target_wgs / std::max<long long>(1, n_out));
         seg = std::min<long long>(seg, std::max<long long>(1, chunks / (kBlock * 4)));
         seg = std::min<long long>(seg, 1024);
@@ -618,8 +642,24 @@ int launch_interp(ngh_context* ctx, Plan& P) {
         ws.val = (float*)ctx->ws;
         ws.idx = (int*)ctx->ws + n;
     }
-    if (P.family == F_RED_ROW) {
-        const unsigned blocks = P.n_out * P.n_seg;
+    unsigned red_blocks = 0;
+    if (P.special >= 0 && !k.probe) {
+        // a pre-built reduction: same grid and workspace as the interpreter's kernel
+        red_blocks = P.family == F_RED_ROW ? P.n_out * P.n_seg
+                                            : (unsigned)((unsigned long long)P.n_bx * (unsigned)k.shape[1] * P.n_seg);
+        NGH_TRY(stat_scratch(ctx, k, red_blocks));
+        HIP_TRY(launch_special_red(P.special, ctx->stream, red_blocks, k, P.family == F_RED_ROW ? P.n_out : P.n_bx,
+                                   P.n_seg, P.seg_len, P.tx, ws, P.cache_policy));
+    } else if (P.family == F_RED_ROW && P.small_rows) {
+        const unsigned rows_per_wg = kBlock / P.tx;
+        red_blocks = (P.n_out + rows_per_wg - 1) / rows_per_wg;
+        NGH_TRY(stat_scratch(ctx, k, red_blocks));
+        if (V == 4)
+            hipLaunchKernelGGL(red_rows_small_interp_kernel<4>, dim3(red_blocks), dim3(kBlock), lds, ctx->stream, k, P.n_out, P.tx);
+        else
+            hipLaunchKernelGGL(red_rows_small_interp_kernel<1>, dim3(red_blocks), dim3(kBlock), lds, ctx->stream, k, P.n_out, P.tx);
+    } else if (P.family == F_RED_ROW) {
+        const unsigned blocks = red_blocks = P.n_out * P.n_seg;
         NGH_TRY(stat_scratch(ctx, k, blocks));
         if (V == 4)
             hipLaunchKernelGGL(red_row_interp_kernel<4>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, P.n_out, P.n_seg, P.seg_len, ws);
@@ -628,17 +668,22 @@ int launch_interp(ngh_context* ctx, Plan& P) {
     } else {
         const unsigned long long blocks = (unsigned long long)P.n_bx * (unsigned)k.shape[1] * P.n_seg;
         if (blocks >= (1ULL << 31)) return fail(NGH_E_UNSUPPORTED, "reduction grid too large");
-        NGH_TRY(stat_scratch(ctx, k, (unsigned)blocks));
-        hipLaunchKernelGGL(red_col_interp_kernel, dim3((unsigned)blocks), dim3(kBlock), lds, ctx->stream, k, P.n_bx, P.n_seg, P.seg_len, ws);
+        red_blocks = (unsigned)blocks;
+        NGH_TRY(stat_scratch(ctx, k, red_blocks));
+        if (V == 4)
+            hipLaunchKernelGGL(red_col_interp_kernel<4>, dim3(red_blocks), dim3(kBlock), interp_lds_bytes(k, 4, 4), ctx->stream, k, P.n_bx, P.n_seg, P.seg_len, P.tx, ws);
+        else
+            hipLaunchKernelGGL(red_col_interp_kernel<1>, dim3(red_blocks), dim3(kBlock), lds, ctx->stream, k, P.n_bx, P.n_seg, P.seg_len, P.tx, ws);
     }
     HIP_TRY(hipGetLastError());
-    if (k.n_stat_slots)
-        NGH_TRY(stat_fold(ctx, k, P.family == F_RED_ROW ? P.n_out * P.n_seg
-                                                        : (unsigned)(P.n_bx * (unsigned)k.shape[1] * P.n_seg)));
+    if (k.n_stat_slots) NGH_TRY(stat_fold(ctx, k, red_blocks));
     if (P.n_seg > 1) {
-        const unsigned blocks = (P.n_out + kBlock - 1) / kBlock;
-        hipLaunchKernelGGL(red_finish_kernel, dim3(blocks), dim3(kBlock), 0, ctx->stream, k, P.n_out, P.n_seg,
-                           P.family == F_RED_ROW ? 1 : 0, ws);
+        if (P.n_seg >= 32)
+            hipLaunchKernelGGL(red_finish_wave_kernel, dim3((P.n_out + kWaves - 1) / kWaves), dim3(kBlock), 0, ctx->stream,
+                               k, P.n_out, P.n_seg, P.family == F_RED_ROW ? 1 : 0, ws);
+        else
+            hipLaunchKernelGGL(red_finish_kernel, dim3((P.n_out + kBlock - 1) / kBlock), dim3(kBlock), 0, ctx->stream,
+                               k, P.n_out, P.n_seg, P.family == F_RED_ROW ? 1 : 0, ws);
         HIP_TRY(hipGetLastError());
     }
     return NGH_OK;
@@ -654,8 +699,11 @@ void describe(const Plan& P, char* out, size_t n) {
             if (P.Vi == 1) snprintf(out, n, "ew_gather_interp_g%d", gather_width(P.k));
             else snprintf(out, n, "ew_interp_v%d%s", P.Vi, P.tail ? "+tail" : "");
             break;
-        case F_RED_ROW: snprintf(out, n, "red_row_interp_v%d_s%u", P.V, P.n_seg); break;
-        case F_RED_COL: snprintf(out, n, "red_col_interp_v1_s%u", P.n_seg); break;
+        case F_RED_ROW:
+            if (P.small_rows) snprintf(out, n, "red_rows_small_interp_v%d_l%u", P.V, P.tx);
+            else snprintf(out, n, "red_row_interp_v%d_s%u", P.V, P.n_seg);
+            break;
+        case F_RED_COL: snprintf(out, n, "red_col_interp_v%d_t%u_s%u", P.V, P.tx, P.n_seg); break;
         case F_EW_TILED: snprintf(out, n, "ew_tiled_interp_t%d_s%d", P.tile, P.k.n_staged); break;
     }
 }
@@ -700,6 +748,7 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->force_interp = env_int("NGH_FORCE_INTERP", 0);
     ctx->flex_self_managed = env_int("NGH_FLEX_SELF_MANAGED", 1);
     ctx->no_tiles = env_int("NGH_NO_TILES", 0);
+    ctx->red_wgs_per_cu = std::max(1, env_int("NGH_RED_WGS_PER_CU", 8));
     ctx->cache_policy = env_int("NGH_CACHE_POLICY", -1);
     ctx->stream_bytes = (long long)env_int("NGH_STREAM_MIB", 128) << 20;
     ctx->moments_wgs_per_cu = std::max(1, env_int("NGH_MOMENTS_WGS_PER_CU", 16));
@@ -714,7 +763,9 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     const void* interp_kernels[] = {(const void*)ew_interp_kernel<8>, (const void*)ew_interp_kernel<4>,
                                     (const void*)ew_gather_interp_kernel<4>, (const void*)ew_gather_interp_kernel<1>,
                                     (const void*)red_row_interp_kernel<4>, (const void*)red_row_interp_kernel<1>,
-                                    (const void*)red_col_interp_kernel, (const void*)ew_tiled_interp_kernel<16>,
+                                    (const void*)red_col_interp_kernel<4>, (const void*)red_col_interp_kernel<1>,
+                                    (const void*)red_rows_small_interp_kernel<4>, (const void*)red_rows_small_interp_kernel<1>,
+                                    (const void*)ew_tiled_interp_kernel<16>,
                                     (const void*)ew_tiled_interp_kernel<32>};
     for (const void* fn : interp_kernels) {
         e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kInterpLdsMax);
@@ -889,7 +940,7 @@ int ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec) {
         if (spec->stages[s].op_end == spec->stages[s].op_begin) continue;
         Plan P;
         NGH_TRY(plan_stage(ctx, *spec, s, P));
-        if (!ctx->force_interp && !P.k.probe) {
+        if (!ctx->force_interp && !P.k.probe && P.family == F_EW) {
             P.special = match_special(P.family, P.V, P.k, P.tail);
             if (P.special >= 0) {
                 const unsigned blocks = streaming_blocks(ctx->cus, ctx->ew_blocks_per_cu, P.n_chunks);
@@ -902,6 +953,10 @@ int ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec) {
                 continue;
             }
         }
+        if (!ctx->force_interp && !P.k.probe && (P.family == F_RED_COL || (P.family == F_RED_ROW && !P.small_rows))) {
+            P.special = match_special(P.family, P.V, P.k, 0);
+            P.cache_policy = stage_cache_policy(ctx, *spec, spec->stages[s]);
+        }
         NGH_TRY(launch_interp(ctx, P));
     }
     return NGH_OK;
@@ -913,9 +968,10 @@ int ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec, int32_t sta
     if (stage < 0 || stage >= spec->n_stages) return fail(NGH_E_INVALID, "stage %d", stage);
     Plan P;
     NGH_TRY(plan_stage(ctx, *spec, stage, P));
-    if (!ctx->force_interp) P.special = match_special(P.family, P.V, P.k, P.tail);
+    if (!ctx->force_interp && !(P.family == F_RED_ROW && P.small_rows) && P.family != F_EW_TILED)
+        P.special = match_special(P.family, P.V, P.k, P.tail);
     describe(P, name128, 128);
-    if (P.special >= 0) {
+    if (P.special >= 0 && P.family == F_EW) {
         static const char* const suffix[4] = {"", "/nt-loads", "/nt-stores", "/nt-loads-stores"};
         const int cp = stage_cache_policy(ctx, *spec, spec->stages[stage]);
         strncat(name128, suffix[cp], 127 - strlen(name128));
