@@ -237,8 +237,9 @@ int  ngh_stats_read(ngh_context* ctx, const int32_t* dev, int32_t n, int32_t* ho
  * ngh_tensor.dev_stats = &state.stats; ngh_flex_prepare / ngh_flex_update run the
  * exponent policy on the device around a kernel, so no statistics travel to the host
  * between kernels (the reference reads them back after every kernel,
- * flexgputransform.py:361-366).  Policy: DESIGN.md section 5; the host mirror is
- * ngraph_hip/flex/hipflex.py.                                                      */
+ * flexgputransform.py:361-366).  Policy: an overflow (max|mantissa| >= 32767) lowers
+ * dec by 2; otherwise dec is the tightest fit of max(h) + 3 * stddev(h) over the last 16
+ * recorded maxima h.  The host mirror is ngraph_hip/flex/hipflex.py.                */
 #define NGH_FLEX_HISTORY 16
 typedef struct ngh_flex_state {
     int32_t stats;          /* max |mantissa| merged by kernels since ngh_flex_prepare   */

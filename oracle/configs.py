@@ -12,7 +12,7 @@ reference front end builds:
   C4  LSTM cell pointwise block         frontends/neon/layer.py:1630-1647 (gate order i,f,o,g :1615)
   C5  flex16 relu(x*w+b)                frontends/neon/activation.py:46; flex rules in flex_model.py
 
-Inputs are seeded as BASELINE.md lists them.  Temporaries are preallocated
+Inputs are seeded per configuration (seeds 0-4, NumPy RandomState).  Temporaries are preallocated
 (the CPU transformer runs out of two preallocated float32 pools,
 cputransform.py:998-1007), so timing one of these functions measures ufunc
 work only.

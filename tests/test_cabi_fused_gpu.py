@@ -3,7 +3,7 @@
 Each case builds an ngh_fused_spec the way the transformer's lowering does,
 launches it with ngh_launch_fused and compares with the CPU oracle
 (oracle/configs.py, oracle/numpy_ops.py) on the same seeded inputs.
-Tolerance: fp32 rtol 1e-5 / atol 1e-6 (the bar BASELINE.json states).
+Tolerance: fp32 rtol 1e-5 / atol 1e-6.
 """
 import numpy as np
 import pytest
