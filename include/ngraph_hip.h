@@ -94,6 +94,10 @@ enum ngh_opcode {
      * loop coordinate; the tensor's stride on that axis is the table's stride along its
      * looked-up axis and take_extent its length there (indices are clamped to it).       */
     NGH_OP_TAKE,
+    /* STORE whose conversion to a FLEX16 mantissa truncates toward zero instead of rounding
+     * to nearest: the fill of a flex tensor, int(value / scale) clipped
+     * (tensor_ops.py:690-707 FlexFillKernel).  Other storage types: same as STORE.        */
+    NGH_OP_STORE_TRUNC,
     NGH_OP_COUNT_
 };
 

@@ -155,6 +155,13 @@ __device__ __forceinline__ int flex_quantize(float v) {
     return (v != v) ? 0 : q;
 }
 
+// the fill rule: int(value / scale) cut toward zero, clipped (tensor_ops.py:690-707)
+__device__ __forceinline__ int flex_quantize_trunc(float v) {
+    v = truncf(v);
+    v = fminf(fmaxf(v, -32768.0f), 32767.0f);
+    return (v != v) ? 0 : (int)v;
+}
+
 __device__ __forceinline__ int iabs(int x) { return x < 0 ? -x : x; }
 
 // bit pattern of |v| (ordered like the value for non-negative floats); NaN counts as 0

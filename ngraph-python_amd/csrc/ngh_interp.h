@@ -165,6 +165,33 @@ __device__ __forceinline__ void run_ops(const KArgs& k, LdsRegs<V>& rf, Extra& e
                 }
                 if (t.stat_slot >= 0) ex.seti(ex_stat(t.stat_slot), max(ex.geti(ex_stat(t.stat_slot)), fmax));
             } break;
+            case NGH_OP_STORE_TRUNC: {
+                const KTensor& t = k.t[o.dst];
+                int fmax = 0;
+                if (t.dtype == NGH_FLEX16 && !k.probe) {
+                    const float sc = 1.0f / tensor_scale(t);
+#pragma unroll
+                    for (int v = 0; v < V; ++v)
+                        if (at.valid(v)) {
+                            const int q = flex_quantize_trunc(sc * rf.get(o.a, v));
+                            reinterpret_cast<short*>(t.p)[at.coord(0, v) * t.s[0] + at.coord(1, v) * t.s[1] +
+                                                          at.coord(2, v) * t.s[2]] = (short)q;
+                            fmax = max(fmax, iabs(q));
+                        }
+                } else {
+                    float x[V];
+#pragma unroll
+                    for (int v = 0; v < V; ++v) x[v] = rf.get(o.a, v);
+                    if (k.probe) {
+#pragma unroll
+                        for (int v = 0; v < V; ++v)
+                            if (at.valid(v)) fmax = max(fmax, probe_bits(x[v]));
+                    } else {
+                        at.store(t, x, fmax);
+                    }
+                }
+                if (t.stat_slot >= 0) ex.seti(ex_stat(t.stat_slot), max(ex.geti(ex_stat(t.stat_slot)), fmax));
+            } break;
             case NGH_OP_TAKE: {
                 // table lookup: the coordinate along one axis comes from a register
                 const KTensor& t = k.t[o.b & 15];

@@ -139,7 +139,7 @@ int validate(const ngh_fused_spec* sp) {
             if (opc == NGH_OP_LOAD) {
                 if (o.a >= sp->n_tensors || !reg_ok(o.dst)) return fail(NGH_E_INVALID, "op %d: bad LOAD", pc);
                 defined[o.dst] = true;
-            } else if (opc == NGH_OP_STORE) {
+            } else if (opc == NGH_OP_STORE || opc == NGH_OP_STORE_TRUNC) {
                 if (o.dst >= sp->n_tensors || !need(o.a)) return fail(NGH_E_INVALID, "op %d: bad STORE", pc);
                 const ngh_tensor& T = sp->tensors[o.dst];
                 for (int a = 0; a < NGH_MAX_AXES; ++a)
@@ -219,7 +219,7 @@ void stage_tensors(const ngh_fused_spec& sp, const ngh_stage& S, bool* loads, bo
     for (int pc = S.op_begin; pc < S.op_end; ++pc) {
         const ngh_op& o = sp.ops[pc];
         if (o.opcode == NGH_OP_LOAD) loads[o.a] = true;
-        if (o.opcode == NGH_OP_STORE) stores[o.dst] = true;
+        if (o.opcode == NGH_OP_STORE || o.opcode == NGH_OP_STORE_TRUNC) stores[o.dst] = true;
     }
 }
 
@@ -349,7 +349,9 @@ int plan_stage(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan
                 P.k.shape[2] = n;
             }
         }
-        if (P.V == 1 && P.tail == 0 && !(ctx && ctx->no_tiles)) {
+        bool plain_stores = true;     // a truncating store writes memory directly, never through a tile
+        for (int pc = S.op_begin; pc < S.op_end; ++pc) plain_stores = plain_stores && sp.ops[pc].opcode != NGH_OP_STORE_TRUNC;
+        if (P.V == 1 && P.tail == 0 && plain_stores && !(ctx && ctx->no_tiles)) {
             // Operands of mixed contiguity: if enough of the traffic is contiguous along a
             // second axis (transposed views), stage those operands through LDS tiles.
             double total = 0.0, along[NGH_MAX_AXES] = {0.0, 0.0, 0.0};

@@ -32,7 +32,7 @@ _OPCODE_NAMES = [
     "add", "sub", "mul", "div", "int_div", "mod", "eq", "ne", "lt", "le", "gt", "ge",
     "pow", "minimum", "maximum",
     "sum", "prod", "max", "min", "argmax", "argmin",
-    "take",
+    "take", "store_trunc",
 ]
 #: op name (the reference's template names, float_ew2.py:31-77) -> opcode
 OPCODES = {name: i for i, name in enumerate(_OPCODE_NAMES)}
@@ -513,8 +513,9 @@ class FusedSpecBuilder(object):
         self.emit("load", dst, t)
         return dst
 
-    def store(self, t, r):
-        self.emit("store", t, r)
+    def store(self, t, r, truncate=False):
+        """truncate: a FLEX16 mantissa is cut toward zero (the fill rule) instead of rounded."""
+        self.emit("store_trunc" if truncate else "store", t, r)
 
     def constant(self, value, dst=None):
         dst = self.reg() if dst is None else dst
@@ -565,6 +566,7 @@ class FusedSpecBuilder(object):
         for name in REDUCTION_OPS:
             src_fields[OPCODES[name]] = (2,)
         src_fields[OPCODES["store"]] = (2,)
+        src_fields[OPCODES["store_trunc"]] = (2,)
         src_fields[OPCODES["take"]] = (2,)
         writes = set(OPCODES[n] for n in UNARY_OPS + BINARY_OPS + ["load", "const", "iota", "take"])
         n_regs = 0

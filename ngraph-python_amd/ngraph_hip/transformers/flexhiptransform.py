@@ -101,6 +101,8 @@ class FlexFusedKernel(FusedKernel):
         super(FlexFusedKernel, self).__init__(*args, **kwargs)
         self.output_flex_entries = []
 
+    fill_store = "store_trunc"   # FlexFillKernel: int(value / scale), clipped (tensor_ops.py:690-707)
+
     def _constant_value(self, value):
         """A scalar constant as the host write path would have stored it: tightest-fit
         exponent, truncated mantissa (flexgputransform.py:183-203)."""

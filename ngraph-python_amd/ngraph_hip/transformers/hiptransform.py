@@ -294,6 +294,8 @@ class FusedKernel(HipKernel):
         self.spec_uses = []         # per spec: [(base tensor description, is read, is written)] per slot
         self.described = None
 
+    fill_store = "store"         # how a Fill writes its value (a flex kernel truncates)
+
     def _constant_value(self, value):
         """The fp32 immediate a scalar constant becomes (a flex kernel quantises it first)."""
         return value
@@ -367,7 +369,7 @@ class FusedKernel(HipKernel):
                 td = op.args[0].forwarded.tensor_description()
                 r = new_reg()
                 program.append(("const", r, float(op.scalar)))
-                program.append(("store", slot(td), r))
+                program.append((self.fill_store, slot(td), r))
                 value_reg[_view_key(td)] = r
                 continue
             if isinstance(op, og.OneHotOp):
@@ -525,8 +527,8 @@ class FusedKernel(HipKernel):
             elif kind == "load":
                 sb.load(ins[2], reg(ins[1]))
                 read.add(ins[2])
-            elif kind == "store":
-                sb.store(ins[1], reg(ins[2]))
+            elif kind in ("store", "store_trunc"):
+                sb.store(ins[1], reg(ins[2]), truncate=(kind == "store_trunc"))
                 written.add(ins[1])
             elif kind == "iota":
                 axis = [i for i, d in enumerate(inner) if d.named == ins[2].name]

@@ -498,3 +498,27 @@ def test_take_needs_an_extent(hip_runtime):
         rt.launch_fused(sb.build())
     for d in (lut_d, idx_d, out_d):
         d.free()
+
+
+def test_truncating_store_is_the_flex_fill_rule(hip_runtime):
+    """STORE_TRUNC: mantissa = int(value / scale) cut toward zero and clipped
+    (tensor_ops.py:690-707), where the ordinary store rounds to nearest."""
+    from ngraph_hip.runtime import NGH_FLEX16
+    rt = hip_runtime
+    n, dec = 1000, 14
+    values = [1.2, -1.2, 0.99999, 5.0, -5.0]               # the last two saturate at dec 14
+    for value in values:
+        for truncate in (True, False):
+            y_d = rt.empty((n,), NGH_FLEX16)
+            stats = rt.stats_alloc(1)
+            sb = FusedSpecBuilder([n])
+            ty = sb.tensor(y_d.ptr, [1], NGH_FLEX16, scale=2.0 ** -dec, dev_stats=stats)
+            sb.store(ty, sb.constant(value), truncate=truncate)
+            rt.launch_fused(sb.build())
+            scaled = np.float32(value) * np.float32(2.0 ** dec)
+            want = int(np.clip(np.trunc(scaled) if truncate else np.rint(scaled), -32768, 32767))
+            got = y_d.get()
+            assert (got == want).all(), (value, truncate, got[:4], want)
+            assert int(rt.stats_read(stats, 1)[0]) == abs(want)
+            y_d.free()
+            rt.free(stats)
