@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define NGH_ABI_VERSION 3
+#define NGH_ABI_VERSION 4
 
 /* ---- limits (float_ew2.py:285-286 MAX_AXES = 3) ------------------------ */
 #define NGH_MAX_AXES      3
@@ -98,6 +98,15 @@ enum ngh_opcode {
      * to nearest: the fill of a flex tensor, int(value / scale) clipped
      * (tensor_ops.py:690-707 FlexFillKernel).  Other storage types: same as STORE.        */
     NGH_OP_STORE_TRUNC,
+    /* random fills (RngFillKernel, tensor_ops.py:621-661; RngOp, op_graph.py:2786-2870):
+     * dst=reg a=stream number.  Each element draws from a counter-based generator
+     * (Philox-4x32-10) keyed by the spec's rng_seed, with counter (linear index of the element
+     * in the spec's axis order, stream, rng_counter): the value of an element does not depend
+     * on how the launch is split over lanes, and a caller that bumps rng_counter per execution
+     * gets fresh numbers every time.  UNIFORM is in [0, 1); NORMAL is standard normal
+     * (Box-Muller).  The streams differ from the reference's (curand / numpy), as those two
+     * differ from each other; only the distributions can be compared.                      */
+    NGH_OP_RNG_UNIFORM, NGH_OP_RNG_NORMAL,
     NGH_OP_COUNT_
 };
 
@@ -172,6 +181,8 @@ typedef struct ngh_fused_spec {
     float       consts[NGH_MAX_CONSTS];
     ngh_op      ops[NGH_MAX_OPS];
     ngh_stage   stages[NGH_MAX_STAGES];
+    uint32_t    rng_seed;      /* NGH_OP_RNG_*: key of the generator            */
+    uint32_t    rng_counter;   /* NGH_OP_RNG_*: execution number (caller bumps)  */
 } ngh_fused_spec;
 
 typedef struct ngh_context ngh_context;

@@ -40,6 +40,7 @@ struct KArgs {
     int       iota_map[3];   // kernel axis holding spec axis k (for NGH_OP_IOTA)
     int       n_stat_slots;
     int       n_staged;      // tiled skeleton: operands staged through LDS tiles
+    unsigned  rng_seed, rng_counter;   // NGH_OP_RNG_*
     int       probe;         // NGH_SPEC_PROBE: record max|value| bits instead of storing
     int*      stat_ptr[4];   // device word of each per-thread accumulator
     int*      stat_partial[4];  // per-workgroup scratch the streaming kernels write instead
@@ -153,6 +154,36 @@ __device__ __forceinline__ int flex_quantize(float v) {
     r = fminf(fmaxf(r, -32768.0f), 32767.0f); // saturate (NaN -> -32768 by fmaxf, fixed below)
     int q = (int)r;
     return (v != v) ? 0 : q;
+}
+
+// ---------------------------------------------------------------------------
+// Philox-4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11):
+// a counter-based generator, so an element's number depends only on (key, counter).
+// ---------------------------------------------------------------------------
+struct Philox4 { unsigned x[4]; };
+
+__device__ __forceinline__ Philox4 philox4x32_10(unsigned c0, unsigned c1, unsigned c2, unsigned c3,
+                                                 unsigned k0, unsigned k1) {
+#pragma unroll
+    for (int round = 0; round < 10; ++round) {
+        const unsigned lo0 = 0xD2511F53u * c0, hi0 = __umulhi(0xD2511F53u, c0);
+        const unsigned lo1 = 0xCD9E8D57u * c2, hi1 = __umulhi(0xCD9E8D57u, c2);
+        const unsigned n0 = hi1 ^ c1 ^ k0, n1 = lo1, n2 = hi0 ^ c3 ^ k1, n3 = lo0;
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    Philox4 r;
+    r.x[0] = c0; r.x[1] = c1; r.x[2] = c2; r.x[3] = c3;
+    return r;
+}
+
+// uniform in [0, 1) with 24 random bits; standard normal by Box-Muller
+__device__ __forceinline__ float rng_uniform01(unsigned bits) { return (float)(bits >> 8) * (1.0f / 16777216.0f); }
+__device__ __forceinline__ float rng_normal(unsigned b0, unsigned b1) {
+    const float u1 = ((float)(b0 >> 8) + 1.0f) * (1.0f / 16777216.0f);       // (0, 1]
+    const float u2 = rng_uniform01(b1);
+    return sqrtf(-2.0f * logf(u1)) * cosf(6.28318530717958647692f * u2);
 }
 
 // the fill rule: int(value / scale) cut toward zero, clipped (tensor_ops.py:690-707)

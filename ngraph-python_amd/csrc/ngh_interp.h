@@ -192,6 +192,20 @@ __device__ __forceinline__ void run_ops(const KArgs& k, LdsRegs<V>& rf, Extra& e
                 }
                 if (t.stat_slot >= 0) ex.seti(ex_stat(t.stat_slot), max(ex.geti(ex_stat(t.stat_slot)), fmax));
             } break;
+            case NGH_OP_RNG_UNIFORM: case NGH_OP_RNG_NORMAL: {
+                // shape of the spec's axes, whatever order the kernel walks them in
+                const unsigned long long n1 = (unsigned long long)k.shape[k.iota_map[1]];
+                const unsigned long long n2 = (unsigned long long)k.shape[k.iota_map[2]];
+#pragma unroll
+                for (int v = 0; v < V; ++v) {
+                    const unsigned long long lin =
+                        ((unsigned long long)at.coord(k.iota_map[0], v) * n1 + (unsigned long long)at.coord(k.iota_map[1], v)) * n2 +
+                        (unsigned long long)at.coord(k.iota_map[2], v);
+                    const Philox4 r = philox4x32_10((unsigned)lin, (unsigned)(lin >> 32), o.a, k.rng_counter,
+                                                    k.rng_seed, 0x1BD11BDAu);
+                    rf.set(o.dst, v, opc == NGH_OP_RNG_UNIFORM ? rng_uniform01(r.x[0]) : rng_normal(r.x[0], r.x[1]));
+                }
+            } break;
             case NGH_OP_TAKE: {
                 // table lookup: the coordinate along one axis comes from a register
                 const KTensor& t = k.t[o.b & 15];

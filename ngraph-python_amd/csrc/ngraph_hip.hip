@@ -148,6 +148,9 @@ int validate(const ngh_fused_spec* sp) {
             } else if (opc == NGH_OP_CONST) {
                 if (o.a >= sp->n_consts || !reg_ok(o.dst)) return fail(NGH_E_INVALID, "op %d: bad CONST", pc);
                 defined[o.dst] = true;
+            } else if (opc == NGH_OP_RNG_UNIFORM || opc == NGH_OP_RNG_NORMAL) {
+                if (!reg_ok(o.dst)) return fail(NGH_E_INVALID, "op %d: bad RNG destination", pc);
+                defined[o.dst] = true;
             } else if (opc == NGH_OP_TAKE) {
                 const int t = o.b & 15, axis = o.b >> 4;
                 if (t >= sp->n_tensors || axis >= sp->rank || !need(o.a) || !reg_ok(o.dst))
@@ -237,6 +240,8 @@ void fill_kargs(const ngh_fused_spec& sp, const ngh_stage& S, const int perm[3],
     k.n_red = S.n_reductions;
     k.red_axis = -1;
     k.probe = (sp.flags & NGH_SPEC_PROBE) ? 1 : 0;
+    k.rng_seed = sp.rng_seed;
+    k.rng_counter = sp.rng_counter;
     for (int r = 0; r < S.n_reductions; ++r) k.red_out[r] = S.red_out[r];
     if (S.n_reductions) k.red_axis = k.iota_map[0];
     bool loads[NGH_MAX_TENSORS], stores[NGH_MAX_TENSORS];

@@ -16,7 +16,8 @@ from ngraph_hip.op_graph.op_graph import (  # noqa: F401
     absolute, add, argmax, argmin, as_op, as_ops, assign, axes_with_order, batch_size, broadcast,
     cast_axes, cast_role, computation, constant, cos, divide, doall, equal, exp, expand_dims, fill,
     flatten, flatten_at, floordivide, greater, greater_equal, less, less_equal, log, max, maximum,
-    mean, min, minimum, mod, multiply, negative, not_equal, one_hot, lookuptable, persistent_tensor,
+    mean, min, minimum, mod, multiply, negative, not_equal, one_hot, lookuptable, uniform, normal,
+    persistent_tensor,
     placeholder, power, prod, reciprocal, safelog, sequential, sigmoid, sigmoidAtomic, sign, sin,
     slice_along_axis, softmax, sqrt, square, squared_L2, subtract, sum, tanh, temporary,
     tensor_size, tensor_slice, unflatten, value_of, variable, variance, Transpose)

@@ -1343,6 +1343,29 @@ def one_hot(x, axis):
     return OneHotOp(x, axis)
 
 
+class RngOp(TensorOp):
+    """A tensor of x's axes filled with fresh random numbers at every execution; x itself is
+    not read (op_graph.py:2786-2812)."""
+
+    def __init__(self, distribution, params, x, **kwargs):
+        if distribution not in ("uniform", "normal"):
+            raise ValueError("unsupported distribution: {}".format(distribution))
+        x = as_op(x)
+        self.distribution = distribution
+        self.params = params
+        super(RngOp, self).__init__(args=(x,), axes=x.axes, **kwargs)
+
+
+def uniform(x, low=0.0, high=1.0):
+    """Uniform numbers in [low, high) with the axes of x (op_graph.py:2843-2855)."""
+    return RngOp(distribution="uniform", params=dict(low=low, high=high), x=x)
+
+
+def normal(x, loc=0.0, scale=1.0):
+    """Normal numbers around loc with standard deviation scale (op_graph.py:2858-2870)."""
+    return RngOp(distribution="normal", params=dict(loc=loc, scale=scale), x=x)
+
+
 class LookupTableOp(TensorOp):
     """Forward lookup: rows (lut_axis 0) or columns (lut_axis 1) of a 2-D table selected by a
     1-D index tensor (op_graph/lookuptable.py:55-115).  `axes` are the output axes; the one at

@@ -12,7 +12,7 @@ import os
 
 import numpy as np
 
-NGH_ABI_VERSION = 3
+NGH_ABI_VERSION = 4
 NGH_MAX_AXES = 3
 NGH_MAX_TENSORS = 12
 NGH_MAX_OPS = 96
@@ -32,7 +32,7 @@ _OPCODE_NAMES = [
     "add", "sub", "mul", "div", "int_div", "mod", "eq", "ne", "lt", "le", "gt", "ge",
     "pow", "minimum", "maximum",
     "sum", "prod", "max", "min", "argmax", "argmin",
-    "take", "store_trunc",
+    "take", "store_trunc", "rng_uniform", "rng_normal",
 ]
 #: op name (the reference's template names, float_ew2.py:31-77) -> opcode
 OPCODES = {name: i for i, name in enumerate(_OPCODE_NAMES)}
@@ -74,7 +74,8 @@ class ngh_fused_spec(ctypes.Structure):
                 ("tensors", ngh_tensor * NGH_MAX_TENSORS),
                 ("consts", ctypes.c_float * NGH_MAX_CONSTS),
                 ("ops", ngh_op * NGH_MAX_OPS),
-                ("stages", ngh_stage * NGH_MAX_STAGES)]
+                ("stages", ngh_stage * NGH_MAX_STAGES),
+                ("rng_seed", ctypes.c_uint32), ("rng_counter", ctypes.c_uint32)]
 
 
 class HipLibraryError(RuntimeError):
@@ -537,6 +538,12 @@ class FusedSpecBuilder(object):
         self.emit(name, dst, a, b)
         return dst
 
+    def rng(self, distribution, stream=0, dst=None):
+        """dst = a fresh random number per element: "uniform" in [0, 1) or standard "normal"."""
+        dst = self.reg() if dst is None else dst
+        self.emit("rng_" + distribution, dst, int(stream))
+        return dst
+
     def take(self, table, index_reg, axis, dst=None):
         """dst = table[.., (int)index_reg along `axis`, ..] (the other coordinates are the loop's)."""
         dst = self.reg() if dst is None else dst
@@ -568,7 +575,8 @@ class FusedSpecBuilder(object):
         src_fields[OPCODES["store"]] = (2,)
         src_fields[OPCODES["store_trunc"]] = (2,)
         src_fields[OPCODES["take"]] = (2,)
-        writes = set(OPCODES[n] for n in UNARY_OPS + BINARY_OPS + ["load", "const", "iota", "take"])
+        writes = set(OPCODES[n] for n in UNARY_OPS + BINARY_OPS +
+                     ["load", "const", "iota", "take", "rng_uniform", "rng_normal"])
         n_regs = 0
         for begin, end, _ in self.stages:
             last_use = {}

@@ -70,7 +70,7 @@ def kernel_op_name(op):
 
 def is_fusable(op):
     return (kernel_op_name(op) is not None or
-            isinstance(op, (og.AssignOp, og.OneHotOp, og.Fill, og.LookupTableOp)))
+            isinstance(op, (og.AssignOp, og.OneHotOp, og.Fill, og.LookupTableOp, og.RngOp)))
 
 
 def iteration_axes(op):
@@ -289,6 +289,9 @@ class FusedKernel(HipKernel):
         self.ops = list(ops)
         self.store_ops = set(store_ops)
         self.name = name
+        self.kernel_number = transformer.n_kernels      # distinguishes the random streams of kernels
+        transformer.n_kernels += 1
+        self.n_rng_streams = 0
         self.specs = []
         self.flex_bindings = []     # (spec index, tensor slot, flex entry, is_output)
         self.spec_uses = []         # per spec: [(base tensor description, is read, is written)] per slot
@@ -317,6 +320,7 @@ class FusedKernel(HipKernel):
         take_axes = []           # output axes whose coordinate a lookup replaces by an index value
         take_strides = {}        # (operand slot, axis) -> the table's stride along its looked-up axis
         self.take_extents = {}   # operand slot -> length of the table's looked-up axis
+        self.n_rng_streams = 0   # random fills in this kernel, each its own stream
 
         # ---- pass 1: collect operands (views) and the program over symbolic registers ----
         operands = []            # [(td, role)] in slot order
@@ -378,6 +382,20 @@ class FusedKernel(HipKernel):
                 program.append(("iota", i, op.axis))
                 r = new_reg()
                 program.append(("eq", r, i, x))
+            elif isinstance(op, og.RngOp):
+                # RngFillKernel (tensor_ops.py:651-661): draw, then scale and shift
+                u = new_reg()
+                program.append(("rng", u, op.distribution, self.n_rng_streams))
+                self.n_rng_streams += 1
+                if op.distribution == "uniform":
+                    mul, add = op.params["high"] - op.params["low"], op.params["low"]
+                else:
+                    mul, add = op.params["scale"], op.params["loc"]
+                c_mul, c_add, m, r = new_reg(), new_reg(), new_reg(), new_reg()
+                program.append(("const", c_mul, float(mul)))
+                program.append(("mul", m, u, c_mul))
+                program.append(("const", c_add, float(add)))
+                program.append(("add", r, m, c_add))
             elif isinstance(op, og.LookupTableOp):
                 # gputransform.py:197-199: ("take", x=idx, y=lut, axis=lut_axis)
                 lut, idx = op.args[0].forwarded, op.args[1].forwarded
@@ -535,6 +553,8 @@ class FusedKernel(HipKernel):
                 if not axis:
                     raise og_unsupported("one-hot axis was merged away")
                 sb.iota(axis[0], reg(ins[1]))
+            elif kind == "rng":
+                sb.rng(ins[2], ins[3], reg(ins[1]))
             elif kind == "take":
                 axis = [i for i, d in enumerate(inner) if d.named == ins[4].name]
                 if not axis:
@@ -550,6 +570,7 @@ class FusedKernel(HipKernel):
                 sb.binary(kind, reg(ins[2]), reg(ins[3]), reg(ins[1]))
         spec = sb.build()
         index = len(self.specs)
+        spec.rng_seed = (t.rng_seed * 0x9E3779B1 + index * 0x85EBCA77 + self.kernel_number) & 0xFFFFFFFF
         for s, td in enumerate(operands):
             entry = t.flex_entry_of(td)
             if entry is not None:
@@ -571,6 +592,8 @@ class FusedKernel(HipKernel):
         rt = self.transformer.runtime
         for spec in self.specs:
             rt.launch_fused(spec)
+            if self.n_rng_streams:
+                spec.rng_counter = (spec.rng_counter + 1) & 0xFFFFFFFF    # fresh numbers next time
 
     def describe(self):
         rt = self.transformer.runtime
@@ -1103,15 +1126,18 @@ class HipTransformer(ComputationGraphTransformer):
 
     kernel_group_class = HipKernelGroup
 
-    def __init__(self, device_id=0, fusion=True, dry_run=False, fuse_moments=None, **kwargs):
+    def __init__(self, device_id=0, fusion=True, dry_run=False, fuse_moments=None, rng_seed=0, **kwargs):
         """dry_run=True lowers graphs to kernel specs without a device (no results can be
-        read back); it exists so the host-side lowering can be inspected and tested."""
+        read back); it exists so the host-side lowering can be inspected and tested.
+        rng_seed keys the random fills (ng.uniform / ng.normal): same seed, same numbers."""
         try:
             self.runtime = DryRunRuntime() if dry_run else HipRuntime(device_id)
         except HipLibraryError as e:
             raise UnsupportedTransformerException("hipgpu needs libngraph_hip.so and an MI355X: %s" % e)
         super(HipTransformer, self).__init__(**kwargs)
         self.fusion = fusion
+        self.rng_seed = int(rng_seed)
+        self.n_kernels = 0
         self.kernel_groups = OrderedDict()
         self.graph_passes = [SimplePrune(), TensorSizeFold(), ConstantFoldPass(), SimplePrune()]
         if fusion if fuse_moments is None else fuse_moments:

@@ -119,6 +119,14 @@ class NumpyTransformer(ComputationGraphTransformer):
                 o, x = view(op), view(op.args[0])
                 o[:] = np.eye(o.shape[0])[:, x.astype(np.int32)]
             return onehot
+        if isinstance(op, og.RngOp):
+            def fill_random():                                       # cputransform.py:580-587
+                out = view(op)
+                if op.distribution == "uniform":
+                    out[()] = np.random.uniform(low=op.params["low"], high=op.params["high"], size=out.shape)
+                else:
+                    out[()] = np.random.normal(loc=op.params["loc"], scale=op.params["scale"], size=out.shape)
+            return fill_random
         if isinstance(op, og.LookupTableOp):
             def lookup():                                            # cpuengine.py:421-422 fprop_lut
                 view(op)[:] = view(op.args[0]).take(view(op.args[1]).astype(int), op.lut_axis)

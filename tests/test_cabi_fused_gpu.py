@@ -522,3 +522,36 @@ def test_truncating_store_is_the_flex_fill_rule(hip_runtime):
             assert int(rt.stats_read(stats, 1)[0]) == abs(want)
             y_d.free()
             rt.free(stats)
+
+
+def test_rng_is_a_function_of_seed_counter_and_element(hip_runtime):
+    """The random fill draws per element from (seed, counter, linear index, stream): the same
+    numbers come out whatever the launch shape, and a new counter or seed gives new ones."""
+    rt = hip_runtime
+    A, B = 96, 1000
+
+    def draw(shape, strides, seed, counter, dist="uniform"):
+        y_d = rt.empty((A * B,))
+        sb = FusedSpecBuilder(shape)
+        ty = sb.tensor(y_d.ptr, strides)
+        sb.store(ty, sb.rng(dist, 0))
+        spec = sb.build()
+        spec.rng_seed, spec.rng_counter = seed, counter
+        rt.launch_fused(spec)
+        out = y_d.get()
+        y_d.free()
+        return out
+
+    flat = draw([A * B], [1], 7, 0)                         # one contiguous axis: vector stores
+    two_d = draw([A, B], [B, 1], 7, 0)                      # same elements as a matrix
+    transposed = draw([B, A], [1, B], 7, 0)                 # walked column by column
+    np.testing.assert_array_equal(flat, two_d)
+    # the transposed walk numbers element (b, a) as b * A + a: the same set, permuted
+    np.testing.assert_array_equal(np.sort(transposed), np.sort(flat))
+    np.testing.assert_array_equal(transposed.reshape(A, B).T.ravel(), flat)
+    assert flat.min() >= 0.0 and flat.max() < 1.0 and abs(flat.mean() - 0.5) < 0.01
+    assert not np.array_equal(flat, draw([A * B], [1], 7, 1))
+    assert not np.array_equal(flat, draw([A * B], [1], 8, 0))
+    np.testing.assert_array_equal(flat, draw([A * B], [1], 7, 0))
+    z = draw([A * B], [1], 7, 0, "normal")
+    assert abs(z.mean()) < 0.02 and abs(z.std() - 1.0) < 0.02

@@ -257,6 +257,40 @@ def test_lookuptable_forward(backend, lut_axis):
         np.testing.assert_allclose(summed, want.sum(axis=lut_axis), rtol=RTOL, atol=1e-5)
 
 
+def test_rng_uniform_ranges(backend):
+    """tests/transformer_dependent/test_rngop.py:36-62: ranges of ng.uniform."""
+    a = axes(M=5, N=8)
+    t = ng.persistent_tensor(a, initial_value=10.0)
+    with executor([ng.uniform(t, low=0.0, high=0.5), ng.uniform(t, low=-0.5, high=0.5)]) as f:
+        pos, posneg = f()
+        assert np.all(pos < 0.5) and np.all(pos >= 0.0) and not np.all(pos == 0.0)
+        assert np.all(posneg < 0.5) and np.all(posneg >= -0.5) and not np.all(posneg >= 0.0)
+        assert not np.array_equal(pos - 0.25, posneg * 0.5)      # two fills, two streams
+
+
+def test_rng_runs_at_every_execution(backend):
+    """test_rngop.py:65-79: a random fill is redone by every call of the computation."""
+    a = axes(A=2, B=2)
+    x = ng.variable(a, initial_value=np.array([[1, 2], [3, 4]]))
+    with executor(ng.sum(ng.uniform(x), out_axes=())) as f:
+        assert np.array(f()).copy() != np.array(f()).copy()
+
+
+def test_rng_normal_moments(backend):
+    """test_rngop.py:82-103 at a size where the moments are tight: mean, spread, and (for the
+    uniform) the variance (high-low)^2/12."""
+    a = axes(M=300, N=400)
+    t = ng.persistent_tensor(a, initial_value=10.0)
+    with executor([ng.normal(t, loc=-0.5, scale=1.0), ng.uniform(t, low=1.0, high=3.0)]) as f:
+        z, u = f()
+        assert abs(z.mean() + 0.5) < 0.02 and abs(z.std() - 1.0) < 0.02
+        assert not np.all(z >= 0.0) and not np.all(z < 0.0)
+        assert abs(np.mean(((z + 0.5)) ** 3)) < 0.05 and abs(np.mean((z + 0.5) ** 4) - 3.0) < 0.15
+        assert abs(u.mean() - 2.0) < 0.01 and abs(u.var() - 4.0 / 12.0) < 0.01
+        # neighbours are uncorrelated
+        assert abs(np.corrcoef(u.ravel()[:-1], u.ravel()[1:])[0, 1]) < 0.02
+
+
 def test_lookuptable_argument_checks():
     a = axes(V=5, F=4, I=3)
     V, F, I = a
