@@ -203,7 +203,9 @@ def main():
     for k, times in prof:
         per_kernel.append({"kernel": "+".join(sum(k.describe(), [])) if hasattr(k, "describe") else
                            type(k).__name__, "ms": float(np.mean(times)),
-                           "bytes": kernel_bytes(k) if hasattr(k, "specs") else 0})
+                           "bytes": kernel_bytes(k) if hasattr(k, "specs") else
+                           # the moments kernel reads x once and writes 3 floats per row
+                           (k.rows * k.R * 4 + k.rows * 12 if hasattr(k, "rows") else 0)})
     dom = max(per_kernel, key=lambda d: d["ms"])
     achieved = dom["bytes"] / (dom["ms"] * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": dom["kernel"], "achieved": round(achieved, 1),

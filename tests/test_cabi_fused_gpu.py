@@ -555,3 +555,30 @@ def test_rng_is_a_function_of_seed_counter_and_element(hip_runtime):
     np.testing.assert_array_equal(flat, draw([A * B], [1], 7, 0))
     z = draw([A * B], [1], 7, 0, "normal")
     assert abs(z.mean()) < 0.02 and abs(z.std() - 1.0) < 0.02
+
+
+@pytest.mark.parametrize("n", [4096, 100003])
+def test_convert_between_fp32_and_flex16(hip_runtime, n):
+    """Storage types may differ inside one kernel: fp32 -> flex16 is the quantising conversion
+    (round to nearest even, saturate, max|mantissa|), flex16 -> fp32 the dequantisation."""
+    from ngraph_hip.runtime import NGH_FLEX16
+    from oracle import flex_model as fm
+    rt = hip_runtime
+    rs = np.random.RandomState(n)
+    x = rs.normal(0, 3.0, n).astype(f32)
+    dec = 12                                               # +-8 range: some elements saturate
+    x_d, q_d, back_d = rt.array(x), rt.empty((n,), NGH_FLEX16), rt.empty((n,))
+    stats = rt.stats_alloc(1)
+    sb = FusedSpecBuilder([n])
+    sb.store(sb.tensor(q_d.ptr, [1], NGH_FLEX16, scale=2.0 ** -dec, dev_stats=stats), sb.load(sb.tensor(x_d.ptr, [1])))
+    rt.launch_fused(sb.build())
+    want = fm.quantize_rni(x, dec)
+    np.testing.assert_array_equal(q_d.get(), want)
+    assert int(rt.stats_read(stats, 1)[0]) == fm.maxabs(want)
+    sb = FusedSpecBuilder([n])
+    sb.store(sb.tensor(back_d.ptr, [1]), sb.load(sb.tensor(q_d.ptr, [1], NGH_FLEX16, scale=2.0 ** -dec)))
+    rt.launch_fused(sb.build())
+    np.testing.assert_array_equal(back_d.get(), fm.dequantize(want, dec))
+    for d in (x_d, q_d, back_d):
+        d.free()
+    rt.free(stats)
