@@ -66,6 +66,19 @@ def _reduction_pattern(fn, out_axis):
     return build
 
 
+def pattern_lstm_cell(t, Hn=1024, Nn=64):
+    # LSTM cell on transposed storage (frontends/neon/layer.py:1630-1647): inputs contiguous
+    # along H, results along N -- the tiled skeleton
+    H, N, G = _axes(H=Hn, N=Nn, G=4 * Hn)
+    gates_st, cprev_st = ng.placeholder([N, G]), ng.placeholder([N, H])
+    gates = ng.axes_with_order(gates_st, [G, N])
+    c_prev = ng.axes_with_order(cprev_st, [H, N])
+    parts = {k: ng.cast_axes(ng.tensor_slice(gates, [slice(j * Hn, (j + 1) * Hn), slice(None)]), [H, N])
+             for j, k in enumerate(("i", "f", "o", "g"))}
+    h, c = neon.lstm_cell(parts, c_prev, H, None)
+    return t.computation([c, h], gates_st, cprev_st)
+
+
 def pattern_lstm_bias_gradient(t):
     # db = sum over N of gates [4H, N] stored transposed (frontends/neon/layer.py:1630-1647)
     N, G = _axes(N=64, G=4096)
@@ -84,6 +97,10 @@ PATTERNS = [
     ("max_along", "hipgpu", _reduction_pattern(ng.max, 0)),
     ("max_across", "hipgpu", _reduction_pattern(ng.max, 1)),
     ("sum_across_small", "hipgpu", pattern_lstm_bias_gradient),
+    ("lstm_cell", "hipgpu", pattern_lstm_cell),
+    # the planner orders ops of large tensors differently (nothing above 65536 elements is
+    # materialised early), which gives the cell a second program
+    ("lstm_cell_large", "hipgpu", lambda t: pattern_lstm_cell(t, 2048, 512)),
 ]
 
 
@@ -104,7 +121,7 @@ def collect():
                     plan = hiplib.plan_fused(spec, stage)
                     st = spec.stages[stage]
                     family = plan["family"]
-                    if family > 2 or (family == 0 and (plan["V"] < 4 or st.n_reductions)):
+                    if family > 3 or (family == 0 and (plan["V"] < 4 or st.n_reductions)):
                         continue
                     if family == 1 and spec.shape[0] // plan["V"] <= 64:
                         continue          # short rows run the several-rows-per-workgroup kernel
@@ -119,6 +136,16 @@ def collect():
                     dtypes = [spec.tensors[i].dtype for i in range(spec.n_tensors)]
                     bcast = [1 if spec.tensors[i].strides[fast] == 0 else 0 for i in range(spec.n_tensors)]
                     stored = set(o[1] for o in ops if o[0] == hiplib.OPCODES["store"])
+                    loaded = set(o[2] for o in ops if o[0] == hiplib.OPCODES["load"])
+                    staged, n_staged = [], 0
+                    for i in range(spec.n_tensors):
+                        st_i = spec.tensors[i].strides
+                        if family == 3 and i in (stored | loaded) and st_i[plan["perm"][1]] == 1 and \
+                                st_i[fast] not in (0, 1):
+                            staged.append(n_staged)
+                            n_staged += 1
+                        else:
+                            staged.append(-1)
                     stat_slot, n_slots = [], 0
                     for i in range(spec.n_tensors):
                         if i in stored and dtypes[i] == hiplib.NGH_FLEX16 and n_slots < 4:
@@ -126,12 +153,14 @@ def collect():
                             n_slots += 1
                         else:
                             stat_slot.append(-1)
-                    key = (tuple(ops), tuple(dtypes), tuple(bcast), plan["V"], family, tuple(red_out))
+                    key = (tuple(ops), tuple(dtypes), tuple(bcast), plan["V"], family, tuple(red_out), tuple(staged))
                     if key in seen:
                         continue
                     seen.add(key)
                     programs.append(("%s_k%d" % (name, k_index), ops, dtypes, bcast, stat_slot,
-                                     n_slots, spec.n_regs, plan["V"], family, red_out))
+                                     n_slots, spec.n_regs, plan["V"], family, red_out, staged,
+                                     [1 if i in loaded else 0 for i in range(spec.n_tensors)],
+                                     [1 if i in stored else 0 for i in range(spec.n_tensors)]))
             k_index += 1
         t.close()
     return programs
@@ -140,7 +169,8 @@ def collect():
 def render(programs):
     lines = ["// GENERATED by gen_programs.py from the host lowering -- do not edit.",
              "// One entry per streaming elementwise op program that gets a pre-built kernel."]
-    for i, (name, ops, dtypes, bcast, stat_slot, n_slots, n_regs, V, family, red_out) in enumerate(programs):
+    for i, (name, ops, dtypes, bcast, stat_slot, n_slots, n_regs, V, family, red_out, staged, loaded,
+            stored) in enumerate(programs):
         lines.append("struct SP%d {  // %s" % (i, name))
         lines.append("    static constexpr int V = %d, n_ops = %d, n_regs = %d, n_tensors = %d, "
                      "n_stat_slots = %d, family = %d, n_red = %d;"
@@ -152,14 +182,23 @@ def render(programs):
         lines.append("    static constexpr int dtypes[%d] = {%s};" % (len(dtypes), ", ".join(map(str, dtypes))))
         lines.append("    static constexpr unsigned char bcast[%d] = {%s};" % (len(bcast), ", ".join(map(str, bcast))))
         lines.append("    static constexpr int stat_slot[%d] = {%s};" % (len(stat_slot), ", ".join(map(str, stat_slot))))
+        lines.append("    static constexpr int n_staged = %d;" % sum(1 for x in staged if x >= 0))
+        lines.append("    static constexpr signed char staged[%d] = {%s};" % (len(staged), ", ".join(map(str, staged))))
+        lines.append("    static constexpr unsigned char loaded[%d] = {%s};" % (len(loaded), ", ".join(map(str, loaded))))
+        lines.append("    static constexpr unsigned char stored[%d] = {%s};" % (len(stored), ", ".join(map(str, stored))))
         lines.append("};")
     lines.append("static const StaticEntry kStaticTable[] = {")
     for i, p in enumerate(programs):
-        launch = ("&launch_static<SP%d>, nullptr" % i) if p[8] == 0 else ("nullptr, &launch_static_red<SP%d>" % i)
+        if p[8] == 0:
+            launch = "&launch_static<SP%d>, nullptr, SP%d::staged, nullptr" % (i, i)
+        elif p[8] == 3:
+            launch = "nullptr, nullptr, SP%d::staged, &launch_static_tiled<SP%d>" % (i, i)
+        else:
+            launch = "nullptr, &launch_static_red<SP%d>, SP%d::staged, nullptr" % (i, i)
         lines.append('    {"%s", SP%d::family, SP%d::V, SP%d::n_ops, SP%d::ops, SP%d::n_tensors, SP%d::dtypes, '
                      'SP%d::bcast, SP%d::n_red, SP%d::red_out, %s},' % (p[0], i, i, i, i, i, i, i, i, i, launch))
     if not programs:
-        lines.append('    {"none", 0, 4, 0, nullptr, 0, nullptr, nullptr, 0, nullptr, nullptr, nullptr},')
+        lines.append('    {"none", 0, 4, 0, nullptr, 0, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr},')
     lines.append("};")
     lines.append("static const int kStaticCount = %d;" % len(programs))
     return "\n".join(lines) + "\n"

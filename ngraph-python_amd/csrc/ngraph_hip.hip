@@ -84,7 +84,7 @@ struct ngh_context {
     int         cache_policy = -1;   // -1: from the operands' cache hints; 0..3 forces bit 0 = non-temporal
                                      // loads, bit 1 = non-temporal stores in pre-built kernels
     long long   stream_bytes = 128ll << 20;  // hints act on stages touching at least this much memory
-    int         moments_wgs_per_cu = 16;
+    int         moments_wgs_per_cu = 8;
     char        name[256] = "";
     uint64_t    total_bytes = 0;
 };
@@ -588,6 +588,10 @@ int launch_interp(ngh_context* ctx, Plan& P) {
         if (P.n_tiles == 0) return NGH_OK;
         const unsigned blocks = std::min<unsigned>(P.n_tiles, (unsigned)(ctx->cus * ctx->ew_blocks_per_cu));
         NGH_TRY(stat_scratch(ctx, P.k, blocks));
+        if (P.special >= 0 && !P.k.probe) {
+            HIP_TRY(launch_special_tiled(P.special, ctx->stream, blocks, P.k, P.tiles_a, P.tiles_b, P.n_tiles, P.tile));
+            return stat_fold(ctx, P.k, blocks);
+        }
         if (P.tile == 16)
             hipLaunchKernelGGL(ew_tiled_interp_kernel<16>, dim3(blocks), dim3(kBlock), tiled_lds_bytes(P.k, 16),
                                ctx->stream, P.k, P.tiles_a, P.tiles_b, P.n_tiles, P.load_mask, P.store_mask);
@@ -758,7 +762,7 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->red_wgs_per_cu = std::max(1, env_int("NGH_RED_WGS_PER_CU", 8));
     ctx->cache_policy = env_int("NGH_CACHE_POLICY", -1);
     ctx->stream_bytes = (long long)env_int("NGH_STREAM_MIB", 128) << 20;
-    ctx->moments_wgs_per_cu = std::max(1, env_int("NGH_MOMENTS_WGS_PER_CU", 16));
+    ctx->moments_wgs_per_cu = std::max(1, env_int("NGH_MOMENTS_WGS_PER_CU", 8));
     hipError_t e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev0);
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev1);
@@ -897,7 +901,8 @@ int ngh_copy_strided(ngh_context* ctx, void* dev_dst, const void* dev_src, int32
     }
     if (total == 0) return NGH_OK;
     if (!dev_dst || !dev_src) return fail(NGH_E_INVALID, "NULL device pointer");
-    if (total >= (1LL << 32)) return fail(NGH_E_UNSUPPORTED, "copy of %lld elements; split it", total);
+    // 32-bit element counters with grid-stride steps: stay well inside the range
+    if (total >= (1LL << 31)) return fail(NGH_E_UNSUPPORTED, "copy of %lld elements; split it", total);
     a.rank = r;
     a.total = (unsigned)total;
     return launch_copy(ctx->stream, ctx->cus, dev_dst, dev_src, a, itemsize) == hipSuccess
@@ -960,7 +965,8 @@ int ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec) {
                 continue;
             }
         }
-        if (!ctx->force_interp && !P.k.probe && (P.family == F_RED_COL || (P.family == F_RED_ROW && !P.small_rows))) {
+        if (!ctx->force_interp && !P.k.probe &&
+            (P.family == F_RED_COL || P.family == F_EW_TILED || (P.family == F_RED_ROW && !P.small_rows))) {
             P.special = match_special(P.family, P.V, P.k, 0);
             P.cache_policy = stage_cache_policy(ctx, *spec, spec->stages[s]);
         }
@@ -975,7 +981,7 @@ int ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec, int32_t sta
     if (stage < 0 || stage >= spec->n_stages) return fail(NGH_E_INVALID, "stage %d", stage);
     Plan P;
     NGH_TRY(plan_stage(ctx, *spec, stage, P));
-    if (!ctx->force_interp && !(P.family == F_RED_ROW && P.small_rows) && P.family != F_EW_TILED)
+    if (!ctx->force_interp && !(P.family == F_RED_ROW && P.small_rows))
         P.special = match_special(P.family, P.V, P.k, P.tail);
     describe(P, name128, 128);
     if (P.special >= 0 && P.family == F_EW) {
