@@ -83,7 +83,7 @@ struct ngh_context {
     int         flex_self_managed = 1;  // ngh_launch_fused_flex may fold the policy into the kernel
     int         cache_policy = -1;   // -1: from the operands' cache hints; 0..3 forces bit 0 = non-temporal
                                      // loads, bit 1 = non-temporal stores in pre-built kernels
-    long long   stream_bytes = 128ll << 20;  // hints act on stages touching at least this much memory
+    long long   stream_bytes = 192ll << 20;  // hints act on stages touching at least this much memory
     int         moments_wgs_per_cu = 8;
     char        name[256] = "";
     uint64_t    total_bytes = 0;
@@ -761,7 +761,7 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->no_tiles = env_int("NGH_NO_TILES", 0);
     ctx->red_wgs_per_cu = std::max(1, env_int("NGH_RED_WGS_PER_CU", 8));
     ctx->cache_policy = env_int("NGH_CACHE_POLICY", -1);
-    ctx->stream_bytes = (long long)env_int("NGH_STREAM_MIB", 128) << 20;
+    ctx->stream_bytes = (long long)env_int("NGH_STREAM_MIB", 192) << 20;
     ctx->moments_wgs_per_cu = std::max(1, env_int("NGH_MOMENTS_WGS_PER_CU", 8));
     hipError_t e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev0);
