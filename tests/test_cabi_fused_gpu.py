@@ -11,6 +11,7 @@ import pytest
 from oracle import configs, numpy_ops
 from ngraph_hip.runtime import FusedSpecBuilder, NGH_F32, NGH_I32
 from ngraph_hip.runtime.hiplib import UNARY_OPS, BINARY_OPS
+from conftest import default_kernel_choice
 
 pytestmark = pytest.mark.gpu
 
@@ -421,7 +422,8 @@ def test_tiled_transposed_operands(hip_runtime, shape3, in_place):
     y_d, w_d = rt.empty((O, A, B)), rt.empty((O, B, A))
     spec = _transpose_program(rt, shape3, x_d, y_d, z_d, w_d, in_place)
     assert hiplib.plan_fused(spec, 0)["family"] == 3
-    assert rt.describe_fused(spec, 0).startswith("ew_tiled_interp")
+    if default_kernel_choice():
+        assert rt.describe_fused(spec, 0).startswith("ew_tiled_interp")
     rt.launch_fused(spec)
     y_w = (x.transpose(0, 2, 1) * f32(2.0) + z).astype(f32)
     w_w = (y_w - f32(1.0)).transpose(0, 2, 1)
@@ -449,7 +451,8 @@ def test_tiled_flex_transposed_output_with_statistics(hip_runtime):
     ty = sb.tensor(y_d.ptr, [1, A], NGH_FLEX16, scale=2.0 ** -dec, dev_stats=stats)
     sb.store(ty, sb.binary("mul", sb.load(tx), sb.constant(3.0)))
     spec = sb.build()
-    assert rt.describe_fused(spec, 0).startswith("ew_tiled_interp")
+    if default_kernel_choice():
+        assert rt.describe_fused(spec, 0).startswith("ew_tiled_interp")
     rt.launch_fused(spec)
     want = fm.quantize_rni((x * f32(3.0)).T, dec)
     np.testing.assert_array_equal(y_d.get(), want)

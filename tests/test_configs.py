@@ -10,6 +10,7 @@ built from the neon formulas on the oracle transformer ("cpu") and on
 """
 import numpy as np
 import pytest
+from conftest import default_kernel_choice
 
 import ngraph_hip as ng
 import ngraph_hip.transformers as ngt
@@ -159,6 +160,8 @@ def test_c4_graph(transformer, Hn, Nn):
 def test_cache_policy_does_not_change_results(policy, monkeypatch):
     """Non-temporal loads / stores are a cache hint only: forcing each of the four variants
     of the pre-built Adam and batch-norm kernels gives bit-identical results."""
+    check_names = default_kernel_choice()        # before this test sets a knob itself
+
     def adam_and_bn():
         out = []
         t = ngt.make_transformer_factory("hipgpu")()
@@ -174,7 +177,8 @@ def test_cache_policy_does_not_change_results(policy, monkeypatch):
         f(g_np)
         f(g_np)
         out.extend(np.array(a) for a in read())
-        assert any("special:adam" in d for k in t.kernel_groups[f].kernels for ds in k.describe() for d in ds)
+        assert not check_names or \
+            any("special:adam" in d for k in t.kernel_groups[f].kernels for ds in k.describe() for d in ds)
         t.close()
         t = ngt.make_transformer_factory("hipgpu")()
         dims = (64, 16, 16, 16)
@@ -185,7 +189,8 @@ def test_cache_policy_does_not_change_results(policy, monkeypatch):
         y, xmean, xvar = neon.batch_norm_train(x, gamma, beta, out_axes=[C])
         f = t.computation([y, xmean, xvar], x)
         out.extend(np.array(a) for a in f(x_np.reshape(dims)))
-        assert any("special:batchnorm" in d for k in t.kernel_groups[f].kernels for ds in k.describe() for d in ds)
+        assert not check_names or \
+            any("special:batchnorm" in d for k in t.kernel_groups[f].kernels for ds in k.describe() for d in ds)
         t.close()
         return out
 

@@ -12,6 +12,7 @@ import os
 
 import numpy as np
 import pytest
+from conftest import default_kernel_choice
 
 import ngraph_hip as ng
 import ngraph_hip.transformers as ngt
@@ -116,7 +117,8 @@ def test_c5_fused_flex_bit_exact_over_8_iterations(n, resident):
                 (i, entry.dec, entry.next_dec, dec_want, next_dec_want)
             np.testing.assert_array_equal(got, fm.dequantize(m_want, dec_want))
         assert len(t.kernel_groups[f].kernels) == 1           # one fused kernel
-        assert "special:flex_relu_fma" in kernel.describe()[0][0]
+        if default_kernel_choice():
+            assert "special:flex_relu_fma" in kernel.describe()[0][0]
     finally:
         t.close()
 
