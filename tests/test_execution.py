@@ -191,6 +191,32 @@ def test_run_twice_bit_equal(backend):
     np.testing.assert_array_equal(a, b)
 
 
+def test_log_softmax_twice_bit_equal(backend):
+    """test_kernel_generator.py:43-71 (exit condition): log(softmax(y)) over the class axis of a
+    16 x 10 tensor, evaluated twice with identical bits, and equal to the NumPy statement."""
+    N, Y = ng.make_axis(16, name="N"), ng.make_axis(10, name="Y")
+    yv = rng.uniform(-3, 3, ng.make_axes([N, Y]))
+    y = ng.constant(yv, ng.make_axes([N, Y]))
+    with executor(ng.log(ng.softmax(y, normalization_axes=y.axes[1]))) as f:
+        a = np.array(f()).copy()
+        b = np.array(f())
+    np.testing.assert_array_equal(a, b)
+    e = np.exp(yv - yv.max(axis=1, keepdims=True))
+    np.testing.assert_allclose(a, np.log(e / e.sum(axis=1, keepdims=True)), rtol=1e-5, atol=1e-6)
+
+
+def test_broadcast_add_over_a_long_trailing_axis(backend):
+    """test_kernel_generator.py:174-203 (kernel cache): x[32,32] broadcast against two
+    [32,32,16384] tensors."""
+    X, Y, C = ng.make_axis(32, name="X"), ng.make_axis(32, name="Y"), ng.make_axis(16384, name="C")
+    xv = rng.uniform(-1, 1, ng.make_axes([X, Y]))
+    yv = rng.uniform(-1, 1, ng.make_axes([X, Y, C]))
+    zv = rng.uniform(-1, 1, ng.make_axes([X, Y, C]))
+    x, y, z = ng.constant(xv, [X, Y]), ng.constant(yv, [X, Y, C]), ng.constant(zv, [X, Y, C])
+    with executor(ng.add(ng.add(x, y), z)) as f:
+        np.testing.assert_allclose(f(), xv.reshape(32, 32, 1) + yv + zv, rtol=1e-6, atol=1e-6)
+
+
 def test_views_reorder_slice_flatten(backend):
     C, H, N = ng.make_axis(4, name="C"), ng.make_axis(6, name="H"), ng.make_axis(5, name="N")
     x = ng.placeholder([C, H, N])
