@@ -44,6 +44,14 @@ def pattern_adam(t):
     return t.computation(updates, grad)
 
 
+def _rule_pattern(make):
+    def build(t):
+        P, = _axes(P=1 << 20)
+        p, grad = ng.variable([P], initial_value=0.0), ng.placeholder([P])
+        return t.computation(make().variable_update(p, grad)[0], grad)
+    return build
+
+
 def pattern_batchnorm(t):
     C, H, W, N = _axes(C=64, H=16, W=16, N=16)
     x = ng.placeholder([C, H, W, N])
@@ -90,6 +98,12 @@ def pattern_lstm_bias_gradient(t):
 PATTERNS = [
     ("c1_tanh_sigmoid", "hipgpu", pattern_c1),
     ("adam", "hipgpu", pattern_adam),
+    ("sgd_momentum", "hipgpu", _rule_pattern(lambda: neon.GradientDescentMomentum(0.1, 0.9))),
+    ("sgd_momentum_wdecay", "hipgpu", _rule_pattern(lambda: neon.GradientDescentMomentum(0.1, 0.9, wdecay=0.01))),
+    ("sgd_nesterov", "hipgpu", _rule_pattern(lambda: neon.GradientDescentMomentum(0.1, 0.9, nesterov=True))),
+    ("rmsprop", "hipgpu", _rule_pattern(lambda: neon.RMSProp())),
+    ("rmsprop_momentum_wdecay", "hipgpu", _rule_pattern(lambda: neon.RMSProp(wdecay=0.01, momentum_coef=0.5))),
+    ("adagrad", "hipgpu", _rule_pattern(lambda: neon.Adagrad())),
     ("batchnorm", "hipgpu", pattern_batchnorm),
     ("flex_relu_fma", "flexhip", pattern_flex_relu),
     ("sum_along", "hipgpu", _reduction_pattern(ng.sum, 0)),

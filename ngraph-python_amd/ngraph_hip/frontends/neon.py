@@ -61,6 +61,68 @@ class Adam(object):
         return updates, m, v
 
 
+class GradientDescentMomentum(object):
+    """SGD with momentum, weight decay, optional Nesterov step and the Kahan-compensated
+    parameter update of frontends/neon/optimizer.py:285-310."""
+
+    def __init__(self, learning_rate, momentum_coef=0.0, wdecay=0.0, nesterov=False):
+        self.lrate = learning_rate
+        self.momentum_coef = momentum_coef
+        self.wdecay = wdecay
+        self.nesterov = nesterov
+
+    def variable_update(self, variable, grad, scale_factor=1):
+        velocity = ng.persistent_tensor(axes=variable.axes, initial_value=0.)
+        lr = - self.lrate * (scale_factor * grad + self.wdecay * variable)
+        updates = [ng.assign(velocity, velocity * self.momentum_coef + lr)]
+        delta = (self.momentum_coef * velocity + lr) if self.nesterov else velocity
+        kahan_c = ng.persistent_tensor(axes=variable.axes, initial_value=0.)
+        kahan_y = ng.persistent_tensor(axes=variable.axes, initial_value=0.)
+        kahan_t = ng.persistent_tensor(axes=variable.axes, initial_value=0.)
+        updates.append(ng.assign(kahan_y, delta - kahan_c))
+        updates.append(ng.assign(kahan_t, variable + kahan_y))
+        updates.append(ng.assign(kahan_c, (kahan_t - variable) - kahan_y))
+        updates.append(ng.assign(variable, kahan_t))
+        return ng.sequential(updates), velocity
+
+
+class RMSProp(object):
+    """frontends/neon/optimizer.py:370-383."""
+
+    def __init__(self, decay_rate=0.95, learning_rate=2e-3, epsilon=1e-6, wdecay=0.0, momentum_coef=0.0):
+        self.decay_rate, self.lrate, self.epsilon = decay_rate, learning_rate, epsilon
+        self.wdecay, self.momentum = wdecay, momentum_coef
+
+    def variable_update(self, variable, grad, scale_factor=1):
+        epsilon, decay = self.epsilon, self.decay_rate
+        state = ng.persistent_tensor(axes=variable.axes, initial_value=1.)
+        velocity = ng.persistent_tensor(axes=variable.axes, initial_value=0.)
+        updates = ng.sequential([
+            ng.assign(state, decay * state + (1.0 - decay) * ng.square(grad)),
+            ng.assign(velocity, velocity * self.momentum +
+                      (self.lrate * scale_factor * grad / ng.sqrt(state + epsilon)) +
+                      self.lrate * self.wdecay * variable),
+            ng.assign(variable, variable - velocity)
+        ])
+        return updates, state, velocity
+
+
+class Adagrad(object):
+    """frontends/neon/optimizer.py:533-542."""
+
+    def __init__(self, learning_rate=0.01, epsilon=1e-6):
+        self.lrate, self.epsilon = learning_rate, epsilon
+
+    def variable_update(self, variable, grad, scale_factor=1):
+        state = ng.persistent_tensor(axes=grad.axes, initial_value=0.)
+        updates = ng.sequential([
+            ng.assign(state, state + ng.square(grad)),
+            ng.assign(variable,
+                      variable - (scale_factor * self.lrate * grad) / (ng.sqrt(state + self.epsilon)))
+        ])
+        return updates, state
+
+
 def lstm_cell(gates, c_prev, hidden_axis, gate_slices):
     """Pointwise part of an LSTM step.
 

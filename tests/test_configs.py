@@ -200,3 +200,57 @@ def test_cache_policy_does_not_change_results(policy, monkeypatch):
     got = adam_and_bn()
     for a, b in zip(got, want):
         np.testing.assert_array_equal(a, b)
+
+
+# ------------------------------------------------------------------ other learning rules
+def _run_rule(transformer, make_updates, n, steps=3):
+    rs = np.random.RandomState(n)
+    p0 = rs.normal(0, 0.1, n).astype(np.float32)
+    grads = [rs.normal(0, 0.01, n).astype(np.float32) for _ in range(steps)]
+    P = ng.make_axis(n, name="P")
+    p, grad = ng.variable([P], initial_value=p0), ng.placeholder([P])
+    updates = make_updates(p, grad)
+    f = transformer.computation(updates, grad)
+    read = transformer.computation(p * 1.0)
+    for g in grads:
+        f(g)
+    return p0, grads, np.array(read())
+
+
+@pytest.mark.parametrize("n", [1 << 16, 100003])
+@pytest.mark.parametrize("nesterov", [False, True])
+def test_sgd_momentum_with_kahan_update(transformer, n, nesterov):
+    """optimizer.py:285-310 restated in float64 (the compensated sum makes fp32 track it)."""
+    opt = neon.GradientDescentMomentum(0.1, momentum_coef=0.9, wdecay=0.01, nesterov=nesterov)
+    p0, grads, got = _run_rule(transformer, lambda p, g: opt.variable_update(p, g)[0], n)
+    p, vel = p0.astype(np.float64), np.zeros(n)
+    for g in grads:
+        lr = -0.1 * (g.astype(np.float64) + 0.01 * p)
+        vel = vel * 0.9 + lr
+        p = p + ((0.9 * vel + lr) if nesterov else vel)
+    np.testing.assert_allclose(got, p, rtol=2e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("n", [1 << 16, 100003])
+def test_rmsprop(transformer, n):
+    opt = neon.RMSProp(decay_rate=0.95, learning_rate=2e-3, epsilon=1e-6, wdecay=0.01, momentum_coef=0.5)
+    p0, grads, got = _run_rule(transformer, lambda p, g: opt.variable_update(p, g)[0], n)
+    p, state, vel = p0.astype(np.float64), np.ones(n), np.zeros(n)
+    for g in grads:
+        g = g.astype(np.float64)
+        state = 0.95 * state + 0.05 * g * g
+        vel = vel * 0.5 + 2e-3 * g / np.sqrt(state + 1e-6) + 2e-3 * 0.01 * p
+        p = p - vel
+    np.testing.assert_allclose(got, p, rtol=2e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("n", [1 << 16, 100003])
+def test_adagrad(transformer, n):
+    opt = neon.Adagrad(learning_rate=0.01, epsilon=1e-6)
+    p0, grads, got = _run_rule(transformer, lambda p, g: opt.variable_update(p, g)[0], n)
+    p, state = p0.astype(np.float64), np.zeros(n)
+    for g in grads:
+        g = g.astype(np.float64)
+        state = state + g * g
+        p = p - 0.01 * g / np.sqrt(state + 1e-6)
+    np.testing.assert_allclose(got, p, rtol=2e-5, atol=1e-6)
