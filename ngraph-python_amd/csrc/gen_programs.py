@@ -104,6 +104,9 @@ PATTERNS = [
     ("rmsprop", "hipgpu", _rule_pattern(lambda: neon.RMSProp())),
     ("rmsprop_momentum_wdecay", "hipgpu", _rule_pattern(lambda: neon.RMSProp(wdecay=0.01, momentum_coef=0.5))),
     ("adagrad", "hipgpu", _rule_pattern(lambda: neon.Adagrad())),
+    ("flex_adam", "flexhip", pattern_adam),
+    ("flex_sgd_momentum", "flexhip", _rule_pattern(lambda: neon.GradientDescentMomentum(0.1, 0.9))),
+    ("flex_rmsprop", "flexhip", _rule_pattern(lambda: neon.RMSProp())),
     ("batchnorm", "hipgpu", pattern_batchnorm),
     ("flex_relu_fma", "flexhip", pattern_flex_relu),
     ("sum_along", "hipgpu", _reduction_pattern(ng.sum, 0)),

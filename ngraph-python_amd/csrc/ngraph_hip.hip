@@ -261,6 +261,8 @@ void fill_kargs(const ngh_fused_spec& sp, const ngh_stage& S, const int perm[3],
         if (stores[t] && T.dtype == NGH_FLEX16 && k.n_stat_slots < 4) {
             K.stat_slot = k.n_stat_slots;
             k.stat_ptr[k.n_stat_slots++] = T.dev_stats;
+        } else if (stores[t] && T.dtype == NGH_FLEX16 && T.dev_stats != nullptr) {
+            k.n_stat_slots = 5;      // more flex results with statistics than slots: plan_stage rejects
         }
     }
     memcpy(k.consts, sp.consts, sizeof(k.consts));
@@ -310,7 +312,16 @@ int gather_width(const KArgs& k) {
     return interp_lds_bytes(k, 4) <= kInterpLdsPreferred ? 4 : 1;
 }
 
+int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan& P);
+
 int plan_stage(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan& P) {
+    NGH_TRY(plan_stage_impl(ctx, sp, stage, P));
+    if (P.k.n_stat_slots > 4)
+        return fail(NGH_E_UNSUPPORTED, "stage %d stores more than 4 flex16 tensors with statistics", stage);
+    return NGH_OK;
+}
+
+int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan& P) {
     const ngh_stage& S = sp.stages[stage];
     bool loads[NGH_MAX_TENSORS], stores[NGH_MAX_TENSORS], used[NGH_MAX_TENSORS];
     stage_tensors(sp, S, loads, stores);

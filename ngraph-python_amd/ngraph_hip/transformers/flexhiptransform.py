@@ -252,6 +252,7 @@ class FlexHipTransformer(HipTransformer):
     default_rtol = 1e-02
     atol_precision_multiplier = 8
     kernel_group_class = FlexHipKernelGroup
+    max_written_views = 4        # a kernel merges max|mantissa| for at most 4 flex results
 
     def __init__(self, fixed_point=False, flex_verbose=False, collect_flex_data=False,
                  resident=False, **kwargs):

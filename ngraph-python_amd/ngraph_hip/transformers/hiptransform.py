@@ -977,7 +977,7 @@ class FusionPlanner(object):
                     groups.append(cur)
                     cur = None
                 if is_fusable(pick):
-                    cur = _Group(pick)
+                    cur = _Group(pick, max_written_views=self.transformer.max_written_views)
                 else:
                     groups.append(_Group(pick, fusable=False))
             else:
@@ -993,10 +993,12 @@ class FusionPlanner(object):
 
 
 class _Group(object):
-    def __init__(self, op, fusable=True):
+    def __init__(self, op, fusable=True, max_written_views=NGH_MAX_TENSORS):
         self.ops = [op]
         self.fusable = fusable
         self.store_ops = set()
+        self.max_written_views = max_written_views    # flex kernels: one statistics slot per result
+        self.n_written_views = 0
         if fusable:
             self.axes = iteration_axes(op)
             self.has_reduce = False
@@ -1048,20 +1050,21 @@ class _Group(object):
         for op in ops:
             if op.is_tensor_op and not isinstance(op, (og.AssignOp, og.Fill)):
                 produced.add(op.tensor_description().base)
-        views = set()
+        views, written = set(), set()
         for op in ops:
             reads, writes = self._operand_views(op)
             for td in reads:
                 if td.base not in produced:
                     views.add(_view_key(td))
             if isinstance(op, (og.AssignOp, og.Fill)):
-                views.update(_view_key(td) for td in writes)
+                written.update(_view_key(td) for td in writes)
             else:
                 base = op.tensor_description().base
                 if base in returned or isinstance(op, og.ReductionOp) or \
                         any(u not in inside for u in readers.get(base, ())):
-                    views.add(_view_key(op.tensor_description()))
-        return len(views)
+                    written.add(_view_key(op.tensor_description()))
+        self.n_written_views = len(written)
+        return len(views | written)
 
     def accepts(self, op, readers, returned):
         if not iteration_axes(op).is_equal_set(self.axes) or \
@@ -1091,6 +1094,8 @@ class _Group(object):
             # a reduction reads its argument through registers; its output must not be re-read here
             pass
         if self._memory_operands(op, readers, returned) > NGH_MAX_TENSORS:
+            return False
+        if self.n_written_views > self.max_written_views:
             return False
         if self.n_ops + 4 > NGH_MAX_OPS or self.n_consts + 2 > NGH_MAX_CONSTS:
             return False
@@ -1125,6 +1130,7 @@ class HipTransformer(ComputationGraphTransformer):
     default_atol = 1e-08
 
     kernel_group_class = HipKernelGroup
+    max_written_views = NGH_MAX_TENSORS      # results one fused kernel may write
 
     def __init__(self, device_id=0, fusion=True, dry_run=False, fuse_moments=None, rng_seed=0, **kwargs):
         """dry_run=True lowers graphs to kernel specs without a device (no results can be
