@@ -498,9 +498,11 @@ class FusedSpecBuilder(object):
         return len(self.consts) - 1
 
     def reg(self):
+        """A fresh symbolic register; build() renumbers them by liveness, and it is the
+        renumbered program that has to fit NGH_MAX_REGS."""
         self.n_regs += 1
-        if self.n_regs > NGH_MAX_REGS:
-            raise ValueError("too many registers in one fused kernel")
+        if self.n_regs > 255:
+            raise ValueError("too many values in one fused kernel")
         return self.n_regs - 1
 
     def emit(self, name, dst=0, a=0, b=0):
@@ -617,6 +619,8 @@ class FusedSpecBuilder(object):
             self.end_stage()
         if compact:
             self._compact_registers()
+        if self.n_regs > NGH_MAX_REGS:
+            raise ValueError("too many registers in one fused kernel (%d live values)" % self.n_regs)
         if len(self.stages) > NGH_MAX_STAGES:
             raise ValueError("too many stages in one fused kernel")
         spec = ngh_fused_spec()

@@ -1099,9 +1099,40 @@ class _Group(object):
             return False
         if self.n_ops + 4 > NGH_MAX_OPS or self.n_consts + 2 > NGH_MAX_CONSTS:
             return False
-        if self.n_ops // 4 + 1 > NGH_MAX_REGS - 4:
+        if self._max_live(self.ops + [op]) + 4 > NGH_MAX_REGS:
             return False
         return True
+
+    @staticmethod
+    def _max_live(ops):
+        """Upper estimate of the registers the group's program keeps alive at once: a value
+        (an op's result, or an operand loaded from memory at its first use) lives until its
+        last use inside the group; constants are loaded where they are used."""
+        index = {op: i for i, op in enumerate(ops)}
+        born, last = {}, {}
+        for i, op in enumerate(ops):
+            srcs = op.args[1:] if isinstance(op, og.AssignOp) else (() if isinstance(op, og.Fill) else op.args)
+            if isinstance(op, (og.RngOp,)):
+                srcs = ()
+            for a in srcs:
+                a = a.forwarded
+                if _scalar_constant_value(a) is not None:
+                    continue
+                prod = _producer(a)
+                key = prod if prod in index and index[prod] < i else _view_key(a.tensor_description())
+                born.setdefault(key, index[prod] if key is prod else i)
+                last[key] = i
+            born.setdefault(op, i)
+            last.setdefault(op, i)
+        events = [0] * (len(ops) + 1)
+        for key, b in born.items():
+            events[b] += 1
+            events[last[key]] -= 1          # dies at its last use: the result may take its register
+        live = peak = 0
+        for i in range(len(ops)):
+            live += events[i]
+            peak = max(peak, live + 3)      # + the op's transient constants and result
+        return peak
 
     def add(self, op):
         self.ops.append(op)

@@ -30,10 +30,24 @@ def test_backend_fails_loudly_without_a_gpu():
 
 
 def test_builder_limits_raise():
+    # 40 values alive at once do not fit the 32 registers of a program ...
     sb = FusedSpecBuilder([8])
+    t = sb.tensor(4096, [1])
+    regs = [sb.load(t) for _ in range(40)]
+    acc = regs[0]
+    for r in regs[1:]:
+        acc = sb.binary("add", acc, r)
+    sb.store(t, acc)
     with pytest.raises(ValueError):
-        for _ in range(40):
-            sb.reg()
+        sb.build()
+    # ... but 40 values of which few are alive together do
+    sb = FusedSpecBuilder([8])
+    t = sb.tensor(4096, [1])
+    acc = sb.load(t)
+    for _ in range(40):
+        acc = sb.unary("neg", acc)
+    sb.store(t, acc)
+    assert sb.build().n_regs <= 2
     with pytest.raises(ValueError):
         FusedSpecBuilder([2, 2, 2, 2])
     sb = FusedSpecBuilder([8])

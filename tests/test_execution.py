@@ -365,3 +365,38 @@ def test_computation_return_shapes_and_errors(backend):
     with pytest.raises(ValueError):
         ng.computation(a, x)                     # placeholder y not supplied
     t.close()
+
+
+def test_long_chains_split_into_several_kernels(backend):
+    """More ops, constants and distinct operands than one kernel spec holds: the planner has to
+    cut the group, and the pieces must still compute the same values."""
+    a = axes(A=33, B=70)
+    xs = [ng.placeholder(a) for _ in range(14)]             # more operands than a spec's 12 slots
+    vals = [rng.uniform(0.5, 1.5, a) for _ in xs]
+    acc, want = xs[0], vals[0].astype(np.float64)
+    for i in range(1, len(xs)):
+        acc = acc * (1.0 + 0.01 * i) + xs[i]                 # a new constant each step (> 16 in all)
+        want = want * (1.0 + 0.01 * i) + vals[i]
+    for j in range(60):                                      # and well over 96 ops
+        acc = ng.tanh(acc * 0.5) + (0.25 + 0.001 * j)
+        want = np.tanh(want * 0.5) + (0.25 + 0.001 * j)
+    with executor(acc, *xs) as f:
+        np.testing.assert_allclose(f(*vals), want, rtol=2e-5, atol=2e-6)
+
+
+def test_more_than_four_reductions_of_one_tensor(backend):
+    a = axes(R=50, N=40)
+    x = ng.placeholder(a)
+    xv = rng.uniform(0.5, 1.5, a)
+    outs = [ng.sum(x, out_axes=[a[1]]), ng.max(x, out_axes=[a[1]]), ng.min(x, out_axes=[a[1]]),
+            ng.prod(x * 0.9, out_axes=[a[1]]), ng.argmax(x, out_axes=[a[1]]), ng.argmin(x, out_axes=[a[1]]),
+            ng.sum(x * x, out_axes=[a[1]])]
+    with executor(outs, x) as f:
+        s, mx, mn, pr, am, an, ss = f(xv)
+    np.testing.assert_allclose(s, xv.sum(0), rtol=1e-5)
+    np.testing.assert_array_equal(mx, xv.max(0))
+    np.testing.assert_array_equal(mn, xv.min(0))
+    np.testing.assert_allclose(pr, (xv * np.float32(0.9)).prod(0), rtol=1e-4)
+    np.testing.assert_array_equal(am, xv.argmax(0))
+    np.testing.assert_array_equal(an, xv.argmin(0))
+    np.testing.assert_allclose(ss, (xv * xv).sum(0), rtol=1e-5)
