@@ -332,6 +332,10 @@ class ComputationGraphTransformer(Transformer):
             # state tensors are reached through reads / writes, not through deps
             for state in (op.states_read | op.states_written):
                 ensure_tensor(state)
+        # a parameter nothing reads still receives its argument at every call
+        for comp in self.computations:
+            for param in comp.computation_op.parameters:
+                ensure_tensor(param)
 
         self.start_transform_allocate()
         for device_buffer in self.device_buffers:

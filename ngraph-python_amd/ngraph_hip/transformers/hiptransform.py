@@ -360,6 +360,7 @@ class FusedKernel(HipKernel):
             return r
 
         red_slots = []
+        reductions_at_end = []
         for op in ops:
             name = kernel_op_name(op)
             if isinstance(op, og.AssignOp):
@@ -418,7 +419,8 @@ class FusedKernel(HipKernel):
                     else:
                         program.append(("assign", r, x))
                 else:
-                    program.append(("reduce", name, x, slot(op.tensor_description())))
+                    # reductions end the stage: collected here, emitted after every elementwise op
+                    reductions_at_end.append(("reduce", name, x, slot(op.tensor_description())))
                     red_slots.append(op)
                     continue
             elif name in og_unary_names:
@@ -432,6 +434,8 @@ class FusedKernel(HipKernel):
             value_reg[op] = r
             if op in self.store_ops:
                 program.append(("store", slot(op.tensor_description()), r))
+
+        program.extend(reductions_at_end)
 
         # ---- pass 2: dims = iteration axes with every operand's stride -----------------------
         def strides_over(td, axes):
@@ -1090,9 +1094,11 @@ class _Group(object):
             w = self.write_views.get(td.base)
             if w is not None and w != {td.parameter_key}:
                 return False
-        if is_red:
-            # a reduction reads its argument through registers; its output must not be re-read here
-            pass
+        if is_red and not self._reduced_axes_mergeable(op):
+            # the operands the fused kernel would read do not walk the reduced axes as one
+            # strided axis: leave the reduction to a kernel of its own, whose argument is a
+            # temporary in a layout that does (ReductionLayoutPass saw to that)
+            return False
         if self._memory_operands(op, readers, returned) > NGH_MAX_TENSORS:
             return False
         if self.n_written_views > self.max_written_views:
@@ -1101,6 +1107,34 @@ class _Group(object):
             return False
         if self._max_live(self.ops + [op]) + 4 > NGH_MAX_REGS:
             return False
+        return True
+
+    def _reduced_axes_mergeable(self, red_op):
+        """Can every memory operand of the group plus `red_op` walk red_op's reduced axes as ONE
+        strided axis, in one common axis order?  (The kernels reduce over a single axis.)"""
+        ops = self.ops + [red_op]
+        produced = set(op.tensor_description().base for op in ops
+                       if op.is_tensor_op and not isinstance(op, (og.AssignOp, og.Fill)))
+        tds = []
+        for op in ops:
+            for td in self._operand_views(op)[0]:
+                if td.base not in produced:
+                    tds.append(td)
+        red = [a for a in red_op.reduction_axes if a.length != 1]
+        if len(red) < 2:
+            return True
+
+        def strides(td):
+            return [td.full_strides[td.axes.index(a)] if a in td.axes else 0 for a in red]
+        rows = [strides(td) for td in tds]
+        rows = [r for r in rows if any(r)]
+        if not rows:
+            return True
+        order = sorted(range(len(red)), key=lambda i: tuple(-r[i] for r in rows))
+        for r in rows:
+            for i, j in zip(order[:-1], order[1:]):
+                if r[i] != r[j] * red[j].length:
+                    return False
         return True
 
     @staticmethod

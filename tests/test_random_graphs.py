@@ -1,0 +1,82 @@
+"""Randomly built graphs (fixed seeds): the HIP transformer against the NumPy oracle
+transformer on the same graph and inputs.  Exercises the fusion planner and the lowering on
+shapes nobody wrote by hand: broadcasts over axis subsets, reordered and sliced views,
+reductions over several axes feeding further elementwise ops, results shared by several
+consumers."""
+import numpy as np
+import pytest
+
+import ngraph_hip as ng
+import ngraph_hip.transformers as ngt
+import oracle.cpu_transformer  # noqa: F401
+
+UNARY = [ng.tanh, ng.negative, ng.absolute, ng.square, ng.sigmoid, lambda x: ng.sqrt(ng.absolute(x) + 0.5),
+         lambda x: ng.exp(x * 0.25), lambda x: ng.log(ng.absolute(x) + 1.0), ng.sign]
+BINARY = [ng.add, ng.subtract, ng.multiply, ng.maximum, ng.minimum, lambda a, b: a / (ng.absolute(b) + 1.0),
+          lambda a, b: ng.greater(a, b), lambda a, b: ng.less_equal(a, b)]
+REDUCE = [ng.sum, ng.max, ng.min, ng.mean]
+
+
+def build(seed):
+    rs = np.random.RandomState(seed)
+    n_axes = rs.randint(2, 5)
+    lengths = [int(rs.choice([1, 2, 3, 5, 8, 16, 33])) for _ in range(n_axes)]
+    all_axes = [ng.make_axis(n, name="ax%d_%d" % (seed, i)) for i, n in enumerate(lengths)]
+    inputs, values = [], []
+    for _ in range(rs.randint(2, 5)):
+        k = rs.randint(1, n_axes + 1)
+        idx = sorted(rs.choice(n_axes, size=k, replace=False))
+        if rs.rand() < 0.4:
+            idx = list(rs.permutation(idx))                       # stored in another axis order
+        axes = [all_axes[i] for i in idx]
+        inputs.append(ng.placeholder(axes))
+        values.append(rs.uniform(-2, 2, [a.length for a in axes]).astype(np.float32))
+    pool = list(inputs)
+    for _ in range(rs.randint(4, 14)):
+        kind = rs.rand()
+        if kind < 0.35:
+            x = pool[rs.randint(len(pool))]
+            node = UNARY[rs.randint(len(UNARY))](x)
+        elif kind < 0.8:
+            a, b = pool[rs.randint(len(pool))], pool[rs.randint(len(pool))]
+            node = BINARY[rs.randint(len(BINARY))](a, b)
+        else:
+            x = pool[rs.randint(len(pool))]
+            if len(x.axes) == 0:
+                continue
+            k = rs.randint(1, len(x.axes) + 1)
+            red = [x.axes[i] for i in sorted(rs.choice(len(x.axes), size=k, replace=False))]
+            node = REDUCE[rs.randint(len(REDUCE))](x, reduction_axes=ng.make_axes(red))
+        pool.append(node)
+    results = [pool[-1]] + [pool[i] for i in rs.choice(np.arange(len(inputs), len(pool)), size=min(2, len(pool) - len(inputs)),
+                                                       replace=False)]
+    return results, inputs, values
+
+
+def run(backend, results, inputs, values, **kwargs):
+    t = ngt.make_transformer_factory(backend, **kwargs)()
+    try:
+        f = t.computation(results, *inputs)
+        return [np.array(r) for r in f(*values)]
+    finally:
+        t.close()
+
+
+@pytest.mark.parametrize("seed", range(200))
+def test_oracle_transformer_agrees_with_itself_unfused(seed):
+    """CPU-only sanity of the generator: every graph builds and evaluates on the oracle."""
+    results, inputs, values = build(seed)
+    out = run("cpu", results, inputs, values)
+    assert all(np.isfinite(o).all() for o in out)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fusion", [True, False], ids=["fused", "unfused"])
+@pytest.mark.parametrize("seed", range(200))
+def test_random_graph_matches_oracle(seed, fusion):
+    results, inputs, values = build(seed)
+    want = run("cpu", results, inputs, values)
+    got = run("hipgpu", results, inputs, values, fusion=fusion)
+    for g, w in zip(got, want):
+        assert g.shape == w.shape
+        np.testing.assert_allclose(g, w, rtol=2e-5, atol=2e-5)
