@@ -1094,7 +1094,7 @@ class _Group(object):
             w = self.write_views.get(td.base)
             if w is not None and w != {td.parameter_key}:
                 return False
-        if is_red and not self._reduced_axes_mergeable(op):
+        if is_red and not self._reduced_axes_mergeable(op, readers, returned):
             # the operands the fused kernel would read do not walk the reduced axes as one
             # strided axis: leave the reduction to a kernel of its own, whose argument is a
             # temporary in a layout that does (ReductionLayoutPass saw to that)
@@ -1109,17 +1109,26 @@ class _Group(object):
             return False
         return True
 
-    def _reduced_axes_mergeable(self, red_op):
-        """Can every memory operand of the group plus `red_op` walk red_op's reduced axes as ONE
-        strided axis, in one common axis order?  (The kernels reduce over a single axis.)"""
+    def _reduced_axes_mergeable(self, red_op, readers, returned):
+        """Can every memory operand of the group plus `red_op` -- what it reads from outside and
+        the elementwise results it has to write out -- walk red_op's reduced axes as ONE strided
+        axis, in one common axis order?  (The kernels reduce over a single axis.)"""
         ops = self.ops + [red_op]
+        inside = set(ops)
         produced = set(op.tensor_description().base for op in ops
                        if op.is_tensor_op and not isinstance(op, (og.AssignOp, og.Fill)))
         tds = []
         for op in ops:
-            for td in self._operand_views(op)[0]:
+            reads, writes = self._operand_views(op)
+            for td in reads:
                 if td.base not in produced:
                     tds.append(td)
+            if isinstance(op, (og.AssignOp, og.Fill)):
+                tds.extend(writes)
+            elif not isinstance(op, og.ReductionOp):
+                base = op.tensor_description().base
+                if base in returned or any(u not in inside for u in readers.get(base, ())):
+                    tds.append(op.tensor_description())
         red = [a for a in red_op.reduction_axes if a.length != 1]
         if len(red) < 2:
             return True

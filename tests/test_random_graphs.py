@@ -80,3 +80,79 @@ def test_random_graph_matches_oracle(seed, fusion):
     for g, w in zip(got, want):
         assert g.shape == w.shape
         np.testing.assert_allclose(g, w, rtol=2e-5, atol=2e-5)
+
+
+# ------------------------------------------------------------------ second generator: larger shapes, views
+def build_views(seed):
+    """Larger tensors (vector, tiled and multi-segment kernels get chosen), up to five axes (the
+    host loops over what does not fit three), sliced and reordered views as operands, argmax /
+    prod reductions with explicit out_axes orders."""
+    rs = np.random.RandomState(seed)
+    n_axes = rs.randint(2, 6)
+    lengths = [int(rs.choice([1, 2, 3, 4, 8, 16, 32, 64, 100])) for _ in range(n_axes)]
+    while np.prod(lengths) > 400000:
+        lengths[int(np.argmax(lengths))] //= 2
+    all_axes = [ng.make_axis(n, name="bx%d_%d" % (seed, i)) for i, n in enumerate(lengths)]
+    inputs, values, pool = [], [], []
+    for _ in range(rs.randint(2, 4)):
+        k = rs.randint(max(1, n_axes - 2), n_axes + 1)
+        idx = list(rs.permutation(n_axes)[:k]) if rs.rand() < 0.5 else sorted(rs.choice(n_axes, size=k, replace=False))
+        axes = [all_axes[i] for i in idx]
+        p = ng.placeholder(axes)
+        inputs.append(p)
+        values.append(rs.uniform(-2, 2, [a.length for a in axes]).astype(np.float32))
+        view = p
+        if rs.rand() < 0.5 and len(axes) > 1:
+            view = ng.axes_with_order(view, [axes[i] for i in rs.permutation(len(axes))])
+        pool.append(view)
+    # a sliced operand: a window of the first input along its first axis, renamed so it can
+    # only meet operands through its other axes
+    first = inputs[0]
+    if first.axes[0].length >= 4:
+        lo = int(rs.randint(0, first.axes[0].length // 2))
+        hi = int(rs.randint(lo + 1, first.axes[0].length + 1))
+        sl = ng.tensor_slice(first, [slice(lo, hi)] + [slice(None)] * (len(first.axes) - 1))
+        pool.append(ng.sum(sl, reduction_axes=ng.make_axes([sl.axes[0]])) if len(sl.axes) > 1 else ng.sum(sl))
+    for _ in range(rs.randint(5, 12)):
+        kind = rs.rand()
+        if kind < 0.3:
+            node = UNARY[rs.randint(len(UNARY))](pool[rs.randint(len(pool))])
+        elif kind < 0.75:
+            node = BINARY[rs.randint(len(BINARY))](pool[rs.randint(len(pool))], pool[rs.randint(len(pool))])
+        else:
+            x = pool[rs.randint(len(pool))]
+            if len(x.axes) == 0:
+                continue
+            which = rs.rand()
+            if which < 0.25:
+                node = ng.argmax(x, reduction_axes=ng.make_axes([x.axes[rs.randint(len(x.axes))]]))
+            elif which < 0.4:
+                node = ng.prod(x * 0.5, reduction_axes=ng.make_axes([x.axes[rs.randint(len(x.axes))]]))
+            else:
+                k = rs.randint(1, len(x.axes) + 1)
+                red = [x.axes[i] for i in sorted(rs.choice(len(x.axes), size=k, replace=False))]
+                kept = [a for a in x.axes if a not in red]
+                out_axes = [kept[i] for i in rs.permutation(len(kept))]
+                node = REDUCE[rs.randint(len(REDUCE))](x, out_axes=ng.make_axes(out_axes))
+        pool.append(node)
+    n_in = len(inputs)
+    picks = rs.choice(np.arange(n_in, len(pool)), size=min(3, len(pool) - n_in), replace=False)
+    return [pool[-1]] + [pool[i] for i in picks], inputs, values
+
+
+@pytest.mark.parametrize("seed", range(1000, 1100))
+def test_view_graphs_evaluate_on_the_oracle(seed):
+    results, inputs, values = build_views(seed)
+    run("cpu", results, inputs, values)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(1000, 1100))
+def test_random_view_graph_matches_oracle(seed):
+    results, inputs, values = build_views(seed)
+    want = run("cpu", results, inputs, values)
+    got = run("hipgpu", results, inputs, values)
+    for g, w in zip(got, want):
+        assert g.shape == w.shape
+        ok = np.isfinite(w)
+        np.testing.assert_allclose(g[ok], w[ok], rtol=1e-4, atol=1e-4)
