@@ -152,9 +152,19 @@ class FlexFusedKernel(FusedKernel):
     def execute_managed(self, rt, dev_table, count):
         if not hasattr(self, "_id_arrays"):
             ids = [e.flex_id for e in self.output_flex_entries]
-            self._id_arrays = rt.make_id_arrays(ids, [1 if i in self.in_place_flex_ids else 0 for i in ids])
+            in_place = [1 if i in self.in_place_flex_ids else 0 for i in ids]
+            self._id_lists = (ids, in_place)
+            self._id_arrays = rt.make_id_arrays(ids, in_place)
+        if len(self.specs) == 1:
+            rt.launch_fused_flex(self.specs[0], dev_table, self._id_arrays, count)
+            return
+        # several launches cover one set of tensors (an outer axis looped on the host): one
+        # exponent for all of them, statistics merged over all of them
+        ids, in_place = self._id_lists
+        rt.flex_prepare(dev_table, ids, in_place)
         for spec in self.specs:
-            rt.launch_fused_flex(spec, dev_table, self._id_arrays, count)
+            rt.launch_fused(spec)
+        rt.flex_update(dev_table, ids, count)
 
     def probe(self):
         """Measure max|fp32 result| of every not yet initialised output without storing."""

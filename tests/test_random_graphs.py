@@ -156,3 +156,96 @@ def test_random_view_graph_matches_oracle(seed):
         assert g.shape == w.shape
         ok = np.isfinite(w)
         np.testing.assert_allclose(g[ok], w[ok], rtol=1e-4, atol=1e-4)
+
+
+# ------------------------------------------------------------------ third generator: state
+def build_state(seed):
+    """Sequences of assignments to a few variables (whole tensors and row windows), each value an
+    expression of the variables' current contents and an input: in-place updates, reads after
+    writes, writes after reads -- what the planner's hazard rules exist for."""
+    rs = np.random.RandomState(seed)
+    A = ng.make_axis(int(rs.choice([4, 16, 33])), name="sa%d" % seed)
+    B = ng.make_axis(int(rs.choice([8, 64, 100])), name="sb%d" % seed)
+    init = [rs.uniform(-1, 1, (A.length, B.length)).astype(np.float32) for _ in range(3)]
+    variables = [ng.variable([A, B], initial_value=v) for v in init]
+    x = ng.placeholder([A, B])
+    xv = rs.uniform(-1, 1, (A.length, B.length)).astype(np.float32)
+
+    def expr(depth=0):
+        if depth > 2 or rs.rand() < 0.3:
+            return variables[rs.randint(3)] if rs.rand() < 0.7 else x
+        if rs.rand() < 0.4:
+            return [ng.tanh, ng.negative, ng.absolute, lambda t: t * 0.5][rs.randint(4)](expr(depth + 1))
+        return [ng.add, ng.subtract, ng.multiply, ng.maximum][rs.randint(4)](expr(depth + 1), expr(depth + 1))
+
+    steps = []
+    for _ in range(rs.randint(3, 9)):
+        target = variables[rs.randint(3)]
+        value = expr()
+        if not hasattr(value, "axes") or len(value.axes) != 2:
+            continue
+        if rs.rand() < 0.3 and A.length >= 4:
+            lo = int(rs.randint(0, A.length - 2))
+            hi = int(rs.randint(lo + 1, A.length + 1))
+            window = [slice(lo, hi), slice(None)]
+            tgt = ng.tensor_slice(target, window)
+            val = ng.cast_axes(ng.tensor_slice(value, window), tgt.axes)
+            steps.append(ng.assign(tgt, val))
+        else:
+            steps.append(ng.assign(target, value))
+    total = ng.sum(variables[0] + variables[1] * 2.0 + variables[2] * 3.0, out_axes=())
+    return ng.sequential(steps + [total]), variables, x, xv
+
+
+def run_state(backend, seed, **kwargs):
+    prog, variables, x, xv = build_state(seed)
+    t = ngt.make_transformer_factory(backend, **kwargs)()
+    try:
+        f = t.computation(prog, x)
+        read = t.computation([v * 1.0 for v in variables])
+        totals = [np.array(f(xv)).copy(), np.array(f(xv * 0.5)).copy()]
+        return totals, [np.array(r) for r in read()]
+    finally:
+        t.close()
+
+
+@pytest.mark.parametrize("seed", range(2000, 2060))
+def test_state_programs_evaluate_on_the_oracle(seed):
+    run_state("cpu", seed)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fusion", [True, False], ids=["fused", "unfused"])
+@pytest.mark.parametrize("seed", range(2000, 2060))
+def test_random_state_program_matches_oracle(seed, fusion):
+    want_tot, want_vars = run_state("cpu", seed)
+    got_tot, got_vars = run_state("hipgpu", seed, fusion=fusion)
+    for g, w in zip(got_vars, want_vars):
+        np.testing.assert_allclose(g, w, rtol=2e-5, atol=2e-5)
+    for g, w in zip(got_tot, want_tot):
+        np.testing.assert_allclose(g, w, rtol=1e-4, atol=1e-3)
+
+
+# ------------------------------------------------------------------ flex: host-managed vs device-resident
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(120))
+def test_flex_random_graph_host_and_device_management_agree(seed):
+    """The same flex graph run three times with growing inputs under host-managed and under
+    device-resident exponent management: results (dequantised values) must agree bit for bit,
+    call after call."""
+    def run_flex(resident):
+        results, inputs, values = build(seed)
+        t = ngt.make_transformer_factory("flexhip", resident=resident)()
+        try:
+            f = t.computation(results, *inputs)
+            out = []
+            for gain in (1.0, 3.0, 0.25):
+                out.append([np.array(r).copy() for r in f(*[v * np.float32(gain) for v in values])])
+            return out
+        finally:
+            t.close()
+
+    host, device = run_flex(False), run_flex(True)
+    for call, (h, d) in enumerate(zip(host, device)):
+        for a, b in zip(h, d):
+            np.testing.assert_array_equal(a, b, err_msg="call %d" % call)
