@@ -249,3 +249,44 @@ def test_flex_random_graph_host_and_device_management_agree(seed):
     for call, (h, d) in enumerate(zip(host, device)):
         for a, b in zip(h, d):
             np.testing.assert_array_equal(a, b, err_msg="call %d" % call)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(2000, 2050))
+def test_flex_state_program_host_and_device_management_agree(seed):
+    """Assignment programs (in-place updates keep their exponent for the kernel that reads and
+    writes them) under both management modes: identical variables after two calls."""
+    def run_flex(resident):
+        prog, variables, x, xv = build_state(seed)
+        t = ngt.make_transformer_factory("flexhip", resident=resident)()
+        try:
+            f = t.computation(prog, x)
+            read = t.computation([v * 1.0 for v in variables])
+            totals = [np.array(f(xv)).copy(), np.array(f(xv * 4.0)).copy(), np.array(f(xv * 0.1)).copy()]
+            return totals, [np.array(r) for r in read()]
+        finally:
+            t.close()
+
+    (h_tot, h_vars), (d_tot, d_vars) = run_flex(False), run_flex(True)
+    for a, b in zip(h_vars, d_vars):
+        np.testing.assert_array_equal(a, b)
+    for a, b in zip(h_tot, d_tot):
+        np.testing.assert_array_equal(a, b)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(1000, 1040))
+def test_flex_view_graph_host_and_device_management_agree(seed):
+    def run_flex(resident):
+        results, inputs, values = build_views(seed)
+        t = ngt.make_transformer_factory("flexhip", resident=resident)()
+        try:
+            f = t.computation(results, *inputs)
+            return [[np.array(r).copy() for r in f(*[v * np.float32(g) for v in values])] for g in (1.0, 2.5, 0.2)]
+        finally:
+            t.close()
+
+    host, device = run_flex(False), run_flex(True)
+    for h, d in zip(host, device):
+        for a, b in zip(h, d):
+            np.testing.assert_array_equal(a, b)
