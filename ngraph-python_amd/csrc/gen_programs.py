@@ -74,6 +74,14 @@ def _reduction_pattern(fn, out_axis):
     return build
 
 
+def _reduction_of(expr, out_axis, n_in=1):
+    def build(t):
+        A, B = _axes(A=4096, B=4096)
+        xs = [ng.placeholder([A, B]) for _ in range(n_in)]
+        return t.computation(expr(*xs, out_axes=[A if out_axis == 0 else B]), *xs)
+    return build
+
+
 def pattern_lstm_cell(t, Hn=1024, Nn=64):
     # LSTM cell on transposed storage (frontends/neon/layer.py:1630-1647): inputs contiguous
     # along H, results along N -- the tiled skeleton
@@ -113,6 +121,12 @@ PATTERNS = [
     ("sum_across", "hipgpu", _reduction_pattern(ng.sum, 1)),
     ("max_along", "hipgpu", _reduction_pattern(ng.max, 0)),
     ("max_across", "hipgpu", _reduction_pattern(ng.max, 1)),
+    ("argmax_along", "hipgpu", _reduction_pattern(ng.argmax, 0)),
+    ("argmax_across", "hipgpu", _reduction_pattern(ng.argmax, 1)),
+    ("sum_of_squares_along", "hipgpu", _reduction_of(lambda x, out_axes: ng.sum(x * x, out_axes=out_axes), 0)),
+    ("sum_of_squares_across", "hipgpu", _reduction_of(lambda x, out_axes: ng.sum(x * x, out_axes=out_axes), 1)),
+    ("dot_along", "hipgpu", _reduction_of(lambda x, y, out_axes: ng.sum(x * y, out_axes=out_axes), 0, 2)),
+    ("dot_across", "hipgpu", _reduction_of(lambda x, y, out_axes: ng.sum(x * y, out_axes=out_axes), 1, 2)),
     ("sum_across_small", "hipgpu", pattern_lstm_bias_gradient),
     ("lstm_cell", "hipgpu", pattern_lstm_cell),
     # the planner orders ops of large tensors differently (nothing above 65536 elements is
