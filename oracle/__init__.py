@@ -9,8 +9,9 @@ it follows.
 
 Pinning status (what checks each restatement beyond itself):
   numpy_ops.py      closed forms: each entry IS the NumPy ufunc call the CPU
-                    transformer emits; tests/test_oracle_ops.py checks every
-                    entry against float64 references and textbook identities.
+                    transformer emits; tests/test_cabi_fused_gpu.py and
+                    tests/test_execution.py check them against float64 references
+                    and NumPy expressions written in each test.
   configs.py        BatchNorm / Adam / LSTM pinned against independent float64
                     restatements of the reference's own test references
                     (neon/tests/test_batchnorm_layer.py:35-58,
@@ -21,8 +22,8 @@ Pinning status (what checks each restatement beyond itself):
                     Exponent policy (next_dec): the reference delegates it to
                     the private `autoflex` package, which is not in the tree;
                     PARITY UNPINNED at source level, pinned at the boundary by
-                    the golden vectors; mismatching vectors are listed in
-                    tests/golden/flex_policy_xfail.json.
+                    all 154 vectors the reference itself enables (the 9 it
+                    disables are flagged inside the fixture).
   cpu_transformer.py evaluates op graphs op by op with numpy_ops; pinned by the
                     NumPy expressions written in each test, as the reference's
                     own tests do.
