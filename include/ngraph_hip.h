@@ -55,6 +55,13 @@ extern "C" {
 #define NGH_FLEX16  1          /* int16 mantissa, shared per-tensor scale   */
 #define NGH_I32     2          /* int32 (argmax / argmin results, indices)  */
 #define NGH_F16     3          /* IEEE half in memory, float in registers   */
+/* Integer storage: converted to float on load; a store converts toward zero and
+ * saturates at the type's range (the device conversion the reference's generated
+ * "(type)reg" assignment compiles to).  Values are exact up to 2^24.            */
+#define NGH_U32     4          /* uint32                                    */
+#define NGH_I16     5          /* int16 (plain integers, no scale)          */
+#define NGH_I8      6          /* int8                                      */
+#define NGH_U8      7          /* uint8 (image bytes on the loader side)    */
 
 /* ---- spec flags ---------------------------------------------------------
  * NGH_SPEC_PROBE: run the program but store NOTHING; instead every FLEX16
@@ -132,7 +139,7 @@ typedef struct ngh_op {
 typedef struct ngh_tensor {
     void*    dev;              /* device address of view element (0,0,0)     */
     int64_t  strides[NGH_MAX_AXES];
-    int32_t  dtype;            /* NGH_F32 / NGH_FLEX16 / NGH_I32 / NGH_F16   */
+    int32_t  dtype;            /* one of the NGH_* storage types            */
     float    scale;            /* FLEX16 only: the tensor's scale 2**-dec.
                                   Loaded value = scale * int16; stored int16 =
                                   rni_sat(value * (1/scale)).  The reference
@@ -210,7 +217,7 @@ int  ngh_memset16(ngh_context* ctx, void* dev, uint16_t value, size_t count);
 
 /* ---- strided copy / dimshuffle: replaces _get_copy_transpose_kernel
  *      (copy_transpose.py:89-282) and DimShuffleKernel (tensor_ops.py:137-204).
- *      Copies an N-d view (rank <= 8) element by element; itemsize 2 or 4.   */
+ *      Copies an N-d view (rank <= 8) element by element; itemsize 1, 2 or 4. */
 int  ngh_copy_strided(ngh_context* ctx, void* dev_dst, const void* dev_src,
                       int32_t rank, const int64_t* shape,
                       const int64_t* dst_strides, const int64_t* src_strides,

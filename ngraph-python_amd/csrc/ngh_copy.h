@@ -202,8 +202,9 @@ inline hipError_t launch_copy_t(hipStream_t stream, int cus, void* dst, const vo
 
 inline hipError_t launch_copy(hipStream_t stream, int cus, void* dst, const void* src, const CopyArgs& a,
                               int itemsize) {
-    return itemsize == 2 ? launch_copy_t<uint16_t>(stream, cus, dst, src, a)
-                         : launch_copy_t<uint32_t>(stream, cus, dst, src, a);
+    return itemsize == 1   ? launch_copy_t<uint8_t>(stream, cus, dst, src, a)
+           : itemsize == 2 ? launch_copy_t<uint16_t>(stream, cus, dst, src, a)
+                           : launch_copy_t<uint32_t>(stream, cus, dst, src, a);
 }
 
 }  // namespace ngh

@@ -213,8 +213,18 @@ __device__ __forceinline__ float load1(const KTensor& t, long long off, float sc
         case NGH_FLEX16: return scale * (float)reinterpret_cast<const short*>(t.p)[off];
         case NGH_I32:    return (float)reinterpret_cast<const int*>(t.p)[off];
         case NGH_F16:    return __half2float(reinterpret_cast<const __half*>(t.p)[off]);
+        case NGH_U32:    return (float)reinterpret_cast<const unsigned*>(t.p)[off];
+        case NGH_I16:    return (float)reinterpret_cast<const short*>(t.p)[off];
+        case NGH_I8:     return (float)reinterpret_cast<const signed char*>(t.p)[off];
+        case NGH_U8:     return (float)reinterpret_cast<const unsigned char*>(t.p)[off];
         default:         return 0.0f;
     }
+}
+
+// float -> integer storage: toward zero, saturating at the type's range, NaN -> 0
+// (what the hardware conversion does for 32-bit results; narrower types clamp first).
+__device__ __forceinline__ int to_int_sat(float v, float lo, float hi) {
+    return (int)fminf(fmaxf(v, lo), hi);
 }
 
 __device__ __forceinline__ void store1(const KTensor& t, long long off, float v, float scale, int& fmax) {
@@ -227,6 +237,10 @@ __device__ __forceinline__ void store1(const KTensor& t, long long off, float v,
         } break;
         case NGH_I32: reinterpret_cast<int*>(t.p)[off] = (int)v; break;
         case NGH_F16: reinterpret_cast<__half*>(t.p)[off] = __float2half(v); break;
+        case NGH_U32: reinterpret_cast<unsigned*>(t.p)[off] = (unsigned)v; break;
+        case NGH_I16: reinterpret_cast<short*>(t.p)[off] = (short)to_int_sat(v, -32768.0f, 32767.0f); break;
+        case NGH_I8:  reinterpret_cast<signed char*>(t.p)[off] = (signed char)to_int_sat(v, -128.0f, 127.0f); break;
+        case NGH_U8:  reinterpret_cast<unsigned char*>(t.p)[off] = (unsigned char)to_int_sat(v, 0.0f, 255.0f); break;
         default: break;
     }
 }
@@ -254,6 +268,24 @@ __device__ __forceinline__ void load4(const KTensor& t, long long off, float sca
             float2 fa = __half22float2(a), fb = __half22float2(b);
             v[0] = fa.x; v[1] = fa.y; v[2] = fb.x; v[3] = fb.y;
         } break;
+        case NGH_U32: {
+            uint4 x = *reinterpret_cast<const uint4*>(reinterpret_cast<const unsigned*>(t.p) + off);
+            v[0] = (float)x.x; v[1] = (float)x.y; v[2] = (float)x.z; v[3] = (float)x.w;
+        } break;
+        case NGH_I16: {
+            short4 x = *reinterpret_cast<const short4*>(reinterpret_cast<const short*>(t.p) + off);
+            v[0] = (float)x.x; v[1] = (float)x.y; v[2] = (float)x.z; v[3] = (float)x.w;
+        } break;
+        case NGH_I8: {
+            const unsigned w = *reinterpret_cast<const unsigned*>(t.p + off);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = (float)(signed char)((w >> (8 * j)) & 0xffu);
+        } break;
+        case NGH_U8: {
+            const unsigned w = *reinterpret_cast<const unsigned*>(t.p + off);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = (float)((w >> (8 * j)) & 0xffu);
+        } break;
         default: v[0] = v[1] = v[2] = v[3] = 0.0f;
     }
 }
@@ -278,6 +310,28 @@ __device__ __forceinline__ void store4(const KTensor& t, long long off, float sc
             __half2 a = __floats2half2_rn(v[0], v[1]), b = __floats2half2_rn(v[2], v[3]);
             uint2 raw; raw.x = *reinterpret_cast<unsigned*>(&a); raw.y = *reinterpret_cast<unsigned*>(&b);
             *reinterpret_cast<uint2*>(reinterpret_cast<__half*>(t.p) + off) = raw;
+        } break;
+        case NGH_U32:
+            *reinterpret_cast<uint4*>(reinterpret_cast<unsigned*>(t.p) + off) =
+                make_uint4((unsigned)v[0], (unsigned)v[1], (unsigned)v[2], (unsigned)v[3]);
+            break;
+        case NGH_I16: {
+            short4 x;
+            x.x = (short)to_int_sat(v[0], -32768.0f, 32767.0f); x.y = (short)to_int_sat(v[1], -32768.0f, 32767.0f);
+            x.z = (short)to_int_sat(v[2], -32768.0f, 32767.0f); x.w = (short)to_int_sat(v[3], -32768.0f, 32767.0f);
+            *reinterpret_cast<short4*>(reinterpret_cast<short*>(t.p) + off) = x;
+        } break;
+        case NGH_I8: {
+            unsigned w = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) w |= ((unsigned)to_int_sat(v[j], -128.0f, 127.0f) & 0xffu) << (8 * j);
+            *reinterpret_cast<unsigned*>(t.p + off) = w;
+        } break;
+        case NGH_U8: {
+            unsigned w = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) w |= ((unsigned)to_int_sat(v[j], 0.0f, 255.0f) & 0xffu) << (8 * j);
+            *reinterpret_cast<unsigned*>(t.p + off) = w;
         } break;
         default: break;
     }

@@ -52,8 +52,9 @@ int fail(int code, const char* fmt, ...) {
 
 int itemsize_of(int dtype) {
     switch (dtype) {
-        case NGH_F32: case NGH_I32: return 4;
-        case NGH_FLEX16: case NGH_F16: return 2;
+        case NGH_F32: case NGH_I32: case NGH_U32: return 4;
+        case NGH_FLEX16: case NGH_F16: case NGH_I16: return 2;
+        case NGH_I8: case NGH_U8: return 1;
         default: return 0;
     }
 }
@@ -890,7 +891,8 @@ int ngh_copy_strided(ngh_context* ctx, void* dev_dst, const void* dev_src, int32
                      int32_t itemsize) {
     if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
     if (rank < 0 || rank > kCopyMaxRank) return fail(NGH_E_INVALID, "rank %d not in 0..%d", rank, kCopyMaxRank);
-    if (itemsize != 2 && itemsize != 4) return fail(NGH_E_INVALID, "itemsize %d (2 or 4)", itemsize);
+    if (itemsize != 1 && itemsize != 2 && itemsize != 4)
+        return fail(NGH_E_INVALID, "itemsize %d (1, 2 or 4)", itemsize);
     if (rank && (!shape || !dst_strides || !src_strides)) return fail(NGH_E_INVALID, "NULL shape/strides");
     CopyArgs a;
     memset(&a, 0, sizeof(a));

@@ -1398,6 +1398,10 @@ def lookuptable(lut, idx, axes, update=True, pad_idx=None):
     return LookupTableOp(lut, idx, axes=axes, update=update, pad_idx=pad_idx)
 
 
+class UnmatchedAxesError(ValueError):
+    """y and t of a cross entropy do not broadcast to matching axes."""
+
+
 class SigmoidOp(ValueOp):
     """sigmoid as the composite reciprocal(exp(-x) + 1) (op_graph.py:4183-4202)."""
 
@@ -1405,22 +1409,86 @@ class SigmoidOp(ValueOp):
         super(SigmoidOp, self).__init__(**kwargs)
         self.x = x
         self.value_tensor = reciprocal(exp(-x) + 1)
+        self.value_tensor.deriv_handler = self
 
 
 def sigmoid(x):
-    return SigmoidOp(x).value_tensor
+    return SigmoidOp(as_op(x)).value_tensor
 
 
 def sigmoidAtomic(x):
     return SigmoidAtomicOp(x)
 
 
+class SoftmaxOp(ValueOp):
+    """softmax as exp(x - max x) / sum of the same (op_graph.py:3819-3846).  The
+    composite is kept reachable from its value (`deriv_handler`) so that a cross
+    entropy can use the shifted input and the normaliser directly."""
+
+    def __init__(self, x, normalization_axes=None, **kwargs):
+        super(SoftmaxOp, self).__init__(**kwargs)
+        if normalization_axes is None:
+            rec = x.axes.recurrent_axis()
+            normalization_axes = x.axes.sample_axes() - (
+                make_axes(rec) if rec is not None else make_axes(()))
+        self.x = x - max(x, reduction_axes=normalization_axes)
+        self.exps = exp(self.x)
+        self.Z = sum(self.exps, reduction_axes=normalization_axes)
+        self.value_tensor = self.exps * reciprocal(self.Z)
+        self.value_tensor.deriv_handler = self
+
+
 def softmax(x, normalization_axes=None, **kwargs):
-    # op_graph.py:3819-3850
-    x = as_op(x)
-    if normalization_axes is None:
-        rec = x.axes.recurrent_axis()
-        normalization_axes = x.axes.sample_axes() - (make_axes(rec) if rec is not None else make_axes(()))
-    x = x - max(x, reduction_axes=normalization_axes)
-    exps = exp(x)
-    return exps * reciprocal(sum(exps, reduction_axes=normalization_axes))
+    return SoftmaxOp(as_op(x), normalization_axes, **kwargs).value_tensor
+
+
+def _check_cross_entropy_axes(y, t):
+    if (not y.axes.is_sub_set(t.axes)) and (not y.axes.is_super_set(t.axes)):
+        raise UnmatchedAxesError(
+            "y and t must broadcast to matching axes: {} vs. {}".format(y.axes, t.axes))
+
+
+def cross_entropy_multi(y, t, usebits=False, out_axes=None, enable_softmax_opt=True,
+                        enable_diff_opt=True):
+    """Cross entropy of the distributions y (model) and t (truth), summed over the
+    sample axes that are not recurrent (op_graph.py:4318-4390).  When y is a
+    softmax, -sum(x t) + log Z on the shifted input replaces -sum(t log y); this
+    relies on sum(t) == 1, as the reference's shortcut does."""
+    y, t = as_op(y), as_op(t)
+    _check_cross_entropy_axes(y, t)
+    if out_axes is None:
+        rec = y.axes.recurrent_axis()
+        index_axes = y.axes.sample_axes() - (make_axes(rec) if rec is not None else make_axes(()))
+        out_axes = y.axes - index_axes
+    handler = getattr(y, "deriv_handler", None)
+    if enable_softmax_opt and isinstance(handler, SoftmaxOp):
+        s = -sum(handler.x * t, out_axes=out_axes)
+        value = minimum(s + log(handler.Z), safelog_cutoff)
+    else:
+        value = -sum(safelog(y) * t, out_axes=out_axes)
+    if usebits:
+        value = value * float(1.0 / np.log(2.0))
+    return value
+
+
+def cross_entropy_binary_inner(y, t, enable_sig_opt=True, enable_diff_opt=True):
+    """Per-element binary cross entropy -(t log y + (1 - t) log(1 - y))
+    (op_graph.py:4392-4451).  When y is a sigmoid of x the equivalent
+    (1 - t) max(x, -cutoff) - log y is built instead."""
+    y, t = as_op(y), as_op(t)
+    _check_cross_entropy_axes(y, t)
+    handler = getattr(y, "deriv_handler", None)
+    if enable_sig_opt and isinstance(handler, SigmoidOp):
+        return (1 - t) * maximum(handler.x, -safelog_cutoff) - safelog(y)
+    return -(safelog(y) * t + safelog(1 - y) * (1 - t))
+
+
+def cross_entropy_binary(y, t, usebits=False, out_axes=None, enable_sig_opt=True,
+                         enable_diff_opt=True):
+    """Binary cross entropy summed over the sample axes (op_graph.py:4454-4478)."""
+    result = sum(cross_entropy_binary_inner(y, t, enable_sig_opt=enable_sig_opt,
+                                            enable_diff_opt=enable_diff_opt),
+                 out_axes=out_axes)
+    if usebits:
+        result = result * float(1.0 / np.log(2.0))
+    return result

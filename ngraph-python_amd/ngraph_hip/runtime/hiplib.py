@@ -22,6 +22,7 @@ NGH_MAX_REDUCTIONS = 4
 NGH_MAX_STAGES = 6
 
 NGH_F32, NGH_FLEX16, NGH_I32, NGH_F16 = 0, 1, 2, 3
+NGH_U32, NGH_I16, NGH_I8, NGH_U8 = 4, 5, 6, 7
 NGH_SPEC_PROBE = 1
 NGH_CACHE_STREAM_LOAD, NGH_CACHE_STREAM_STORE = 1, 2
 
@@ -171,7 +172,8 @@ def _check(lib, rc):
         raise HipLibraryError(rc, msg.decode("utf-8", "replace") if msg else "")
 
 
-_NP_DTYPES = {NGH_F32: np.float32, NGH_FLEX16: np.int16, NGH_I32: np.int32, NGH_F16: np.float16}
+_NP_DTYPES = {NGH_F32: np.float32, NGH_FLEX16: np.int16, NGH_I32: np.int32, NGH_F16: np.float16,
+              NGH_U32: np.uint32, NGH_I16: np.int16, NGH_I8: np.int8, NGH_U8: np.uint8}
 
 
 class DeviceArray(object):
@@ -280,7 +282,9 @@ class HipRuntime(object):
         host = np.asarray(host)
         if ngh_dtype is None:
             ngh_dtype = {np.dtype(np.float32): NGH_F32, np.dtype(np.int16): NGH_FLEX16,
-                         np.dtype(np.int32): NGH_I32, np.dtype(np.float16): NGH_F16}[host.dtype]
+                         np.dtype(np.int32): NGH_I32, np.dtype(np.float16): NGH_F16,
+                         np.dtype(np.uint32): NGH_U32, np.dtype(np.int8): NGH_I8,
+                         np.dtype(np.uint8): NGH_U8}[host.dtype]
         return DeviceArray(self, host.shape, ngh_dtype).set(host)
 
     def copy_strided(self, dst, src, shape, dst_strides, src_strides, itemsize):

@@ -28,7 +28,8 @@ import numpy as np
 from ngraph_hip.op_graph import op_graph as og
 from ngraph_hip.op_graph.op_graph import Op, OrderedSet
 from ngraph_hip.runtime.hiplib import (HipRuntime, DryRunRuntime, HipLibraryError, FusedSpecBuilder, NGH_F32,
-                                       NGH_FLEX16, NGH_I32, NGH_F16, NGH_MAX_TENSORS,
+                                       NGH_FLEX16, NGH_I32, NGH_F16, NGH_U32, NGH_I16, NGH_I8, NGH_U8,
+                                       NGH_MAX_TENSORS,
                                        NGH_MAX_OPS, NGH_MAX_CONSTS, NGH_MAX_REGS,
                                        NGH_MAX_REDUCTIONS, NGH_CACHE_STREAM_LOAD,
                                        NGH_CACHE_STREAM_STORE)
@@ -1228,12 +1229,12 @@ class HipTransformer(ComputationGraphTransformer):
     def ngh_dtype(self, dtype):
         if not isinstance(dtype, np.dtype):
             return NGH_FLEX16
-        if dtype == np.float32:
-            return NGH_F32
-        if dtype == np.int32:
-            return NGH_I32
-        if dtype == np.float16:
-            return NGH_F16
+        # float_ew2.py:615-641 lists the storage types a compound kernel may touch
+        for np_type, code in ((np.float32, NGH_F32), (np.int32, NGH_I32), (np.float16, NGH_F16),
+                              (np.uint32, NGH_U32), (np.int16, NGH_I16), (np.int8, NGH_I8),
+                              (np.uint8, NGH_U8)):
+            if dtype == np_type:
+                return code
         raise TypeError("hipgpu: unsupported tensor dtype %s" % dtype)
 
     def flex_entry_of(self, tensor_description):

@@ -585,3 +585,54 @@ def test_convert_between_fp32_and_flex16(hip_runtime, n):
     for d in (x_d, q_d, back_d):
         d.free()
     rt.free(stats)
+
+
+INT_TYPES = [("NGH_I32", np.int32), ("NGH_U32", np.uint32), ("NGH_I16", np.int16), ("NGH_I8", np.int8),
+             ("NGH_U8", np.uint8)]
+
+
+@pytest.mark.parametrize("type_name,np_type", INT_TYPES)
+@pytest.mark.parametrize("shape", [(4096,), (7, 33), (3, 64, 48)])
+def test_integer_storage_types(hip_runtime, type_name, np_type, shape):
+    """Integer tensors are converted to float on load and back on store (float_ew2.py:615-641
+    declares the same storage types).  A store truncates toward zero and saturates at the
+    type's range; inside the range that is NumPy's astype, which is what the CPU transformer
+    does."""
+    import ngraph_hip.runtime as runtime
+    code = getattr(runtime, type_name)
+    rt = hip_runtime
+    info = np.iinfo(np_type)
+    lo, hi = max(info.min, -(1 << 20)), min(info.max, 1 << 20)      # exact in fp32
+    rs = np.random.RandomState(len(shape) + info.bits)
+    src = rs.randint(lo, hi + 1, size=shape).astype(np_type)
+    x = rs.uniform(-1.5, 1.5, size=shape).astype(f32) * f32(min(hi, 1 << 15))
+    st = contiguous_strides(shape)
+    src_d, x_d = rt.array(src, code), rt.array(x)
+    as_float_d, as_int_d = rt.empty(shape), rt.empty(shape, code)
+    sb = FusedSpecBuilder(shape)
+    v = sb.load(sb.tensor(src_d.ptr, st, code))
+    sb.store(sb.tensor(as_float_d.ptr, st), sb.binary("mul", v, sb.constant(0.5)))
+    sb.store(sb.tensor(as_int_d.ptr, st, code), sb.load(sb.tensor(x_d.ptr, st)))
+    rt.launch_fused(sb.build())
+    np.testing.assert_array_equal(as_float_d.get(), src.astype(f32) * f32(0.5))
+    want = np.clip(np.trunc(x.astype(np.float64)), info.min, info.max).astype(np_type)
+    np.testing.assert_array_equal(as_int_d.get(), want)
+    inside = (x > info.min) & (x < info.max)
+    np.testing.assert_array_equal(as_int_d.get()[inside], x[inside].astype(np_type))
+    for d in (src_d, x_d, as_float_d, as_int_d):
+        d.free()
+
+
+@pytest.mark.parametrize("np_type", [np.int8, np.uint8])
+def test_byte_views_copy(hip_runtime, np_type):
+    """The strided copy moves 1-byte elements too (transposed and sliced views)."""
+    rt = hip_runtime
+    rs = np.random.RandomState(5)
+    src = rs.randint(0, 100, size=(70, 130)).astype(np_type)
+    import ngraph_hip.runtime as runtime
+    code = runtime.NGH_I8 if np_type is np.int8 else runtime.NGH_U8
+    src_d, dst_d = rt.array(src), rt.empty((130, 70), code)
+    rt.copy_strided(dst_d.ptr, src_d.ptr, (130, 70), (70, 1), (1, 130), 1)
+    np.testing.assert_array_equal(dst_d.get(), src.T)
+    src_d.free()
+    dst_d.free()

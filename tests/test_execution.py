@@ -400,3 +400,129 @@ def test_more_than_four_reductions_of_one_tensor(backend):
     np.testing.assert_array_equal(am, xv.argmax(0))
     np.testing.assert_array_equal(an, xv.argmin(0))
     np.testing.assert_allclose(ss, (xv * xv).sum(0), rtol=1e-5)
+
+
+# ---- cross entropies (reference tests/transformer_dependent/test_execution.py:584-598, 786-813, 863-897)
+
+def _np_softmax(x, axis):
+    e = np.exp(x - x.max(axis=axis, keepdims=True))
+    return e / e.sum(axis=axis, keepdims=True)
+
+
+def test_cross_entropy_binary_logistic_shortcut(backend):
+    C, N = ng.make_axis(3, name="C"), ng.make_axis(8, name="N")
+    p_u, p_v = ng.placeholder([C, N]), ng.placeholder([C, N])
+    u = rng.uniform(-3.0, 3.0, p_u.axes)
+    v = _np_softmax(rng.uniform(-3.0, 3.0, p_u.axes), 0).astype(np.float32)
+    y = 1.0 / (1.0 + np.exp(-u.astype(np.float64)))
+    want = -(v * np.log(y) + (1.0 - v) * np.log(1.0 - y))
+    short = ng.cross_entropy_binary_inner(ng.sigmoid(p_u), p_v)
+    plain = ng.cross_entropy_binary_inner(ng.sigmoid(p_u), p_v, enable_sig_opt=False)
+    total = ng.cross_entropy_binary(ng.sigmoid(p_u), p_v, usebits=True)
+    with executor([short, plain, total], p_u, p_v) as f:
+        s, p, tot = f(u, v)
+    np.testing.assert_allclose(s, want, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(p, want, rtol=1e-4, atol=1e-6)
+    np.testing.assert_allclose(tot, want.sum(axis=0) / np.log(2.0), rtol=1e-5)
+
+
+@pytest.mark.parametrize("recurrent", [False, True])
+def test_cross_entropy_softmax(backend, recurrent):
+    C, N = ng.make_axis(3, name="C"), ng.make_axis(8, name="N")
+    ax = [C, ng.make_axis(4, name="REC"), N] if recurrent else [C, N]
+    p_x, p_t = ng.placeholder(ax), ng.placeholder(ax)
+    x = rng.uniform(0, 1, p_x.axes)
+    t = _np_softmax(rng.uniform(0, 1, p_t.axes), 0).astype(np.float32)
+    want = -(np.log(_np_softmax(x.astype(np.float64), 0)) * t).sum(axis=0)
+    short = ng.cross_entropy_multi(ng.softmax(p_x), p_t)
+    plain = ng.cross_entropy_multi(ng.softmax(p_x), p_t, enable_softmax_opt=False)
+    with executor([short, plain], p_x, p_t) as f:
+        s, p = f(x, t)
+    assert s.shape == want.shape
+    np.testing.assert_allclose(s, want, rtol=1e-5)
+    np.testing.assert_allclose(p, want, rtol=1e-5)
+
+
+def test_cross_entropy_softmax_large_input(backend):
+    C, N = ng.make_axis(3, name="C"), ng.make_axis(8, name="N")
+    p_x, p_t = ng.placeholder([C, N]), ng.placeholder([C, N])
+    r = np.random.RandomState(3)
+    x = (np.eye(3)[r.choice(3, 8)].T * rng.uniform(-10, 10, p_x.axes) * 25).astype(np.float32)
+    t = np.eye(3)[r.choice(3, 8)].T.astype(np.float32)
+    x64 = x.astype(np.float64)
+    logsm = x64 - x64.max(axis=0) - np.log(np.exp(x64 - x64.max(axis=0)).sum(axis=0))
+    want = np.minimum(-(logsm * t).sum(axis=0), 50.0)
+    with executor(ng.cross_entropy_multi(ng.softmax(p_x), p_t), p_x, p_t) as f:
+        np.testing.assert_allclose(f(x, t), want, atol=1e-7, rtol=1e-4)
+
+
+def test_cross_entropy_axis_checks_and_order(backend):
+    C, N = ng.make_axis(5, name="C"), ng.make_axis(8, name="N")
+    y = ng.placeholder([C, N])
+    with pytest.raises(ng.UnmatchedAxesError):
+        ng.cross_entropy_multi(y, ng.placeholder([ng.make_axis(5), N]))
+    with pytest.raises(ng.UnmatchedAxesError):
+        ng.cross_entropy_binary_inner(y, ng.placeholder([ng.make_axis(5), N]))
+    t1, t2 = ng.placeholder([C, N]), ng.placeholder([N, C])
+    yv = rng.uniform(0, 1, y.axes)
+    t1v = np.eye(8, dtype=np.float32)[:5, :]
+    with executor([ng.cross_entropy_multi(ng.softmax(y), t1),
+                   ng.cross_entropy_multi(ng.softmax(y), t2)], y, t1, t2) as f:
+        a, b = f(yv, t1v, np.ascontiguousarray(t1v.T))
+    np.testing.assert_allclose(a, b, rtol=1e-6)
+
+
+# ---- small forward cases (reference test_execution.py:990-1065, 1122-1150, 1208-1216)
+
+def test_clip(backend):
+    a = axes(W=4, H=5)
+    p_x = ng.placeholder(a)
+    x = (2 * rng.uniform(0, 1, a) - 1) * 20
+    with executor(ng.minimum(ng.maximum(p_x, -10), 10), p_x) as f:
+        np.testing.assert_array_equal(f(x), np.clip(x, -10, 10))
+
+
+def test_elementwise_fp16_in_and_out(backend):
+    a = axes(A=2, B=2)
+    h1 = ng.constant(np.array([[1.0, 2.0], [4.0, 12.0]], dtype="float16"), a, dtype=np.dtype(np.float16))
+    h2 = ng.constant(np.array([[1.0, 2.0], [6.0, 12.0]], dtype="float16"), a, dtype=np.dtype(np.float16))
+    f1 = ng.constant(np.array([[1.0, 2.0], [4.0, 12.0]], dtype="float32"), a)
+    f2 = ng.constant(np.array([[1.0, 2.0], [6.0, 12.0]], dtype="float32"), a)
+    with executor([ng.multiply(h1, h2), ng.multiply(f1, f2, dtype=np.dtype(np.float16))]) as f:
+        r_in, r_out = f()
+    np.testing.assert_array_equal(r_in, [[1.0, 4.0], [24.0, 144.0]])
+    np.testing.assert_array_equal(r_out, [[1.0, 4.0], [24.0, 144.0]])
+    assert r_out.dtype == np.float16
+
+
+def test_fill_slice(backend):
+    a = axes(A=2, B=8)
+    x = ng.placeholder(a)
+    b = ng.sequential([ng.fill(x[:, 1], 0), ng.value_of(x)])
+    with executor(b, x) as f:
+        got = f(np.array([[1, 2, 3, 4, 5, 6, 7, 8], [8, 7, 6, 5, 4, 3, 2, 1]], dtype=np.float32))
+    np.testing.assert_array_equal(got, [[1, 0, 3, 4, 5, 6, 7, 8], [8, 0, 6, 5, 4, 3, 2, 1]])
+
+
+def test_empty_transformer_initializes(backend):
+    t = ngt.make_transformer()
+    t.initialize()
+    t.close()
+
+
+def test_variance_sqrt_inverse_forward(backend):
+    C, N = ng.make_axis(7, name="C"), ng.make_axis(16, name="N")
+    x, tg = ng.placeholder([C, N]), ng.placeholder([C, N])
+    stat = ng.reciprocal(ng.sqrt(ng.variance(x, reduction_axes=x.axes.batch_axes()) + 1e-3))
+    err = ng.sum(stat - tg, out_axes=())
+    xv, tv = rng.uniform(-1, 1, x.axes), rng.uniform(-1, 1, x.axes)
+    with executor(err, x, tg) as f:
+        got = f(xv, tv)
+    want = np.sum(1.0 / np.sqrt(np.var(xv.astype(np.float64), axis=1, keepdims=True) + 1e-3) - tv)
+    np.testing.assert_allclose(got, want, atol=1e-4, rtol=1e-4)
+
+
+def test_multiply_uint32_scalar(backend):
+    x = ng.placeholder((), dtype=np.uint32)
+    with executor(0.5 * x * 0.5, x) as f:
+        assert f(1) == 0.25
