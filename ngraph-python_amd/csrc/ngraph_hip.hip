@@ -96,6 +96,8 @@ struct ngh_context {
 // ---------------------------------------------------------------------------
 namespace {
 
+constexpr long long kMaxStageElems = 1LL << 33;
+
 int validate(const ngh_fused_spec* sp) {
     if (!sp) return fail(NGH_E_INVALID, "spec is NULL");
     if (sp->abi_version != NGH_ABI_VERSION)
@@ -105,6 +107,8 @@ int validate(const ngh_fused_spec* sp) {
     for (int a = 0; a < NGH_MAX_AXES; ++a) {
         if (sp->shape[a] < 0) return fail(NGH_E_INVALID, "negative shape on axis %d", a);
         if (a >= sp->rank && sp->shape[a] != 1) return fail(NGH_E_INVALID, "axis %d beyond rank must have length 1", a);
+        if (sp->shape[a] > kMaxStageElems || (sp->shape[a] > 0 && total > kMaxStageElems / sp->shape[a]))
+            return fail(NGH_E_UNSUPPORTED, "iteration space exceeds 2^33 elements");
         total *= sp->shape[a];
     }
     if (sp->n_tensors < 0 || sp->n_tensors > NGH_MAX_TENSORS) return fail(NGH_E_INVALID, "n_tensors %d", sp->n_tensors);
@@ -117,8 +121,13 @@ int validate(const ngh_fused_spec* sp) {
         if (itemsize_of(T.dtype) == 0) return fail(NGH_E_INVALID, "tensor %d: unknown dtype %d", t, T.dtype);
         if (total > 0 && T.dev == nullptr) return fail(NGH_E_INVALID, "tensor %d: NULL device pointer", t);
         if (((uintptr_t)T.dev) % itemsize_of(T.dtype)) return fail(NGH_E_INVALID, "tensor %d: misaligned pointer", t);
-        for (int a = 0; a < NGH_MAX_AXES; ++a)
+        __int128 reach = 0;      // byte offset of the last element the view can name
+        for (int a = 0; a < NGH_MAX_AXES; ++a) {
             if (T.strides[a] < 0) return fail(NGH_E_UNSUPPORTED, "tensor %d: negative stride", t);
+            if (sp->shape[a] > 1) reach += (__int128)(sp->shape[a] - 1) * T.strides[a];
+        }
+        if (reach * itemsize_of(T.dtype) >= ((__int128)1 << 47))
+            return fail(NGH_E_UNSUPPORTED, "tensor %d: view spans more than 2^47 bytes", t);
     }
     int next = 0;
     for (int s = 0; s < sp->n_stages; ++s) {
@@ -328,7 +337,7 @@ int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage,
     stage_tensors(sp, S, loads, stores);
     for (int t = 0; t < NGH_MAX_TENSORS; ++t) used[t] = loads[t] || stores[t];
     long long total = sp.shape[0] * sp.shape[1] * sp.shape[2];
-    if (total >= (1LL << 31) * 4LL) return fail(NGH_E_UNSUPPORTED, "stage view of %lld elements exceeds 2^33", total);
+    if (total >= kMaxStageElems) return fail(NGH_E_UNSUPPORTED, "stage view of %lld elements exceeds 2^33", total);
 
     if (S.n_reductions == 0) {
         // fast axis = the one along which most memory traffic is contiguous: every
@@ -897,10 +906,17 @@ int ngh_copy_strided(ngh_context* ctx, void* dev_dst, const void* dev_src, int32
     CopyArgs a;
     memset(&a, 0, sizeof(a));
     long long total = 1;
+    bool empty = false;
+    for (int i = 0; i < rank; ++i) {
+        if (shape[i] < 0) return fail(NGH_E_INVALID, "negative shape");
+        empty = empty || shape[i] == 0;
+    }
+    if (empty) return NGH_OK;
     // drop length-1 axes, merge axes that are contiguous in both views
     int r = 0;
     for (int i = 0; i < rank; ++i) {
-        if (shape[i] < 0) return fail(NGH_E_INVALID, "negative shape");
+        if (shape[i] >= (1LL << 31) || total > (1LL << 31) / shape[i])
+            return fail(NGH_E_UNSUPPORTED, "copy of more than 2^31 elements; split it");
         total *= shape[i];
         if (shape[i] == 1) continue;
         if (r > 0 && a.ds[r - 1] == dst_strides[i] * shape[i] && a.ss[r - 1] == src_strides[i] * shape[i]) {
@@ -912,7 +928,6 @@ int ngh_copy_strided(ngh_context* ctx, void* dev_dst, const void* dev_src, int32
             ++r;
         }
     }
-    if (total == 0) return NGH_OK;
     if (!dev_dst || !dev_src) return fail(NGH_E_INVALID, "NULL device pointer");
     // 32-bit element counters with grid-stride steps: stay well inside the range
     if (total >= (1LL << 31)) return fail(NGH_E_UNSUPPORTED, "copy of %lld elements; split it", total);

@@ -150,23 +150,39 @@ def test_misaligned_and_broadcast_operands(hip_runtime):
 @gpu
 @pytest.mark.parametrize("shape", [(5, 7, 11), (64, 64), (128, 70), (3, 130, 66), (2, 3, 4, 5), (256, 192),
                                    (4, 96, 200), (8, 1024)])
-@pytest.mark.parametrize("itemsize", [4, 2])
+@pytest.mark.parametrize("itemsize", [4, 2, 1])
 def test_strided_copy_all_permutations(hip_runtime, shape, itemsize):
     """Dimshuffle: every axis permutation against numpy.transpose (tensor_ops.py:137-204)."""
+    from ngraph_hip.runtime import NGH_U8
     rt = hip_runtime
-    dt = np.float32 if itemsize == 4 else np.int16
-    src = (np.arange(int(np.prod(shape))) % 30011).astype(dt).reshape(shape)
-    s_d = rt.array(src, NGH_F32 if itemsize == 4 else NGH_FLEX16)
+    dt = {4: np.float32, 2: np.int16, 1: np.uint8}[itemsize]
+    code = {4: NGH_F32, 2: NGH_FLEX16, 1: NGH_U8}[itemsize]
+    src = (np.arange(int(np.prod(shape))) % (251 if itemsize == 1 else 30011)).astype(dt).reshape(shape)
+    s_d = rt.array(src, code)
     perms = list(itertools.permutations(range(len(shape))))
     for perm in perms[:: max(1, len(perms) // 8)] + [perms[-1]]:
         want = np.ascontiguousarray(src.transpose(perm))
-        d_d = rt.empty(want.shape, NGH_F32 if itemsize == 4 else NGH_FLEX16)
+        d_d = rt.empty(want.shape, code)
         src_strides = [src.strides[p] // itemsize for p in perm]
         dst_strides = [s // itemsize for s in want.strides]
         rt.copy_strided(d_d.ptr, s_d.ptr, want.shape, dst_strides, src_strides, itemsize)
         np.testing.assert_array_equal(d_d.get(), want)
         d_d.free()
     s_d.free()
+
+
+@gpu
+def test_strided_copy_argument_checks(hip_runtime):
+    from ngraph_hip.runtime import HipLibraryError
+    rt = hip_runtime
+    a = rt.empty((16,))
+    rt.copy_strided(a.ptr, a.ptr, (1 << 40, 0, 3), (0, 0, 1), (0, 0, 1), 4)       # empty: nothing to do
+    for shape in [(1 << 62, 4), (1 << 31, 1), (1 << 16, 1 << 16), (-1, 4)]:
+        with pytest.raises(HipLibraryError):
+            rt.copy_strided(a.ptr, a.ptr, shape, (0, 1), (0, 1), 4)
+    with pytest.raises(HipLibraryError):
+        rt.copy_strided(a.ptr, a.ptr, (4,), (1,), (1,), 8)
+    a.free()
 
 
 @gpu
