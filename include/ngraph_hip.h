@@ -287,9 +287,18 @@ int  ngh_flex_update(ngh_context* ctx, ngh_flex_state* dev, const int32_t* ids, 
                      int32_t count);
 
 /* ngh_flex_prepare + ngh_launch_fused + ngh_flex_update in one call (one host transition per
- * kernel instead of three).                                                            */
+ * kernel instead of three; flexgputransform.py:347-366 is the loop it replaces).  When a
+ * pre-built streaming kernel covers the spec, the library may go further and leave the
+ * statistics of the launch unfolded: the next launch that writes the same tensors folds them
+ * in its first instructions, and every other entry point that reads or writes a record, or
+ * launches a kernel whose operands point into one, first brings it up to date.  A record read
+ * through ngh_flex_states_read is therefore always current; device memory of a table must not
+ * be copied out by other means while ngh_flex_unsettled reports a non-zero count.          */
 int  ngh_launch_fused_flex(ngh_context* ctx, const ngh_fused_spec* spec, ngh_flex_state* dev,
                            const int32_t* ids, const int32_t* in_place, int32_t n_ids, int32_t count);
+/* number of records whose statistics are still unfolded (no counterpart in the reference,
+ * whose policy runs on the host after every kernel)                                        */
+int  ngh_flex_unsettled(ngh_context* ctx, int32_t* out_count);
 
 /* ---- timing (HIP events on the context's stream; used by the bench) ----- */
 int  ngh_timer_begin(ngh_context* ctx);

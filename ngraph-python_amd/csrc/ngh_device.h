@@ -31,6 +31,17 @@ struct KTensor {
     int          pad_;
 };
 
+// One statistics slot of a launch with deferred statistics (see ngh_flex.h).
+struct FlexLazySlot {
+    const ngh_flex_state*     in;         // page holding the record as of the previous write
+    ngh_flex_state*           out;        // page this launch leaves the record in
+    const unsigned long long* words_in;   // group words of the previous write, NULL = nothing pending
+    unsigned long long*       words_out;
+    unsigned                  tag_in, tag_out;
+    int                       count_in;   // the previous write's `count`
+    int                       in_place;
+};
+
 struct KArgs {
     long long shape[3];
     int       n_tensors, op_begin, op_end, n_regs;
@@ -50,6 +61,10 @@ struct KArgs {
     int       flex_count;
     unsigned* tickets;              // arrival counters, zero between launches
     int*      group_max;            // per slot and group: merged max|mantissa|, zero between launches
+    int          flex_lazy;         // != 0: deferred statistics, lazy[] is set instead of flex_state[];
+                                    // the value is the number of compute units
+    FlexLazySlot lazy[4];
+    int          lazy_blocks_per_cu;
     KTensor   t[NGH_MAX_TENSORS];
     float     consts[NGH_MAX_CONSTS];
     ngh_op    ops[NGH_MAX_OPS];

@@ -7,13 +7,14 @@
 // scales from it and merge statistics into it, and two one-wavefront kernels apply the
 // exponent policy on the device, so a sequence of flex kernels runs without the host.
 //
-// The arithmetic below is written as explicit sequential double-precision steps because the
+// The policy arithmetic is a sequence of double-precision steps, each rounded once, because the
 // host mirror (ngraph_hip/flex/hipflex.py, _policy_step) executes the same steps in the same
-// order; the two must stay line-for-line equivalent.
+// order; the two must stay equivalent (the library is built with -ffp-contract=off).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include "ngraph_hip.h"
+#include "ngh_device.h"
 
 namespace ngh {
 
@@ -46,40 +47,109 @@ __device__ __forceinline__ int flex_write_dec(const ngh_flex_state& s, int in_pl
     return (!in_place && s.initialized && s.next_dec >= 0) ? s.next_dec : s.dec;
 }
 
-// After a write with s.dec / s.scale: record max|mantissa| and choose the next exponent.
-__device__ inline void flex_policy_record(ngh_flex_state& s, int maxabs, int count) {
-    s.last_maxabs = maxabs;
-    s.last_count = count;
-    s.initialized = 1;
-    const double value = (double)maxabs * (double)s.scale;
-    int pos = s.hist_pos;
-    if (maxabs >= kFlexPclip) {
-        s.history[pos] = 2.0 * value;
-        s.hist_pos = (pos + 1) % NGH_FLEX_HISTORY;
-        if (s.hist_len < NGH_FLEX_HISTORY) s.hist_len += 1;
-        const int d = s.dec - 2;
-        s.next_dec = d < kFlexMinDec ? kFlexMinDec : d;
-        return;
+// The record's scalar fields, as a kernel holds them while it works on a record.
+struct FlexFields {
+    int   stats, dec, next_dec, initialized;
+    float scale;
+    int   hist_len, hist_pos, last_maxabs, last_count;
+};
+
+// Entry j of a value held one per lane, as a wavefront-uniform number (j is the same in
+// every lane).
+__device__ __forceinline__ double flex_lane_value(double v, int j) {
+    const int lo = __builtin_amdgcn_readlane(__double2loint(v), j);
+    const int hi = __builtin_amdgcn_readlane(__double2hiint(v), j);
+    return __hiloint2double(hi, lo);
+}
+
+// After a write with f.dec / f.scale: record max|mantissa| and choose the next exponent.
+// One wavefront with all 64 lanes active works on a record: every lane holds the same fields,
+// lane j (j < NGH_FLEX_HISTORY) holds entry j of the ring of recent maxima in `h`.  The sums
+// run over the entries in index order, one rounding per step, exactly as the host mirror's
+// loops do; only the per-entry work (subtracting the mean, squaring) is done by all lanes at
+// once.
+__device__ __forceinline__ void flex_policy_step(FlexFields& f, double& h, int maxabs, int count) {
+    const int lane = threadIdx.x & 63;
+    const int dec_now = f.dec;
+    const double value = (double)maxabs * (double)f.scale;
+    const int pos = f.hist_pos;
+    const bool clipped = maxabs >= kFlexPclip;
+    if (lane == pos) h = clipped ? 2.0 * value : value;
+    const int n = f.hist_len < NGH_FLEX_HISTORY ? f.hist_len + 1 : NGH_FLEX_HISTORY;
+    int next_dec;
+    if (clipped) {
+        const int d = dec_now - 2;
+        next_dec = d < kFlexMinDec ? kFlexMinDec : d;
+    } else {
+        // Rolled loops on purpose: this code runs once per launch with a cold instruction cache,
+        // and fetching a long unrolled sequence costs more than executing it.
+        double mx = flex_lane_value(h, 0), sum = 0.0;
+#pragma unroll 1
+        for (int j = 0; j < n; ++j) {
+            const double hj = flex_lane_value(h, j);
+            mx = hj > mx ? hj : mx;
+            sum = sum + hj;
+        }
+        const double mean = sum / (double)n;
+        const double d = h - mean;
+        const double dd = d * d;
+        double ss = 0.0;
+#pragma unroll 1
+        for (int j = 0; j < n; ++j) ss = ss + flex_lane_value(dd, j);
+        const double sd = sqrt(ss / (double)n);
+        const int dec = flex_fit_dec(mx + 3.0 * sd);
+        next_dec = dec < 0 ? dec_now : dec;
     }
-    s.history[pos] = value;
-    s.hist_pos = (pos + 1) % NGH_FLEX_HISTORY;
-    if (s.hist_len < NGH_FLEX_HISTORY) s.hist_len += 1;
-    const int n = s.hist_len;
-    double mx = s.history[0], sum = 0.0;
-    for (int j = 0; j < n; ++j) {
-        const double h = s.history[j];
-        mx = h > mx ? h : mx;
-        sum = sum + h;
-    }
-    const double mean = sum / (double)n;
-    double ss = 0.0;
-    for (int j = 0; j < n; ++j) {
-        const double d = s.history[j] - mean;
-        ss = ss + d * d;
-    }
-    const double sd = sqrt(ss / (double)n);
-    const int dec = flex_fit_dec(mx + 3.0 * sd);
-    s.next_dec = dec < 0 ? s.dec : dec;
+    f.last_maxabs = maxabs;
+    f.last_count = count;
+    f.initialized = 1;
+    f.hist_pos = (pos + 1) % NGH_FLEX_HISTORY;
+    f.hist_len = n;
+    f.next_dec = next_dec;
+}
+
+__device__ __forceinline__ FlexFields flex_fields_of(const ngh_flex_state& s) {
+    FlexFields f;
+    f.stats = s.stats; f.dec = s.dec; f.next_dec = s.next_dec; f.initialized = s.initialized;
+    f.scale = s.scale; f.hist_len = s.hist_len; f.hist_pos = s.hist_pos;
+    f.last_maxabs = s.last_maxabs; f.last_count = s.last_count;
+    return f;
+}
+
+__device__ __forceinline__ void flex_fields_to(ngh_flex_state& s, const FlexFields& f) {
+    s.stats = f.stats; s.dec = f.dec; s.next_dec = f.next_dec; s.initialized = f.initialized;
+    s.scale = f.scale; s.hist_len = f.hist_len; s.hist_pos = f.hist_pos;
+    s.last_maxabs = f.last_maxabs; s.last_count = f.last_count;
+}
+
+// A record as one wavefront holds it.
+struct FlexInWave {
+    FlexFields f;
+    double     h;       // lane j < NGH_FLEX_HISTORY: ring entry j
+};
+
+__device__ __forceinline__ FlexInWave flex_wave_load(const ngh_flex_state& s) {
+    FlexInWave r;
+    r.f = flex_fields_of(s);
+    r.h = s.history[threadIdx.x & (NGH_FLEX_HISTORY - 1)];
+    return r;
+}
+
+__device__ __forceinline__ void flex_wave_store(ngh_flex_state& s, const FlexInWave& r) {
+    const int lane = threadIdx.x & 63;
+    if (lane == 0) flex_fields_to(s, r.f);
+    if (lane < NGH_FLEX_HISTORY) s.history[lane] = r.h;
+}
+
+// whole wavefront: policy step on a record in memory
+__device__ __forceinline__ void flex_policy_record(ngh_flex_state& s, int maxabs, int count) {
+    FlexInWave r = flex_wave_load(s);
+    flex_policy_step(r.f, r.h, maxabs, count);
+    flex_wave_store(s, r);
+}
+
+__device__ __forceinline__ int flex_write_dec(const FlexFields& f, int in_place) {
+    return (!in_place && f.initialized && f.next_dec >= 0) ? f.next_dec : f.dec;
 }
 
 // Before a kernel: outputs that are fully overwritten take the exponent the policy chose;
@@ -96,11 +166,10 @@ __global__ void flex_prepare_kernel(ngh_flex_state* st, const FlexIds ids) {
     s.stats = 0;
 }
 
-// After a kernel: record max|mantissa| and choose the next exponent.
-__global__ void flex_update_kernel(ngh_flex_state* st, const FlexIds ids, int count) {
-    const int i = threadIdx.x;
-    if (i >= ids.n) return;
-    ngh_flex_state& s = st[ids.id[i]];
+// After a kernel: record max|mantissa| and choose the next exponent.  One wavefront per id.
+__global__ __launch_bounds__(64) void flex_update_kernel(ngh_flex_state* st, const FlexIds ids, int count) {
+    if ((int)blockIdx.x >= ids.n) return;
+    ngh_flex_state& s = st[ids.id[blockIdx.x]];
     flex_policy_record(s, s.stats, count);
 }
 
@@ -177,15 +246,106 @@ __device__ __forceinline__ void flex_epilogue(ngh_flex_state* const (&state)[4],
         }
 #pragma unroll
         for (int d = 32; d > 0; d >>= 1) gm = max(gm, __shfl_xor(gm, d, 64));
-        if (lane == 0) {
-            ngh_flex_state& st = *state[s];
-            const int dec = flex_write_dec(st, in_place[s]);
-            st.dec = dec;
-            st.scale = flex_scale_of(dec);
-            st.stats = gm;
-            flex_policy_record(st, gm, count);
-        }
+        FlexInWave r = flex_wave_load(*state[s]);
+        const int dec = flex_write_dec(r.f, in_place[s]);
+        r.f.dec = dec;
+        r.f.scale = flex_scale_of(dec);
+        r.f.stats = gm;
+        flex_policy_step(r.f, r.h, gm, count);
+        flex_wave_store(*state[s], r);
     }
+}
+
+// ---------------------------------------------------------------------------
+// Deferred statistics: no work at all after the last store.
+//
+// flex_epilogue's chain of dependent atomics runs after the slowest workgroup has finished
+// streaming, so it adds to every launch.  Here a workgroup only sends its max|mantissa| to one
+// of kFlexGroups words with an atomic that returns nothing, and the fold and the policy step
+// are done by whoever needs the record next: the prologue of the next kernel that writes the
+// tensor (every workgroup computes the same new record in registers, workgroup 0 stores it),
+// or flex_settle_kernel when something else is about to look at the record.
+//
+// A record therefore has two pages (the ABI's record, and a shadow) and two sets of group
+// words.  A launch reads one page and one set and writes the other page and the other set, so
+// no workgroup of a launch reads anything another workgroup of the same launch writes.  Words
+// carry the write's sequence number in their upper half: a word left by an older write
+// compares lower and reads as "no contribution", so the sets never need clearing.
+// ---------------------------------------------------------------------------
+constexpr int kFlexWordPad = 16;                                  // 64-bit words per 128-byte line
+constexpr int kFlexWordsPerSet = kFlexGroups * kFlexWordPad;
+constexpr int kFlexWordsPerRecord = 2 * kFlexWordsPerSet;
+
+// What a wavefront holds of a record between asking for it and needing it.
+struct FlexLazyLoaded {
+    FlexInWave         r;
+    unsigned long long word;    // this lane's group word of the pending write
+};
+
+// Issue the loads of a record and of the pending group words (one word per lane).
+__device__ __forceinline__ void flex_lazy_fetch(const FlexLazySlot& a, FlexLazyLoaded& l) {
+    l.r = flex_wave_load(*a.in);
+    // the words were written by the previous kernel's atomics and by nobody in this launch: an
+    // ordinary (cacheable) load sees them, and thousands of workgroups asking do not all go to
+    // memory
+    l.word = a.words_in ? a.words_in[(threadIdx.x & 63) * kFlexWordPad] : 0ull;
+}
+
+// Fold what is pending into the record (whole wavefront).
+__device__ __forceinline__ void flex_lazy_fold(const FlexLazySlot& a, FlexLazyLoaded& l) {
+    if (!a.words_in) return;
+    int gm = ((unsigned)(l.word >> 32) == a.tag_in) ? (int)(unsigned)(l.word & 0xffffffffull) : 0;
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) gm = max(gm, __shfl_xor(gm, d, 64));
+    l.r.f.stats = gm;
+    flex_policy_step(l.r.f, l.r.h, gm, a.count_in);
+}
+
+// The rest of a streaming kernel's prologue (whole wavefront): fold, choose the exponent of this
+// write, leave the record in the other page if `store`, return the scale the kernel writes with.
+__device__ __forceinline__ float flex_lazy_finish(const FlexLazySlot& a, FlexLazyLoaded& l, bool store) {
+    flex_lazy_fold(a, l);
+    const int dec = flex_write_dec(l.r.f, a.in_place);
+    l.r.f.dec = dec;
+    l.r.f.scale = flex_scale_of(dec);
+    if (store) flex_wave_store(*a.out, l.r);
+    return l.r.f.scale;
+}
+
+template <int NS>
+__device__ __forceinline__ void flex_lazy_epilogue(const FlexLazySlot* slots, const int (&fmax)[4],
+                                                   int (*lds)[4] /* [NS][waves] */) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        int m = fmax[s];
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) m = max(m, __shfl_xor(m, d, 64));
+        if (lane == 0) lds[s][wave] = m;
+    }
+    __syncthreads();
+    if (threadIdx.x >= NS) return;
+    const int s = threadIdx.x;
+    const int bm = max(max(lds[s][0], lds[s][1]), max(lds[s][2], lds[s][3]));
+    const unsigned long long v = ((unsigned long long)slots[s].tag_out << 32) | (unsigned)bm;
+    (void)__hip_atomic_fetch_max(slots[s].words_out + (blockIdx.x % kFlexGroups) * kFlexWordPad, v,
+                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Bring records back to their plain form: fold what is pending and leave the result in the
+// ABI's record.  One wavefront per entry.
+struct FlexSettleArgs {
+    int          n;
+    FlexLazySlot slot[kFlexMaxIds];       // out = the ABI's record
+};
+
+__global__ __launch_bounds__(64) void flex_settle_kernel(const FlexSettleArgs args) {
+    if ((int)blockIdx.x >= args.n) return;
+    const FlexLazySlot& a = args.slot[blockIdx.x];
+    FlexLazyLoaded l;
+    flex_lazy_fetch(a, l);
+    flex_lazy_fold(a, l);
+    flex_wave_store(*a.out, l.r);
 }
 
 }  // namespace ngh

@@ -66,7 +66,31 @@ int env_int(const char* name, int dflt) {
 
 }  // namespace
 
+// Host-side bookkeeping of deferred statistics (ngh_flex.h): where each record of a table
+// allocated by ngh_flex_states_alloc currently lives and whether a fold is outstanding.
+struct FlexRecordHost {
+    uint8_t  page = 0;      // 0 = the ABI's record, 1 = the shadow page
+    uint8_t  pending = 0;   // group words of write `seq` have not been folded in yet
+    uint32_t seq = 0;       // number of deferred writes so far (tag of the latest one)
+    int32_t  count = 0;     // that write's `count`
+    bool unsettled() const { return page != 0 || pending != 0; }
+};
+
+struct FlexTable {
+    ngh_flex_state*     base = nullptr;
+    int32_t             n = 0;
+    ngh_flex_state*     shadow = nullptr;   // second page of every record
+    unsigned long long* words = nullptr;    // per record: 2 sets of kFlexGroups padded words
+    std::vector<FlexRecordHost> rec;
+    ngh_flex_state* page(int32_t id, int which) const { return (which ? shadow : base) + id; }
+    unsigned long long* set(int32_t id, uint32_t seq) const {
+        return words + ((size_t)id * 2 + (seq & 1u)) * ngh::kFlexWordsPerSet;
+    }
+};
+
 struct ngh_context {
+    std::vector<FlexTable> flex_tables;
+    int         flex_unsettled = 0;  // records not in their plain form
     int         device = 0;
     int         cus = 0;
     hipStream_t stream = nullptr;
@@ -81,11 +105,13 @@ struct ngh_context {
     int         force_interp = 0;    // never pick a specialised kernel
     int         red_wgs_per_cu = 8;  // workgroups per CU a split reduction aims for
     int         no_tiles = 0;        // never use the LDS-tiled elementwise skeleton
-    int         flex_self_managed = 1;  // ngh_launch_fused_flex may fold the policy into the kernel
+    int         flex_self_managed = 2;  // ngh_launch_fused_flex: 0 = prepare / kernel / update launches,
+                                     // 1 = policy at the end of the kernel, 2 = statistics deferred to the next user
     int         cache_policy = -1;   // -1: from the operands' cache hints; 0..3 forces bit 0 = non-temporal
                                      // loads, bit 1 = non-temporal stores in pre-built kernels
     long long   stream_bytes = 192ll << 20;  // hints act on stages touching at least this much memory
     int         moments_wgs_per_cu = 8;
+    int         flex_lazy_blocks_per_cu = 6;  // grid of a launch with deferred statistics
     char        name[256] = "";
     uint64_t    total_bytes = 0;
 };
@@ -97,6 +123,7 @@ struct ngh_context {
 namespace {
 
 constexpr long long kMaxStageElems = 1LL << 33;
+constexpr int kFlexMaxLazyRecords = 4096;   // tables up to this size get pages and words for deferred statistics
 
 int validate(const ngh_fused_spec* sp) {
     if (!sp) return fail(NGH_E_INVALID, "spec is NULL");
@@ -542,6 +569,94 @@ int ensure_ws(ngh_context* ctx, size_t bytes) {
 
 // Arrival counters for kernels whose last workgroup finishes the job.  They are zero whenever
 // no such kernel is running: allocated zeroed, and each kernel resets what it used.
+// ---------------------------------------------------------------------------
+// Deferred flex statistics: host side.  A record is "unsettled" while its current contents
+// live in the shadow page or a fold of group words is outstanding; anything but the next
+// deferred launch writing it needs it settled (one small kernel) first.
+// ---------------------------------------------------------------------------
+FlexTable* flex_table_of(ngh_context* ctx, const void* p, int32_t* id) {
+    for (auto& T : ctx->flex_tables) {
+        const char* b = (const char*)T.base;
+        if ((const char*)p >= b && (const char*)p < b + (size_t)T.n * sizeof(ngh_flex_state)) {
+            *id = (int32_t)(((const char*)p - b) / sizeof(ngh_flex_state));
+            return &T;
+        }
+    }
+    return nullptr;
+}
+
+int flex_settle_flush(ngh_context* ctx, FlexSettleArgs& a) {
+    if (a.n == 0) return NGH_OK;
+    hipLaunchKernelGGL(flex_settle_kernel, dim3((unsigned)a.n), dim3(64), 0, ctx->stream, a);
+    HIP_TRY(hipGetLastError());
+    a.n = 0;
+    return NGH_OK;
+}
+
+// queue record `id` of T for settling (flushes when the batch is full)
+int flex_settle_add(ngh_context* ctx, FlexTable& T, int32_t id, FlexSettleArgs& a) {
+    FlexRecordHost& R = T.rec[(size_t)id];
+    if (!R.unsettled()) return NGH_OK;
+    for (int i = 0; i < a.n; ++i)
+        if (a.slot[i].out == T.base + id) return NGH_OK;
+    FlexLazySlot& sl = a.slot[a.n++];
+    memset(&sl, 0, sizeof(sl));
+    sl.in = T.page(id, R.page);
+    sl.out = T.base + id;
+    sl.words_in = R.pending ? T.set(id, R.seq) : nullptr;
+    sl.tag_in = R.seq;
+    sl.count_in = R.count;
+    R.page = 0;
+    R.pending = 0;
+    ctx->flex_unsettled -= 1;
+    if (a.n == kFlexMaxIds) return flex_settle_flush(ctx, a);
+    return NGH_OK;
+}
+
+int flex_settle_range(ngh_context* ctx, const ngh_flex_state* dev, int32_t first, int32_t n) {
+    if (ctx->flex_unsettled == 0) return NGH_OK;
+    FlexSettleArgs a;
+    a.n = 0;
+    for (auto& T : ctx->flex_tables) {
+        if (T.base != dev) continue;
+        const int32_t end = std::min<int64_t>((int64_t)first + n, T.n);
+        for (int32_t id = std::max(first, 0); id < end; ++id) NGH_TRY(flex_settle_add(ctx, T, id, a));
+    }
+    return flex_settle_flush(ctx, a);
+}
+
+int flex_settle_ids(ngh_context* ctx, const ngh_flex_state* dev, const int32_t* ids, int32_t n_ids) {
+    if (ctx->flex_unsettled == 0) return NGH_OK;
+    FlexSettleArgs a;
+    a.n = 0;
+    for (auto& T : ctx->flex_tables) {
+        if (T.base != dev) continue;
+        for (int i = 0; i < n_ids; ++i)
+            if (ids[i] >= 0 && ids[i] < T.n) NGH_TRY(flex_settle_add(ctx, T, ids[i], a));
+    }
+    return flex_settle_flush(ctx, a);
+}
+
+// settle every record a spec's operands point into (scale or statistics word); with
+// `writer` set, operands that carry one of that launch's statistics slots are left alone
+// (the launch works on those records itself)
+int flex_settle_spec(ngh_context* ctx, const ngh_fused_spec& sp, const KArgs* writer = nullptr) {
+    if (ctx->flex_unsettled == 0) return NGH_OK;
+    FlexSettleArgs a;
+    a.n = 0;
+    for (int t = 0; t < sp.n_tensors; ++t) {
+        if (writer && writer->t[t].stat_slot >= 0) continue;
+        const void* ptrs[2] = {sp.tensors[t].dev_scale, sp.tensors[t].dev_stats};
+        for (const void* p : ptrs) {
+            if (!p) continue;
+            int32_t id = 0;
+            FlexTable* T = flex_table_of(ctx, p, &id);
+            if (T) NGH_TRY(flex_settle_add(ctx, *T, id, a));
+        }
+    }
+    return flex_settle_flush(ctx, a);
+}
+
 int ensure_tickets(ngh_context* ctx, size_t n) {
     if (n <= ctx->n_tickets) return NGH_OK;
     if (ctx->tickets) {
@@ -778,7 +893,8 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     snprintf(ctx->name, sizeof(ctx->name), "%s (%s)", prop.name, prop.gcnArchName);
     ctx->ew_blocks_per_cu = std::max(1, env_int("NGH_EW_BLOCKS_PER_CU", 64));
     ctx->force_interp = env_int("NGH_FORCE_INTERP", 0);
-    ctx->flex_self_managed = env_int("NGH_FLEX_SELF_MANAGED", 1);
+    ctx->flex_self_managed = env_int("NGH_FLEX_SELF_MANAGED", 2);
+    ctx->flex_lazy_blocks_per_cu = std::max(1, env_int("NGH_FLEX_LAZY_BLOCKS_PER_CU", 6));
     ctx->no_tiles = env_int("NGH_NO_TILES", 0);
     ctx->red_wgs_per_cu = std::max(1, env_int("NGH_RED_WGS_PER_CU", 8));
     ctx->cache_policy = env_int("NGH_CACHE_POLICY", -1);
@@ -817,6 +933,10 @@ int ngh_shutdown(ngh_context* ctx) {
     if (ctx->ws) (void)hipFree(ctx->ws);
     if (ctx->stat_ws) (void)hipFree(ctx->stat_ws);
     if (ctx->tickets) (void)hipFree(ctx->tickets);
+    for (auto& T : ctx->flex_tables) {
+        if (T.shadow) (void)hipFree(T.shadow);
+        if (T.words) (void)hipFree(T.words);
+    }
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
     if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -850,6 +970,15 @@ int ngh_free(ngh_context* ctx, void* dev) {
     if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
     if (!dev) return NGH_OK;
     HIP_TRY(hipStreamSynchronize(ctx->stream));
+    for (size_t i = 0; i < ctx->flex_tables.size(); ++i) {
+        FlexTable& T = ctx->flex_tables[i];
+        if ((void*)T.base != dev) continue;
+        for (const auto& r : T.rec) ctx->flex_unsettled -= r.unsettled() ? 1 : 0;
+        if (T.shadow) (void)hipFree(T.shadow);
+        if (T.words) (void)hipFree(T.words);
+        ctx->flex_tables.erase(ctx->flex_tables.begin() + i);
+        break;
+    }
     HIP_TRY(hipFree(dev));
     return NGH_OK;
 }
@@ -976,6 +1105,7 @@ static int stage_cache_policy(const ngh_context* ctx, const ngh_fused_spec& sp, 
 int ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec) {
     if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
     NGH_TRY(validate(spec));
+    NGH_TRY(flex_settle_spec(ctx, *spec));
     for (int s = 0; s < spec->n_stages; ++s) {
         if (spec->stages[s].op_end == spec->stages[s].op_begin) continue;
         Plan P;
@@ -1097,13 +1227,41 @@ int ngh_flex_states_alloc(ngh_context* ctx, int32_t n, ngh_flex_state** out_dev)
         s.scale = 1.0f / 256.0f;
     }
     *out_dev = (ngh_flex_state*)p;
-    return ngh_memcpy_h2d(ctx, p, init.data(), init.size() * sizeof(ngh_flex_state));
+    NGH_TRY(ngh_memcpy_h2d(ctx, p, init.data(), init.size() * sizeof(ngh_flex_state)));
+    // second page and group words for deferred statistics (16 KiB a record; large tables go without
+    // and their launches fold at the end of the kernel instead)
+    FlexTable T;
+    T.base = (ngh_flex_state*)p;
+    T.n = n;
+    T.rec.resize((size_t)n);
+    if (n <= kFlexMaxLazyRecords) {
+        const size_t wbytes = (size_t)n * kFlexWordsPerRecord * sizeof(unsigned long long);
+        if (hipMalloc((void**)&T.shadow, (size_t)n * sizeof(ngh_flex_state)) != hipSuccess ||
+            hipMalloc((void**)&T.words, wbytes) != hipSuccess) {
+            (void)hipGetLastError();
+            if (T.shadow) (void)hipFree(T.shadow);
+            T.shadow = nullptr;
+            T.words = nullptr;
+        } else {
+            HIP_TRY(hipMemsetAsync(T.words, 0, wbytes, ctx->stream));
+            HIP_TRY(hipMemsetAsync(T.shadow, 0, (size_t)n * sizeof(ngh_flex_state), ctx->stream));
+        }
+    }
+    ctx->flex_tables.push_back(std::move(T));
+    return NGH_OK;
+}
+
+int ngh_flex_unsettled(ngh_context* ctx, int32_t* out_count) {
+    if (!ctx || !out_count) return fail(NGH_E_INVALID, "ngh_flex_unsettled: NULL argument");
+    *out_count = ctx->flex_unsettled;
+    return NGH_OK;
 }
 
 int ngh_flex_states_write(ngh_context* ctx, ngh_flex_state* dev, int32_t first, int32_t n,
                           const ngh_flex_state* host) {
     if (n <= 0) return NGH_OK;
     if (!dev || !host || first < 0) return fail(NGH_E_INVALID, "ngh_flex_states_write: bad argument");
+    NGH_TRY(flex_settle_range(ctx, dev, first, n));      // the copy must be the last writer
     return ngh_memcpy_h2d(ctx, dev + first, host, (size_t)n * sizeof(ngh_flex_state));
 }
 
@@ -1111,6 +1269,7 @@ int ngh_flex_states_read(ngh_context* ctx, const ngh_flex_state* dev, int32_t fi
                          ngh_flex_state* host) {
     if (n <= 0) return NGH_OK;
     if (!dev || !host || first < 0) return fail(NGH_E_INVALID, "ngh_flex_states_read: bad argument");
+    NGH_TRY(flex_settle_range(ctx, dev, first, n));
     return ngh_memcpy_d2h(ctx, host, dev + first, (size_t)n * sizeof(ngh_flex_state));
 }
 
@@ -1135,6 +1294,7 @@ int ngh_flex_prepare(ngh_context* ctx, ngh_flex_state* dev, const int32_t* ids, 
     if (n_ids == 0) return NGH_OK;
     FlexIds f;
     NGH_TRY(make_flex_ids(ids, in_place, n_ids, f));
+    NGH_TRY(flex_settle_ids(ctx, dev, ids, n_ids));
     hipLaunchKernelGGL(flex_prepare_kernel, dim3(1), dim3(64), 0, ctx->stream, dev, f);
     HIP_TRY(hipGetLastError());
     return NGH_OK;
@@ -1145,7 +1305,8 @@ int ngh_flex_update(ngh_context* ctx, ngh_flex_state* dev, const int32_t* ids, i
     if (n_ids == 0) return NGH_OK;
     FlexIds f;
     NGH_TRY(make_flex_ids(ids, nullptr, n_ids, f));
-    hipLaunchKernelGGL(flex_update_kernel, dim3(1), dim3(64), 0, ctx->stream, dev, f, (int)count);
+    NGH_TRY(flex_settle_ids(ctx, dev, ids, n_ids));
+    hipLaunchKernelGGL(flex_update_kernel, dim3((unsigned)n_ids), dim3(64), 0, ctx->stream, dev, f, (int)count);
     HIP_TRY(hipGetLastError());
     return NGH_OK;
 }
@@ -1176,10 +1337,55 @@ static int try_self_managed_launch(ngh_context* ctx, const ngh_fused_spec* spec,
         P.k.flex_state[s] = dev + id;
         P.k.flex_in_place[s] = in_place ? in_place[j] : 0;
     }
-    NGH_TRY(ensure_tickets(ctx, (size_t)kFlexTicketWords + kFlexGroupMaxWords));
-    P.k.flex_count = count;
-    P.k.tickets = ctx->tickets;
-    P.k.group_max = (int*)(ctx->tickets + kFlexTicketWords);
+    // records the kernel writes: slot s <-> record slot_id[s]
+    int32_t slot_id[4] = {0, 0, 0, 0};
+    for (int s = 0; s < P.k.n_stat_slots; ++s) slot_id[s] = (int32_t)(P.k.flex_state[s] - dev);
+    FlexTable* T = nullptr;
+    if (ctx->flex_self_managed >= 2) {
+        int32_t id0 = 0;
+        T = flex_table_of(ctx, dev, &id0);
+        if (T && (T->base != dev || !T->words)) T = nullptr;
+        for (int s = 0; T && s < P.k.n_stat_slots; ++s)
+            if (slot_id[s] >= T->n || T->rec[(size_t)slot_id[s]].seq >= 0xfffffff0u) T = nullptr;
+        // a tensor that is read and then rewritten at a new scale needs its record settled
+        // before the first load: not worth deferring
+        bool loads[NGH_MAX_TENSORS], stores[NGH_MAX_TENSORS];
+        stage_tensors(*spec, spec->stages[0], loads, stores);
+        for (int t = 0; T && t < P.k.n_tensors; ++t)
+            if (P.k.t[t].stat_slot >= 0 && loads[t] && !P.k.flex_in_place[P.k.t[t].stat_slot]) T = nullptr;
+    }
+    if (T) {
+        // deferred statistics: everything the kernel merely reads must be in its plain form
+        NGH_TRY(flex_settle_spec(ctx, *spec, &P.k));
+        for (int s = 0; s < P.k.n_stat_slots; ++s) {
+            const int32_t id = slot_id[s];
+            FlexRecordHost& R = T->rec[(size_t)id];
+            FlexLazySlot& sl = P.k.lazy[s];
+            sl.in = T->page(id, R.page);
+            sl.out = T->page(id, R.page ^ 1);
+            sl.words_in = R.pending ? T->set(id, R.seq) : nullptr;
+            sl.tag_in = R.seq;
+            sl.count_in = R.count;
+            sl.in_place = P.k.flex_in_place[s];
+            if (!R.unsettled()) ctx->flex_unsettled += 1;
+            R.seq += 1;
+            R.page ^= 1;
+            R.pending = 1;
+            R.count = count;
+            sl.tag_out = R.seq;
+            sl.words_out = T->set(id, R.seq);
+            P.k.flex_state[s] = nullptr;
+        }
+        P.k.lazy_blocks_per_cu = ctx->flex_lazy_blocks_per_cu;
+        P.k.flex_lazy = ctx->cus > 0 ? ctx->cus : 1;   // also the distance between workgroups of one CU
+    } else {
+        NGH_TRY(flex_settle_spec(ctx, *spec));
+        NGH_TRY(flex_settle_ids(ctx, dev, slot_id, P.k.n_stat_slots));
+        NGH_TRY(ensure_tickets(ctx, (size_t)kFlexTicketWords + kFlexGroupMaxWords));
+        P.k.flex_count = count;
+        P.k.tickets = ctx->tickets;
+        P.k.group_max = (int*)(ctx->tickets + kFlexTicketWords);
+    }
     const unsigned blocks = streaming_blocks(ctx->cus, ctx->ew_blocks_per_cu, P.n_chunks);
     hipError_t e = launch_special(P.special, ctx->stream, blocks, P.k, P.n_chunks, P.chunks_per_row,
                                   stage_cache_policy(ctx, *spec, spec->stages[0]));

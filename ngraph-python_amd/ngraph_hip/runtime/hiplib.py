@@ -121,6 +121,7 @@ _SYMBOLS = {
     "ngh_flex_update": [_vp, _vp, ctypes.POINTER(ctypes.c_int32), _i32, _i32],
     "ngh_launch_fused_flex": [_vp, ctypes.POINTER(ngh_fused_spec), _vp, ctypes.POINTER(ctypes.c_int32),
                               ctypes.POINTER(ctypes.c_int32), _i32, _i32],
+    "ngh_flex_unsettled": [_vp, ctypes.POINTER(ctypes.c_int32)],
     "ngh_timer_begin": [_vp],
     "ngh_timer_end": [_vp, ctypes.POINTER(ctypes.c_float)],
 }
@@ -365,6 +366,12 @@ class HipRuntime(object):
         _check(self.lib, self.lib.ngh_launch_fused_flex(self.ctx, ctypes.byref(spec), ctypes.c_void_p(dev),
                                                         ids, in_place, n, int(count)))
 
+    def flex_unsettled(self):
+        """Records whose latest statistics the library has not folded in yet."""
+        n = ctypes.c_int32()
+        _check(self.lib, self.lib.ngh_flex_unsettled(self.ctx, ctypes.byref(n)))
+        return n.value
+
     # -- timing ------------------------------------------------------------
     def timer_begin(self):
         _check(self.lib, self.lib.ngh_timer_begin(self.ctx))
@@ -451,6 +458,9 @@ class DryRunRuntime(object):
 
     def launch_fused_flex(self, spec, dev, id_arrays, count):
         self.launch_fused(spec)
+
+    def flex_unsettled(self):
+        return 0
 
 
 class FusedSpecBuilder(object):

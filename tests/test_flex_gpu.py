@@ -236,3 +236,124 @@ def test_flex_learning_rules_prebuilt_equals_interpreter(rule, resident, monkeyp
     # state tensors start from zeros at the default exponent (resolution 2**-8) and only then
     # adapt, so the first steps are coarse: a sanity bound, not a precision claim
     assert np.abs(v_static - p).max() < 0.02, np.abs(v_static - p).max()
+
+
+# ---- exponent management across launches with nobody looking in between --------------------
+# The library can leave the statistics of a launch unfolded until the next launch that writes
+# the tensor, or until something else needs the record.  Whatever it does, records, mantissas
+# and consumers must see exactly what the launch-by-launch policy of the host gives.
+
+_POLICY_MODES = [("host", None, None), ("three-launches", "0", None), ("end-of-kernel", "1", None),
+                 ("deferred", "2", None), ("deferred-small-grid", "2", "1")]
+
+
+def _entry_state(entry):
+    return (entry.dec, entry.next_dec, entry.last_maxabs, tuple(entry.history))
+
+
+def _with_policy_mode(monkeypatch, mode, grid):
+    monkeypatch.delenv("NGH_FLEX_SELF_MANAGED", raising=False)
+    monkeypatch.delenv("NGH_FLEX_LAZY_BLOCKS_PER_CU", raising=False)
+    if mode is not None:
+        monkeypatch.setenv("NGH_FLEX_SELF_MANAGED", mode)
+    if grid is not None:
+        monkeypatch.setenv("NGH_FLEX_LAZY_BLOCKS_PER_CU", grid)
+
+
+@pytest.mark.parametrize("n", [1 << 18, 100003 * 8])
+def test_device_only_iterations_agree_across_policy_modes(n, monkeypatch):
+    x0, w, b = configs.c5_inputs(n, seed=11)
+    x0 = (x0 * 30.0).astype(np.float32)           # saturates at the first exponent: the policy has to move
+    seen = {}
+    for name, mode, grid in _POLICY_MODES:
+        _with_policy_mode(monkeypatch, mode, grid)
+        t = ngt.make_transformer_factory("flexhip", resident=name != "host")()
+        try:
+            f, _, _ = _c5_graph(t, n)
+            f(x0, w, b)
+            group = t.kernel_groups[f]
+            states = []
+            for it in range(7):
+                group()
+                if name.startswith("deferred") and default_kernel_choice():
+                    assert t.runtime.flex_unsettled() == 1        # y's record, and only that
+                elif name != "host":
+                    assert t.runtime.flex_unsettled() == 0
+                if it in (2, 6):                    # look twice: after a few launches, and at the end
+                    view = t.get_op_tensor_view(f.computation_op.values[0])
+                    states.append((_entry_state(view.flex_entry), view._read_raw().copy()))
+            seen[name] = states
+        finally:
+            t.close()
+    ref = seen["host"]
+    assert ref[0][0] != ref[1][0]                   # the exponent state did evolve in between
+    for name, states in seen.items():
+        for (st, mant), (st_ref, mant_ref) in zip(states, ref):
+            assert st == st_ref, (name, st, st_ref)
+            np.testing.assert_array_equal(mant, mant_ref, err_msg=name)
+
+
+def test_consumer_of_a_tensor_with_unfolded_statistics(monkeypatch):
+    """A second computation reads, on the device, the scale of a tensor whose last writes left
+    their statistics unfolded; a host fill of the same tensor in between must also win."""
+    n = 1 << 18
+    x0, w, b = configs.c5_inputs(n, seed=12)
+    seen = {}
+    for name, mode, grid in _POLICY_MODES:
+        _with_policy_mode(monkeypatch, mode, grid)
+        t = ngt.make_transformer_factory("flexhip", resident=name != "host")()
+        try:
+            P = ng.make_axis(n, name="P")
+            x, wp, bp = ng.placeholder([P]), ng.placeholder([P]), ng.placeholder([P])
+            v = ng.persistent_tensor([P], initial_value=0.0)
+            write = t.computation(ng.assign(v, neon.rectlin(x * wp + bp)), x, wp, bp)
+            read = t.computation(v * 0.5 + 1.0)
+            write((x0 * 20.0).astype(np.float32), w, b)
+            group = t.kernel_groups[write]
+            for _ in range(3):
+                group()
+            first = np.array(read())
+            for _ in range(2):
+                group()
+            view = t.get_op_tensor_view(v)
+            second = (np.array(read()), _entry_state(view.flex_entry), view._read_raw().copy())
+            seen[name] = (first, second)
+        finally:
+            t.close()
+    ref_first, ref_second = seen["host"]
+    for name, (first, second) in seen.items():
+        np.testing.assert_array_equal(first, ref_first, err_msg=name)
+        np.testing.assert_array_equal(second[0], ref_second[0], err_msg=name)
+        assert second[1] == ref_second[1], (name, second[1], ref_second[1])
+        np.testing.assert_array_equal(second[2], ref_second[2], err_msg=name)
+
+
+def test_in_place_rule_iterated_on_the_device_agrees_across_policy_modes(monkeypatch):
+    from ngraph_hip.frontends import neon as neon_front
+    n = 1 << 18
+    rs = np.random.RandomState(5)
+    p0 = rs.normal(0, 0.1, n).astype(np.float32)
+    g = rs.normal(0, 0.05, n).astype(np.float32)
+    seen = {}
+    for name, mode, grid in _POLICY_MODES:
+        _with_policy_mode(monkeypatch, mode, grid)
+        t = ngt.make_transformer_factory("flexhip", resident=name != "host")()
+        try:
+            P = ng.make_axis(n, name="P")
+            p, grad = ng.variable([P], initial_value=p0), ng.placeholder([P])
+            updates = neon_front.GradientDescentMomentum(0.1, 0.9).variable_update(p, grad)[0]
+            f = t.computation(updates, grad)
+            f(g)
+            group = t.kernel_groups[f]
+            for _ in range(5):
+                group()
+            if name.startswith("deferred") and default_kernel_choice():
+                assert t.runtime.flex_unsettled() >= 1
+            view = t.get_op_tensor_view(p)
+            seen[name] = (_entry_state(view.flex_entry), view._read_raw().copy())
+            assert name == "host" or t.runtime.flex_unsettled() == 0
+        finally:
+            t.close()
+    for name, (st, mant) in seen.items():
+        assert st == seen["host"][0], (name, st, seen["host"][0])
+        np.testing.assert_array_equal(mant, seen["host"][1], err_msg=name)
