@@ -97,11 +97,15 @@ struct GatherAt {   // element v at (i0[v], i1[v], i2[v]); only the first nv cou
     unsigned i0[V], i1[V], i2[V];
     int nv;
     __device__ __forceinline__ bool valid(int v) const { return v < nv; }
-    __device__ __forceinline__ float iota(int ka, int v) const {
-        return (float)(ka == 2 ? i2[v] : (ka == 1 ? i1[v] : i0[v]));
+    // Picked with masks, not with `ka == 2 ? i2[v] : ...`: the compiler turns that into one load
+    // at a run-time offset into this struct, which moves the whole struct to scratch memory.
+    __device__ __forceinline__ unsigned pick(int ka, int v) const {
+        const unsigned m1 = 0u - (unsigned)(ka == 1), m2 = 0u - (unsigned)(ka == 2);
+        return (i0[v] & ~(m1 | m2)) | (i1[v] & m1) | (i2[v] & m2);
     }
+    __device__ __forceinline__ float iota(int ka, int v) const { return (float)pick(ka, v); }
     __device__ __forceinline__ int red_index(int, int) const { return 0; }   // not used with reductions
-    __device__ __forceinline__ long long coord(int ka, int v) const { return ka == 2 ? i2[v] : (ka == 1 ? i1[v] : i0[v]); }
+    __device__ __forceinline__ long long coord(int ka, int v) const { return pick(ka, v); }
     __device__ __forceinline__ void load(const KTensor& t, float (&x)[V]) const {
         const float sc = (t.dtype == NGH_FLEX16) ? tensor_scale(t) : 1.0f;
 #pragma unroll
