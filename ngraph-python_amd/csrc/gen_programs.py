@@ -152,13 +152,17 @@ def collect():
                     plan = hiplib.plan_fused(spec, stage)
                     st = spec.stages[stage]
                     family = plan["family"]
-                    if family > 3 or (family == 0 and (plan["V"] < 4 or st.n_reductions)):
+                    total = spec.shape[0] * spec.shape[1] * spec.shape[2]
+                    # A one-element stage (a learning rule's step counter and rate factor) is worth a
+                    # program of its own: the interpreter fetches the code of every op kind it meets
+                    # with a cold instruction cache, several microseconds for twenty scalar ops.
+                    scalar = total == 1 and family == 0 and not st.n_reductions
+                    if family > 3 or (family == 0 and not scalar and (plan["V"] < 4 or st.n_reductions)):
                         continue
                     if family == 1 and spec.shape[0] // plan["V"] <= 64:
                         continue          # short rows run the several-rows-per-workgroup kernel
-                    total = spec.shape[0] * spec.shape[1] * spec.shape[2]
-                    if total < 4096:
-                        continue          # tiny stages are launch-bound; the interpreter is fine
+                    if total < 4096 and not scalar:
+                        continue          # small stages are launch-bound; the interpreter is fine
                     if any(o.opcode >= hiplib.OPCODES["take"] for o in spec.ops[st.op_begin:st.op_end]):
                         continue          # lookups only run in the interpreter
                     ops = [(o.opcode, o.dst, o.a, o.b) for o in spec.ops[st.op_begin:st.op_end]]
