@@ -1126,7 +1126,8 @@ class _Group(object):
                     tds.append(td)
             if isinstance(op, (og.AssignOp, og.Fill)):
                 tds.extend(writes)
-            elif not isinstance(op, og.ReductionOp):
+            elif not (isinstance(op, og.ReductionOp) and op.reduction_axes.size > 1):
+                # (a reduction over axes of length 1 is an elementwise assignment)
                 base = op.tensor_description().base
                 if base in returned or any(u not in inside for u in readers.get(base, ())):
                     tds.append(op.tensor_description())

@@ -146,8 +146,35 @@ def test_view_graphs_evaluate_on_the_oracle(seed):
     run("cpu", results, inputs, values)
 
 
+def _lower_without_a_device(results, inputs):
+    """Plan and lower every kernel of the computation with the dry-run runtime: whatever the
+    planner groups, the lowering must be able to express (no GPU involved)."""
+    t = ngt.make_transformer_factory("hipgpu", dry_run=True)()
+    try:
+        f = t.computation(results, *inputs)
+        t.initialize()
+        for kernel in t.kernel_groups[f].kernels:
+            kernel.bind_buffers()
+    finally:
+        t.close()
+
+
+# 6789: a reduction over a length-1 axis (an elementwise assignment whose result is written out)
+# next to a reduction over all axes of a permuted view
+@pytest.mark.parametrize("seed", list(range(1000, 1400)) + [6789])
+def test_view_graphs_lower_without_a_device(seed):
+    results, inputs, _ = build_views(seed)
+    _lower_without_a_device(results, inputs)
+
+
+@pytest.mark.parametrize("seed", range(200, 500))
+def test_graphs_lower_without_a_device(seed):
+    results, inputs, _ = build(seed)
+    _lower_without_a_device(results, inputs)
+
+
 @pytest.mark.gpu
-@pytest.mark.parametrize("seed", range(1000, 1100))
+@pytest.mark.parametrize("seed", list(range(1000, 1100)) + [6789])
 def test_random_view_graph_matches_oracle(seed):
     results, inputs, values = build_views(seed)
     want = run("cpu", results, inputs, values)
