@@ -123,6 +123,7 @@ struct ngh_context {
 namespace {
 
 constexpr long long kMaxStageElems = 1LL << 33;
+constexpr long long kSmallReduction = 1LL << 19;   // elements: below this a reduction stays one launch
 constexpr int kFlexMaxLazyRecords = 4096;   // tables up to this size get pages and words for deferred statistics
 
 int validate(const ngh_fused_spec* sp) {
@@ -522,6 +523,9 @@ int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage,
         long long seg = std::max<long long>(1, target_wgs / std::max<long long>(1, base_wgs));
         seg = std::min<long long>(seg, std::max<long long>(1, R / (rows_per_pass * 8)));
         seg = std::min<long long>(seg, 4096);
+        // a small problem is bound by launches: a second one (the fold of the segments) costs more
+        // than the parallelism the segments buy
+        if (R * n_out <= kSmallReduction) seg = 1;
         P.seg_len = (unsigned)((R + seg - 1) / seg);
         P.n_seg = (unsigned)((R + P.seg_len - 1) / std::max(1u, P.seg_len));
         if (P.n_seg == 0) P.n_seg = 1;
@@ -545,6 +549,7 @@ int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage,
         long long seg = std::max<long long>(1, target_wgs / std::max<long long>(1, n_out));
         seg = std::min<long long>(seg, std::max<long long>(1, chunks / (kBlock * 4)));
         seg = std::min<long long>(seg, 1024);
+        if (R * n_out <= kSmallReduction && n_out >= 16) seg = 1;
         P.seg_len = (unsigned)((chunks + seg - 1) / seg);
         P.n_seg = (unsigned)((chunks + P.seg_len - 1) / std::max(1u, P.seg_len));
         if (P.n_seg == 0) P.n_seg = 1;
