@@ -948,7 +948,11 @@ class AssignableTensorOp(TensorOp):
             if callable(initial_value):
                 initial_value = initial_value(self.axes)
             if isinstance(initial_value, TensorOp):
-                raise ValueError("initial_value must be a number or array, not an Op")
+                # a constant op stands for its value (op_graph.py:2338-2344)
+                tensor = initial_value.forwarded.tensor
+                if not getattr(tensor, "is_constant", False) or tensor.const is None:
+                    raise ValueError("initial_value must be convertible to a NumPy tensor")
+                initial_value = tensor.const
             # a private copy: later changes to the caller's array must not reach the graph
             self.initial_value = np.array(initial_value, dtype=np.float64 if not isinstance(
                 self.dtype, np.dtype) else self.dtype, copy=True)
@@ -1021,7 +1025,8 @@ def placeholder(axes, dtype=None, initial_value=None, **kwargs):
 
 
 def temporary(axes, dtype=None, **kwargs):
-    return AssignableTensorOp(axes=make_axes(axes), is_constant=False, is_input=True,
+    # op_graph.py:2501-2519: storage a computation may reuse; not an input
+    return AssignableTensorOp(axes=make_axes(axes), is_constant=False, is_input=False,
                               is_persistent=False, is_trainable=False, dtype=dtype, **kwargs)
 
 
