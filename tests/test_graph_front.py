@@ -352,3 +352,40 @@ def test_axes_with_order_argument_checks():
     for bad in ([B], [A, B, C], [A, C], [A, B, B]):
         with pytest.raises(ValueError):
             ng.axes_with_order(x, bad)
+
+
+# ---- tensor_size, expand_dims, cast_axes (test_tensor_size.py:28-41, test_reshaping.py:31-98, 298-318)
+def test_tensor_size(backend):
+    x = ng.placeholder([ng.make_axis(3), ng.make_axis(4)])
+    with executor(ng.tensor_size(x), x) as f:
+        assert f(np.arange(12, dtype=np.float32).reshape(3, 4)) == 12
+    # the default counts the sample axes only; the batch axis has its own count
+    xb = ng.placeholder([ng.make_axis(3), ng.make_axis(4, name="N")])
+    with executor([ng.tensor_size(xb), ng.batch_size(xb)], xb) as f:
+        size, batch = f(np.arange(12, dtype=np.float32).reshape(3, 4))
+    assert size == 3 and batch == 4
+
+
+@pytest.mark.parametrize("tensor", [[[2, 5], [13, 5]], 2])
+@pytest.mark.parametrize("new_length", [1, 2, 3, 4])
+def test_expand_dims(backend, tensor, new_length):
+    data = np.array(tensor, dtype=np.float32)
+    for dim in range(data.ndim + 1):
+        x = ng.placeholder([ng.make_axis(n) for n in data.shape])
+        expanded = ng.expand_dims(x, ng.make_axis(new_length), dim)
+        want = np.ndarray(buffer=data, dtype=data.dtype,
+                          shape=data.shape[:dim] + (new_length,) + data.shape[dim:],
+                          strides=data.strides[:dim] + (0,) + data.strides[dim:])
+        with executor(expanded, x) as f:
+            np.testing.assert_array_equal(f(data), want)
+
+
+def test_cast_axes(backend):
+    C, D = ng.make_axis(2), ng.make_axis(3)
+    x = ng.placeholder([C, D])
+    with pytest.raises(ValueError):
+        ng.cast_axes(x, [D, C])
+    y = x + ng.cast_axes(x[1, :], [D])          # the slice, named D again, broadcasts along C
+    with executor(y, x) as f:
+        np.testing.assert_allclose(f(np.array([[10, 20, 30], [1, 2, 3]], dtype=np.float32)),
+                                   [[11, 22, 33], [2, 4, 6]])
