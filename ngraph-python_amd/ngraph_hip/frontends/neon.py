@@ -7,6 +7,9 @@ graphs the backend fuses are the ones the reference would hand it:
 * `adam_update`       ngraph/frontends/neon/optimizer.py:446-470
 * `lstm_cell`         ngraph/frontends/neon/layer.py:1630-1647 (gate order i,f,o,g :1615)
 * `rectlin`           ngraph/frontends/neon/activation.py:46
+
+plus the other elementwise pieces a training step is made of on this path: the activation
+classes, Dropout, two cost formulas and the learning rules.
 """
 import numpy as np
 
@@ -15,6 +18,89 @@ import ngraph_hip as ng
 
 def rectlin(x, slope=0):
     return ng.maximum(x, 0) + slope * ng.minimum(0, x)
+
+
+# ---- activations (ngraph/frontends/neon/activation.py:21-190): elementwise composites that
+# ---- the backend fuses into their producer ---------------------------------------------------
+class Rectlin(object):
+    def __init__(self, slope=0, **kwargs):
+        self.slope = slope
+
+    def __call__(self, x):
+        return ng.maximum(x, 0) + self.slope * ng.minimum(0, x)
+
+
+class Rectlinclip(object):
+    def __init__(self, slope=0, cutoff=20.0, name=None):
+        self.cutoff, self.slope = cutoff, slope
+
+    def __call__(self, x):
+        return ng.minimum(ng.maximum(x, 0) + self.slope * ng.minimum(x, 0), self.cutoff)
+
+
+class Identity(object):
+    def __call__(self, x):
+        return x
+
+
+class Explin(object):
+    def __init__(self, alpha=1.0):
+        self.alpha = alpha
+
+    def __call__(self, x):
+        return ng.maximum(x, 0) + self.alpha * (ng.exp(ng.minimum(x, 0)) - 1)
+
+
+class Normalizer(object):
+    def __init__(self, divisor=128.):
+        self.divisor = divisor
+
+    def __call__(self, x):
+        return x / self.divisor
+
+
+class Softmax(object):
+    def __call__(self, x):
+        return ng.softmax(x)
+
+
+class Tanh(object):
+    def __call__(self, x):
+        return ng.tanh(x)
+
+
+class Logistic(object):
+    def __call__(self, x):
+        return ng.sigmoid(x)
+
+
+class Dropout(object):
+    """Training: a fresh uniform mask per execution, `(u <= keep) * x`; inference: `keep * x`
+    (ngraph/frontends/neon/layer.py:1272-1303).  The random fill is an op of the fused kernel,
+    so mask and product are one launch."""
+
+    inference_mode = False
+
+    def __init__(self, keep=0.5, **kwargs):
+        self.keep = keep
+        self.mask = None
+
+    def __call__(self, in_obj):
+        if Dropout.inference_mode:
+            return self.keep * in_obj
+        if self.mask is None:
+            self.mask = ng.persistent_tensor(axes=in_obj.axes.sample_axes())
+        self.mask = ng.uniform(self.mask, low=0.0, high=1.0) <= self.keep
+        return self.mask * in_obj
+
+
+# ---- costs as the reference's tests build them (neon/tests/test_costs.py:46-76) ---------------
+def sum_squared(y, t):
+    return ng.squared_L2(y - t, out_axes=()) / 2
+
+
+def mean_squared(y, t):
+    return ng.mean(ng.square(y - t), out_axes=()) / 2.
 
 
 def batch_norm_train(in_obj, gamma, beta, out_axes, eps=1e-5):
