@@ -23,6 +23,7 @@ from ngraph_hip.op_graph.op_graph import (  # noqa: F401
     tensor_size, tensor_slice, unflatten, value_of, variable, variance, Transpose,
     cross_entropy_multi, cross_entropy_binary, cross_entropy_binary_inner, UnmatchedAxesError)
 from ngraph_hip.op_graph.op_graph import ContiguousOp as _ContiguousOp
+from ngraph_hip.op_graph.autodiff import deriv  # noqa: F401
 
 
 def contiguous(x):

@@ -1,8 +1,8 @@
 """Activations, costs and dropout of the neon front: elementwise composites on the fused path.
 
 Inputs and reference formulas follow ngraph/frontends/neon/tests/test_activations.py:64-170,
-test_costs.py:27-91 and test_dropout.py:31-85 (forward values only; this front has no
-autodiff).
+test_costs.py:27-91 and test_dropout.py:31-85 (forward values; derivatives are covered by
+tests/test_autodiff.py).
 """
 import numpy as np
 import pytest
