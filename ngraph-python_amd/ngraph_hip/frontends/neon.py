@@ -118,10 +118,85 @@ def batch_norm_train(in_obj, gamma, beta, out_axes, eps=1e-5):
     return y, xmean, xvar
 
 
-class Adam(object):
+# ---- a training step out of a cost (ngraph/frontends/neon/optimizer.py:50-120, 159-209) -------
+def clip_gradient_norm(grad_list, clip_norm=None):
+    """Factor <= 1 that brings the joint L2 norm of the gradients down to clip_norm."""
+    if clip_norm is None:
+        return 1
+    s = None
+    for g in grad_list:
+        term = ng.squared_L2(g, out_axes=None)
+        s = term if s is None else s + term
+    return clip_norm / ng.maximum(ng.sqrt(s), clip_norm)
+
+
+def clip_gradient_value(grad, clip_value=None):
+    if clip_value is None:
+        return grad
+    return ng.minimum(ng.maximum(grad, -abs(clip_value)), abs(clip_value))
+
+
+def clip_weight_value(weight, clip_value=None, min_value_override=None):
+    if clip_value is None:
+        return weight
+    if min_value_override is None:
+        min_value_override = -abs(clip_value)
+    return ng.minimum(ng.maximum(weight, min_value_override), abs(clip_value))
+
+
+def trainable_variables(op):
+    """The trainable variables `op` is computed from, in graph order."""
+    from ngraph_hip.op_graph.op_graph import Op, AssignableTensorOp
+    found = []
+    for o in Op.ordered_ops([op]):
+        for s in o.states_read:
+            if isinstance(s, AssignableTensorOp) and s.is_trainable and s not in found:
+                found.append(s)
+    return found
+
+
+class Optimizer(object):
+    """What the reference's LearningRateOptimizer.__call__ does with a cost: gradients of the
+    summed cost divided by the batch size, optional clipping, one update per variable; the
+    returned op runs gradients, updates and weight clipping in that order."""
+
+    gradient_clip_norm = None
+    gradient_clip_value = None
+    weight_clip_value = None
+
+    def minimize(self, cost_func, variables=None):
+        batch_cost = ng.sum(cost_func, out_axes=())
+        batch_axis = cost_func.axes.batch_axis()
+        batch_size = 1 if batch_axis is None else batch_axis.length
+        if variables is None:
+            variables = trainable_variables(batch_cost)
+        self.prepare()
+        grads = [ng.deriv(batch_cost, v) / batch_size for v in variables]
+        scale_factor = clip_gradient_norm(grads, self.gradient_clip_norm)
+        grads = [clip_gradient_value(g, self.gradient_clip_value) for g in grads]
+        updates = []
+        for variable, grad in zip(variables, grads):
+            out = self.variable_update(variable, grad, scale_factor)
+            updates.append(out[0] if isinstance(out, tuple) else out)
+        steps = list(updates)
+        if self.weight_clip_value is not None:
+            steps += [ng.assign(v, clip_weight_value(v, self.weight_clip_value)) for v in variables]
+        return ng.sequential(steps + [batch_cost])
+
+    def prepare(self):
+        pass
+
+    def _set_clipping(self, gradient_clip_norm=None, gradient_clip_value=None, weight_clip_value=None):
+        self.gradient_clip_norm = gradient_clip_norm
+        self.gradient_clip_value = gradient_clip_value
+        self.weight_clip_value = weight_clip_value
+
+
+class Adam(Optimizer):
     """Adam learning rule; `__call__` advances t, `variable_update` builds one update."""
 
-    def __init__(self, learning_rate=1e-3, beta_1=0.9, beta_2=0.999, epsilon=1e-8):
+    def __init__(self, learning_rate=1e-3, beta_1=0.9, beta_2=0.999, epsilon=1e-8, **clipping):
+        self._set_clipping(**clipping)
         self.lrate = learning_rate
         self.beta_1 = ng.constant(beta_1, dtype=np.float32)
         self.beta_2 = ng.constant(beta_2, dtype=np.float32)
@@ -129,6 +204,10 @@ class Adam(object):
         self.t = ng.persistent_tensor(axes=(), initial_value=0)
         self.step = None
         self.ell = None
+
+    def prepare(self):
+        if self.ell is None:
+            self()
 
     def __call__(self):
         self.step = ng.sequential([ng.assign(self.t, self.t + 1), self.t])
@@ -147,11 +226,12 @@ class Adam(object):
         return updates, m, v
 
 
-class GradientDescentMomentum(object):
+class GradientDescentMomentum(Optimizer):
     """SGD with momentum, weight decay, optional Nesterov step and the Kahan-compensated
     parameter update of frontends/neon/optimizer.py:285-310."""
 
-    def __init__(self, learning_rate, momentum_coef=0.0, wdecay=0.0, nesterov=False):
+    def __init__(self, learning_rate, momentum_coef=0.0, wdecay=0.0, nesterov=False, **clipping):
+        self._set_clipping(**clipping)
         self.lrate = learning_rate
         self.momentum_coef = momentum_coef
         self.wdecay = wdecay
@@ -172,10 +252,11 @@ class GradientDescentMomentum(object):
         return ng.sequential(updates), velocity
 
 
-class RMSProp(object):
+class RMSProp(Optimizer):
     """frontends/neon/optimizer.py:370-383."""
 
-    def __init__(self, decay_rate=0.95, learning_rate=2e-3, epsilon=1e-6, wdecay=0.0, momentum_coef=0.0):
+    def __init__(self, decay_rate=0.95, learning_rate=2e-3, epsilon=1e-6, wdecay=0.0, momentum_coef=0.0, **clipping):
+        self._set_clipping(**clipping)
         self.decay_rate, self.lrate, self.epsilon = decay_rate, learning_rate, epsilon
         self.wdecay, self.momentum = wdecay, momentum_coef
 
@@ -193,10 +274,11 @@ class RMSProp(object):
         return updates, state, velocity
 
 
-class Adagrad(object):
+class Adagrad(Optimizer):
     """frontends/neon/optimizer.py:533-542."""
 
-    def __init__(self, learning_rate=0.01, epsilon=1e-6):
+    def __init__(self, learning_rate=0.01, epsilon=1e-6, **clipping):
+        self._set_clipping(**clipping)
         self.lrate, self.epsilon = learning_rate, epsilon
 
     def variable_update(self, variable, grad, scale_factor=1):

@@ -106,3 +106,73 @@ def test_dropout_inference(backend):
     x = np.random.RandomState(1).uniform(size=(32, 2)).astype(np.float32)
     with executor(out_op, inp) as f:
         np.testing.assert_allclose(f(x), x * 0.5, rtol=1e-6)
+
+
+# ---- optimizers driven by a cost (neon/tests/test_optimizer.py:139-330 compares with NumPy
+# ---- reference classes; here the closed form is written out per rule) --------------------------
+def _quadratic_problem():
+    """cost_n = sum_f (w_f * x_fn - t_fn)^2 / 2: the gradient of the batch sum, divided by the
+    batch size, is mean_n (w x - t) x."""
+    F, N = ng.make_axis(5, name="F"), ng.make_axis(8, name="N")
+    rs = np.random.RandomState(4)
+    xv, tv = rs.normal(0, 1, (5, 8)).astype(np.float32), rs.normal(0, 1, (5, 8)).astype(np.float32)
+    w0 = rs.normal(0, 0.5, 5).astype(np.float32)
+    x, t = ng.placeholder([F, N]), ng.placeholder([F, N])
+    w = ng.variable([F], initial_value=w0)
+    cost = ng.sum(ng.square(w * x - t), out_axes=[N]) / 2
+
+    def grad(wn):
+        return ((wn[:, None] * xv - tv) * xv).mean(axis=1)
+    return (x, t, w, cost), (xv, tv, w0.astype(np.float64)), grad
+
+
+@pytest.mark.parametrize("rule", ["sgd", "sgd_momentum_clip", "rmsprop", "adagrad", "adam", "clip_norm"])
+def test_optimizer_minimises_a_cost(backend, rule):
+    (x, t, w, cost), (xv, tv, wn), grad = _quadratic_problem()
+    steps = 4
+    if rule == "sgd":
+        opt = neon.GradientDescentMomentum(0.1)
+        def ref(wn, state):
+            return wn - 0.1 * grad(wn), state
+    elif rule == "sgd_momentum_clip":
+        opt = neon.GradientDescentMomentum(0.1, momentum_coef=0.9, gradient_clip_value=0.3, weight_clip_value=0.6)
+        def ref(wn, state):
+            vel = state.get("v", 0.0) * 0.9 - 0.1 * np.clip(grad(wn), -0.3, 0.3)
+            return np.clip(wn + vel, -0.6, 0.6), {"v": vel}
+    elif rule == "rmsprop":
+        opt = neon.RMSProp(learning_rate=0.01)
+        def ref(wn, state):
+            g = grad(wn)
+            s = 0.95 * state.get("s", 1.0) + 0.05 * g * g
+            return wn - 0.01 * g / np.sqrt(s + 1e-6), {"s": s}
+    elif rule == "adagrad":
+        opt = neon.Adagrad(learning_rate=0.1)
+        def ref(wn, state):
+            g = grad(wn)
+            s = state.get("s", 0.0) + g * g
+            return wn - 0.1 * g / np.sqrt(s + 1e-6), {"s": s}
+    elif rule == "adam":
+        opt = neon.Adam(learning_rate=0.05)
+        def ref(wn, state):
+            g, k = grad(wn), state.get("k", 0) + 1
+            m = 0.9 * state.get("m", 0.0) + 0.1 * g
+            v = 0.999 * state.get("v", 0.0) + 0.001 * g * g
+            ell = 0.05 * np.sqrt(1 - 0.999 ** k) / (1 - 0.9 ** k)
+            return wn - ell * m / (np.sqrt(v) + 1e-8), {"k": k, "m": m, "v": v}
+    else:
+        opt = neon.GradientDescentMomentum(0.1, gradient_clip_norm=0.5)
+        def ref(wn, state):
+            g = grad(wn)
+            return wn - 0.1 * g * (0.5 / max(np.sqrt((g * g).sum()), 0.5)), state
+    train = opt.minimize(cost)
+    read = w * 1.0
+    t_ = ngt.make_transformer()
+    try:
+        f, r = t_.computation(train, x, t), t_.computation(read)
+        state = {}
+        for _ in range(steps):
+            f(xv, tv)
+            wn, state = ref(wn, state)
+        np.testing.assert_allclose(r(), wn, rtol=2e-4, atol=2e-6)
+    finally:
+        t_.close()
