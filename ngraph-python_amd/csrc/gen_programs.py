@@ -60,6 +60,17 @@ def pattern_batchnorm(t):
     return t.computation([y, xmean, xvar], x)
 
 
+def pattern_batchnorm_bprop(t):
+    # backward of the same layer from an upstream error: two reductions in one pass (dbeta,
+    # dgamma) and one elementwise pass (dx)
+    C, H, W, N = _axes(C=64, H=16, W=16, N=16)
+    x, err = ng.placeholder([C, H, W, N]), ng.placeholder([C, H, W, N])
+    gamma, beta = ng.variable([C], initial_value=1.0), ng.variable([C], initial_value=0.0)
+    y, _, _ = neon.batch_norm_train(x, gamma, beta, out_axes=[C])
+    return t.computation([ng.deriv(y, x, error=err), ng.deriv(y, gamma, error=err),
+                          ng.deriv(y, beta, error=err)], x, err)
+
+
 def pattern_flex_relu(t):
     P, = _axes(P=1 << 20)
     x, w, b = ng.placeholder([P]), ng.placeholder([P]), ng.placeholder([P])
@@ -116,6 +127,7 @@ PATTERNS = [
     ("flex_sgd_momentum", "flexhip", _rule_pattern(lambda: neon.GradientDescentMomentum(0.1, 0.9))),
     ("flex_rmsprop", "flexhip", _rule_pattern(lambda: neon.RMSProp())),
     ("batchnorm", "hipgpu", pattern_batchnorm),
+    ("batchnorm_bprop", "hipgpu", pattern_batchnorm_bprop),
     ("flex_relu_fma", "flexhip", pattern_flex_relu),
     ("sum_along", "hipgpu", _reduction_pattern(ng.sum, 0)),
     ("sum_across", "hipgpu", _reduction_pattern(ng.sum, 1)),

@@ -240,13 +240,18 @@ def adjoints_of(dependent, error):
             continue
         processed.add(key)
         target = key if isinstance(o, og.ValueOp) else o
-        rule = RULES.get(type(target).__name__)
-        if rule is None:
-            continue
         adjoint = adjoints[key]
         if getattr(target, "scale", None) is not None:
             adjoint = adjoint * target.scale
-        rule(target, adjoints, adjoint, *[a.forwarded for a in target.args])
+        # a composite may differentiate itself as a whole (op_graph.py:1153-1160 deriv_handler):
+        # sigmoid, softmax, the cross entropies of either, batch normalisation
+        handler = getattr(target, "deriv_handler", None)
+        if handler is not None and handler is not target:
+            handler.generate_adjoints(_add_delta, adjoints, adjoint)
+            continue
+        rule = RULES.get(type(target).__name__)
+        if rule is not None:
+            rule(target, adjoints, adjoint, *[a.forwarded for a in target.args])
     return adjoints
 
 
@@ -254,12 +259,22 @@ def deriv(dependent, independent, error=None):
     """The op computing [d dependent / d independent](error); it has independent's axes.
     `error` defaults to the scalar 1: a tensor-valued dependent needs an explicit error."""
     dependent, independent = og.as_op(dependent), og.as_op(independent)
+    # One backward graph per (dependent, error): derivatives with respect to several tensors share
+    # it (there is no common-subexpression elimination to merge separate copies later).  The default
+    # error is one constant per dependent for the same reason (op_graph.py:4275-4282); being a
+    # scalar, it only suits a scalar dependent.
+    cache = dependent.forwarded.__dict__.setdefault("_adjoint_cache", {})
     if error is None:
-        error = og.constant(1.0)      # so only a scalar can do without one (op_graph.py:4275-4282)
+        if "one" not in cache:
+            cache["one"] = og.constant(1.0)
+        error = cache["one"]
     error = og.as_op(error)
     if not error.axes.is_equal_set(dependent.axes):
         raise ValueError("Dependent and error must have the same set of axes")
-    adjoints = adjoints_of(dependent, error)
+    error_key = id(_key(error))          # a placeholder is wrapped anew at every use
+    if error_key not in cache:
+        cache[error_key] = (error, adjoints_of(dependent, error))
+    adjoints = cache[error_key][1]
     key = _key(independent)
     if key not in adjoints:
         return og.constant(0, independent.axes)       # not connected (op_graph.py:4286-4287)

@@ -1416,6 +1416,10 @@ class SigmoidOp(ValueOp):
         self.value_tensor = reciprocal(exp(-x) + 1)
         self.value_tensor.deriv_handler = self
 
+    def generate_adjoints(self, add_delta, adjoints, delta):
+        # op_graph.py:4200-4202
+        add_delta(adjoints, self.x, delta * self.value_tensor * (1.0 - self.value_tensor))
+
 
 def sigmoid(x):
     return SigmoidOp(as_op(x)).value_tensor
@@ -1441,6 +1445,13 @@ class SoftmaxOp(ValueOp):
         self.Z = sum(self.exps, reduction_axes=normalization_axes)
         self.value_tensor = self.exps * reciprocal(self.Z)
         self.value_tensor.deriv_handler = self
+        self.normalization_axes = normalization_axes
+
+    def generate_adjoints(self, add_delta, adjoints, delta):
+        # op_graph.py:3832-3846
+        z = delta * self.value_tensor
+        zs = sum(z, reduction_axes=self.normalization_axes)
+        add_delta(adjoints, self.x, z - zs * self.value_tensor)
 
 
 def softmax(x, normalization_axes=None, **kwargs):
@@ -1469,11 +1480,35 @@ def cross_entropy_multi(y, t, usebits=False, out_axes=None, enable_softmax_opt=T
     if enable_softmax_opt and isinstance(handler, SoftmaxOp):
         s = -sum(handler.x * t, out_axes=out_axes)
         value = minimum(s + log(handler.Z), safelog_cutoff)
+        if enable_diff_opt:
+            value.deriv_handler = _SoftmaxCrossEntropyAdjoint(handler, s)
     else:
         value = -sum(safelog(y) * t, out_axes=out_axes)
     if usebits:
         value = value * float(1.0 / np.log(2.0))
     return value
+
+
+class _SoftmaxCrossEntropyAdjoint(object):
+    """d/dx of -sum(x t) + log Z is -t + softmax(x) (op_graph.py:4363-4365)."""
+
+    def __init__(self, softmax_op, s):
+        self.softmax_op, self.s = softmax_op, s
+
+    def generate_adjoints(self, add_delta, adjoints, delta):
+        add_delta(adjoints, self.s, delta)
+        add_delta(adjoints, self.softmax_op.x, self.softmax_op.value_tensor * delta)
+
+
+class _SigmoidCrossEntropyAdjoint(object):
+    """Binary cross entropy of a sigmoid: d/dx = (y - t), d/dt = x (op_graph.py:4425-4427)."""
+
+    def __init__(self, sigmoid_op, y, t):
+        self.sigmoid_op, self.y, self.t = sigmoid_op, y, t
+
+    def generate_adjoints(self, add_delta, adjoints, delta):
+        add_delta(adjoints, self.sigmoid_op.x, (self.y - self.t) * delta)
+        add_delta(adjoints, self.t, self.sigmoid_op.x * delta)
 
 
 def cross_entropy_binary_inner(y, t, enable_sig_opt=True, enable_diff_opt=True):
@@ -1483,9 +1518,13 @@ def cross_entropy_binary_inner(y, t, enable_sig_opt=True, enable_diff_opt=True):
     y, t = as_op(y), as_op(t)
     _check_cross_entropy_axes(y, t)
     handler = getattr(y, "deriv_handler", None)
-    if enable_sig_opt and isinstance(handler, SigmoidOp):
-        return (1 - t) * maximum(handler.x, -safelog_cutoff) - safelog(y)
-    return -(safelog(y) * t + safelog(1 - y) * (1 - t))
+    value = -(safelog(y) * t + safelog(1 - y) * (1 - t))
+    if isinstance(handler, SigmoidOp):
+        if enable_sig_opt:
+            value = (1 - t) * maximum(handler.x, -safelog_cutoff) - safelog(y)
+        if enable_diff_opt:
+            value.deriv_handler = _SigmoidCrossEntropyAdjoint(handler, y, t)
+    return value
 
 
 def cross_entropy_binary(y, t, usebits=False, out_axes=None, enable_sig_opt=True,

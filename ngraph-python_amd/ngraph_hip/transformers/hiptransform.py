@@ -113,6 +113,15 @@ def _producer(op):
             return cur
 
 
+def _memory_elements(td):
+    """Distinct elements a view touches (a broadcast axis repeats the same ones)."""
+    n = 1
+    for length, stride in zip(td.shape, td.full_strides):
+        if stride != 0:
+            n *= length
+    return n
+
+
 def _view_key(td):
     return (td.base, td.parameter_key)
 
@@ -991,10 +1000,113 @@ class FusionPlanner(object):
             release(pick)
         if cur:
             groups.append(cur)
+        if self.fusion:
+            groups = self._recompute_across_groups(groups, readers, returned)
         for g in groups:
             if g.fusable:
                 g.decide_stores(readers, returned)
         return groups
+
+    # -- recomputation instead of a round trip through memory -------------------------------------
+    max_recompute_ops = 6
+
+    def _recompute_across_groups(self, groups, readers, returned):
+        """An elementwise result that later kernels need is normally written out and read back: two
+        passes over a large tensor.  When the few ops that produce it can be repeated in those
+        kernels from operands that are in memory anyway, at the price of at most one more large
+        operand to read, repeating them is cheaper -- the rule of the reference's compound
+        kernels, which re-emit the elementwise producers needed after a reduction
+        (float_ew2.py:553-612), applied across kernels."""
+        where = {}
+        for gi, g in enumerate(groups):
+            for op in g.ops:
+                where[op] = gi
+        plain = lambda op: (kernel_op_name(op) is not None and not isinstance(op, og.ReductionOp))
+        for gi, g in enumerate(groups):
+            if not g.fusable:
+                continue
+            for op in list(g.ops):
+                if not plain(op) or iteration_axes(op).size <= self.small_tensor:
+                    continue
+                base = op.tensor_description().base
+                if base in returned:
+                    continue
+                inside = set(groups[gi].ops)
+                outside = [u for u in readers.get(base, ()) if u not in inside]
+                if not outside:
+                    continue
+                targets = sorted(set(where.get(u, -1) for u in outside))
+                if targets[0] <= gi or not all(groups[hi].fusable for hi in targets):
+                    continue
+                chain = self._producer_chain(op, groups[gi], plain)
+                if chain is None or len(chain) > self.max_recompute_ops:
+                    continue
+                leaves = self._outside_operands(chain)
+                if self._written_between(leaves, groups, gi, targets[-1]):
+                    continue
+                rebuilt = {}
+                for hi in targets:
+                    h = groups[hi]
+                    have = set(_view_key(td) for o in h.ops for td in h._operand_views(o)[0])
+                    extra_large = [td for td in leaves
+                                   if _view_key(td) not in have and _memory_elements(td) > self.small_tensor]
+                    if len(extra_large) > 1:
+                        break
+                    ops = [o for o in chain if o not in h.ops] + h.ops
+                    new = _Group(ops[0], max_written_views=h.max_written_views)
+                    if not all(new.accepts(o, readers, returned) and (new.add(o) or True) for o in ops[1:]):
+                        break
+                    # the repeated ops are private to the kernel: whoever else needs them has them
+                    new.never_store = set(h.never_store) | set(o for o in chain if o not in h.ops)
+                    rebuilt[hi] = new
+                else:
+                    for hi, new in rebuilt.items():
+                        groups[hi] = new
+                    groups[gi].never_store.add(op)
+        return groups
+
+    @staticmethod
+    def _producer_chain(op, group, plain):
+        """The ops of `group`, in its order, that `op` is computed from inside the group; None if
+        one of them is not a plain elementwise op."""
+        index = {o: i for i, o in enumerate(group.ops)}
+        need, stack = set(), [op]
+        while stack:
+            o = stack.pop()
+            if o in need:
+                continue
+            if not plain(o):
+                return None
+            need.add(o)
+            for a in o.args:
+                prod = _producer(a.forwarded)
+                if prod in index and index[prod] < index[o]:
+                    stack.append(prod)
+        return [o for o in group.ops if o in need]
+
+    @staticmethod
+    def _outside_operands(chain):
+        inside = set(o.tensor_description().base for o in chain)
+        out = []
+        for o in chain:
+            for a in o.args:
+                a = a.forwarded
+                if _scalar_constant_value(a) is not None:
+                    continue
+                td = a.tensor_description()
+                if td.base not in inside:
+                    out.append(td)
+        return out
+
+    @staticmethod
+    def _written_between(leaves, groups, first, last):
+        bases = set(td.base for td in leaves)
+        for g in groups[first:last + 1]:
+            for o in g.ops:
+                if isinstance(o, (og.AssignOp, og.Fill)) and \
+                        o.args[0].forwarded.tensor_description().base in bases:
+                    return True
+        return False
 
 
 class _Group(object):
@@ -1002,6 +1114,7 @@ class _Group(object):
         self.ops = [op]
         self.fusable = fusable
         self.store_ops = set()
+        self.never_store = set()      # results every outside reader recomputes for itself
         self.max_written_views = max_written_views    # flex kernels: one statistics slot per result
         self.n_written_views = 0
         if fusable:
@@ -1191,6 +1304,8 @@ class _Group(object):
                 continue
             base = op.tensor_description().base
             users = readers.get(base, ())
+            if op in self.never_store:
+                continue
             if base in returned or any(u not in inside for u in users):
                 self.store_ops.add(op)
             elif isinstance(op, og.ReductionOp):

@@ -210,3 +210,61 @@ def test_a_training_step_built_from_deriv(backend):
         wn = wn - 0.5 * (xv * (p - tv)).sum(axis=1) / 16.0
     np.testing.assert_allclose(losses, want, rtol=2e-5)
     assert losses[-1] < losses[0]
+
+
+def test_batch_norm_backward_closed_form(backend):
+    """neon.batch_norm_train differentiates itself as a whole (two reductions in one pass, one
+    elementwise pass); checked against the textbook formulas in float64 and against numeric
+    derivatives of the op-by-op composite."""
+    from ngraph_hip.frontends import neon
+    C, H, N = ng.make_axis(4, name="C"), ng.make_axis(5, name="H"), ng.make_axis(6, name="N")
+    x, e = ng.placeholder([C, H, N]), ng.placeholder([C, H, N])
+    gv = np.array([1.0, 2.0, 0.5, 1.5], np.float32)
+    g, b = ng.variable([C], initial_value=gv), ng.variable([C], initial_value=np.zeros(4, np.float32))
+    y, _, _ = neon.batch_norm_train(x, g, b, [C])
+    rs = np.random.RandomState(0)
+    xv, ev = rs.normal(0.5, 2, (4, 5, 6)).astype(np.float32), rs.normal(0, 1, (4, 5, 6)).astype(np.float32)
+    with executor([ng.deriv(y, x, error=e), ng.deriv(y, g, error=e), ng.deriv(y, b, error=e)], x, e) as f:
+        dx, dg, db = f(xv, ev)
+    x64, e64 = xv.reshape(4, -1).astype(np.float64), ev.reshape(4, -1).astype(np.float64)
+    rstd = 1 / np.sqrt(x64.var(1, keepdims=True) + 1e-5)
+    xh = (x64 - x64.mean(1, keepdims=True)) * rstd
+    dg_want, db_want = (e64 * xh).sum(1), e64.sum(1)
+    dx_want = gv[:, None] * rstd * (e64 - db_want[:, None] / 30 - xh * dg_want[:, None] / 30)
+    np.testing.assert_allclose(dx.reshape(4, -1), dx_want, rtol=1e-4, atol=2e-6)
+    np.testing.assert_allclose(dg, dg_want, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(db, db_want, rtol=1e-5, atol=1e-5)
+    # the same layer written out op by op, differentiated rule by rule
+    flat_mean = ng.mean(x, out_axes=[C])
+    flat_var = ng.variance(x, out_axes=[C])
+    y_plain = g * ((x - flat_mean) * ng.reciprocal(ng.sqrt(flat_var + 1e-5))) + b
+    with executor(ng.deriv(y_plain, x, error=e), x, e) as f:
+        np.testing.assert_allclose(f(xv, ev), dx, rtol=1e-3, atol=1e-5)
+
+
+def test_recomputation_replaces_a_round_trip_through_memory():
+    """Planner property, no GPU: the normalised input of the batch-norm backward is needed by the
+    reduction kernel and by the elementwise kernel after it; the second recomputes it from x
+    instead of reading a copy the first would have to write."""
+    from ngraph_hip.frontends import neon
+    from ngraph_hip.runtime.hiplib import OPCODES
+    t = ngt.make_transformer_factory("hipgpu", dry_run=True)()
+    try:
+        C, R = ng.make_axis(16, name="C"), ng.make_axis(16384, name="R")
+        x, e = ng.placeholder([C, R]), ng.placeholder([C, R])
+        g, b = ng.variable([C], initial_value=1.0), ng.variable([C], initial_value=0.0)
+        y, _, _ = neon.batch_norm_train(x, g, b, [C])
+        f = t.computation([ng.deriv(y, x, error=e), ng.deriv(y, g, error=e), ng.deriv(y, b, error=e)], x, e)
+        t.initialize()
+        big_stores = 0
+        for kernel in t.kernel_groups[f].kernels:
+            kernel.bind_buffers()
+            for spec in getattr(kernel, "specs", []):
+                if spec.shape[0] * spec.shape[1] * spec.shape[2] < 16 * 16384:
+                    continue
+                big_stores += sum(1 for i in range(spec.n_ops) if spec.ops[i].opcode == OPCODES["store"]
+                                  and all(spec.tensors[spec.ops[i].dst].strides[a] != 0 or spec.shape[a] == 1
+                                          for a in range(3)))
+        assert big_stores == 1          # dx, and nothing else of that size
+    finally:
+        t.close()
