@@ -324,7 +324,9 @@ class FusedKernel(HipKernel):
         ops = self.ops
         first = ops[0]
         reductions = [op for op in ops if isinstance(op, og.ReductionOp) and op.reduction_axes.size > 1]
-        it_axes = iteration_axes(first)
+        # (a kernel may carry a few ops over a subset of its axes, absorbed from a smaller kernel:
+        # they are simply repeated along the missing axes)
+        it_axes = iteration_axes(max(ops, key=lambda o: (len(iteration_axes(o)), iteration_axes(o).size)))
         red_axes = reductions[0].reduction_axes if reductions else og.make_axes(())
         onehot_axes = [op.axis for op in ops if isinstance(op, og.OneHotOp)]
         take_axes = []           # output axes whose coordinate a lookup replaces by an index value
@@ -1002,10 +1004,29 @@ class FusionPlanner(object):
             groups.append(cur)
         if self.fusion:
             groups = self._recompute_across_groups(groups, readers, returned)
+            groups = self._absorb_small_groups(groups, readers, returned)
+            self._check_order(groups)
         for g in groups:
             if g.fusable:
                 g.decide_stores(readers, returned)
         return groups
+
+    @staticmethod
+    def _check_order(groups):
+        """Every value is produced before it is used: in an earlier kernel, or earlier in the same
+        one.  (The passes that move ops between kernels must keep this; a violation is a planner
+        bug, not a property of the user's graph.)"""
+        seen = set()
+        produced_somewhere = set(o for g in groups for o in g.ops)
+        for g in groups:
+            for o in g.ops:
+                for a in o.args:
+                    prod = _producer(a.forwarded)
+                    if prod in produced_somewhere and prod not in seen and prod is not o and \
+                            not isinstance(o, (og.AssignOp, og.Fill)):
+                        raise RuntimeError("planner: {} is used by {} before any kernel computes it"
+                                           .format(prod, o))
+                seen.add(o)
 
     # -- recomputation instead of a round trip through memory -------------------------------------
     max_recompute_ops = 6
@@ -1052,18 +1073,76 @@ class FusionPlanner(object):
                                    if _view_key(td) not in have and _memory_elements(td) > self.small_tensor]
                     if len(extra_large) > 1:
                         break
-                    ops = [o for o in chain if o not in h.ops] + h.ops
-                    new = _Group(ops[0], max_written_views=h.max_written_views)
-                    if not all(new.accepts(o, readers, returned) and (new.add(o) or True) for o in ops[1:]):
-                        break
                     # the repeated ops are private to the kernel: whoever else needs them has them
-                    new.never_store = set(h.never_store) | set(o for o in chain if o not in h.ops)
+                    new = _Group.rebuilt(h, chain, readers, returned, h.private)
+                    if new is None:
+                        break
                     rebuilt[hi] = new
                 else:
                     for hi, new in rebuilt.items():
                         groups[hi] = new
                     groups[gi].never_store.add(op)
         return groups
+
+    cheap_ops = ("add", "sub", "mul", "div", "neg", "abs", "sqrt", "rcp", "sqr", "minimum", "maximum", "assign")
+
+    def _absorb_small_groups(self, groups, readers, returned):
+        """A kernel over a few elements (per-channel factors between two passes over a big tensor)
+        costs a launch, several microseconds, for nanoseconds of work.  When it consists of a few
+        cheap elementwise ops and everything it produces is only read by later kernels whose axes
+        include its own, those kernels repeat its ops themselves -- per element, from operands
+        that are broadcast loads -- and the small kernel disappears."""
+        holders = {}        # an op may have been repeated in several kernels by now
+        for gi, g in enumerate(groups):
+            for op in g.ops:
+                holders.setdefault(op, set()).add(gi)
+        gone = set()
+        for gi, g in enumerate(groups):
+            if not g.fusable or len(g.ops) > self.max_recompute_ops or \
+                    g.axes.size > self.small_tensor or \
+                    not all(kernel_op_name(o) in self.cheap_ops for o in g.ops):
+                continue
+            inside = set(g.ops)
+            targets, ok = set(), True
+            for op in g.ops:
+                base = op.tensor_description().base
+                if base in returned:
+                    ok = False
+                    break
+                for u in readers.get(base, ()):
+                    if u in inside:
+                        continue
+                    for hi in holders.get(u, (-1,)):
+                        if hi <= gi or hi in gone or not groups[hi].fusable or \
+                                not g.axes.is_sub_set(groups[hi].axes) or \
+                                groups[hi].axes.size <= self.small_tensor:
+                            ok = False
+                            break
+                        targets.add(hi)
+                    if not ok:
+                        break
+                if not ok:
+                    break
+            if not ok or not targets:
+                continue
+            if self._written_between(self._outside_operands(g.ops), groups, gi, max(targets)):
+                continue
+            rebuilt = {}
+            for hi in sorted(targets):
+                h = groups[hi]
+                new = _Group.rebuilt(h, g.ops, readers, returned, inside | h.private)
+                if new is None:
+                    break
+                rebuilt[hi] = new
+            else:
+                for hi, new in rebuilt.items():
+                    groups[hi] = new
+                    for o in inside:
+                        holders[o].add(hi)
+                for o in inside:
+                    holders[o].discard(gi)
+                gone.add(gi)
+        return [g for gi, g in enumerate(groups) if gi not in gone]
 
     @staticmethod
     def _producer_chain(op, group, plain):
@@ -1110,7 +1189,8 @@ class FusionPlanner(object):
 
 
 class _Group(object):
-    def __init__(self, op, fusable=True, max_written_views=NGH_MAX_TENSORS):
+    def __init__(self, op, fusable=True, max_written_views=NGH_MAX_TENSORS, axes=None, private=()):
+        self.private = set(private)   # repeated ops: their results only ever live in registers
         self.ops = [op]
         self.fusable = fusable
         self.store_ops = set()
@@ -1118,7 +1198,8 @@ class _Group(object):
         self.max_written_views = max_written_views    # flex kernels: one statistics slot per result
         self.n_written_views = 0
         if fusable:
-            self.axes = iteration_axes(op)
+            self.axes = iteration_axes(op) if axes is None else axes
+            self.absorbed = set()     # ops over a subset of the axes, repeated along the others
             self.has_reduce = False
             self.red_axes = None
             self.read_views = {}     # base -> set(view keys)
@@ -1150,8 +1231,9 @@ class _Group(object):
         reads, writes = self._operand_views(op)
         for td in reads:
             self.read_views.setdefault(td.base, set()).add(td.parameter_key)
-        for td in writes:
-            self.write_views.setdefault(td.base, set()).add(td.parameter_key)
+        if op not in self.private:
+            for td in writes:
+                self.write_views.setdefault(td.base, set()).add(td.parameter_key)
         self.n_ops += 4
         self.n_consts += sum(1 for a in op.args if _scalar_constant_value(a.forwarded) is not None)
         if isinstance(op, og.ReductionOp) and op.reduction_axes.size > 1:
@@ -1184,10 +1266,33 @@ class _Group(object):
         self.n_written_views = len(written)
         return len(views | written)
 
-    def accepts(self, op, readers, returned):
-        if not iteration_axes(op).is_equal_set(self.axes) or \
-                iteration_axes(op).lengths != tuple(self.axes[self.axes.index(a)].length
-                                                    for a in iteration_axes(op)):
+    def axes_fit(self, op, absorb=False):
+        """Does op iterate over the group's axes -- or, for a cheap op of a smaller kernel that is
+        repeated along the axes it lacks (`absorb`), over some of them?"""
+        axes = iteration_axes(op)
+        if not (axes.is_sub_set(self.axes) if absorb else axes.is_equal_set(self.axes)):
+            return False
+        return axes.lengths == tuple(self.axes[self.axes.index(a)].length for a in axes)
+
+    @classmethod
+    def rebuilt(cls, h, first, readers, returned, private):
+        """The group `h` with the ops `first` (repeated from an earlier kernel, results private to
+        this one) put in front; None if the rules of a group do not allow it."""
+        # `first` is closed under its producers and reads only memory no kernel from its own to this
+        # one writes, so those of its ops that h already repeats can move to the front with it
+        ops = list(first) + [o for o in h.ops if o not in first]
+        new = cls(ops[0], max_written_views=h.max_written_views, axes=h.axes, private=private)
+        if not new.axes_fit(ops[0], ops[0] in new.private):
+            return None
+        for o in ops[1:]:
+            if not new.accepts(o, readers, returned, absorb=o in new.private):
+                return None
+            new.add(o)
+        new.never_store = set(h.never_store) | set(o for o in first if o not in h.ops)
+        return new
+
+    def accepts(self, op, readers, returned, absorb=False):
+        if not self.axes_fit(op, absorb):
             return False
         is_red = isinstance(op, og.ReductionOp) and op.reduction_axes.size > 1
         if self.has_reduce:

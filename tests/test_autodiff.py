@@ -266,5 +266,49 @@ def test_recomputation_replaces_a_round_trip_through_memory():
                                   and all(spec.tensors[spec.ops[i].dst].strides[a] != 0 or spec.shape[a] == 1
                                           for a in range(3)))
         assert big_stores == 1          # dx, and nothing else of that size
+        # the per-channel factors between the passes (gamma * rstd, the two sums over m) are
+        # repeated inside the dx kernel instead of costing launches of their own
+        assert len(t.kernel_groups[f].kernels) == 3     # statistics, the two sums, dx
     finally:
         t.close()
+
+
+@pytest.mark.gpu
+def test_per_channel_factors_absorbed_into_the_big_kernels():
+    """Small elementwise kernels between passes over a large tensor are repeated inside their
+    consumers (operands become broadcast loads); values against float64 closed forms, on axes
+    that do not merge into one row axis."""
+    from ngraph_hip.frontends import neon
+    C, H, N = ng.make_axis(8, name="C"), ng.make_axis(48, name="H"), ng.make_axis(256, name="N")
+    x, e = ng.placeholder([C, H, N]), ng.placeholder([C, H, N])
+    rs = np.random.RandomState(3)
+    gv = rs.uniform(0.5, 2, 8).astype(np.float32)
+    g, b = ng.variable([C], initial_value=gv), ng.variable([C], initial_value=np.zeros(8, np.float32))
+    y, _, _ = neon.batch_norm_train(x, g, b, [C])
+    xv = rs.normal(0.5, 2, (8, 48, 256)).astype(np.float32)
+    ev = rs.normal(0, 1, (8, 48, 256)).astype(np.float32)
+    t = ngt.make_transformer_factory("hipgpu")()
+    try:
+        f = t.computation([ng.deriv(y, x, error=e), ng.deriv(y, g, error=e), ng.deriv(y, b, error=e)], x, e)
+        # a per-channel scale feeding a large elementwise result and a reduction
+        s = ng.variable([C], initial_value=gv)
+        k = ng.sqrt(s * s + 1.0) * 0.5
+        f2 = t.computation([x * k, ng.sum(e * k, out_axes=[C])], x, e)
+        dx, dg, db = f(xv, ev)
+        assert len(t.kernel_groups[f].kernels) == 3
+        xs, es = f2(xv, ev)
+        assert len(t.kernel_groups[f2].kernels) == 1      # the scale chain, x * k and the sum
+    finally:
+        t.close()
+    m = 48 * 256
+    x64, e64 = xv.reshape(8, -1).astype(np.float64), ev.reshape(8, -1).astype(np.float64)
+    rstd = 1 / np.sqrt(x64.var(1, keepdims=True) + 1e-5)
+    xh = (x64 - x64.mean(1, keepdims=True)) * rstd
+    dg_want, db_want = (e64 * xh).sum(1), e64.sum(1)
+    dx_want = gv[:, None] * rstd * (e64 - db_want[:, None] / m - xh * dg_want[:, None] / m)
+    np.testing.assert_allclose(dx.reshape(8, -1), dx_want, rtol=1e-4, atol=2e-6)
+    np.testing.assert_allclose(dg, dg_want, rtol=1e-5, atol=1e-3)
+    np.testing.assert_allclose(db, db_want, rtol=1e-5, atol=1e-3)
+    k64 = np.sqrt(gv.astype(np.float64) ** 2 + 1.0) * 0.5
+    np.testing.assert_allclose(xs.reshape(8, -1), x64 * k64[:, None], rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(es, (e64 * k64[:, None]).sum(1), rtol=1e-5, atol=1e-3)

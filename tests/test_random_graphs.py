@@ -317,3 +317,46 @@ def test_flex_view_graph_host_and_device_management_agree(seed):
     for h, d in zip(host, device):
         for a, b in zip(h, d):
             np.testing.assert_array_equal(a, b)
+
+
+# ------------------------------------------------------------------ the planner's large-tensor rules on small graphs
+@pytest.fixture
+def everything_is_large(monkeypatch):
+    """Repeating a producer chain in a later kernel and folding a small kernel into its consumers
+    are rules for tensors above a size threshold, which the generators' shapes stay below.  With
+    the threshold at a few elements the same rules apply to these graphs."""
+    import ngraph_hip.transformers.hiptransform as ht
+    monkeypatch.setattr(ht.FusionPlanner, "small_tensor", 6)
+
+
+@pytest.mark.parametrize("seed", range(300))
+def test_graphs_lower_without_a_device_under_large_tensor_rules(seed, everything_is_large):
+    for builder in (build, build_views):
+        results, inputs, _ = builder(seed)
+        _lower_without_a_device(results, inputs)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(150))
+def test_random_graphs_match_oracle_under_large_tensor_rules(seed, everything_is_large):
+    results, inputs, values = build(seed)
+    for g, w in zip(run("hipgpu", results, inputs, values), run("cpu", results, inputs, values)):
+        np.testing.assert_allclose(g, w, rtol=2e-5, atol=2e-5)
+    results, inputs, values = build_views(seed)
+    for g, w in zip(run("hipgpu", results, inputs, values), run("cpu", results, inputs, values)):
+        ok = np.isfinite(w)
+        np.testing.assert_allclose(g[ok], w[ok], rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(500, 650))
+def test_state_programs_match_oracle_under_large_tensor_rules(seed, everything_is_large):
+    """Moving a computation into a later kernel must respect every write in between: an
+    assignment to a window of a variable the moved ops read, a kernel iterating over a window
+    of the moved op's axes."""
+    want_tot, want_vars = run_state("cpu", seed)
+    got_tot, got_vars = run_state("hipgpu", seed)
+    for g, w in zip(got_vars, want_vars):
+        np.testing.assert_allclose(g, w, rtol=2e-5, atol=2e-5)
+    for g, w in zip(got_tot, want_tot):
+        np.testing.assert_allclose(g, w, rtol=1e-4, atol=1e-3)
