@@ -275,8 +275,11 @@ def test_device_only_iterations_agree_across_policy_modes(n, monkeypatch):
             states = []
             for it in range(7):
                 group()
-                if name.startswith("deferred") and default_kernel_choice():
-                    assert t.runtime.flex_unsettled() == 1        # y's record, and only that
+                if name.startswith("deferred"):
+                    if default_kernel_choice():
+                        assert t.runtime.flex_unsettled() == 1    # y's record, and only that
+                    else:           # a forced kernel choice may or may not take the one-launch path
+                        assert t.runtime.flex_unsettled() in (0, 1)
                 elif name != "host":
                     assert t.runtime.flex_unsettled() == 0
                 if it in (2, 6):                    # look twice: after a few launches, and at the end
