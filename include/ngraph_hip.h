@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define NGH_ABI_VERSION 4
+#define NGH_ABI_VERSION 5
 
 /* ---- limits (float_ew2.py:285-286 MAX_AXES = 3) ------------------------ */
 #define NGH_MAX_AXES      3
@@ -231,6 +231,23 @@ int  ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec);
  * of `spec` (diagnostics and tests): writes a NUL-terminated name.          */
 int  ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec,
                         int32_t stage, char* name128);
+
+/* ---- run-time compiled programs: replaces the NVRTC step of the reference, which writes the
+ *      CUDA C of a kernel and compiles it when the transformer is initialised
+ *      (float_ew2.py:1553-1653 CudaSourceFile.add_kernel / compile).  Here the host side writes
+ *      the op programs of a computation that the library has no compiled kernel for as C++
+ *      tables, compiles them with hipcc into a program library, and hands its path over; from
+ *      then on ngh_launch_fused finds those kernels the way it finds the built-in ones (a
+ *      structural comparison, float_ew2.py:1486-1529 / :1560-1567 being the reference's hash
+ *      lookup), in every context of the process.  The library stays loaded.  out_added, when
+ *      not NULL, receives the number of programs that were new.  A library built from other
+ *      sources than this one (NGH_ABI_VERSION, layout of the argument block) is rejected with
+ *      NGH_E_INVALID.  A program library exports one function, named ngh_program_library,
+ *      taking (int abi, unsigned entry_bytes, unsigned args_bytes, const void** out_entries)
+ *      and returning the number of entries, or -1 when the three numbers are not its own.  */
+int  ngh_programs_load(ngh_context* ctx, const char* path, int32_t* out_added);
+/* number of compiled programs the process knows: built in, loaded */
+int  ngh_programs_count(int32_t* built_in, int32_t* loaded);
 
 /* Per-row mean and (biased) variance of a [rows, R] fp32 matrix with contiguous rows in ONE
  * read of x (x_cache_hint: NGH_CACHE_* bits for x): fuses the reductions behind ng.mean + ng.variance

@@ -20,7 +20,7 @@ import numpy as np  # noqa: E402
 import ngraph_hip as ng  # noqa: E402
 import ngraph_hip.transformers as ngt  # noqa: E402
 from ngraph_hip.frontends import neon  # noqa: E402
-from ngraph_hip.runtime import hiplib  # noqa: E402
+from ngraph_hip.runtime.programs import stage_programs, render  # noqa: E402
 
 OUT = os.path.join(HERE, "ngh_programs.inc")
 
@@ -148,7 +148,7 @@ PATTERNS = [
 
 
 def collect():
-    """[(name, ops, dtypes, bcast, stat_slot, n_regs)] for every streaming stage of every pattern."""
+    """Program records for every stage of every pattern that a compiled kernel can run."""
     programs, seen = [], set()
     for name, backend, build in PATTERNS:
         if backend not in ngt.transformer_choices():
@@ -156,103 +156,20 @@ def collect():
         t = ngt.make_transformer_factory(backend, dry_run=True)()
         f = build(t)
         t.initialize()
-        k_index = 0
-        for kernel in t.kernel_groups[f].kernels:
+        kernels = t.kernel_groups[f].kernels
+        for kernel in kernels:
             kernel.bind_buffers()
-            for spec in getattr(kernel, "specs", [])[:1]:
-                for stage in range(spec.n_stages):
-                    plan = hiplib.plan_fused(spec, stage)
-                    st = spec.stages[stage]
-                    family = plan["family"]
-                    total = spec.shape[0] * spec.shape[1] * spec.shape[2]
-                    # A one-element stage (a learning rule's step counter and rate factor) is worth a
-                    # program of its own: the interpreter fetches the code of every op kind it meets
-                    # with a cold instruction cache, several microseconds for twenty scalar ops.
-                    scalar = total == 1 and family == 0 and not st.n_reductions
-                    if family > 3 or (family == 0 and not scalar and (plan["V"] < 4 or st.n_reductions)):
-                        continue
-                    if family == 1 and spec.shape[0] // plan["V"] <= 64:
-                        continue          # short rows run the several-rows-per-workgroup kernel
-                    if total < 4096 and not scalar:
-                        continue          # small stages are launch-bound; the interpreter is fine
-                    if any(o.opcode >= hiplib.OPCODES["take"] for o in spec.ops[st.op_begin:st.op_end]):
-                        continue          # lookups only run in the interpreter
-                    ops = [(o.opcode, o.dst, o.a, o.b) for o in spec.ops[st.op_begin:st.op_end]]
-                    fast = plan["perm"][2]
-                    red_out = [st.red_out[r] for r in range(st.n_reductions)]
-                    dtypes = [spec.tensors[i].dtype for i in range(spec.n_tensors)]
-                    bcast = [1 if spec.tensors[i].strides[fast] == 0 else 0 for i in range(spec.n_tensors)]
-                    stored = set(o[1] for o in ops if o[0] == hiplib.OPCODES["store"])
-                    loaded = set(o[2] for o in ops if o[0] == hiplib.OPCODES["load"])
-                    staged, n_staged = [], 0
-                    for i in range(spec.n_tensors):
-                        st_i = spec.tensors[i].strides
-                        if family == 3 and i in (stored | loaded) and st_i[plan["perm"][1]] == 1 and \
-                                st_i[fast] not in (0, 1):
-                            staged.append(n_staged)
-                            n_staged += 1
-                        else:
-                            staged.append(-1)
-                    stat_slot, n_slots = [], 0
-                    for i in range(spec.n_tensors):
-                        if i in stored and dtypes[i] == hiplib.NGH_FLEX16 and n_slots < 4:
-                            stat_slot.append(n_slots)
-                            n_slots += 1
-                        else:
-                            stat_slot.append(-1)
-                    key = (tuple(ops), tuple(dtypes), tuple(bcast), plan["V"], family, tuple(red_out), tuple(staged))
-                    if key in seen:
-                        continue
-                    seen.add(key)
-                    programs.append(("%s_k%d" % (name, k_index), ops, dtypes, bcast, stat_slot,
-                                     n_slots, spec.n_regs, plan["V"], family, red_out, staged,
-                                     [1 if i in loaded else 0 for i in range(spec.n_tensors)],
-                                     [1 if i in stored else 0 for i in range(spec.n_tensors)]))
-            k_index += 1
+        programs += stage_programs(kernels, name, seen)
         t.close()
     return programs
 
 
-def render(programs):
-    lines = ["// GENERATED by gen_programs.py from the host lowering -- do not edit.",
-             "// One entry per streaming elementwise op program that gets a pre-built kernel."]
-    for i, (name, ops, dtypes, bcast, stat_slot, n_slots, n_regs, V, family, red_out, staged, loaded,
-            stored) in enumerate(programs):
-        lines.append("struct SP%d {  // %s" % (i, name))
-        lines.append("    static constexpr int V = %d, n_ops = %d, n_regs = %d, n_tensors = %d, "
-                     "n_stat_slots = %d, family = %d, n_red = %d;"
-                     % (V, len(ops), max(n_regs, 1), len(dtypes), n_slots, family, len(red_out)))
-        lines.append("    static constexpr int red_out[%d] = {%s};"
-                     % (max(len(red_out), 1), ", ".join(map(str, red_out or [0]))))
-        lines.append("    static constexpr ngh_op ops[%d] = {%s};"
-                     % (len(ops), ", ".join("{%d,%d,%d,%d}" % o for o in ops)))
-        lines.append("    static constexpr int dtypes[%d] = {%s};" % (len(dtypes), ", ".join(map(str, dtypes))))
-        lines.append("    static constexpr unsigned char bcast[%d] = {%s};" % (len(bcast), ", ".join(map(str, bcast))))
-        lines.append("    static constexpr int stat_slot[%d] = {%s};" % (len(stat_slot), ", ".join(map(str, stat_slot))))
-        lines.append("    static constexpr int n_staged = %d;" % sum(1 for x in staged if x >= 0))
-        lines.append("    static constexpr signed char staged[%d] = {%s};" % (len(staged), ", ".join(map(str, staged))))
-        lines.append("    static constexpr unsigned char loaded[%d] = {%s};" % (len(loaded), ", ".join(map(str, loaded))))
-        lines.append("    static constexpr unsigned char stored[%d] = {%s};" % (len(stored), ", ".join(map(str, stored))))
-        lines.append("};")
-    lines.append("static const StaticEntry kStaticTable[] = {")
-    for i, p in enumerate(programs):
-        if p[8] == 0:
-            launch = "&launch_static<SP%d>, nullptr, SP%d::staged, nullptr" % (i, i)
-        elif p[8] == 3:
-            launch = "nullptr, nullptr, SP%d::staged, &launch_static_tiled<SP%d>" % (i, i)
-        else:
-            launch = "nullptr, &launch_static_red<SP%d>, SP%d::staged, nullptr" % (i, i)
-        lines.append('    {"%s", SP%d::family, SP%d::V, SP%d::n_ops, SP%d::ops, SP%d::n_tensors, SP%d::dtypes, '
-                     'SP%d::bcast, SP%d::n_red, SP%d::red_out, %s},' % (p[0], i, i, i, i, i, i, i, i, i, launch))
-    if not programs:
-        lines.append('    {"none", 0, 4, 0, nullptr, 0, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr},')
-    lines.append("};")
-    lines.append("static const int kStaticCount = %d;" % len(programs))
-    return "\n".join(lines) + "\n"
+HEADER = ["// GENERATED by gen_programs.py from the host lowering -- do not edit.",
+          "// One entry per streaming elementwise op program that gets a pre-built kernel."]
 
 
 if __name__ == "__main__":
-    text = render(collect())
+    text = render(collect(), HEADER)
     if "--check" in sys.argv:
         sys.exit(0 if open(OUT).read() == text else 1)
     with open(OUT, "w") as fh:

@@ -1,0 +1,126 @@
+// The table of compiled op programs: the ones built into the library (ngh_programs.inc) and the
+// ones loaded at run time from program libraries (ngh_programs_load).
+//
+// Counterpart of the reference's kernel cache (ngraph/transformers/gpu/float_ew2.py:1486-1529
+// _ops_to_hash, :1560-1567 compiled-kernel lookup): there a structural hash of the op list finds
+// a kernel that NVRTC already compiled for this process, here a structural comparison finds a
+// kernel hipcc compiled -- with the library, or later into a program library by the host side
+// (ngraph_hip/runtime/jit.py).  Anything without an entry runs on the interpreter.
+#pragma once
+#include <atomic>
+#include <deque>
+#include <mutex>
+
+#include "ngh_special.h"
+
+namespace ngh {
+
+#include "ngh_programs.inc"
+
+// Entries of loaded program libraries.  Append-only: an index, once handed out, stays valid for
+// the life of the process (a deque never moves its elements), and the libraries stay loaded.
+struct LoadedPrograms {
+    std::mutex              lock;
+    std::deque<StaticEntry> entries;
+    std::atomic<int>        count{0};
+};
+inline LoadedPrograms& loaded_programs() {
+    static LoadedPrograms table;
+    return table;
+}
+
+inline const StaticEntry& special_entry(int i) {
+    return i < kStaticCount ? kStaticTable[i] : loaded_programs().entries[i - kStaticCount];
+}
+
+inline const char* special_name(int i) { return special_entry(i).name; }
+
+inline bool entry_matches(const StaticEntry& e, int family, int V, const KArgs& k) {
+    const int n_ops = k.op_end - k.op_begin;
+    if (e.family != family || e.V != V || e.n_ops != n_ops || e.n_tensors != k.n_tensors || e.n_red != k.n_red)
+        return false;
+    bool same = true;
+    for (int r = 0; r < e.n_red && same; ++r) same = e.red_out[r] == k.red_out[r];
+    for (int j = 0; j < n_ops && same; ++j) {
+        const ngh_op &a = e.ops[j], &b = k.ops[k.op_begin + j];
+        same = a.opcode == b.opcode && a.dst == b.dst && a.a == b.a && a.b == b.b;
+    }
+    for (int t = 0; t < k.n_tensors && same; ++t)
+        same = e.dtypes[t] == k.t[t].dtype && (e.bcast[t] != 0) == (k.t[t].s[2] == 0) &&
+               (family != 3 || e.staged[t] == k.t[t].stage_slot);
+    return same;
+}
+
+// family: 0 streaming elementwise (V >= 4), 1 / 2 reductions, 3 tiled elementwise
+inline int match_special(int family, int V, const KArgs& k, long long /*tail*/) {
+    // V == 1 entries exist for one-element stages only (every operand "broadcast")
+    const bool one_element = k.shape[0] * k.shape[1] * k.shape[2] == 1;
+    if (family > 3 || (family == 0 && ((V < 4 && !one_element) || k.n_red != 0))) return -1;
+    for (int i = 0; i < kStaticCount; ++i)
+        if (entry_matches(kStaticTable[i], family, V, k)) return i;
+    LoadedPrograms& L = loaded_programs();
+    const int n = L.count.load(std::memory_order_acquire);
+    for (int i = 0; i < n; ++i)
+        if (entry_matches(L.entries[i], family, V, k)) return kStaticCount + i;
+    return -1;
+}
+
+// Same program (what match_special compares), whatever the name.
+inline bool same_program(const StaticEntry& a, const StaticEntry& b) {
+    if (a.family != b.family || a.V != b.V || a.n_ops != b.n_ops || a.n_tensors != b.n_tensors || a.n_red != b.n_red)
+        return false;
+    for (int r = 0; r < a.n_red; ++r) if (a.red_out[r] != b.red_out[r]) return false;
+    for (int j = 0; j < a.n_ops; ++j)
+        if (a.ops[j].opcode != b.ops[j].opcode || a.ops[j].dst != b.ops[j].dst || a.ops[j].a != b.ops[j].a ||
+            a.ops[j].b != b.ops[j].b)
+            return false;
+    for (int t = 0; t < a.n_tensors; ++t)
+        if (a.dtypes[t] != b.dtypes[t] || (a.bcast[t] != 0) != (b.bcast[t] != 0) ||
+            (a.family == 3 && a.staged[t] != b.staged[t]))
+            return false;
+    return true;
+}
+
+// Add the entries of a loaded library that the table does not hold yet; returns how many were new.
+inline int add_loaded_programs(const StaticEntry* entries, int n) {
+    LoadedPrograms& L = loaded_programs();
+    std::lock_guard<std::mutex> guard(L.lock);
+    int added = 0;
+    for (int i = 0; i < n; ++i) {
+        bool known = false;
+        for (int j = 0; j < kStaticCount && !known; ++j) known = same_program(kStaticTable[j], entries[i]);
+        for (size_t j = 0; j < L.entries.size() && !known; ++j) known = same_program(L.entries[j], entries[i]);
+        if (known) continue;
+        L.entries.push_back(entries[i]);
+        L.count.store((int)L.entries.size(), std::memory_order_release);
+        ++added;
+    }
+    return added;
+}
+
+inline unsigned streaming_blocks(int cus, int blocks_per_cu, unsigned n_chunks) {
+    unsigned blocks = (n_chunks + kBlock - 1) / kBlock;
+    const unsigned cap = (unsigned)(cus * blocks_per_cu);
+    return blocks > cap ? cap : blocks;
+}
+
+inline hipError_t launch_special_tiled(int i, hipStream_t stream, unsigned blocks, const KArgs& k, unsigned tiles_a,
+                                       unsigned tiles_b, unsigned n_tiles, int tile) {
+    special_entry(i).launch_tiled(stream, blocks, k, tiles_a, tiles_b, n_tiles, tile);
+    return hipGetLastError();
+}
+
+inline hipError_t launch_special_red(int i, hipStream_t stream, unsigned blocks, const KArgs& k, unsigned n_first,
+                                     unsigned n_seg, unsigned seg_len, unsigned TX, RedWs ws, int cache_policy) {
+    special_entry(i).launch_red(stream, blocks, k, n_first, n_seg, seg_len, TX, ws, cache_policy);
+    return hipGetLastError();
+}
+
+inline hipError_t launch_special(int i, hipStream_t stream, unsigned blocks, const KArgs& k,
+                                 unsigned n_chunks, unsigned chunks_per_row, int cache_policy) {
+    if (n_chunks == 0) return hipSuccess;
+    special_entry(i).launch(stream, blocks, k, n_chunks, chunks_per_row, cache_policy);
+    return hipGetLastError();
+}
+
+}  // namespace ngh

@@ -2,6 +2,7 @@
 // planner that maps one stage of a fused spec onto a kernel skeleton, and the
 // launches.  See include/ngraph_hip.h for the contract of every entry point.
 #include <hip/hip_runtime.h>
+#include <dlfcn.h>
 
 #include <algorithm>
 #include <cstdarg>
@@ -15,7 +16,7 @@
 #include "ngh_device.h"
 #include "ngh_interp.h"
 #include "ngh_copy.h"
-#include "ngh_special.h"
+#include "ngh_table.h"
 #include "ngh_moments.h"
 #include "ngh_flex.h"
 
@@ -1152,6 +1153,37 @@ int ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec, int32_t sta
         const int cp = stage_cache_policy(ctx, *spec, spec->stages[stage]);
         strncat(name128, suffix[cp], 127 - strlen(name128));
     }
+    return NGH_OK;
+}
+
+int ngh_programs_load(ngh_context* ctx, const char* path, int32_t* out_added) {
+    if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
+    if (!path || !*path) return fail(NGH_E_INVALID, "path is NULL or empty");
+    HIP_TRY(hipSetDevice(ctx->device));
+    void* handle = dlopen(path, RTLD_NOW | RTLD_LOCAL);
+    if (!handle) return fail(NGH_E_INVALID, "cannot load program library %s: %s", path, dlerror());
+    typedef int (*table_fn)(int, unsigned, unsigned, const void**);
+    table_fn table = (table_fn)dlsym(handle, "ngh_program_library");
+    if (!table) {
+        dlclose(handle);
+        return fail(NGH_E_INVALID, "%s exports no ngh_program_library", path);
+    }
+    const void* entries = nullptr;
+    const int n = table(NGH_ABI_VERSION, (unsigned)sizeof(StaticEntry), (unsigned)sizeof(KArgs), &entries);
+    if (n < 0 || (n > 0 && !entries)) {
+        dlclose(handle);
+        return fail(NGH_E_INVALID, "%s was built from other sources than this library (ABI %d, entry %zu bytes, "
+                    "argument block %zu bytes)", path, NGH_ABI_VERSION, sizeof(StaticEntry), sizeof(KArgs));
+    }
+    // the handle is kept for the life of the process: table entries point into the library
+    const int added = add_loaded_programs((const StaticEntry*)entries, n);
+    if (out_added) *out_added = added;
+    return NGH_OK;
+}
+
+int ngh_programs_count(int32_t* built_in, int32_t* loaded) {
+    if (built_in) *built_in = kStaticCount;
+    if (loaded) *loaded = loaded_programs().count.load();
     return NGH_OK;
 }
 

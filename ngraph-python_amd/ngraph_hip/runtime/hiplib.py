@@ -12,7 +12,7 @@ import os
 
 import numpy as np
 
-NGH_ABI_VERSION = 4
+NGH_ABI_VERSION = 5
 NGH_MAX_AXES = 3
 NGH_MAX_TENSORS = 12
 NGH_MAX_OPS = 96
@@ -122,6 +122,8 @@ _SYMBOLS = {
     "ngh_launch_fused_flex": [_vp, ctypes.POINTER(ngh_fused_spec), _vp, ctypes.POINTER(ctypes.c_int32),
                               ctypes.POINTER(ctypes.c_int32), _i32, _i32],
     "ngh_flex_unsettled": [_vp, ctypes.POINTER(ctypes.c_int32)],
+    "ngh_programs_load": [_vp, ctypes.c_char_p, ctypes.POINTER(ctypes.c_int32)],
+    "ngh_programs_count": [ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32)],
     "ngh_timer_begin": [_vp],
     "ngh_timer_end": [_vp, ctypes.POINTER(ctypes.c_float)],
 }
@@ -372,6 +374,14 @@ class HipRuntime(object):
         _check(self.lib, self.lib.ngh_flex_unsettled(self.ctx, ctypes.byref(n)))
         return n.value
 
+    # -- compiled programs ---------------------------------------------------
+    def programs_load(self, path):
+        """Add the compiled programs of a program library (runtime/jit.py) to the library's
+        table; returns how many were new."""
+        n = ctypes.c_int32()
+        _check(self.lib, self.lib.ngh_programs_load(self.ctx, os.fsencode(path), ctypes.byref(n)))
+        return n.value
+
     # -- timing ------------------------------------------------------------
     def timer_begin(self):
         _check(self.lib, self.lib.ngh_timer_begin(self.ctx))
@@ -392,6 +402,7 @@ class DryRunRuntime(object):
         self.lib = load_library()
         self._next = 1 << 32
         self.launched = []
+        self.program_libraries = []
 
     def close(self):
         pass
@@ -460,6 +471,10 @@ class DryRunRuntime(object):
         self.launch_fused(spec)
 
     def flex_unsettled(self):
+        return 0
+
+    def programs_load(self, path):
+        self.program_libraries.append(path)      # compiled, not loaded: there is no device
         return 0
 
 
@@ -668,3 +683,11 @@ class FusedSpecBuilder(object):
             for j, t in enumerate(reds):
                 s.red_out[j] = t
         return spec
+
+
+def programs_count():
+    """(built in, loaded) compiled programs the process knows."""
+    lib = load_library()
+    a, b = ctypes.c_int32(), ctypes.c_int32()
+    _check(lib, lib.ngh_programs_count(ctypes.byref(a), ctypes.byref(b)))
+    return a.value, b.value

@@ -1,0 +1,110 @@
+"""Compiled op programs: from lowered kernels to the C++ tables the kernels are instantiated on.
+
+A stage of a lowered fused kernel that one of the streaming / reduction / tiled skeletons can run
+is described by a record (op list, operand types, which operands are broadcast along the fast
+axis, vector width, skeleton); `render` writes records as the `struct SPn` tables and the entry
+table that `csrc/ngh_special.h` instantiates kernels on.  Two users: `csrc/gen_programs.py`
+writes the table that is built into the library, `jit.py` writes tables for the programs of a
+user's computation and compiles them at run time (the reference generates and compiles CUDA C per
+computation, float_ew2.py:1135-1483, :1553-1653).
+"""
+from ngraph_hip.runtime import hiplib
+
+
+def stage_programs(kernels, name, seen=None, min_elements=4096):
+    """Records for every stage of `kernels` (lowered, buffers bound) that can run as a compiled
+    program; `seen` holds the structural keys already recorded."""
+    programs = []
+    seen = set() if seen is None else seen
+    k_index = 0
+    for kernel in kernels:
+        for spec in getattr(kernel, "specs", [])[:1]:
+            for stage in range(spec.n_stages):
+                plan = hiplib.plan_fused(spec, stage)
+                st = spec.stages[stage]
+                family = plan["family"]
+                total = spec.shape[0] * spec.shape[1] * spec.shape[2]
+                # A one-element stage (a learning rule's step counter and rate factor) is worth a
+                # program of its own: the interpreter fetches the code of every op kind it meets
+                # with a cold instruction cache, several microseconds for twenty scalar ops.
+                scalar = total == 1 and family == 0 and not st.n_reductions
+                if family > 3 or (family == 0 and not scalar and (plan["V"] < 4 or st.n_reductions)):
+                    continue
+                if family == 1 and spec.shape[0] // plan["V"] <= 64:
+                    continue          # short rows run the several-rows-per-workgroup kernel
+                if total < min_elements and not scalar:
+                    continue          # small stages are launch-bound; the interpreter is fine
+                if any(o.opcode >= hiplib.OPCODES["take"] for o in spec.ops[st.op_begin:st.op_end]):
+                    continue          # lookups only run in the interpreter
+                ops = [(o.opcode, o.dst, o.a, o.b) for o in spec.ops[st.op_begin:st.op_end]]
+                fast = plan["perm"][2]
+                red_out = [st.red_out[r] for r in range(st.n_reductions)]
+                dtypes = [spec.tensors[i].dtype for i in range(spec.n_tensors)]
+                bcast = [1 if spec.tensors[i].strides[fast] == 0 else 0 for i in range(spec.n_tensors)]
+                stored = set(o[1] for o in ops if o[0] == hiplib.OPCODES["store"])
+                loaded = set(o[2] for o in ops if o[0] == hiplib.OPCODES["load"])
+                staged, n_staged = [], 0
+                for i in range(spec.n_tensors):
+                    st_i = spec.tensors[i].strides
+                    if family == 3 and i in (stored | loaded) and st_i[plan["perm"][1]] == 1 and \
+                            st_i[fast] not in (0, 1):
+                        staged.append(n_staged)
+                        n_staged += 1
+                    else:
+                        staged.append(-1)
+                stat_slot, n_slots = [], 0
+                for i in range(spec.n_tensors):
+                    if i in stored and dtypes[i] == hiplib.NGH_FLEX16 and n_slots < 4:
+                        stat_slot.append(n_slots)
+                        n_slots += 1
+                    else:
+                        stat_slot.append(-1)
+                key = (tuple(ops), tuple(dtypes), tuple(bcast), plan["V"], family, tuple(red_out), tuple(staged))
+                if key in seen:
+                    continue
+                seen.add(key)
+                programs.append(("%s_k%d" % (name, k_index), ops, dtypes, bcast, stat_slot,
+                                 n_slots, spec.n_regs, plan["V"], family, red_out, staged,
+                                 [1 if i in loaded else 0 for i in range(spec.n_tensors)],
+                                 [1 if i in stored else 0 for i in range(spec.n_tensors)],
+                                 plan["special"]))
+        k_index += 1
+    return programs
+
+
+def render(programs, header, prefix="SP", table="kStaticTable", count="kStaticCount"):
+    """C++ text: one `struct <prefix>n` per record, the entry table and its length."""
+    lines = list(header)
+    for i, (name, ops, dtypes, bcast, stat_slot, n_slots, n_regs, V, family, red_out, staged, loaded,
+            stored, _) in enumerate(programs):
+        lines.append("struct %s%d {  // %s" % (prefix, i, name))
+        lines.append("    static constexpr int V = %d, n_ops = %d, n_regs = %d, n_tensors = %d, "
+                     "n_stat_slots = %d, family = %d, n_red = %d;"
+                     % (V, len(ops), max(n_regs, 1), len(dtypes), n_slots, family, len(red_out)))
+        lines.append("    static constexpr int red_out[%d] = {%s};"
+                     % (max(len(red_out), 1), ", ".join(map(str, red_out or [0]))))
+        lines.append("    static constexpr ngh_op ops[%d] = {%s};"
+                     % (len(ops), ", ".join("{%d,%d,%d,%d}" % o for o in ops)))
+        lines.append("    static constexpr int dtypes[%d] = {%s};" % (len(dtypes), ", ".join(map(str, dtypes))))
+        lines.append("    static constexpr unsigned char bcast[%d] = {%s};" % (len(bcast), ", ".join(map(str, bcast))))
+        lines.append("    static constexpr int stat_slot[%d] = {%s};" % (len(stat_slot), ", ".join(map(str, stat_slot))))
+        lines.append("    static constexpr int n_staged = %d;" % sum(1 for x in staged if x >= 0))
+        lines.append("    static constexpr signed char staged[%d] = {%s};" % (len(staged), ", ".join(map(str, staged))))
+        lines.append("    static constexpr unsigned char loaded[%d] = {%s};" % (len(loaded), ", ".join(map(str, loaded))))
+        lines.append("    static constexpr unsigned char stored[%d] = {%s};" % (len(stored), ", ".join(map(str, stored))))
+        lines.append("};")
+    lines.append("static const StaticEntry %s[] = {" % table)
+    for i, p in enumerate(programs):
+        if p[8] == 0:
+            launch = "&launch_static<{0}>, nullptr, {0}::staged, nullptr".format(prefix + str(i))
+        elif p[8] == 3:
+            launch = "nullptr, nullptr, {0}::staged, &launch_static_tiled<{0}>".format(prefix + str(i))
+        else:
+            launch = "nullptr, &launch_static_red<{0}>, {0}::staged, nullptr".format(prefix + str(i))
+        lines.append('    {{"{1}", {0}::family, {0}::V, {0}::n_ops, {0}::ops, {0}::n_tensors, {0}::dtypes, '
+                     '{0}::bcast, {0}::n_red, {0}::red_out, {2}}},'.format(prefix + str(i), p[0], launch))
+    if not programs:
+        lines.append('    {"none", 0, 4, 0, nullptr, 0, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr},')
+    lines.append("};")
+    lines.append("static const int %s = %d;" % (count, len(programs)))
+    return "\n".join(lines) + "\n"

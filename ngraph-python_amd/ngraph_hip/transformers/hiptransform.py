@@ -837,6 +837,12 @@ class HipKernelGroup(object):
             if not k.buffers_bound:
                 k.bind_buffers()
         self.assign_cache_hints()
+        if self.transformer.jit:
+            # compile what would otherwise run on the interpreter (float_ew2.py:1553-1653: the
+            # reference compiles every kernel of a computation at this point)
+            from ngraph_hip.runtime import jit
+            jit.ensure_programs(self.transformer.runtime, self.kernels, self.name,
+                                min_elements=self.transformer.jit_min_elements)
         self._bound = True
 
     def assign_cache_hints(self):
@@ -1428,10 +1434,17 @@ class HipTransformer(ComputationGraphTransformer):
     kernel_group_class = HipKernelGroup
     max_written_views = NGH_MAX_TENSORS      # results one fused kernel may write
 
-    def __init__(self, device_id=0, fusion=True, dry_run=False, fuse_moments=None, rng_seed=0, **kwargs):
+    def __init__(self, device_id=0, fusion=True, dry_run=False, fuse_moments=None, rng_seed=0, jit=None,
+                 jit_min_elements=4096, **kwargs):
         """dry_run=True lowers graphs to kernel specs without a device (no results can be
         read back); it exists so the host-side lowering can be inspected and tested.
-        rng_seed keys the random fills (ng.uniform / ng.normal): same seed, same numbers."""
+        rng_seed keys the random fills (ng.uniform / ng.normal): same seed, same numbers.
+        jit=True compiles, when a computation is first run, kernels for those of its stages
+        (of at least jit_min_elements elements) that the library has no compiled program for;
+        default: the NGH_JIT environment variable, else off."""
+        from ngraph_hip.runtime import jit as _jit
+        self.jit = _jit.enabled_by_default() if jit is None else bool(jit)
+        self.jit_min_elements = int(jit_min_elements)
         try:
             self.runtime = DryRunRuntime() if dry_run else HipRuntime(device_id)
         except HipLibraryError as e:

@@ -1,0 +1,104 @@
+"""Graphs whose kernels the tests of run-time compiled programs (test_jit.py) compile.
+
+`precompile()` lowers every case without a device and compiles its program libraries into the
+cache, so that a build on a machine without a GPU leaves nothing to compile for the GPU tests
+(they compile on the spot if the cache lacks a library).
+"""
+import numpy as np
+
+import ngraph_hip as ng
+import ngraph_hip.transformers as ngt
+
+
+def _ab(a=512, b=1024):
+    return ng.make_axis(a, name="A"), ng.make_axis(b, name="B")
+
+
+def case_elementwise():
+    A, B = _ab()
+    x, y, w = ng.placeholder([A, B]), ng.placeholder([A, B]), ng.placeholder([A, B])
+    z = ng.tanh(x * y + 0.5) / (ng.absolute(y) + 1.0)
+    return [z * w, ng.maximum(z, w) - x], [x, y, w]
+
+
+def case_column_reduction_with_store():
+    A, B = _ab()
+    x, y = ng.placeholder([A, B]), ng.placeholder([A, B])
+    z = ng.tanh(x * y + 0.5) / (ng.absolute(y) + 1.0)
+    return [z, ng.max(z, out_axes=[B]), ng.argmax(z * x, out_axes=[B])], [x, y]
+
+
+def case_row_reduction_with_store():
+    A, B = _ab()
+    x, y = ng.placeholder([A, B]), ng.placeholder([A, B])
+    z = ng.sqrt(ng.absolute(x * y) + 0.25)
+    return [z, ng.sum(z * z, out_axes=[A]), ng.min(z, out_axes=[A])], [x, y]
+
+
+def case_transposed_operand():
+    A, B = _ab()
+    xs, x, y = ng.placeholder([B, A]), ng.placeholder([A, B]), ng.placeholder([A, B])
+    return [ng.sigmoid(ng.axes_with_order(xs, [A, B]) * x) + y], [xs, x, y]
+
+
+def case_softmax():
+    A, B = _ab()
+    x = ng.placeholder([A, B])
+    e = ng.exp(x - ng.max(x, out_axes=[A]))
+    return [e / ng.sum(e, out_axes=[A])], [x]
+
+
+def case_mixed_storage_types():
+    A, B = _ab()
+    x, h = ng.placeholder([A, B]), ng.placeholder([A, B], dtype=np.float16)
+    i = ng.placeholder([A, B], dtype=np.int32)
+    return [ng.minimum(x * h, 4.0) + i, ng.sum(h * x, out_axes=[B])], [x, h, i]
+
+
+def case_ragged():
+    # extents that leave a tail after the vector-wide part and rows that are not a multiple of 4
+    A, B = ng.make_axis(301, name="A"), ng.make_axis(77, name="B")
+    x, y = ng.placeholder([A, B]), ng.placeholder([A, B])
+    return [ng.exp(-ng.square(x)) * y + 1.0, ng.sum(x * y + 1.0, out_axes=[A])], [x, y]
+
+
+FP32_CASES = [case_elementwise, case_column_reduction_with_store, case_row_reduction_with_store,
+              case_transposed_operand, case_softmax, case_mixed_storage_types, case_ragged]
+
+
+def flex_case():
+    P = ng.make_axis(1 << 16, name="P")
+    x, w, b = ng.placeholder([P]), ng.placeholder([P]), ng.placeholder([P])
+    return [ng.tanh(x * w) + b], [x, w, b]
+
+
+def inputs_for(placeholders, seed):
+    vals = []
+    for i, p in enumerate(placeholders):
+        rs = np.random.RandomState(seed + i)
+        if p.dtype == np.int32:
+            vals.append(rs.randint(-5, 6, p.axes.lengths).astype(np.int32))
+        else:
+            vals.append(rs.uniform(-1, 1, p.axes.lengths).astype(p.dtype))
+    return vals
+
+
+def precompile(verbose=False):
+    """Compile the program libraries of every case (no device needed); returns their paths."""
+    paths = []
+    for backend, cases in (("hipgpu", FP32_CASES), ("flexhip", [flex_case])):
+        if backend not in ngt.transformer_choices():
+            continue
+        for case in cases:
+            t = ngt.make_transformer_factory(backend, dry_run=True, jit=True)()
+            try:
+                results, inputs = case()
+                f = t.computation(results, *inputs)
+                t.initialize()
+                t.kernel_groups[f].bind()
+                paths += t.runtime.program_libraries
+                if verbose:
+                    print(case.__name__, t.runtime.program_libraries)
+            finally:
+                t.close()
+    return paths

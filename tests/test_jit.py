@@ -1,0 +1,155 @@
+"""Run-time compiled programs: a computation's stages that the library has no compiled kernel for
+are written out as program tables, compiled by hipcc and loaded (the reference's counterpart is
+the NVRTC compilation of generated CUDA C, float_ew2.py:1553-1653).  A compiled program must give
+what the interpreter gives for the same spec, to the last bit (same skeleton, same op
+definitions, same order of operations)."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+import ngraph_hip as ng
+import ngraph_hip.transformers as ngt
+from ngraph_hip.runtime import hiplib, jit
+from conftest import default_kernel_choice
+
+import jit_cases
+
+
+def _dry_kernels(case, backend="hipgpu"):
+    t = ngt.make_transformer_factory(backend, dry_run=True)()
+    results, inputs = case()
+    f = t.computation(results, *inputs)
+    t.initialize()
+    kernels = t.kernel_groups[f].kernels
+    for k in kernels:
+        k.bind_buffers()
+    return t, kernels
+
+
+def test_uncovered_programs_are_found_and_rendered():
+    t, kernels = _dry_kernels(jit_cases.case_elementwise)
+    try:
+        programs = jit.uncovered_programs(kernels, "case")
+        assert len(programs) == 1 and programs[0][8] == 0          # one streaming elementwise stage
+        text = jit.source_text(programs)
+        assert 'extern "C" int ngh_program_library' in text and "launch_static<LP0>" in text
+        # a built-in program is not compiled again
+        t2, k2 = _dry_kernels(lambda: (lambda x: ([ng.sum(x, out_axes=[x.axes[0]])], [x]))(
+            ng.placeholder([ng.make_axis(4096, name="A"), ng.make_axis(4096, name="B")])))
+        try:
+            assert jit.uncovered_programs(k2, "sum") == []
+        finally:
+            t2.close()
+    finally:
+        t.close()
+
+
+def test_program_library_compiles_and_checks_its_caller(tmp_path, monkeypatch):
+    """hipcc cross-compiles a program library without a device; its entry point refuses a caller
+    built from other sources (ABI number, structure sizes)."""
+    monkeypatch.setenv("NGH_PROGRAM_CACHE", str(tmp_path))
+    t, kernels = _dry_kernels(jit_cases.case_row_reduction_with_store)
+    try:
+        programs = jit.uncovered_programs(kernels, "case")
+        assert programs
+        path = jit.compile_programs(programs)
+        assert os.path.dirname(path) == str(tmp_path)
+        assert jit.compile_programs(programs) == path                  # second time: from the cache
+        lib = ctypes.CDLL(path)
+        fn = lib.ngh_program_library
+        fn.argtypes = [ctypes.c_int, ctypes.c_uint, ctypes.c_uint, ctypes.POINTER(ctypes.c_void_p)]
+        out = ctypes.c_void_p()
+        assert fn(hiplib.NGH_ABI_VERSION + 1, 0, 0, ctypes.byref(out)) == -1
+        assert fn(hiplib.NGH_ABI_VERSION, 1, 1, ctypes.byref(out)) == -1
+    finally:
+        t.close()
+
+
+def test_jit_is_off_unless_asked_for(monkeypatch):
+    monkeypatch.delenv("NGH_JIT", raising=False)
+    t = ngt.make_transformer_factory("hipgpu", dry_run=True)()
+    assert not t.jit
+    t.close()
+    monkeypatch.setenv("NGH_JIT", "1")
+    t = ngt.make_transformer_factory("hipgpu", dry_run=True)()
+    assert t.jit
+    t.close()
+
+
+def _run(backend, case, seed, **kwargs):
+    t = ngt.make_transformer_factory(backend, **kwargs)()
+    try:
+        results, inputs = case()
+        f = t.computation(results, *inputs)
+        out = [np.array(r).copy() for r in f(*jit_cases.inputs_for(inputs, seed))]
+        groups = getattr(t, "kernel_groups", None)
+        names = [d for k in groups[f].kernels for ds in k.describe() for d in ds] if groups else []
+        return out, names
+    finally:
+        t.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", jit_cases.FP32_CASES, ids=lambda c: c.__name__)
+def test_compiled_programs_agree_with_the_interpreter(case):
+    import oracle.cpu_transformer  # noqa: F401
+    want, _ = _run("cpu", case, 5)
+    interp, names_interp = _run("hipgpu", case, 5, jit=False)
+    compiled, names = _run("hipgpu", case, 5, jit=True)
+    for a, b, w in zip(interp, compiled, want):
+        np.testing.assert_array_equal(a, b)
+        np.testing.assert_allclose(b, w, rtol=1e-5, atol=1e-5)
+    if default_kernel_choice():
+        # every stage large enough to be worth a compiled kernel has one now
+        assert not any("interp" in n for n in names if "tail" not in n), names
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("resident", [False, True], ids=["host-policy", "device-policy"])
+def test_compiled_flex_program_agrees_with_the_interpreter(resident):
+    """A flex kernel compiled at run time carries statistics slots like the built-in ones: in
+    device-resident mode it takes the one-launch path with deferred statistics."""
+    def run(use_jit):
+        t = ngt.make_transformer_factory("flexhip", resident=resident, jit=use_jit)()
+        try:
+            results, inputs = jit_cases.flex_case()
+            f = t.computation(results, *inputs)
+            vals = jit_cases.inputs_for(inputs, 9)
+            outs = [np.array(f(vals[0] * g, vals[1], vals[2])).copy() for g in (1.0, 4.0, 30.0, 0.1, 1.0)]
+            names = [d for k in t.kernel_groups[f].kernels for ds in k.describe() for d in ds]
+            return outs, names
+        finally:
+            t.close()
+    a, _ = run(False)
+    b, names = run(True)
+    for x, y in zip(a, b):
+        np.testing.assert_array_equal(x, y)
+    if default_kernel_choice():
+        assert any(n.startswith("special:") for n in names), names
+
+
+@pytest.mark.gpu
+def test_loading_a_program_library_twice_adds_nothing():
+    from ngraph_hip.runtime import HipRuntime
+    t, kernels = _dry_kernels(jit_cases.case_softmax)
+    try:
+        # (earlier tests of this process may have loaded these very programs)
+        built_in = hiplib.programs_count()[0]
+        programs = [p for p in jit.uncovered_programs(kernels, "case", include_covered=True)
+                    if not 0 <= p[-1] < built_in]
+        assert len(programs) == 2
+        path = jit.compile_programs(programs)
+    finally:
+        t.close()
+    rt = HipRuntime(0)
+    try:
+        rt.programs_load(path)
+        built_in, loaded = hiplib.programs_count()
+        assert rt.programs_load(path) == 0
+        assert hiplib.programs_count() == (built_in, loaded)
+        with pytest.raises(hiplib.HipLibraryError):
+            rt.programs_load(os.path.join(os.path.dirname(path), "no_such_library.so"))
+    finally:
+        rt.close()
