@@ -7,8 +7,8 @@ structural hash (:1486-1529).  The library here carries compiled kernels for the
 dominate training graphs and an interpreter for everything else; this module closes the gap for
 a user's own graphs: the stage programs that no compiled kernel covers are written out as the
 same C++ tables the built-in ones are made from, compiled by hipcc into a *program library*
-(one shared object per set of programs, named by a hash of the tables, the kernel headers and
-the compiler flags) and handed to the library with `ngh_programs_load`.  The object files are
+(one shared object per program, named by a hash of its table, the kernel headers and the
+compiler flags) and handed to the library with `ngh_programs_load`.  The object files are
 kept, so a program is compiled once per machine, not once per process.
 
 Opt-in (`make_transformer_factory("hipgpu", jit=True)` or NGH_JIT=1): compiling takes seconds
@@ -118,4 +118,15 @@ def ensure_programs(runtime, kernels, name, min_elements=4096, verbose=False):
     programs = uncovered_programs(kernels, name, min_elements)
     if not programs:
         return 0
-    return runtime.programs_load(compile_programs(programs, verbose=verbose))
+    # One library per program: what a library holds, and so its name in the cache, depends on the
+    # program alone and not on which other programs this process happened to have loaded before.
+    if len(programs) == 1:
+        paths = [compile_programs(programs, verbose=verbose)]
+    else:
+        from multiprocessing.pool import ThreadPool          # the work is in hipcc subprocesses
+        pool = ThreadPool(min(len(programs), max(1, min(8, (os.cpu_count() or 2) // 2))))
+        try:
+            paths = pool.map(lambda p: compile_programs([p], verbose=verbose), programs)
+        finally:
+            pool.close()
+    return sum(runtime.programs_load(path) for path in paths)

@@ -646,6 +646,9 @@ class CopyKernel(HipKernel):
         return [(self.op.args[0].forwarded.tensor_description().base, True, False),
                 (self.op.tensor_description().base, False, True)]
 
+    def describe(self):
+        return [["copy_strided"]]
+
     def execute(self):
         self.transformer.runtime.copy_strided(self.dst.ptr, self.src.ptr, self.shape,
                                               self.dst_strides, self.src_strides, self.dst.itemsize)

@@ -72,6 +72,16 @@ def flex_case():
     return [ng.tanh(x * w) + b], [x, w, b]
 
 
+# random graphs of tests/test_random_graphs.py: small shapes, so every stage counts as worth
+# compiling (jit_min_elements=1); the odd programs a generator finds and a person would not write
+RANDOM_SEEDS = list(range(8))
+
+
+def random_case(seed, views):
+    import test_random_graphs as T
+    return (T.build_views if views else T.build)(seed)
+
+
 def inputs_for(placeholders, seed):
     vals = []
     for i, p in enumerate(placeholders):
@@ -99,6 +109,17 @@ def precompile(verbose=False):
                 paths += t.runtime.program_libraries
                 if verbose:
                     print(case.__name__, t.runtime.program_libraries)
+            finally:
+                t.close()
+    for seed in RANDOM_SEEDS:
+        for views in (False, True):
+            t = ngt.make_transformer_factory("hipgpu", dry_run=True, jit=True, jit_min_elements=1)()
+            try:
+                results, inputs, _ = random_case(seed, views)
+                f = t.computation(results, *inputs)
+                t.initialize()
+                t.kernel_groups[f].bind()
+                paths += t.runtime.program_libraries
             finally:
                 t.close()
     return paths

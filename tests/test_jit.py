@@ -107,6 +107,22 @@ def test_compiled_programs_agree_with_the_interpreter(case):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("views", [False, True], ids=["plain", "views"])
+@pytest.mark.parametrize("seed", jit_cases.RANDOM_SEEDS)
+def test_random_graphs_compiled_agree_with_the_interpreter(seed, views):
+    def run(**kwargs):
+        t = ngt.make_transformer_factory("hipgpu", **kwargs)()
+        try:
+            results, inputs, values = jit_cases.random_case(seed, views)
+            f = t.computation(results, *inputs)
+            return [np.array(r).copy() for r in f(*values)]
+        finally:
+            t.close()
+    for a, b in zip(run(jit=False), run(jit=True, jit_min_elements=1)):
+        np.testing.assert_array_equal(a, b)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("resident", [False, True], ids=["host-policy", "device-policy"])
 def test_compiled_flex_program_agrees_with_the_interpreter(resident):
     """A flex kernel compiled at run time carries statistics slots like the built-in ones: in
@@ -140,13 +156,16 @@ def test_loading_a_program_library_twice_adds_nothing():
         programs = [p for p in jit.uncovered_programs(kernels, "case", include_covered=True)
                     if not 0 <= p[-1] < built_in]
         assert len(programs) == 2
-        path = jit.compile_programs(programs)
+        paths = [jit.compile_programs([p]) for p in programs]
+        path = paths[0]
     finally:
         t.close()
     rt = HipRuntime(0)
     try:
-        rt.programs_load(path)
+        for p in paths:
+            rt.programs_load(p)
         built_in, loaded = hiplib.programs_count()
+        assert loaded >= 2
         assert rt.programs_load(path) == 0
         assert hiplib.programs_count() == (built_in, loaded)
         with pytest.raises(hiplib.HipLibraryError):
