@@ -25,7 +25,7 @@ import numpy as np  # noqa: E402
 HBM_PEAK_GBS = 8000.0
 # HBM bytes one launch of the C2 normalise kernel moves, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE scaled by a device copy of known size (profiles/c2_batchnorm_pmc_traffic.md)
-MEASURED_TRAFFIC = {"special:batchnorm": 411154943}
+MEASURED_TRAFFIC = {"special:batchnorm": 411173686}
 
 
 def build_c2(ng, neon, t, dims):
@@ -141,6 +141,45 @@ def other_configs(ng, ngt, neon, configs, steps, warmup):
     return out
 
 
+def user_graphs(ng, An=8192, Bn=8192):
+    """(name, results, inputs, passes over an An x Bn fp32 tensor) of graphs the library has no
+    built-in program for: what a user's own elementwise / reduction code looks like."""
+    A, B = ng.make_axis(An, name="A"), ng.make_axis(Bn, name="B")
+    x, y, w = ng.placeholder([A, B]), ng.placeholder([A, B]), ng.placeholder([A, B])
+    z = ng.tanh(x * y + 0.5) / (ng.absolute(y) + 1.0)
+    yield "chain_3in_2out", [z * w, ng.maximum(z, w) - x], [x, y, w], 5
+    yield "gelu_tanh_form", [0.5 * x * (1.0 + ng.tanh(0.79788456 * (x + 0.044715 * x * x * x)))], [x], 2
+    yield "chain_with_column_max", [z, ng.max(z, out_axes=[B])], [x, y], 3
+    yield "row_sum_of_squared_difference", [ng.sum(ng.square(x - y), out_axes=[A])], [x, y], 2
+    e = ng.exp(x - ng.max(x, out_axes=[A]))
+    yield "softmax_rows", [e / ng.sum(e, out_axes=[A])], [x], 4
+
+
+def compiled_vs_interpreted(ng, ngt, steps, warmup, An=8192, Bn=8192):
+    """The same computations on the interpreter and with kernels compiled at run time
+    (make_transformer_factory(..., jit=True)): ms per step, algorithmic GB/s, kernels."""
+    out = {}
+    for name, results, inputs, passes in user_graphs(ng, An, Bn):
+        row = {}
+        for mode in (False, True):
+            t = ngt.make_transformer_factory("hipgpu", jit=mode)()
+            try:
+                f = t.computation(results, *inputs)
+                f(*[np.random.RandomState(1 + i).uniform(-1, 1, p.axes.lengths).astype(np.float32)
+                    for i, p in enumerate(inputs)])
+                group = t.kernel_groups[f]
+                group()
+                t.runtime.sync()
+                ms = time_steps(t.runtime, group, steps, warmup)
+                row["compiled" if mode else "interpreted"] = {
+                    "ms_per_step": round(ms, 5), "GB/s": round(passes * An * Bn * 4 / (ms * 1e-3) / 1e9, 1),
+                    "kernels": [d for k in group.kernels for ds in k.describe() for d in ds]}
+            finally:
+                t.close()
+        out[name] = row
+    return out
+
+
 def cpu_baseline_c2(dims, budget_s=20.0):
     from oracle import configs
     C, R = dims[0], dims[1] * dims[2] * dims[3]
@@ -165,6 +204,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--all", action="store_true", help="also time configs C1, C3, C4, C5")
+    ap.add_argument("--compiled", action="store_true",
+                    help="also time five user graphs on the interpreter and with kernels compiled "
+                         "at run time (needs hipcc unless the program cache already holds them)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
                     help="also issue N device-to-device copies of x (205 520 896 bytes each): a "
@@ -243,6 +285,8 @@ def main():
     t.close()
     if args.all:
         out["other_configs"] = other_configs(ng, ngt, neon, configs, max(5, args.steps // 3), 2)
+    if args.compiled:
+        out["compiled_at_run_time"] = compiled_vs_interpreted(ng, ngt, max(5, args.steps // 5), 2)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_c2(dims)
     print(json.dumps(out))

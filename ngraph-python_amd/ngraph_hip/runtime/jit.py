@@ -72,7 +72,9 @@ def _sources_digest():
 def source_text(programs):
     header = ["// Program library: op programs of a user's computation, compiled at run time.",
               '#include "ngh_special.h"', "", "namespace ngh {", ""]
-    return render(programs, header, prefix="LP", table="kLoadedTable", count="kLoadedCount") + _TRAILER
+    # the struct's name shows in the kernel's name (profilers group by it): make it the program's
+    tag = "".join(c if c.isalnum() else "_" for c in programs[0][0]) if programs else "none"
+    return render(programs, header, prefix="LP_%s_" % tag, table="kLoadedTable", count="kLoadedCount") + _TRAILER
 
 
 def compile_programs(programs, verbose=False):
