@@ -8,7 +8,7 @@
 // (ngraph_hip/runtime/jit.py).  Anything without an entry runs on the interpreter.
 #pragma once
 #include <atomic>
-#include <deque>
+#include <cstdint>
 #include <mutex>
 
 #include "ngh_special.h"
@@ -17,16 +17,32 @@ namespace ngh {
 
 #include "ngh_programs.inc"
 
-// Entries of loaded program libraries.  Append-only: an index, once handed out, stays valid for
-// the life of the process (a deque never moves its elements), and the libraries stay loaded.
+// Entries of loaded program libraries.  Append-only and in place: a slot is filled, then
+// published by the count (release / acquire), so readers need no lock and an index, once handed
+// out, stays valid for the life of the process; the libraries stay loaded.
+constexpr int kMaxLoadedPrograms = 4096;
 struct LoadedPrograms {
-    std::mutex              lock;
-    std::deque<StaticEntry> entries;
-    std::atomic<int>        count{0};
+    std::mutex       lock;                       // writers only
+    StaticEntry      entries[kMaxLoadedPrograms];
+    uint64_t         hash[kMaxLoadedPrograms];   // of what match_special compares: a quick reject
+    std::atomic<int> count{0};
 };
 inline LoadedPrograms& loaded_programs() {
     static LoadedPrograms table;
     return table;
+}
+
+inline uint64_t mix_hash(uint64_t h, uint64_t v) {
+    h ^= v + 0x9e3779b97f4a7c15ull + (h << 6) + (h >> 2);
+    return h;
+}
+inline uint64_t program_hash(int family, int V, int n_ops, const ngh_op* ops, int n_tensors, int n_red) {
+    uint64_t h = mix_hash(mix_hash(mix_hash(mix_hash((uint64_t)family, (uint64_t)V), (uint64_t)n_ops),
+                                   (uint64_t)n_tensors), (uint64_t)n_red);
+    for (int j = 0; j < n_ops; ++j)
+        h = mix_hash(h, ((uint64_t)(uint32_t)ops[j].opcode << 48) ^ ((uint64_t)(uint32_t)ops[j].dst << 32) ^
+                            ((uint64_t)(uint32_t)ops[j].a << 16) ^ (uint64_t)(uint32_t)ops[j].b);
+    return h;
 }
 
 inline const StaticEntry& special_entry(int i) {
@@ -60,8 +76,10 @@ inline int match_special(int family, int V, const KArgs& k, long long /*tail*/) 
         if (entry_matches(kStaticTable[i], family, V, k)) return i;
     LoadedPrograms& L = loaded_programs();
     const int n = L.count.load(std::memory_order_acquire);
+    if (n == 0) return -1;
+    const uint64_t h = program_hash(family, V, k.op_end - k.op_begin, k.ops + k.op_begin, k.n_tensors, k.n_red);
     for (int i = 0; i < n; ++i)
-        if (entry_matches(L.entries[i], family, V, k)) return kStaticCount + i;
+        if (L.hash[i] == h && entry_matches(L.entries[i], family, V, k)) return kStaticCount + i;
     return -1;
 }
 
@@ -81,18 +99,23 @@ inline bool same_program(const StaticEntry& a, const StaticEntry& b) {
     return true;
 }
 
-// Add the entries of a loaded library that the table does not hold yet; returns how many were new.
+// Add the entries of a loaded library that the table does not hold yet; returns how many were
+// new, or -1 when the table is full.
 inline int add_loaded_programs(const StaticEntry* entries, int n) {
     LoadedPrograms& L = loaded_programs();
     std::lock_guard<std::mutex> guard(L.lock);
     int added = 0;
     for (int i = 0; i < n; ++i) {
+        const int have = L.count.load(std::memory_order_relaxed);
         bool known = false;
         for (int j = 0; j < kStaticCount && !known; ++j) known = same_program(kStaticTable[j], entries[i]);
-        for (size_t j = 0; j < L.entries.size() && !known; ++j) known = same_program(L.entries[j], entries[i]);
+        for (int j = 0; j < have && !known; ++j) known = same_program(L.entries[j], entries[i]);
         if (known) continue;
-        L.entries.push_back(entries[i]);
-        L.count.store((int)L.entries.size(), std::memory_order_release);
+        if (have == kMaxLoadedPrograms) return -1;
+        L.entries[have] = entries[i];
+        L.hash[have] = program_hash(entries[i].family, entries[i].V, entries[i].n_ops, entries[i].ops,
+                                    entries[i].n_tensors, entries[i].n_red);
+        L.count.store(have + 1, std::memory_order_release);
         ++added;
     }
     return added;

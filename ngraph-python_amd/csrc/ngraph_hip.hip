@@ -1177,6 +1177,7 @@ int ngh_programs_load(ngh_context* ctx, const char* path, int32_t* out_added) {
     }
     // the handle is kept for the life of the process: table entries point into the library
     const int added = add_loaded_programs((const StaticEntry*)entries, n);
+    if (added < 0) return fail(NGH_E_UNSUPPORTED, "the program table is full (%d loaded programs)", kMaxLoadedPrograms);
     if (out_added) *out_added = added;
     return NGH_OK;
 }

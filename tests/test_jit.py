@@ -170,5 +170,8 @@ def test_loading_a_program_library_twice_adds_nothing():
         assert hiplib.programs_count() == (built_in, loaded)
         with pytest.raises(hiplib.HipLibraryError):
             rt.programs_load(os.path.join(os.path.dirname(path), "no_such_library.so"))
+        # a shared object that is no program library
+        with pytest.raises(hiplib.HipLibraryError, match="ngh_program_library"):
+            rt.programs_load(hiplib.library_path())
     finally:
         rt.close()
