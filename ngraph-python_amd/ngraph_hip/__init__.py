@@ -21,7 +21,8 @@ from ngraph_hip.op_graph.op_graph import (  # noqa: F401
     placeholder, power, prod, reciprocal, safelog, sequential, sigmoid, sigmoidAtomic, sign, sin,
     slice_along_axis, softmax, sqrt, square, squared_L2, subtract, sum, tanh, temporary,
     tensor_size, tensor_slice, unflatten, value_of, variable, variance, Transpose,
-    cross_entropy_multi, cross_entropy_binary, cross_entropy_binary_inner, UnmatchedAxesError)
+    cross_entropy_multi, cross_entropy_binary, cross_entropy_binary_inner, UnmatchedAxesError,
+    stack, concat_along_axis)
 from ngraph_hip.op_graph.op_graph import ContiguousOp as _ContiguousOp
 from ngraph_hip.op_graph.autodiff import deriv  # noqa: F401
 

@@ -245,7 +245,8 @@ def adjoints_of(dependent, error):
             adjoint = adjoint * target.scale
         # a composite may differentiate itself as a whole (op_graph.py:1153-1160 deriv_handler):
         # sigmoid, softmax, the cross entropies of either, batch normalisation
-        handler = getattr(target, "deriv_handler", None)
+        # (the value of a stack / concat may be the plain read of its storage: look on the read too)
+        handler = getattr(o, "deriv_handler", None) or getattr(target, "deriv_handler", None)
         if handler is not None and handler is not target:
             handler.generate_adjoints(_add_delta, adjoints, adjoint)
             continue

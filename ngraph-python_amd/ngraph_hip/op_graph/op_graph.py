@@ -23,6 +23,7 @@ Autodiff, dot / convolution / pooling / lookup ops are outside this path.
 """
 from __future__ import division
 from collections import OrderedDict, defaultdict
+import builtins
 import numbers
 
 import numpy as np
@@ -1452,6 +1453,90 @@ class SoftmaxOp(ValueOp):
         z = delta * self.value_tensor
         zs = sum(z, reduction_axes=self.normalization_axes)
         add_delta(adjoints, self.x, z - zs * self.value_tensor)
+
+
+class StackOp(SequentialOp):
+    """Joins identically-axed tensors along a new axis inserted at `pos`: every argument is
+    assigned, on the device, into its slice of a temporary that has the new axis first, and the
+    result is that temporary with the axes in the requested order (op_graph.py:2567-2619)."""
+
+    def __init__(self, x_list, axis, pos=0, **kwargs):
+        super(StackOp, self).__init__(**kwargs)
+        self.pos = pos
+        self.x_list = tuple(as_op(arg) for arg in x_list)
+        if axis.length != len(self.x_list):
+            raise ValueError("Axis must have the same length as x_list")
+        arg_axes = self.x_list[0].axes
+        result_axes = arg_axes[:pos] + make_axes(axis) + arg_axes[pos:]
+        storage_axes = make_axes((axis,) + tuple(arg_axes))
+        self.storage = temporary(axes=storage_axes, dtype=self.x_list[0].dtype).named("stack")
+        slices = [slice(None)] * len(arg_axes)
+        self.ops = [assign(tensor_slice(self.storage, [i] + slices, axes=arg_axes), axes_with_order(arg, arg_axes))
+                    for i, arg in enumerate(self.x_list)] + \
+                   [axes_with_order(value_of(self.storage), result_axes)]
+        self.value_tensor.deriv_handler = self
+
+    def generate_adjoints(self, add_delta, adjoints, delta):
+        s = [slice(None)] * len(self.storage.axes)
+        delta = axes_with_order(delta, self.value_tensor.axes)
+        for i, x in enumerate(self.x_list):
+            s[self.pos] = i
+            piece = tensor_slice(delta, tuple(s), axes=delta.axes[:self.pos] + delta.axes[self.pos + 1:])
+            add_delta(adjoints, x, axes_with_order(piece, x.axes))
+
+
+def stack(x_list, axis, pos=0):
+    return StackOp(x_list, axis, pos).value_tensor
+
+
+class ConcatOp(SequentialOp):
+    """Concatenates tensors along one axis each (same name, lengths may differ; the other axes
+    are common): assignments into windows of a temporary (op_graph.py:2636-2708)."""
+
+    def __init__(self, x_list, axis_list, **kwargs):
+        super(ConcatOp, self).__init__(**kwargs)
+        self.x_list = tuple(as_op(arg) for arg in x_list)
+        self.axis_list = list(axis_list)
+        arg_axes = self.x_list[0].axes
+        ax = self.axis_list[0]
+        common_axes = arg_axes - make_axes(ax)
+        for ii, x in enumerate(self.x_list):
+            if len(x.axes - common_axes) > 1:
+                raise RuntimeError("Tensor {} has more than 1 axis not in common with other tensors".format(ii))
+        self.concat_axis = make_axis(builtins.sum(a.length for a in self.axis_list), name=ax.name)
+        ind = arg_axes.index(ax)
+        axes_0, axes_1 = arg_axes[:ind], arg_axes[ind + 1:]
+        result_axes = axes_0 + make_axes(self.concat_axis) + axes_1
+        self.storage_axes = make_axes([self.concat_axis] + list(axes_0) + list(axes_1))
+        self.storage = temporary(axes=self.storage_axes, dtype=self.x_list[0].dtype).named("concat")
+        slices = [slice(None)] * (len(self.storage_axes) - 1)
+        ops, start = [], 0
+        for x, a in zip(self.x_list, self.axis_list):
+            piece_axes = make_axes([a] + list(self.storage_axes[1:]))
+            window = tensor_slice(self.storage, [slice(start, start + a.length)] + slices, axes=piece_axes)
+            ops.append(assign(window, axes_with_order(x, piece_axes)))
+            start += a.length
+        self.ops = ops + [axes_with_order(value_of(self.storage), result_axes)]
+        self.value_tensor.deriv_handler = self
+
+    def generate_adjoints(self, add_delta, adjoints, delta):
+        slices = [slice(None)] * (len(self.storage_axes) - 1)
+        storage_delta = axes_with_order(delta, self.storage_axes)
+        start = 0
+        for x, a in zip(self.x_list, self.axis_list):
+            piece_axes = make_axes([a] + list(self.storage_axes[1:]))
+            piece = tensor_slice(storage_delta, [slice(start, start + a.length)] + slices, axes=piece_axes)
+            add_delta(adjoints, x, axes_with_order(piece, x.axes))
+            start += a.length
+
+
+def concat_along_axis(x_list, axis):
+    """The tensors of x_list joined along `axis`, which each of them has (by name); axes ordered
+    as in the first (op_graph.py:2711-2737)."""
+    if len(x_list) < 1:
+        return x_list
+    x_list = [as_op(x) for x in x_list]
+    return ConcatOp(x_list, [x.axes[x.axes.index(axis)] for x in x_list]).value_tensor
 
 
 def softmax(x, normalization_axes=None, **kwargs):

@@ -312,3 +312,59 @@ def test_per_channel_factors_absorbed_into_the_big_kernels():
     k64 = np.sqrt(gv.astype(np.float64) ** 2 + 1.0) * 0.5
     np.testing.assert_allclose(xs.reshape(8, -1), x64 * k64[:, None], rtol=1e-5, atol=1e-6)
     np.testing.assert_allclose(es, (e64 * k64[:, None]).sum(1), rtol=1e-5, atol=1e-3)
+
+
+# ---- stack / concat: assignments into slices of a temporary, on the device ---------------------
+@pytest.mark.parametrize("pos", [0, 1, 2])
+def test_stack_and_its_derivative(backend, pos):
+    """test_stack_tensor.py:29-56: value against numpy.stack, symbolic against numeric derivative
+    with respect to every argument."""
+    W, H, I = ng.make_axis(4, name="W"), ng.make_axis(5, name="H"), ng.make_axis(3, name="I")
+    axes = ng.make_axes([W, H])
+    gen = RandomTensorGenerator(0, np.float32)
+    a_v = [gen.uniform(0, 1, axes) for _ in range(I.length)]
+    a = [ng.placeholder(axes) for _ in a_v]
+    s = ng.stack(a, I, pos)
+    with ExecutorFactory() as ex:
+        value = ex.executor(s, *a)
+        nums = [ex.numeric_derivative(s, p, 1e-3, *[q for q in a if q is not p]) for p in a]
+        syms = [ex.derivative(s, p, *[q for q in a if q is not p]) for p in a]
+        np.testing.assert_array_equal(value(*a_v), np.stack(a_v, axis=pos))
+        for i, (num, sym) in enumerate(zip(nums, syms)):
+            others = [v for j, v in enumerate(a_v) if j != i]
+            np.testing.assert_allclose(num(a_v[i], *others), sym(a_v[i], *others), rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("num_vars,num_axes,concat_pos", [(1, 2, 1), (2, 3, 2), (15, 5, 1)])
+def test_concatenate_and_its_derivative(backend, num_vars, num_axes, concat_pos):
+    """test_op_graph_transformer_dependent.py:25-42, 166-177."""
+    rs = np.random.RandomState(num_vars)
+    common = [ng.make_axis(2, name="c%d" % i) for i in range(num_axes - 1)]
+    ax = ng.make_axis(int(rs.randint(3, 10)), name="cat")
+    axes = ng.make_axes(common[:concat_pos] + [ax] + common[concat_pos:])
+    np_list = [rs.uniform(0, 1, axes.lengths).astype(np.float32) for _ in range(num_vars)]
+    x_list = [ng.constant(v, axes=axes) for v in np_list]
+    with ExecutorFactory() as ex:
+        v = ng.concat_along_axis(x_list, x_list[0].axes[concat_pos])
+        d = ng.deriv(v, x_list[0], error=ng.constant(np.ones(v.axes.lengths, np.float32), axes=v.axes))
+        e_v, e_d = ex.executor([v, d])()
+        np.testing.assert_array_equal(e_v, np.concatenate(np_list, axis=concat_pos))
+        np.testing.assert_array_equal(e_d, np.ones(axes.lengths))
+
+
+def test_concat_different_axis_lengths_and_state(backend):
+    """test_op_graph_transformer_dependent.py:180-196 (axes of one name, different lengths),
+    test_ssa.py:93-106 (persistent tensors)."""
+    ax1, ax2 = ng.make_axis(3, name="concat"), ng.make_axis(2, name="concat")
+    ax3 = ng.make_axis(10, name="other")
+    x, y = ng.placeholder([ax1, ax3]), ng.placeholder([ax2, ax3])
+    rs = np.random.RandomState(0)
+    np_x, np_y = rs.rand(3, 10).astype(np.float32), rs.rand(2, 10).astype(np.float32)
+    A, B = ng.make_axis(3, name="A"), ng.make_axis(4, name="B")
+    x0 = ng.persistent_tensor([A, B], initial_value=-np.ones((3, 4), np.float32))
+    x1 = ng.persistent_tensor([A, B], initial_value=np.ones((3, 4), np.float32))
+    with ExecutorFactory() as ex:
+        f = ex.executor(ng.concat_along_axis([x, y], ax1), x, y)
+        g = ex.executor(ng.concat_along_axis([x0, x1], A))
+        np.testing.assert_array_equal(f(np_x, np_y), np.concatenate([np_x, np_y], axis=0))
+        np.testing.assert_array_equal(g(), np.concatenate([-np.ones((3, 4)), np.ones((3, 4))], axis=0))
