@@ -159,7 +159,7 @@ def collect():
         kernels = t.kernel_groups[f].kernels
         for kernel in kernels:
             kernel.bind_buffers()
-        programs += stage_programs(kernels, name, seen)
+        programs += stage_programs(kernels, name, seen, vector_only=True)
         t.close()
     return programs
 

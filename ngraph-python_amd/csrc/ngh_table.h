@@ -67,11 +67,10 @@ inline bool entry_matches(const StaticEntry& e, int family, int V, const KArgs& 
     return same;
 }
 
-// family: 0 streaming elementwise (V >= 4), 1 / 2 reductions, 3 tiled elementwise
+// family: 0 streaming elementwise (V >= 4: vector access; V == 1: one element per lane, any
+// strides), 1 / 2 reductions, 3 tiled elementwise
 inline int match_special(int family, int V, const KArgs& k, long long /*tail*/) {
-    // V == 1 entries exist for one-element stages only (every operand "broadcast")
-    const bool one_element = k.shape[0] * k.shape[1] * k.shape[2] == 1;
-    if (family > 3 || (family == 0 && ((V < 4 && !one_element) || k.n_red != 0))) return -1;
+    if (family > 3 || (family == 0 && ((V != 1 && V < 4) || k.n_red != 0))) return -1;
     for (int i = 0; i < kStaticCount; ++i)
         if (entry_matches(kStaticTable[i], family, V, k)) return i;
     LoadedPrograms& L = loaded_programs();

@@ -1363,6 +1363,8 @@ static int try_self_managed_launch(ngh_context* ctx, const ngh_fused_spec* spec,
     NGH_TRY(plan_stage(ctx, *spec, 0, P));
     P.special = match_special(P.family, P.V, P.k, P.tail);
     if (P.special < 0 || P.tail || P.n_chunks == 0 || P.k.n_stat_slots != n_ids || n_ids < 1) return NGH_OK;
+    // (the one-launch kernels work on vector-wide chunks; a one-element stage is the exception)
+    if (P.V < 4 && P.k.shape[0] * P.k.shape[1] * P.k.shape[2] != 1) return NGH_OK;
     for (int s = 0; s < P.k.n_stat_slots; ++s) {
         const ptrdiff_t off = (const char*)P.k.stat_ptr[s] - (const char*)dev;
         if (!P.k.stat_ptr[s] || off < 0 || off % (ptrdiff_t)sizeof(ngh_flex_state)) return NGH_OK;

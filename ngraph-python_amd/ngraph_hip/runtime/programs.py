@@ -11,9 +11,10 @@ computation, float_ew2.py:1135-1483, :1553-1653).
 from ngraph_hip.runtime import hiplib
 
 
-def stage_programs(kernels, name, seen=None, min_elements=4096):
+def stage_programs(kernels, name, seen=None, min_elements=4096, vector_only=False):
     """Records for every stage of `kernels` (lowered, buffers bound) that can run as a compiled
-    program; `seen` holds the structural keys already recorded."""
+    program; `seen` holds the structural keys already recorded; `vector_only` leaves out
+    elementwise stages without vector access (other than one-element ones)."""
     programs = []
     seen = set() if seen is None else seen
     k_index = 0
@@ -28,7 +29,12 @@ def stage_programs(kernels, name, seen=None, min_elements=4096):
                 # program of its own: the interpreter fetches the code of every op kind it meets
                 # with a cold instruction cache, several microseconds for twenty scalar ops.
                 scalar = total == 1 and family == 0 and not st.n_reductions
-                if family > 3 or (family == 0 and not scalar and (plan["V"] < 4 or st.n_reductions)):
+                # An elementwise stage without vector access (V == 1: strided or misaligned views)
+                # runs one element per lane with the operands' own strides; as a built-in program
+                # only the one-element case is worth a table entry (`vector_only`).
+                if family > 3 or (family == 0 and (st.n_reductions or plan["V"] in (2, 3))):
+                    continue
+                if family == 0 and plan["V"] == 1 and not scalar and vector_only:
                     continue
                 if family == 1 and spec.shape[0] // plan["V"] <= 64:
                     continue          # short rows run the several-rows-per-workgroup kernel

@@ -62,8 +62,19 @@ def case_ragged():
     return [ng.exp(-ng.square(x)) * y + 1.0, ng.sum(x * y + 1.0, out_axes=[A])], [x, y]
 
 
+def case_misaligned_slices():
+    # windows that start one element into rows of odd length: no vector access, so the
+    # compiled program takes one element per lane with the operands' own strides
+    A, B = ng.make_axis(300, name="A"), ng.make_axis(1025, name="B")
+    x, y = ng.placeholder([A, B]), ng.placeholder([A, B])
+    xs = ng.tensor_slice(x, [slice(None), slice(1, 1025)])
+    ys = ng.cast_axes(ng.tensor_slice(y, [slice(None), slice(0, 1024)]), xs.axes)
+    return [ng.tanh(xs * ys + 0.5) * ng.sigmoid(xs)], [x, y]
+
+
 FP32_CASES = [case_elementwise, case_column_reduction_with_store, case_row_reduction_with_store,
-              case_transposed_operand, case_softmax, case_mixed_storage_types, case_ragged]
+              case_transposed_operand, case_softmax, case_mixed_storage_types, case_ragged,
+              case_misaligned_slices]
 
 
 def flex_case():
