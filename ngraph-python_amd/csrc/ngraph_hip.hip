@@ -798,11 +798,15 @@ int launch_interp(ngh_context* ctx, Plan& P) {
     unsigned red_blocks = 0;
     if (P.special >= 0 && !k.probe) {
         // a pre-built reduction: same grid and workspace as the interpreter's kernel
-        red_blocks = P.family == F_RED_ROW ? P.n_out * P.n_seg
-                                            : (unsigned)((unsigned long long)P.n_bx * (unsigned)k.shape[1] * P.n_seg);
+        const bool small = P.family == F_RED_ROW && P.small_rows;
+        const unsigned rows_per_wg = small ? kBlock / P.tx : 1;
+        red_blocks = small ? (P.n_out + rows_per_wg - 1) / rows_per_wg
+                   : P.family == F_RED_ROW ? P.n_out * P.n_seg
+                                           : (unsigned)((unsigned long long)P.n_bx * (unsigned)k.shape[1] * P.n_seg);
         NGH_TRY(stat_scratch(ctx, k, red_blocks));
+        // (a row reduction takes no TX unless its rows are short: TX lanes per row then)
         HIP_TRY(launch_special_red(P.special, ctx->stream, red_blocks, k, P.family == F_RED_ROW ? P.n_out : P.n_bx,
-                                   P.n_seg, P.seg_len, P.tx, ws, P.cache_policy));
+                                   P.n_seg, P.seg_len, P.family == F_RED_ROW && !small ? 0u : P.tx, ws, P.cache_policy));
     } else if (P.family == F_RED_ROW && P.small_rows) {
         const unsigned rows_per_wg = kBlock / P.tx;
         red_blocks = (P.n_out + rows_per_wg - 1) / rows_per_wg;
@@ -1130,7 +1134,7 @@ int ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec) {
             }
         }
         if (!ctx->force_interp && !P.k.probe &&
-            (P.family == F_RED_COL || P.family == F_EW_TILED || (P.family == F_RED_ROW && !P.small_rows))) {
+            (P.family == F_RED_COL || P.family == F_EW_TILED || P.family == F_RED_ROW)) {
             P.special = match_special(P.family, P.V, P.k, 0);
             P.cache_policy = stage_cache_policy(ctx, *spec, spec->stages[s]);
         }
@@ -1145,7 +1149,7 @@ int ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec, int32_t sta
     if (stage < 0 || stage >= spec->n_stages) return fail(NGH_E_INVALID, "stage %d", stage);
     Plan P;
     NGH_TRY(plan_stage(ctx, *spec, stage, P));
-    if (!ctx->force_interp && !(P.family == F_RED_ROW && P.small_rows))
+    if (!ctx->force_interp)
         P.special = match_special(P.family, P.V, P.k, P.tail);
     describe(P, name128, 128);
     if (P.special >= 0 && P.family == F_EW) {

@@ -36,8 +36,8 @@ def stage_programs(kernels, name, seen=None, min_elements=4096, vector_only=Fals
                     continue
                 if family == 0 and plan["V"] == 1 and not scalar and vector_only:
                     continue
-                if family == 1 and spec.shape[0] // plan["V"] <= 64:
-                    continue          # short rows run the several-rows-per-workgroup kernel
+                if family == 1 and spec.shape[0] // plan["V"] <= 64 and vector_only:
+                    continue          # short rows (several per workgroup): no table entry of their own
                 if total < min_elements and not scalar:
                     continue          # small stages are launch-bound; the interpreter is fine
                 if any(o.opcode >= hiplib.OPCODES["take"] for o in spec.ops[st.op_begin:st.op_end]):

@@ -72,9 +72,19 @@ def case_misaligned_slices():
     return [ng.tanh(xs * ys + 0.5) * ng.sigmoid(xs)], [x, y]
 
 
+def case_short_rows():
+    # softmax and its cross entropy over 100 classes: rows short enough that several share a
+    # workgroup (the short-row reduction kernel)
+    C, N = ng.make_axis(100, name="C"), ng.make_axis(2048, name="N")
+    x, tgt = ng.placeholder([N, C]), ng.placeholder([N, C])
+    e = ng.exp(x - ng.max(x, out_axes=[N]))
+    sm = e / ng.sum(e, out_axes=[N])
+    return [sm, ng.sum(-tgt * ng.log(sm), out_axes=[N]), ng.argmax(x, out_axes=[N])], [x, tgt]
+
+
 FP32_CASES = [case_elementwise, case_column_reduction_with_store, case_row_reduction_with_store,
               case_transposed_operand, case_softmax, case_mixed_storage_types, case_ragged,
-              case_misaligned_slices]
+              case_misaligned_slices, case_short_rows]
 
 
 def flex_case():
