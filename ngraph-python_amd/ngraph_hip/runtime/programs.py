@@ -40,8 +40,12 @@ def stage_programs(kernels, name, seen=None, min_elements=4096, vector_only=Fals
                     continue          # short rows (several per workgroup): no table entry of their own
                 if total < min_elements and not scalar:
                     continue          # small stages are launch-bound; the interpreter is fine
-                if any(o.opcode >= hiplib.OPCODES["take"] for o in spec.ops[st.op_begin:st.op_end]):
-                    continue          # lookups only run in the interpreter
+                codes = set(o.opcode for o in spec.ops[st.op_begin:st.op_end])
+                if codes & {hiplib.OPCODES["take"], hiplib.OPCODES["store_trunc"]}:
+                    continue          # lookups and truncating stores only run in the interpreter
+                if codes & {hiplib.OPCODES["rng_uniform"], hiplib.OPCODES["rng_normal"]} and \
+                        (family == 3 or vector_only):
+                    continue          # random fills: not through the tiles, no built-in entries
                 ops = [(o.opcode, o.dst, o.a, o.b) for o in spec.ops[st.op_begin:st.op_end]]
                 fast = plan["perm"][2]
                 red_out = [st.red_out[r] for r in range(st.n_reductions)]

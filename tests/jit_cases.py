@@ -82,9 +82,18 @@ def case_short_rows():
     return [sm, ng.sum(-tgt * ng.log(sm), out_axes=[N]), ng.argmax(x, out_axes=[N])], [x, tgt]
 
 
+def case_dropout():
+    # a random mask made in the kernel (Philox keyed by seed, execution count and element
+    # index): the compiled program must draw the very numbers the interpreter draws
+    A, B = _ab()
+    x = ng.placeholder([A, B])
+    keep = ng.less_equal(ng.uniform(ng.temporary([A, B]), 0.0, 1.0), 0.75)
+    return [x * keep * (1.0 / 0.75), ng.sum(keep, out_axes=[A])], [x]
+
+
 FP32_CASES = [case_elementwise, case_column_reduction_with_store, case_row_reduction_with_store,
               case_transposed_operand, case_softmax, case_mixed_storage_types, case_ragged,
-              case_misaligned_slices, case_short_rows]
+              case_misaligned_slices, case_short_rows, case_dropout]
 
 
 def flex_case():

@@ -100,7 +100,11 @@ def test_compiled_programs_agree_with_the_interpreter(case):
     compiled, names = _run("hipgpu", case, 5, jit=True)
     for a, b, w in zip(interp, compiled, want):
         np.testing.assert_array_equal(a, b)
-        np.testing.assert_allclose(b, w, rtol=1e-5, atol=1e-5)
+        if case is jit_cases.case_dropout:
+            # the oracle draws from NumPy's generator: only the distribution is comparable
+            assert abs(np.count_nonzero(compiled[0]) / compiled[0].size - 0.75) < 0.01
+        else:
+            np.testing.assert_allclose(b, w, rtol=1e-5, atol=1e-5)
     if default_kernel_choice():
         # every stage large enough to be worth a compiled kernel has one now
         assert not any("interp" in n for n in names if "tail" not in n), names
