@@ -25,7 +25,7 @@ import numpy as np  # noqa: E402
 HBM_PEAK_GBS = 8000.0
 # HBM bytes one launch of the C2 normalise kernel moves, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE scaled by a device copy of known size (profiles/c2_batchnorm_pmc_traffic.md)
-MEASURED_TRAFFIC = {"special:batchnorm": 411173686}
+MEASURED_TRAFFIC = {"special:batchnorm": 411176158}
 
 
 def build_c2(ng, neon, t, dims):
