@@ -102,13 +102,13 @@ def flex_case():
     return [ng.tanh(x * w) + b], [x, w, b]
 
 
-# random graphs of tests/test_random_graphs.py: small shapes, so every stage counts as worth
+# random graphs of tests/graph_generators.py: small shapes, so every stage counts as worth
 # compiling (jit_min_elements=1); the odd programs a generator finds and a person would not write
 RANDOM_SEEDS = list(range(8))
 
 
 def random_case(seed, views):
-    import test_random_graphs as T
+    import graph_generators as T
     return (T.build_views if views else T.build)(seed)
 
 
