@@ -49,8 +49,7 @@ def enabled_by_default():
 def cache_dir():
     """Where program libraries are kept: NGH_PROGRAM_CACHE, else next to libngraph_hip.so."""
     path = os.environ.get("NGH_PROGRAM_CACHE") or os.path.join(_PKG, "lib", "programs")
-    if not os.path.isdir(path):
-        os.makedirs(path)
+    os.makedirs(path, exist_ok=True)          # (several threads may get here at once)
     return path
 
 

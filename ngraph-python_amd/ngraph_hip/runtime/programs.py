@@ -41,11 +41,11 @@ def stage_programs(kernels, name, seen=None, min_elements=4096, vector_only=Fals
                 if total < min_elements and not scalar:
                     continue          # small stages are launch-bound; the interpreter is fine
                 codes = set(o.opcode for o in spec.ops[st.op_begin:st.op_end])
-                if codes & {hiplib.OPCODES["take"], hiplib.OPCODES["store_trunc"]}:
-                    continue          # lookups and truncating stores only run in the interpreter
-                if codes & {hiplib.OPCODES["rng_uniform"], hiplib.OPCODES["rng_normal"]} and \
-                        (family == 3 or vector_only):
-                    continue          # random fills: not through the tiles, no built-in entries
+                if hiplib.OPCODES["store_trunc"] in codes:
+                    continue          # the truncating store of a flex fill only runs in the interpreter
+                if codes & {hiplib.OPCODES["take"], hiplib.OPCODES["rng_uniform"], hiplib.OPCODES["rng_normal"]} \
+                        and (family == 3 or vector_only):
+                    continue          # lookups, random fills: not through the tiles, no built-in entries
                 ops = [(o.opcode, o.dst, o.a, o.b) for o in spec.ops[st.op_begin:st.op_end]]
                 fast = plan["perm"][2]
                 red_out = [st.red_out[r] for r in range(st.n_reductions)]

@@ -91,9 +91,17 @@ def case_dropout():
     return [x * keep * (1.0 / 0.75), ng.sum(keep, out_axes=[A])], [x]
 
 
+def case_lookup_table():
+    # rows of a table selected by an index tensor (LookupTableOp fprop), scaled afterwards
+    V_, F, N = ng.make_axis(1000, name="V"), ng.make_axis(64, name="F"), ng.make_axis(256, name="N")
+    lut, idx = ng.placeholder([V_, F]), ng.placeholder([N], dtype=np.int32)
+    w = ng.placeholder([N, F])
+    return [ng.lookuptable(lut, idx, ng.make_axes([N, F]), update=False) * w + 1.0], [lut, idx, w]
+
+
 FP32_CASES = [case_elementwise, case_column_reduction_with_store, case_row_reduction_with_store,
               case_transposed_operand, case_softmax, case_mixed_storage_types, case_ragged,
-              case_misaligned_slices, case_short_rows, case_dropout]
+              case_misaligned_slices, case_short_rows, case_dropout, case_lookup_table]
 
 
 def flex_case():
@@ -117,7 +125,8 @@ def inputs_for(placeholders, seed):
     for i, p in enumerate(placeholders):
         rs = np.random.RandomState(seed + i)
         if p.dtype == np.int32:
-            vals.append(rs.randint(-5, 6, p.axes.lengths).astype(np.int32))
+            hi = 1000 if len(p.axes) == 1 else 6          # an index tensor / integer operands
+            vals.append(rs.randint(0 if len(p.axes) == 1 else -5, hi, p.axes.lengths).astype(np.int32))
         else:
             vals.append(rs.uniform(-1, 1, p.axes.lengths).astype(p.dtype))
     return vals

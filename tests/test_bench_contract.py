@@ -47,3 +47,26 @@ def test_transformer_fails_loudly_without_a_gpu():
             "        print('raised')\n") % (ROOT, os.path.join(ROOT, "ngraph-python_amd"))
     p = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
     assert p.stdout.strip() in ("raised", "has-gpu"), (p.stdout, p.stderr)
+
+
+def test_user_graphs_of_the_compiled_leg_have_no_built_in_programs():
+    """`bench.py --compiled` compares interpreter and run-time compiled kernels: each of its
+    graphs must lower, and must have at least one stage the library carries no kernel for
+    (else the comparison would measure nothing)."""
+    sys.path.insert(0, ROOT)
+    import bench
+    import ngraph_hip as ng
+    import ngraph_hip.transformers as ngt
+    from ngraph_hip.runtime import jit
+    for name, results, inputs, passes in bench.user_graphs(ng, 512, 1024):
+        t = ngt.make_transformer_factory("hipgpu", dry_run=True)()
+        try:
+            f = t.computation(results, *inputs)
+            t.initialize()
+            kernels = t.kernel_groups[f].kernels
+            for k in kernels:
+                k.bind_buffers()
+            assert jit.uncovered_programs(kernels, name), name
+            assert passes >= 2
+        finally:
+            t.close()
