@@ -90,7 +90,13 @@ def compile_programs(programs, verbose=False):
     with open(src, "w") as fh:
         fh.write(text)
     tmp = "%s.%d.tmp" % (lib, os.getpid())
-    cmd = [find_hipcc()] + list(flags) + ["-I", INCLUDE, "-I", CSRC, src, "-o", tmp]
+    try:
+        hipcc = find_hipcc()
+    except RuntimeError:
+        raise RuntimeError("run-time compilation (jit=True / NGH_JIT=1) needs hipcc on this machine, or the "
+                           "program library %s in the cache; without jit the same stages run on the "
+                           "interpreter" % os.path.basename(lib))
+    cmd = [hipcc] + list(flags) + ["-I", INCLUDE, "-I", CSRC, src, "-o", tmp]
     if verbose:
         print(" ".join(cmd))
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, universal_newlines=True)

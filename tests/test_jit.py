@@ -67,6 +67,21 @@ def test_program_library_compiles_and_checks_its_caller(tmp_path, monkeypatch):
         t.close()
 
 
+def test_missing_compiler_is_reported_as_such(tmp_path, monkeypatch):
+    import build_ext
+
+    def no_hipcc():
+        raise RuntimeError("hipcc not found")
+    monkeypatch.setenv("NGH_PROGRAM_CACHE", str(tmp_path))
+    monkeypatch.setattr(build_ext, "find_hipcc", no_hipcc)
+    t, kernels = _dry_kernels(jit_cases.case_elementwise)
+    try:
+        with pytest.raises(RuntimeError, match="needs hipcc"):
+            jit.compile_programs(jit.uncovered_programs(kernels, "case"))
+    finally:
+        t.close()
+
+
 def test_jit_is_off_unless_asked_for(monkeypatch):
     monkeypatch.delenv("NGH_JIT", raising=False)
     t = ngt.make_transformer_factory("hipgpu", dry_run=True)()
