@@ -330,8 +330,12 @@ __global__ __launch_bounds__(kBlock) void ew_interp_kernel(const KArgs k, unsign
 // 256 elements apart, so each of its accesses is as coalesced as the strides
 // allow and every op is decoded once for G elements.
 // ---------------------------------------------------------------------------
+// `first` is the linear index of the launch's first element: the tail of a 1-D stage whose body
+// a vector kernel has done starts there, with every coordinate (index values, random-number
+// counters, table lookups) that of the whole view.
 template <int G>
-__global__ __launch_bounds__(kBlock) void ew_gather_interp_kernel(const KArgs k, unsigned long long total) {
+__global__ __launch_bounds__(kBlock) void ew_gather_interp_kernel(const KArgs k, unsigned long long total,
+                                                                  unsigned long long first) {
     extern __shared__ float lds[];
     LdsRegs<G> rf{lds + threadIdx.x, kBlock};
     Extra ex{lds + (size_t)k.n_regs * G * kBlock + threadIdx.x, kBlock};
@@ -343,12 +347,13 @@ __global__ __launch_bounds__(kBlock) void ew_gather_interp_kernel(const KArgs k,
         at.nv = 0;
 #pragma unroll
         for (int v = 0; v < G; ++v) {
-            const unsigned long long q = base + (unsigned)v * kBlock + threadIdx.x;
+            unsigned long long q = base + (unsigned)v * kBlock + threadIdx.x;
             at.i0[v] = at.i1[v] = at.i2[v] = 0;
             if (q < total) {
                 at.nv = v + 1;
+                q += first;
                 unsigned row;
-                if (total <= 0xffffffffull) {
+                if (first + total <= 0xffffffffull) {
                     row = (unsigned)q / d2;
                     at.i2[v] = (unsigned)q - row * d2;
                 } else {

@@ -708,19 +708,18 @@ int stat_fold(ngh_context* ctx, const KArgs& k, unsigned blocks) {
 }
 
 int launch_tail(ngh_context* ctx, const Plan& P) {
+    // The same view as the body's, all of it, entered at element `body`: operand pointers stay
+    // where they are, so index values, random-number counters and the table of a lookup (whose
+    // stride on this axis is the table's own) see the coordinates of the whole view.
     KArgs kt = P.k;
     const long long body = P.k.shape[2];
-    kt.shape[2] = P.tail;
-    for (int t = 0; t < kt.n_tensors; ++t) kt.t[t].p += body * kt.t[t].s[2] * itemsize_of(kt.t[t].dtype);
-    // IOTA along the split axis would restart at 0 in the tail
-    for (int pc = kt.op_begin; pc < kt.op_end; ++pc)
-        if (kt.ops[pc].opcode == NGH_OP_IOTA && kt.iota_map[kt.ops[pc].a] == 2)
-            return fail(NGH_E_UNSUPPORTED, "IOTA along a split 1-D axis");
+    kt.shape[2] = body + P.tail;
+    if (kt.shape[2] > 0xffffffffLL) return fail(NGH_E_UNSUPPORTED, "1-D stage of %lld elements with a scalar tail", kt.shape[2]);
     const size_t lds = interp_lds_bytes(kt, 1);
     if (lds > kInterpLdsMax) return fail(NGH_E_UNSUPPORTED, "program needs %zu bytes of LDS registers", lds);
     NGH_TRY(stat_scratch(ctx, kt, 1));
     hipLaunchKernelGGL(ew_gather_interp_kernel<1>, dim3(1), dim3(kBlock), lds, ctx->stream, kt,
-                       (unsigned long long)P.tail);
+                       (unsigned long long)P.tail, (unsigned long long)body);
     HIP_TRY(hipGetLastError());
     return stat_fold(ctx, kt, 1);
 }
@@ -768,9 +767,9 @@ int launch_interp(ngh_context* ctx, Plan& P) {
             blocks = std::min<unsigned>(blocks, (unsigned)(ctx->cus * ctx->ew_blocks_per_cu));
             NGH_TRY(stat_scratch(ctx, k, blocks));
             if (G == 4)
-                hipLaunchKernelGGL(ew_gather_interp_kernel<4>, dim3(blocks), dim3(kBlock), interp_lds_bytes(k, 4), ctx->stream, k, total);
+                hipLaunchKernelGGL(ew_gather_interp_kernel<4>, dim3(blocks), dim3(kBlock), interp_lds_bytes(k, 4), ctx->stream, k, total, 0ull);
             else
-                hipLaunchKernelGGL(ew_gather_interp_kernel<1>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, total);
+                hipLaunchKernelGGL(ew_gather_interp_kernel<1>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, total, 0ull);
             HIP_TRY(hipGetLastError());
             NGH_TRY(stat_fold(ctx, k, blocks));
         } else if (P.n_chunks) {
@@ -1328,6 +1327,17 @@ int make_flex_ids(const int32_t* ids, const int32_t* in_place, int32_t n_ids, Fl
     }
     return NGH_OK;
 }
+// ids are record numbers counted from `dev`: when `dev` lies in a table this context allocated,
+// none may point past its end (the kernels index records without a bound of their own)
+int check_flex_ids(ngh_context* ctx, const ngh_flex_state* dev, const int32_t* ids, int32_t n_ids) {
+    int32_t first = 0;
+    const FlexTable* T = flex_table_of(ctx, dev, &first);
+    if (!T) return NGH_OK;
+    for (int i = 0; i < n_ids; ++i)
+        if (ids[i] < 0 || (int64_t)first + ids[i] >= T->n)
+            return fail(NGH_E_INVALID, "flex id %d outside the table of %d records", ids[i], T->n);
+    return NGH_OK;
+}
 }  // namespace
 
 int ngh_flex_prepare(ngh_context* ctx, ngh_flex_state* dev, const int32_t* ids, const int32_t* in_place,
@@ -1336,6 +1346,7 @@ int ngh_flex_prepare(ngh_context* ctx, ngh_flex_state* dev, const int32_t* ids, 
     if (n_ids == 0) return NGH_OK;
     FlexIds f;
     NGH_TRY(make_flex_ids(ids, in_place, n_ids, f));
+    NGH_TRY(check_flex_ids(ctx, dev, ids, n_ids));
     NGH_TRY(flex_settle_ids(ctx, dev, ids, n_ids));
     hipLaunchKernelGGL(flex_prepare_kernel, dim3(1), dim3(64), 0, ctx->stream, dev, f);
     HIP_TRY(hipGetLastError());
@@ -1347,6 +1358,7 @@ int ngh_flex_update(ngh_context* ctx, ngh_flex_state* dev, const int32_t* ids, i
     if (n_ids == 0) return NGH_OK;
     FlexIds f;
     NGH_TRY(make_flex_ids(ids, nullptr, n_ids, f));
+    NGH_TRY(check_flex_ids(ctx, dev, ids, n_ids));
     NGH_TRY(flex_settle_ids(ctx, dev, ids, n_ids));
     hipLaunchKernelGGL(flex_update_kernel, dim3((unsigned)n_ids), dim3(64), 0, ctx->stream, dev, f, (int)count);
     HIP_TRY(hipGetLastError());
@@ -1443,6 +1455,8 @@ int ngh_launch_fused_flex(ngh_context* ctx, const ngh_fused_spec* spec, ngh_flex
     if (!ctx || !dev) return fail(NGH_E_INVALID, "ngh_launch_fused_flex: NULL argument");
     NGH_TRY(validate(spec));
     if (n_ids > 0 && !ids) return fail(NGH_E_INVALID, "ngh_launch_fused_flex: ids is NULL");
+    if (n_ids < 0 || n_ids > kFlexMaxIds) return fail(NGH_E_INVALID, "n_ids %d not in 0..%d", n_ids, kFlexMaxIds);
+    NGH_TRY(check_flex_ids(ctx, dev, ids, n_ids));
     bool done = false;
     NGH_TRY(try_self_managed_launch(ctx, spec, dev, ids, in_place, n_ids, count, &done));
     if (done) return NGH_OK;

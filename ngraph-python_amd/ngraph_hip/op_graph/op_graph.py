@@ -1105,8 +1105,10 @@ safelog_cutoff = 50.0
 
 
 def safelog(x, limit=-safelog_cutoff):
-    # op_graph.py:3070-3072
-    return log(maximum(x, np.exp(limit)))
+    """log(x) cut off below at `limit`: maximum(log(x + exp(limit)), limit)
+    (op_graph.py:3070-3072).  safelog(0) is `limit`; a negative x gives NaN, as log does."""
+    offset = np.exp(limit)
+    return maximum(log(x + offset), limit)
 
 
 def reciprocal(x):

@@ -72,7 +72,9 @@ def unary(name, x):
         np.reciprocal(t, out=out)
         return out
     if name == "safelog":
-        # float_ew2.py:48; graph-level safelog = log(maximum(x, exp(-50))) (op_graph.py:3054-3072)
+        # the kernel template of float_ew2.py:48, (x > 0) ? logf(x) : -50.  The graph-level
+        # ng.safelog is a composite of other ops, maximum(log(x + exp(limit)), limit)
+        # (op_graph.py:3070-3072), and never reaches this template.
         with np.errstate(all="ignore"):
             np.log(x, out=out)
         out[~(x > 0)] = f32(-50.0)

@@ -490,6 +490,44 @@ def test_take_lookup(hip_runtime, lut_axis, I, F, V):
         d.free()
 
 
+@pytest.mark.parametrize("N,V", [(37, 50), (1000003, 50), (19, 3)])
+def test_take_lookup_along_a_single_axis_with_a_scalar_tail(hip_runtime, N, V):
+    """out[i] = lut[idx[i]] as a 1-D stage whose length is not a multiple of the vector width:
+    the vector body and the scalar tail both index the table from its first element."""
+    rt = hip_runtime
+    rs = np.random.RandomState(N)
+    lut = rs.normal(0, 1, V).astype(f32)
+    idx = rs.randint(0, V, N).astype(f32)
+    idx[-3:] = [V - 1, V - 2, V + 5]                      # the tail reads the table's end
+    idx[0] = -2.0
+    lut_d, idx_d, out_d = rt.array(lut), rt.array(idx), rt.empty((N,))
+    sb = FusedSpecBuilder([N])
+    ti = sb.tensor(idx_d.ptr, [1])
+    tl = sb.tensor(lut_d.ptr, [1], take_extent=V)
+    to = sb.tensor(out_d.ptr, [1])
+    sb.store(to, sb.take(tl, sb.load(ti), 0))
+    spec = sb.build()
+    from ngraph_hip.runtime.hiplib import plan_fused
+    assert plan_fused(spec)["tail"] == N % 4
+    rt.launch_fused(spec)
+    np.testing.assert_array_equal(out_d.get(), lut.take(np.clip(idx, 0, V - 1).astype(int)))
+    for d in (lut_d, idx_d, out_d):
+        d.free()
+
+
+def test_iota_along_a_single_axis_with_a_scalar_tail(hip_runtime):
+    """The index value of an element in the tail is its index in the whole view."""
+    rt = hip_runtime
+    n = 4099
+    y_d = rt.empty((n,))
+    sb = FusedSpecBuilder([n])
+    ty = sb.tensor(y_d.ptr, [1])
+    sb.store(ty, sb.iota(0))
+    rt.launch_fused(sb.build())
+    np.testing.assert_array_equal(y_d.get(), np.arange(n, dtype=f32))
+    y_d.free()
+
+
 def test_take_needs_an_extent(hip_runtime):
     from ngraph_hip.runtime.hiplib import HipLibraryError
     rt = hip_runtime
@@ -558,6 +596,20 @@ def test_rng_is_a_function_of_seed_counter_and_element(hip_runtime):
     np.testing.assert_array_equal(flat, draw([A * B], [1], 7, 0))
     z = draw([A * B], [1], 7, 0, "normal")
     assert abs(z.mean()) < 0.02 and abs(z.std() - 1.0) < 0.02
+    # a length that leaves a scalar tail: element i draws what element i of any longer or
+    # shorter fill draws, so the tail continues the body's sequence instead of restarting it
+    n = A * B - 5
+    y_d = rt.empty((n,))
+    sb = FusedSpecBuilder([n])
+    sb.store(sb.tensor(y_d.ptr, [1]), sb.rng("uniform", 0))
+    spec = sb.build()
+    spec.rng_seed, spec.rng_counter = 7, 0
+    rt.launch_fused(spec)
+    odd = y_d.get()
+    y_d.free()
+    assert n % 4 == 3
+    np.testing.assert_array_equal(odd, flat[:n])
+    assert not np.array_equal(odd[-3:], odd[:3])
 
 
 @pytest.mark.parametrize("n", [4096, 100003])
@@ -636,3 +688,26 @@ def test_byte_views_copy(hip_runtime, np_type):
     np.testing.assert_array_equal(dst_d.get(), src.T)
     src_d.free()
     dst_d.free()
+
+
+def test_flex_ids_past_the_end_of_the_table_are_rejected(hip_runtime):
+    """Record numbers are checked against the table they index before any kernel runs."""
+    from ngraph_hip.runtime.hiplib import HipLibraryError
+    rt = hip_runtime
+    table = rt.flex_states_alloc(3)
+    try:
+        rt.flex_prepare(table, [0, 2], [0, 0])
+        rt.flex_update(table, [2], 1)
+        for bad in ([3], [0, 7], [1 << 20]):
+            with pytest.raises(HipLibraryError) as e:
+                rt.flex_prepare(table, bad, [0] * len(bad))
+            assert e.value.code == -1
+            with pytest.raises(HipLibraryError):
+                rt.flex_update(table, bad, 1)
+        # counted from a record inside the table: two records are left after the first
+        with pytest.raises(HipLibraryError):
+            rt.flex_update(table + 168, [2], 1)
+        rt.flex_update(table + 168, [1], 1)
+        rt.sync()
+    finally:
+        rt.free(table)

@@ -76,6 +76,22 @@ def test_unary_positive_domain(backend, ng_fn, np_fn):
         np.testing.assert_allclose(f(xv), np_fn(xv), rtol=RTOL, atol=ATOL)
 
 
+def test_safelog_follows_the_reference_statement_sequence(backend):
+    """ng.safelog(x, limit) = maximum(log(x + exp(limit)), limit) (op_graph.py:3070-3072): zero
+    gives the limit, a value below exp(limit) gives about the limit, a negative value NaN."""
+    xv = np.array([0.0, 1e-30, 1e-22, np.exp(-50.0), 1e-10, 0.5, 1.0, 7.25, 3e4, -1e-3, -2.0], np.float32)
+    ax = axes(W=xv.size)
+    x = ng.placeholder(ax)
+    for limit in (-50.0, -10.0):
+        with np.errstate(all="ignore"):
+            t = np.add(xv, np.float32(np.exp(limit)), dtype=np.float32)
+            want = np.maximum(np.log(t, dtype=np.float32), np.float32(limit))
+        with executor(ng.safelog(x, limit), x) as f:
+            got = f(xv)
+        assert np.isnan(want[-2:]).all() and want[0] == np.float32(limit)
+        np.testing.assert_allclose(got, want, rtol=RTOL, atol=ATOL, equal_nan=True)
+
+
 BINARY = [(ng.add, np.add), (ng.subtract, np.subtract), (ng.multiply, np.multiply),
           (ng.divide, np.divide), (ng.maximum, np.maximum), (ng.minimum, np.minimum),
           (ng.equal, np.equal), (ng.not_equal, np.not_equal), (ng.greater, np.greater),

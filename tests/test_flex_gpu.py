@@ -61,10 +61,6 @@ def test_reference_flex_vector(flex_unfused, case):
         vset = ng.sequential([ng.assign(v, p), v])
         with executor(vset, p) as ex:
             execute_calculation(operands, operands[0][0], ex)
-    elif op == "safelog":
-        # graph-level safelog = log(maximum(x, exp(-50))) needs exp(-50), far below flex range
-        # (the reference's GPU path has a dedicated template, float_ew2.py:48); not a flex case
-        pytest.skip("safelog's cut-off constant exp(-50) is not representable in flex16")
     elif len(operands[0]) == 2:
         template_one_placeholder(operands, NG_OPS[op])
     else:

@@ -73,6 +73,14 @@ def _run_case(case):
                           ("rcp", "out", "a")], shapes)
         sim.tensors["one"].host_write(1.0)
         return [sim.run({"x": s["in"][0]}, "out") for s in steps]
+    if op == "safelog":
+        # ng.safelog is maximum(log(x + exp(-50)), -50) (op_graph.py:3070-3072): three kernels on
+        # the unfused flex transformer, the two constants written from the host like any tensor
+        shapes = {"x": shp, "off": (), "lim": (), "a": shp, "l": shp, "out": shp}
+        sim = fm.FlexSim([("add", "a", "x", "off"), ("log", "l", "a"), ("maximum", "out", "l", "lim")], shapes)
+        sim.tensors["off"].host_write(np.exp(-50.0))
+        sim.tensors["lim"].host_write(-50.0)
+        return [sim.run({"x": s["in"][0]}, "out") for s in steps]
     if len(first) == 1:
         red = op in ("sum", "prod", "max", "min", "argmax", "argmin")
         sim = fm.FlexSim([(op, "out", "x")], {"x": shp, "out": () if red else shp})
