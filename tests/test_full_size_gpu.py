@@ -1,0 +1,149 @@
+"""The three large benchmark configurations at their full sizes, through the graph path with the
+library's own kernel choice, against oracle/configs.py and oracle/flex_model.py.
+
+  C2  batch-norm forward over x fp32 (256, 56, 56, 64), gamma, beta ~ U(0.5, 1.5)
+      (frontends/neon/layer.py:1242-1257)
+  C3  Adam over 25.6 M fp32 parameters, warm step then step 2 (frontends/neon/optimizer.py:457-468)
+  C5  flex16 relu(x*w+b) over 16 M elements, 8 iterations, in both exponent-management modes
+      (float_ew2.py:261-281 for the rounding and the statistics)
+
+Tolerances are the ones the fp32 configurations are specified with, rtol 1e-5 / atol 1e-6, for
+every output including the normalised y; flex results are compared bit for bit.  Each test also
+checks that the kernels that ran are the ones the benchmark times at these sizes (the variants
+with cache hints only exist above 192 MiB of operands).
+"""
+import numpy as np
+import pytest
+from conftest import default_kernel_choice
+
+import ngraph_hip as ng
+import ngraph_hip.transformers as ngt
+from ngraph_hip.frontends import neon
+from oracle import configs
+from oracle import flex_model as fm
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-5, 1e-6
+
+
+def _kernel_names(t, f):
+    return [d for k in t.kernel_groups[f].kernels for ds in k.describe() for d in ds]
+
+
+def test_c2_batchnorm_at_full_size():
+    dims = (256, 56, 56, 64)
+    Cn, R = dims[0], dims[1] * dims[2] * dims[3]
+    x_np, gamma_np, beta_np = configs.c2_inputs(Cn, R, seed=1)
+    y_w, mean_w, var_w = configs.c2_cpu(x_np, gamma_np, beta_np)
+    t = ngt.make_transformer_factory("hipgpu")()
+    try:
+        C, H, W, N = (ng.make_axis(n, name=k) for k, n in zip("CHWN", dims))
+        x = ng.placeholder([C, H, W, N])
+        gamma = ng.variable([C], initial_value=gamma_np)
+        beta = ng.variable([C], initial_value=beta_np)
+        y, xmean, xvar = neon.batch_norm_train(x, gamma, beta, out_axes=[C])
+        f = t.computation([y, xmean, xvar], x)
+        y_g, mean_g, var_g = f(x_np.reshape(dims))
+        y_g = np.array(y_g).reshape(Cn, R)
+        names = _kernel_names(t, f)
+    finally:
+        t.close()
+    if default_kernel_choice():
+        assert names == ["moments_f32", "special:batchnorm_k1/nt-stores"], names
+    np.testing.assert_allclose(mean_g, mean_w, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(var_g, var_w, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(y_g, y_w, rtol=RTOL, atol=ATOL)
+    # ... and against float64, which neither side computes in: the one-pass variance of the
+    # device (pivot-shifted sums) and the two-pass one of the oracle both stay inside the bound
+    x64 = x_np.astype(np.float64)
+    mean64, var64 = x64.mean(axis=1), x64.var(axis=1)
+    np.testing.assert_allclose(mean_g, mean64, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(var_g, var64, rtol=RTOL, atol=ATOL)
+    for c in range(0, Cn, 17):
+        y64 = gamma_np[c] * ((x64[c] - mean64[c]) / np.sqrt(var64[c] + 1e-5)) + beta_np[c]
+        np.testing.assert_allclose(y_g[c], y64, rtol=RTOL, atol=ATOL)
+
+
+def test_c3_adam_at_full_size():
+    n = 25600000
+    p_np, g_np, m_np, v_np = configs.c3_inputs(n, seed=2)
+    t = ngt.make_transformer_factory("hipgpu")()
+    try:
+        P = ng.make_axis(n, name="P")
+        p = ng.variable([P], initial_value=p_np)
+        grad = ng.placeholder([P])
+        opt = neon.Adam()
+        opt()
+        updates, m, v = opt.variable_update(p, grad)
+        f = t.computation(updates, grad)
+        read = t.computation([p * 1.0, m * 1.0, v * 1.0])
+        ws = configs.Workspace()
+        for step in (1, 2):                      # the warm step (t = 1), then the step that is timed
+            configs.c3_cpu(p_np, g_np, m_np, v_np, step, ws=ws)
+            f(g_np)
+        p_g, m_g, v_g = (np.array(a) for a in read())
+        names = _kernel_names(t, f)
+    finally:
+        t.close()
+    if default_kernel_choice():
+        assert any(d.startswith("special:adam") and d.endswith("/nt-loads") for d in names), names
+    np.testing.assert_allclose(m_g, m_np, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(v_g, v_np, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(p_g, p_np, rtol=RTOL, atol=ATOL)
+    # the update is far below atol for these inputs (lr 1e-3): also compare it on its own scale
+    p0 = configs.c3_inputs(n, seed=2)[0]
+    np.testing.assert_allclose(p_g - p0, p_np - p0, rtol=1e-4, atol=1e-9)
+
+
+@pytest.mark.parametrize("resident", [False, True], ids=["host-policy", "device-policy"])
+def test_c5_flex_at_full_size_over_8_iterations(resident):
+    n = 16 * 1024 * 1024
+    x_np, w_np, b_np = configs.c5_inputs(n, seed=4)
+    # the oracle: x, w, b written from the host, y written by the kernel, 8 times
+    tx, tw, tb, ty = (fm._SimTensor((n,)) for _ in range(4))
+    tw.host_write(w_np)
+    tb.host_write(b_np)
+    tx.host_write(x_np)
+    assert tx.stored_dec == 12                     # x quantised at 2**-12, as the configuration says
+    want = []
+    ws = configs.Workspace()
+    for _ in range(8):
+        tx.host_write(x_np)
+        ty.kernel_write(lambda: configs.c5_cpu_float(tx.load(), tw.load(), tb.load(), ws=ws))
+        want.append((ty.mantissa.copy(), ty.stored_dec, fm.maxabs(ty.mantissa), ty.policy.dec))
+
+    t = ngt.make_transformer_factory("flexhip", resident=resident)()
+    try:
+        P = ng.make_axis(n, name="P")
+        x, w, b = ng.placeholder([P]), ng.placeholder([P]), ng.placeholder([P])
+        f = t.computation(neon.rectlin(x * w + b), x, w, b)
+        for i in range(8):
+            got = f(x_np, w_np, b_np)
+            y_view = t.get_op_tensor_view(f.computation_op.values[0])
+            entry = y_view.flex_entry
+            m_want, dec_want, maxabs_want, next_dec_want = want[i]
+            assert entry.last_maxabs == maxabs_want, (i, entry.last_maxabs, maxabs_want)
+            assert (entry.dec, entry.next_dec) == (dec_want, next_dec_want), \
+                (i, entry.dec, entry.next_dec, dec_want, next_dec_want)
+            np.testing.assert_array_equal(y_view._read_raw(), m_want, err_msg="iteration %d mantissas" % i)
+            np.testing.assert_array_equal(got, fm.dequantize(m_want, dec_want))
+        names = _kernel_names(t, f)
+        # eight more iterations without the host in between (what the benchmark times): the
+        # kernel group is launched back to back, nothing is read until the end
+        group = t.kernel_groups[f]
+        for _ in range(8):
+            group()
+            ty.kernel_write(lambda: configs.c5_cpu_float(tx.load(), tw.load(), tb.load(), ws=ws))
+        y_view = t.get_op_tensor_view(f.computation_op.values[0])
+        mant = y_view._read_raw()
+        entry = y_view.flex_entry
+        if resident:
+            t.flex_manager.pull()
+        assert (entry.dec, entry.next_dec, entry.last_maxabs) == \
+            (ty.stored_dec, ty.policy.dec, fm.maxabs(ty.mantissa))
+        np.testing.assert_array_equal(mant, ty.mantissa)
+    finally:
+        t.close()
+    if default_kernel_choice():
+        assert names == ["special:flex_relu_fma_k0"], names
