@@ -257,6 +257,18 @@ int  ngh_programs_count(int32_t* built_in, int32_t* loaded);
 int  ngh_moments_f32(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t R, int64_t row_stride,
                      float* dev_mean, float* dev_var, float* dev_rstd, float eps, uint32_t x_cache_hint);
 
+/* ngh_moments_f32 for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid it).  No counterpart in the reference.  Same
+ * arguments, same kernel and same results, but the per-segment partial sums and the per-row
+ * arrival counters live in a fixed array inside the library (768 KiB per device, held until the
+ * process ends) instead of context-owned allocations, and the call allocates and frees
+ * nothing.  Limits: rows <= 65536 and rows x segments <= 65536 (segments = what it takes to
+ * put 8 workgroups on every compute unit, at most 4096 a row); beyond them the call fails
+ * with NGH_E_UNSUPPORTED and launches nothing.  Every call on a device shares that device's
+ * array: calls that overlap there (two contexts, two host threads) race.                   */
+int  ngh_moments_f32_noalloc(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t R, int64_t row_stride,
+                             float* dev_mean, float* dev_var, float* dev_rstd, float eps, uint32_t x_cache_hint);
+
 /* How stage `stage` would be launched, without a device (host-side tooling and
  * tests): out8 = {kernel family (0 streaming, 1 reduce along the contiguous axis,
  * 2 reduce across it, 3 streaming through LDS tiles for transposed operands), vector width, spec axis on kernel axes 0,1,2, tail length,

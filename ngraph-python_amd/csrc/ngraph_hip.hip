@@ -67,6 +67,18 @@ int env_int(const char* name, int dflt) {
 
 }  // namespace
 
+// Scratch of ngh_moments_f32_noalloc, the entry point for callers that cannot allocate: the
+// per-segment partial sums (one 8-byte word per row and segment) and the per-row arrival
+// counters that ngh_moments_f32 keeps in context-owned allocations.  Every device the library
+// runs on holds one copy until the process ends; its address on a device is looked up once,
+// in ngh_init, with that device current, and only that address is ever handed to a kernel.
+constexpr size_t kNoAllocPartials = 65536;   // rows x segments of one call
+constexpr size_t kNoAllocRows = 65536;       // rows of one call
+constexpr size_t kNoAllocScratchBytes = kNoAllocPartials * sizeof(unsigned long long) + kNoAllocRows * sizeof(unsigned);
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+constexpr int kMaxDevices = 64;
+static void* g_scratch_of_device[kMaxDevices] = {nullptr};
+
 // Host-side bookkeeping of deferred statistics (ngh_flex.h): where each record of a table
 // allocated by ngh_flex_states_alloc currently lives and whether a fold is outstanding.
 struct FlexRecordHost {
@@ -94,6 +106,7 @@ struct ngh_context {
     int         flex_unsettled = 0;  // records not in their plain form
     int         device = 0;
     int         cus = 0;
+    void*       noalloc_scratch = nullptr;   // this device's copy of `scratch`
     hipStream_t stream = nullptr;
     hipEvent_t  ev0 = nullptr, ev1 = nullptr;
     void*       ws = nullptr;        // partial results of split reductions
@@ -895,7 +908,15 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     HIP_TRY(hipGetDeviceProperties(&prop, device_id));
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0 && !env_int("NGH_ALLOW_ANY_ARCH", 0))
         return fail(NGH_E_NODEVICE, "device %d is %s; this library is built for gfx950 only", device_id, prop.gcnArchName);
+    if (device_id >= kMaxDevices) return fail(NGH_E_UNSUPPORTED, "device %d: at most %d devices", device_id, kMaxDevices);
+    if (!g_scratch_of_device[device_id]) {
+        void* p = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(NGH_E_RUNTIME, "hipGetSymbolAddress returned no address for the scratch array");
+        g_scratch_of_device[device_id] = p;
+    }
     ngh_context* ctx = new ngh_context();
+    ctx->noalloc_scratch = g_scratch_of_device[device_id];
     ctx->device = device_id;
     ctx->cus = prop.multiProcessorCount;
     ctx->total_bytes = prop.totalGlobalMem;
@@ -1191,37 +1212,79 @@ int ngh_programs_count(int32_t* built_in, int32_t* loaded) {
     return NGH_OK;
 }
 
-int ngh_moments_f32(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t R, int64_t row_stride,
-                    float* dev_mean, float* dev_var, float* dev_rstd, float eps, uint32_t x_cache_hint) {
-    if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
+namespace {
+// How ngh_moments_f32 splits rows into segments: enough workgroups to fill the chip, but at
+// least 4 unrolled sweeps per segment.
+struct MomentsPlan { unsigned R4, seg_chunks, n_seg; };
+
+int plan_moments(const ngh_context* ctx, const float* dev_x, int64_t rows, int64_t R, int64_t row_stride,
+                 const float* dev_mean, const float* dev_var, MomentsPlan& m) {
     if (rows < 0 || R <= 0) return fail(NGH_E_INVALID, "rows %lld, R %lld", (long long)rows, (long long)R);
     if (rows == 0) return NGH_OK;
     if (!dev_x || !dev_mean || !dev_var) return fail(NGH_E_INVALID, "NULL device pointer");
     if (((uintptr_t)dev_x) % 16 || row_stride % 4)
         return fail(NGH_E_UNSUPPORTED, "rows must start on 16-byte boundaries");
     if (rows >= (1LL << 24) || R >= (1LL << 32)) return fail(NGH_E_UNSUPPORTED, "extent too large");
-    const unsigned R4 = (unsigned)(R / 4);
-    // enough workgroups to fill the chip, but at least 4 unrolled sweeps per segment
+    m.R4 = (unsigned)(R / 4);
     long long seg = std::max<long long>(1, (long long)ctx->cus * ctx->moments_wgs_per_cu / rows);
-    seg = std::min<long long>(seg, std::max<long long>(1, R4 / (kMomBlock * kMomUnroll * 2)));
+    seg = std::min<long long>(seg, std::max<long long>(1, m.R4 / (kMomBlock * kMomUnroll * 2)));
     seg = std::min<long long>(seg, 4096);
-    const unsigned seg_chunks = std::max(1u, (unsigned)((R4 + seg - 1) / seg));
-    const unsigned n_seg = std::max(1u, (unsigned)((R4 + seg_chunks - 1) / seg_chunks));
-    NGH_TRY(ensure_ws(ctx, (size_t)rows * n_seg * sizeof(float2)));
-    NGH_TRY(ensure_tickets(ctx, (size_t)rows));
-    float2* partial = (float2*)ctx->ws;
+    m.seg_chunks = std::max(1u, (unsigned)((m.R4 + seg - 1) / seg));
+    m.n_seg = std::max(1u, (unsigned)((m.R4 + m.seg_chunks - 1) / m.seg_chunks));
+    return NGH_OK;
+}
+
+int launch_moments(ngh_context* ctx, const MomentsPlan& m, const float* dev_x, int64_t rows, int64_t R,
+                   int64_t row_stride, float2* partial, unsigned* tickets, float* dev_mean, float* dev_var,
+                   float* dev_rstd, float eps, uint32_t x_cache_hint) {
     const bool stream_x = ctx->cache_policy >= 0
                               ? (ctx->cache_policy & 1)
                               : ((x_cache_hint & NGH_CACHE_STREAM_LOAD) && rows * R * 4 >= ctx->stream_bytes);
-    const dim3 grid((unsigned)(rows * n_seg));
+    const dim3 grid((unsigned)(rows * m.n_seg));
     if (stream_x)
         hipLaunchKernelGGL(moments_kernel<true>, grid, dim3(kMomBlock), 0, ctx->stream, dev_x, (long long)row_stride,
-                           (unsigned)R, R4, n_seg, seg_chunks, partial, ctx->tickets, dev_mean, dev_var, dev_rstd, eps);
+                           (unsigned)R, m.R4, m.n_seg, m.seg_chunks, partial, tickets, dev_mean, dev_var, dev_rstd, eps);
     else
         hipLaunchKernelGGL(moments_kernel<false>, grid, dim3(kMomBlock), 0, ctx->stream, dev_x, (long long)row_stride,
-                           (unsigned)R, R4, n_seg, seg_chunks, partial, ctx->tickets, dev_mean, dev_var, dev_rstd, eps);
+                           (unsigned)R, m.R4, m.n_seg, m.seg_chunks, partial, tickets, dev_mean, dev_var, dev_rstd, eps);
     HIP_TRY(hipGetLastError());
     return NGH_OK;
+}
+}  // namespace
+
+int ngh_moments_f32(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t R, int64_t row_stride,
+                    float* dev_mean, float* dev_var, float* dev_rstd, float eps, uint32_t x_cache_hint) {
+    if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
+    MomentsPlan m;
+    NGH_TRY(plan_moments(ctx, dev_x, rows, R, row_stride, dev_mean, dev_var, m));
+    if (rows == 0) return NGH_OK;
+    NGH_TRY(ensure_ws(ctx, (size_t)rows * m.n_seg * sizeof(float2)));
+    NGH_TRY(ensure_tickets(ctx, (size_t)rows));
+    return launch_moments(ctx, m, dev_x, rows, R, row_stride, (float2*)ctx->ws, ctx->tickets, dev_mean, dev_var,
+                          dev_rstd, eps, x_cache_hint);
+}
+
+int ngh_moments_f32_noalloc(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t R, int64_t row_stride,
+                            float* dev_mean, float* dev_var, float* dev_rstd, float eps, uint32_t x_cache_hint) {
+    if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
+    MomentsPlan m;
+    NGH_TRY(plan_moments(ctx, dev_x, rows, R, row_stride, dev_mean, dev_var, m));
+    if (rows == 0) return NGH_OK;
+    if ((size_t)rows > kNoAllocRows || (size_t)rows * m.n_seg > kNoAllocPartials)
+        return fail(NGH_E_UNSUPPORTED, "ngh_moments_f32_noalloc: %lld rows in %u segments each exceed the fixed scratch "
+                    "(%zu rows, %zu partial sums); use ngh_moments_f32", (long long)rows, m.n_seg, kNoAllocRows,
+                    kNoAllocPartials);
+    unsigned char* base = (unsigned char*)ctx->noalloc_scratch;    // the device address, never the symbol
+    float2* partial = (float2*)base;
+    unsigned* tickets = (unsigned*)(base + kNoAllocPartials * sizeof(unsigned long long));
+    // The array keeps what the last call left: the counters of the rows must start at zero (a fill
+    // kernel rather than a memset, so that the call can be captured into a graph); the partial
+    // sums need no clearing, every one that is read has been written by this launch.
+    const unsigned blocks = (unsigned)((rows + kBlock - 1) / kBlock);
+    hipLaunchKernelGGL(fill_kernel<uint32_t>, dim3(blocks), dim3(kBlock), 0, ctx->stream, tickets, 0u, (size_t)rows);
+    HIP_TRY(hipGetLastError());
+    return launch_moments(ctx, m, dev_x, rows, R, row_stride, partial, tickets, dev_mean, dev_var, dev_rstd, eps,
+                          x_cache_hint);
 }
 
 int ngh_plan_fused(const ngh_fused_spec* spec, int32_t stage, int32_t* out8) {

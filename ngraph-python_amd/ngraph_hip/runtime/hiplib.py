@@ -110,6 +110,8 @@ _SYMBOLS = {
     "ngh_describe_fused": [_vp, ctypes.POINTER(ngh_fused_spec), _i32, ctypes.c_char_p],
     "ngh_moments_f32": [_vp, _vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, _vp, _vp, _vp, ctypes.c_float,
                         ctypes.c_uint32],
+    "ngh_moments_f32_noalloc": [_vp, _vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, _vp, _vp, _vp,
+                                ctypes.c_float, ctypes.c_uint32],
     "ngh_plan_fused": [ctypes.POINTER(ngh_fused_spec), _i32, ctypes.POINTER(ctypes.c_int32)],
     "ngh_stats_alloc": [_vp, _i32, ctypes.POINTER(_vp)],
     "ngh_stats_reset": [_vp, _vp, _i32],
@@ -315,6 +317,13 @@ class HipRuntime(object):
                                                   int(row_stride), ctypes.c_void_p(mean),
                                                   ctypes.c_void_p(var), ctypes.c_void_p(rstd or None),
                                                   float(eps), int(x_cache_hint)))
+
+    def moments_f32_noalloc(self, x, rows, R, row_stride, mean, var, rstd=None, eps=0.0, x_cache_hint=0):
+        """moments_f32 on the library's fixed scratch: allocates nothing, limited in size."""
+        _check(self.lib, self.lib.ngh_moments_f32_noalloc(self.ctx, ctypes.c_void_p(x), int(rows), int(R),
+                                                          int(row_stride), ctypes.c_void_p(mean),
+                                                          ctypes.c_void_p(var), ctypes.c_void_p(rstd or None),
+                                                          float(eps), int(x_cache_hint)))
 
     # -- flex statistics ---------------------------------------------------
     def stats_alloc(self, n):
