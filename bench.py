@@ -1,12 +1,17 @@
 #!/usr/bin/env python
-"""Benchmark of the fused elementwise / reduction path on one MI355X.
+"""Benchmark of the fused elementwise / reduction / flex16 path on one MI355X.
 
-One step = one pass of the batch-norm forward graph (statistics + normalise)
-over x[256, 56, 56, 64] fp32, inputs resident in HBM.  Prints ONE JSON line:
-whole-job achieved HBM GB/s (algorithmic bytes / wall time per step), the
-roofline of the dominant kernel from HIP-event timings taken in this run, and
-the NumPy oracle timed on the host cores as the CPU baseline.  `--all` adds
-the other four configurations to the line under "other_configs".
+The headline step is one pass of the batch-norm forward graph (statistics + normalise) over
+x[256, 56, 56, 64] fp32 with inputs resident in HBM (configuration C2); the same run also
+times the other two configurations of at least 64 MB, the Adam update over 25.6 M parameters
+(C3) and the flex16 relu(x*w+b) over 16 M elements, 8 iterations a step (C5).  Prints ONE JSON
+line: whole-job achieved HBM GB/s of C2 (algorithmic bytes / wall time per step), and per
+configuration the step time over several blocks of steps (median, min, max), the roofline of
+its dominant kernel from HIP-event timings taken in this run -- back to back ("warm": part of
+the operands is still in the 256 MiB last-level cache from the launch before) and with that
+cache displaced before every launch ("cold") -- and the NumPy oracle timed on the host cores as
+the CPU baseline.  `--all` adds the two small configurations (C1, C4), `--compiled` five user
+graphs on the interpreter and with kernels compiled at run time.
 """
 from __future__ import print_function
 import argparse
@@ -23,20 +28,23 @@ for _p in (ROOT, os.path.join(ROOT, "ngraph-python_amd")):
 import numpy as np  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes one launch of the C2 normalise kernel moves, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE scaled by a device copy of known size (profiles/c2_batchnorm_pmc_traffic.md)
-MEASURED_TRAFFIC = {"special:batchnorm": 411176158}
+DISPLACE_BYTES = 512 << 20      # a device copy of this size between launches empties the last-level cache
+
+# Bytes one launch requests from the memory side of L2, recorded with rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (each scaled by a device copy of known size) -- not measured by this run.  A figure
+# is only reported for the very kernel and shape it was recorded on.
+RECORDED_TRAFFIC = {
+    ("C2", "special:batchnorm_k1/nt-stores", 51380224): (411176158, "profiles/c2_batchnorm_pmc_traffic.md"),
+}
 
 
-def build_c2(ng, neon, t, dims):
-    C, H, W, N = (ng.make_axis(n, name=k) for k, n in zip("CHWN", dims))
-    x = ng.placeholder([C, H, W, N])
-    gamma = ng.variable([C], initial_value=np.ones(dims[0], np.float32))
-    beta = ng.variable([C], initial_value=np.zeros(dims[0], np.float32))
-    y, xmean, xvar = neon.batch_norm_train(x, gamma, beta, out_axes=[C])
-    return t.computation([y, xmean, xvar], x), x, gamma, beta
+def recorded_traffic(config, kernel, elements):
+    hit = RECORDED_TRAFFIC.get((config, kernel, elements))
+    return {"traffic": hit[0] if hit else None,
+            "traffic_source": ("requested bytes at L2 -> fabric, recorded in %s" % hit[1]) if hit else None}
 
 
+# ------------------------------------------------------------------------------------- timing
 def time_steps(rt, run, steps, warmup):
     for _ in range(warmup):
         run()
@@ -48,10 +56,42 @@ def time_steps(rt, run, steps, warmup):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
+def step_blocks(rt, run, steps, warmup, blocks):
+    """[ms per step] of `blocks` timed blocks of exactly `steps` steps; the first follows `warmup`
+    untimed steps."""
+    out = [time_steps(rt, run, steps, warmup)]
+    for _ in range(blocks - 1):
+        out.append(time_steps(rt, run, steps, 0))
+    return out
+
+
+def spread(ms):
+    return {"blocks": len(ms), "median_ms": round(float(np.median(ms)), 5), "min_ms": round(min(ms), 5),
+            "max_ms": round(max(ms), 5)}
+
+
+class Displacer(object):
+    """Empties the last-level cache: a device-to-device copy between two 512 MiB buffers."""
+
+    def __init__(self, rt):
+        self.rt = rt
+        self.a, self.b = rt.malloc(DISPLACE_BYTES), rt.malloc(DISPLACE_BYTES)
+        rt.memset32(self.a, 0, DISPLACE_BYTES // 4)
+
+    def __call__(self):
+        self.rt.memcpy_d2d(self.b, self.a, DISPLACE_BYTES)
+
+    def free(self):
+        self.rt.free(self.a)
+        self.rt.free(self.b)
+
+
 def kernel_bytes(kernel):
-    """Algorithmic bytes of one launch of a fused kernel: every operand once."""
+    """Algorithmic bytes of one launch of a kernel: every operand once per direction."""
+    if hasattr(kernel, "rows"):                         # the moments kernel reads x once, writes 3 floats a row
+        return kernel.rows * kernel.R * 4 + kernel.rows * 12
     total = 0
-    for spec in kernel.specs:
+    for spec in getattr(kernel, "specs", []):
         shape = [spec.shape[i] for i in range(3)]
         for i in range(spec.n_tensors):
             t = spec.tensors[i]
@@ -61,40 +101,161 @@ def kernel_bytes(kernel):
                     n *= shape[a]
             loads = sum(1 for o in spec.ops[:spec.n_ops] if o.opcode == 1 and o.a == i)
             stores = sum(1 for o in spec.ops[:spec.n_ops] if o.opcode == 2 and o.dst == i)
-            itemsize = 2 if t.dtype in (1, 3) else 4
+            itemsize = {0: 4, 2: 4, 4: 4, 6: 1, 7: 1}.get(t.dtype, 2)
             total += n * itemsize * (min(loads, 1) + min(stores, 1))
     return total
 
 
-def other_configs(ng, ngt, neon, configs, steps, warmup):
-    """C1, C3, C4, C5 with inputs resident: ms per step and algorithmic GB/s (for information;
-    the headline line is C2)."""
-    out = {}
+def kernel_name(kernel):
+    return "+".join(sum(kernel.describe(), [])) if hasattr(kernel, "describe") else type(kernel).__name__
 
-    def run(name, t, f, nbytes, elems, per_step=1):
-        group = t.kernel_groups[f]
+
+def profile_kernels(group, rt, repeats, inner, displace=None):
+    """Per kernel: algorithmic bytes and HIP-event duration per launch on the launch stream.
+    Warm: `inner` launches back to back between one pair of events.  Cold (`displace` given):
+    the cache is emptied before every launch, outside the event pair, one launch per pair."""
+    out = []
+    if displace is None:
+        for k, times in group.profile(repeats=repeats, inner=inner):
+            out.append({"kernel": kernel_name(k), "bytes": kernel_bytes(k), "ms": float(np.median(times))})
+        return out
+    for k in group.kernels:
+        times = []
+        for _ in range(repeats):
+            displace()
+            group.setup_kernel_execute(k)
+            rt.timer_begin()
+            k.execute()
+            times.append(rt.timer_end())
+            group.after_kernel_execute(k)
+        out.append({"kernel": kernel_name(k), "bytes": kernel_bytes(k), "ms": float(np.median(times))})
+    return out
+
+
+def event_pair_overhead_ms(rt, repeats=20):
+    """What a pair of events around nothing reads: the floor under every one-launch timing."""
+    times = []
+    for _ in range(repeats):
+        rt.timer_begin()
+        times.append(rt.timer_end())
+    return float(np.median(times))
+
+
+def cold_step_ms(group, rt, displace, repeats):
+    times = []
+    for _ in range(repeats):
+        displace()
+        rt.timer_begin()
         group()
-        t.runtime.sync()
-        ms = time_steps(t.runtime, group, steps, warmup)
-        kern = []
-        for k, times in group.profile(repeats=5):
-            kern.append({"kernel": "+".join(sum(k.describe(), [])), "ms": round(float(np.mean(times)), 5)})
-        out[name] = {"ms_per_step": round(ms, 5), "GB/s": round(nbytes * per_step / (ms * 1e-3) / 1e9, 1),
-                     "frac_of_hbm_peak": round(nbytes * per_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                     "elements_per_s": round(elems * per_step / (ms * 1e-3), 1), "kernels": kern}
-        t.close()
+        times.append(rt.timer_end())
+    return float(np.median(times))
 
-    # C1
+
+def roofline_of(config, kernels_warm, kernels_cold, elements):
+    """Roofline block of the kernel with the longest warm duration."""
+    i = max(range(len(kernels_warm)), key=lambda j: kernels_warm[j]["ms"])
+    dom = kernels_warm[i]
+    achieved = dom["bytes"] / (dom["ms"] * 1e-3) / 1e9
+    out = {"bound": "hbm", "kernel": dom["kernel"], "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+           "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+           "algorithmic_bytes_per_launch": dom["bytes"], "avg_launch_ms": round(dom["ms"], 5),
+           "timing": "HIP events on the launch stream, median over event pairs of 10 back-to-back launches"}
+    out.update(recorded_traffic(config, dom["kernel"], elements))
+    if kernels_cold:
+        c = kernels_cold[i]
+        cold = c["bytes"] / (c["ms"] * 1e-3) / 1e9
+        out["cold"] = {"achieved": round(cold, 1), "frac": round(cold / HBM_PEAK_GBS, 4),
+                       "avg_launch_ms": round(c["ms"], 5),
+                       "timing": "one launch per event pair after a 512 MiB device copy has displaced the "
+                                 "last-level cache (the event pair adds a few microseconds)"}
+    return out
+
+
+def config_block(name, workload, step_ms, nbytes, elems, kernels_warm, kernels_cold, cold_ms, roof_elems,
+                 per_step=1):
+    ms = float(np.median(step_ms))
+    blk = {"workload": workload, "ms_per_step": spread(step_ms),
+           "GB/s": round(nbytes * per_step / (ms * 1e-3) / 1e9, 1),
+           "frac_of_hbm_peak": round(nbytes * per_step / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+           "elements_per_s": round(elems * per_step / (ms * 1e-3), 1),
+           "algorithmic_bytes_per_step": nbytes * per_step,
+           "kernels": [dict({"kernel": k["kernel"], "ms": round(k["ms"], 5), "bytes": k["bytes"],
+                             "GB/s": round(k["bytes"] / (k["ms"] * 1e-3) / 1e9, 1)},
+                            **({"cold_ms": round(kernels_cold[i]["ms"], 5),
+                                "cold_GB/s": round(k["bytes"] / (kernels_cold[i]["ms"] * 1e-3) / 1e9, 1)}
+                               if kernels_cold else {}))
+                       for i, k in enumerate(kernels_warm)],
+           "roofline": roofline_of(name, kernels_warm, kernels_cold, roof_elems)}
+    if cold_ms is not None:
+        blk["cold_step"] = {"ms": round(cold_ms, 5), "GB/s": round(nbytes * per_step / (cold_ms * 1e-3) / 1e9, 1),
+                            "frac_of_hbm_peak": round(nbytes * per_step / (cold_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    return blk
+
+
+# ------------------------------------------------------------------------------------- configurations
+C2_DIMS = (256, 56, 56, 64)
+
+
+def build_c2(ng, neon, t, dims, gamma_np, beta_np):
+    C, H, W, N = (ng.make_axis(n, name=k) for k, n in zip("CHWN", dims))
+    x = ng.placeholder([C, H, W, N])
+    gamma = ng.variable([C], initial_value=gamma_np)
+    beta = ng.variable([C], initial_value=beta_np)
+    y, xmean, xvar = neon.batch_norm_train(x, gamma, beta, out_axes=[C])
+    return t.computation([y, xmean, xvar], x), x
+
+
+def bench_c2(ng, ngt, neon, configs, args, want_cold, copy_calibration=0):
+    dims = C2_DIMS
+    n_elems = int(np.prod(dims))
+    nbytes = 3 * n_elems * 4                                  # statistics read + normalise read + write
     t = ngt.make_transformer_factory("hipgpu")()
-    x_np, a, b = configs.c1_inputs((1024, 1024))
-    H, W = ng.make_axis(1024, name="H"), ng.make_axis(1024, name="W")
-    x, pa, pb = ng.placeholder([H, W]), ng.placeholder(()), ng.placeholder(())
-    f = t.computation(ng.tanh(pa * x + pb) * ng.sigmoid(x), x, pa, pb)
-    f(x_np, a, b)
-    run("C1", t, f, 8388608, 1048576)
-    # C3
-    t = ngt.make_transformer_factory("hipgpu")()
+    rt = t.runtime
+    x_np, gamma_np, beta_np = configs.c2_inputs(dims[0], n_elems // dims[0], seed=1)
+    f, x = build_c2(ng, neon, t, dims, gamma_np, beta_np)
+    t.initialize()
+    t.get_op_tensor_view(x)[...] = x_np.reshape(dims)        # inputs resident before timing
+    group = t.kernel_groups[f]
+    group()                                                    # binds buffers, first launch
+    rt.sync()
+    step_ms = step_blocks(rt, group, args.steps, args.warmup, args.blocks)
+    warm = profile_kernels(group, rt, repeats=max(args.steps // 10, 5), inner=10)
+    cold, cold_ms = None, None
+    overhead = event_pair_overhead_ms(rt)
+    if want_cold:
+        d = Displacer(rt)
+        cold = profile_kernels(group, rt, repeats=15, inner=1, displace=d)
+        cold_ms = cold_step_ms(group, rt, d, 15)
+        d.free()
+    if copy_calibration:
+        y_view = t.get_op_tensor_view(f.computation_op.values[0])
+        x_view = t.get_op_tensor_view(x)
+        for _ in range(copy_calibration):
+            rt.memcpy_d2d(y_view.ptr, x_view.ptr, n_elems * 4)
+        rt.sync()
+    group()
+    rt.sync()
+    # Parity at full size through a property that does not depend on it: per channel the
+    # normalised output has mean beta and variance gamma^2 * var / (var + eps).  (The element by
+    # element comparison with the oracle at this size is tests/test_full_size_gpu.py.)
+    y = t.get_op_tensor_view(f.computation_op.values[0]).get(None).reshape(dims[0], -1).astype(np.float64)
+    var = x_np.astype(np.float64).var(axis=1)
+    g64, b64 = gamma_np.astype(np.float64), beta_np.astype(np.float64)
+    assert np.abs(y.mean(axis=1) - b64).max() < 1e-4, "normalised output: per-channel mean is not beta"
+    assert np.abs(y.var(axis=1) - g64 * g64 * var / (var + 1e-5)).max() < 1e-3, \
+        "normalised output: per-channel variance is not gamma^2 var / (var + eps)"
+    t.close()
+    workload = ("C2 batch-norm forward: x fp32 [256,56,56,64] ~N(0.5,2), gamma, beta ~U(0.5,1.5), statistics over "
+                "H,W,N then normalise; algorithmic bytes 616562688 per step")
+    blk = config_block("C2", workload, step_ms, nbytes, n_elems, warm, cold, cold_ms, n_elems)
+    blk["empty_event_pair_ms"] = round(overhead, 5)
+    return blk, x_np, gamma_np, beta_np
+
+
+def bench_c3(ng, ngt, neon, configs, args, want_cold):
     n = 25600000
+    t = ngt.make_transformer_factory("hipgpu")()
+    rt = t.runtime
     p_np, g_np, _, _ = configs.c3_inputs(n)
     P = ng.make_axis(n, name="P")
     p, grad = ng.variable([P], initial_value=p_np), ng.placeholder([P])
@@ -103,8 +264,97 @@ def other_configs(ng, ngt, neon, configs, steps, warmup):
     updates, _, _ = opt.variable_update(p, grad)
     f = t.computation(updates, grad)
     f(g_np)                                   # the warm step (t = 1); inputs stay resident
-    run("C3", t, f, 716800000, n)
-    # C4
+    group = t.kernel_groups[f]
+    steps = max(args.steps // 2, 5)
+    step_ms = step_blocks(rt, group, steps, args.warmup, args.blocks)
+    warm = profile_kernels(group, rt, repeats=max(steps // 10, 5), inner=10)
+    cold, cold_ms = None, None
+    if want_cold:
+        d = Displacer(rt)
+        cold = profile_kernels(group, rt, repeats=15, inner=1, displace=d)
+        cold_ms = cold_step_ms(group, rt, d, 15)
+        d.free()
+    t.close()
+    workload = ("C3 Adam update in place over 25.6 M fp32 parameters (p, m, v read and written, grad read): "
+                "algorithmic bytes 716800000 per step; timed from step 2 on")
+    return config_block("C3", workload, step_ms, 716800000, n, warm, cold, cold_ms, n)
+
+
+class _Times(object):
+    """A kernel group whose step is `n` runs of another group (C5: 8 iterations a step)."""
+
+    def __init__(self, group, n):
+        self.group, self.n, self.kernels = group, n, group.kernels
+
+    def __call__(self):
+        for _ in range(self.n):
+            self.group()
+
+
+def bench_c5(ng, ngt, neon, configs, args, want_cold):
+    n = 16 * 1024 * 1024
+    t = ngt.make_transformer_factory("flexhip")()
+    rt = t.runtime
+    x_np, w_np, b_np = configs.c5_inputs(n)
+    P = ng.make_axis(n, name="P")
+    x, w, b = ng.placeholder([P]), ng.placeholder([P]), ng.placeholder([P])
+    f = t.computation(neon.rectlin(x * w + b), x, w, b)
+    f(x_np, w_np, b_np)
+    group = t.kernel_groups[f]
+    group()
+    rt.sync()
+    eight = _Times(group, 8)
+    steps = max(args.steps // 4, 5)
+    step_ms = step_blocks(rt, eight, steps, args.warmup, args.blocks)
+    # the kernel as it runs inside a step: 8 iterations between one pair of events
+    times = []
+    for _ in range(max(steps // 5, 5)):
+        rt.timer_begin()
+        eight()
+        times.append(rt.timer_end() / 8)
+    name = "+".join(kernel_name(k) for k in group.kernels)
+    warm = [{"kernel": name, "bytes": 134217728, "ms": float(np.median(times))}]
+    cold, cold_ms = None, None
+    if want_cold:
+        d = Displacer(rt)
+        times = []
+        for _ in range(15):
+            d()
+            rt.timer_begin()
+            group()
+            times.append(rt.timer_end())
+        cold = [{"kernel": name, "bytes": 134217728, "ms": float(np.median(times))}]
+        d.free()
+    mode = "device-resident" if t.flex_manager.resident else "host-managed"
+    t.close()
+    workload = ("C5 flex16 y = relu(x*w+b) over 16777216 elements, int16 mantissas with per-tensor exponents, "
+                "max|mantissa| feeding the exponent update, 8 iterations per step (%s exponent management, the "
+                "default of the flexhip transformer); algorithmic bytes 134217728 per iteration" % mode)
+    blk = config_block("C5", workload, step_ms, 134217728, n, warm, cold, cold_ms, n, per_step=8)
+    blk["flex16_elements_per_s"] = blk["elements_per_s"]
+    return blk
+
+
+def small_configs(ng, ngt, neon, configs, steps, warmup):
+    """C1 and C4 with inputs resident: launch-bound sizes, for information."""
+    out = {}
+
+    def run(name, t, f, nbytes, elems):
+        group = t.kernel_groups[f]
+        group()
+        t.runtime.sync()
+        ms = step_blocks(t.runtime, group, steps, warmup, 3)
+        kern = profile_kernels(group, t.runtime, repeats=5, inner=10)
+        out[name] = config_block(name, name, ms, nbytes, elems, kern, None, None, elems)
+        t.close()
+
+    t = ngt.make_transformer_factory("hipgpu")()
+    x_np, a, b = configs.c1_inputs((1024, 1024))
+    H, W = ng.make_axis(1024, name="H"), ng.make_axis(1024, name="W")
+    x, pa, pb = ng.placeholder([H, W]), ng.placeholder(()), ng.placeholder(())
+    f = t.computation(ng.tanh(pa * x + pb) * ng.sigmoid(x), x, pa, pb)
+    f(x_np, a, b)
+    run("C1", t, f, 8388608, 1048576)
     t = ngt.make_transformer_factory("hipgpu")()
     Hn, Nn = 1024, 64
     gates_np, cprev_np = configs.c4_inputs(Hn, Nn)
@@ -117,30 +367,10 @@ def other_configs(ng, ngt, neon, configs, steps, warmup):
     f = t.computation([c, h, ng.sum(gates, out_axes=[G])], gates_st, cprev_st)
     f(gates_np, cprev_np)
     run("C4", t, f, 1851392, 327680)
-    # C5: 8 iterations of the fused flex kernel; statistics and the exponent update stay on the device
-    t = ngt.make_transformer_factory("flexhip", resident=True)()
-    n = 16 * 1024 * 1024
-    x_np, w_np, b_np = configs.c5_inputs(n)
-    P = ng.make_axis(n, name="P")
-    x, w, b = ng.placeholder([P]), ng.placeholder([P]), ng.placeholder([P])
-    f = t.computation(neon.rectlin(x * w + b), x, w, b)
-    f(x_np, w_np, b_np)
-    group = t.kernel_groups[f]
-
-    class Eight(object):
-        kernels = group.kernels
-
-        def __call__(self):
-            for _ in range(8):
-                group()
-
-        def profile(self, repeats):
-            return group.profile(repeats)
-    t.kernel_groups[f] = Eight()
-    run("C5", t, f, 134217728, n, per_step=8)
     return out
 
 
+# ------------------------------------------------------------------------------------- user graphs
 def user_graphs(ng, An=8192, Bn=8192):
     """(name, results, inputs, passes over an An x Bn fp32 tensor) of graphs the library has no
     built-in program for: what a user's own elementwise / reduction code looks like."""
@@ -156,23 +386,28 @@ def user_graphs(ng, An=8192, Bn=8192):
 
 
 def compiled_vs_interpreted(ng, ngt, steps, warmup, An=8192, Bn=8192):
-    """The same computations on the interpreter and with kernels compiled at run time
-    (make_transformer_factory(..., jit=True)): ms per step, algorithmic GB/s, kernels."""
+    """The same computations with the transformer's default kernel choice (programs compiled at
+    run time for large stages), on the interpreter alone (jit=False) and with compilation
+    forced for every stage (jit=True): ms per step, algorithmic GB/s, kernels."""
     out = {}
     for name, results, inputs, passes in user_graphs(ng, An, Bn):
         row = {}
-        for mode in (False, True):
+        # (interpreter first: a compiled program, once loaded, serves every transformer of the process)
+        for label, mode in (("interpreted", False), ("default", None), ("compiled", True)):
             t = ngt.make_transformer_factory("hipgpu", jit=mode)()
             try:
                 f = t.computation(results, *inputs)
                 f(*[np.random.RandomState(1 + i).uniform(-1, 1, p.axes.lengths).astype(np.float32)
                     for i, p in enumerate(inputs)])
                 group = t.kernel_groups[f]
+                if hasattr(group, "wait_for_programs"):
+                    group.wait_for_programs()
                 group()
                 t.runtime.sync()
-                ms = time_steps(t.runtime, group, steps, warmup)
-                row["compiled" if mode else "interpreted"] = {
+                ms = float(np.median(step_blocks(t.runtime, group, steps, warmup, 3)))
+                row[label] = {
                     "ms_per_step": round(ms, 5), "GB/s": round(passes * An * Bn * 4 / (ms * 1e-3) / 1e9, 1),
+                    "frac_of_hbm_peak": round(passes * An * Bn * 4 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                     "kernels": [d for k in group.kernels for ds in k.describe() for d in ds]}
             finally:
                 t.close()
@@ -180,10 +415,8 @@ def compiled_vs_interpreted(ng, ngt, steps, warmup, An=8192, Bn=8192):
     return out
 
 
-def cpu_baseline_c2(dims, budget_s=20.0):
-    from oracle import configs
-    C, R = dims[0], dims[1] * dims[2] * dims[3]
-    x, gamma, beta = configs.c2_inputs(C, R, seed=1)
+# ------------------------------------------------------------------------------------- CPU baseline
+def cpu_baseline_c2(configs, x, gamma, beta, budget_s=20.0):
     ws = configs.Workspace()
     configs.c2_cpu(x, gamma, beta, ws=ws)                       # warm, allocates the pools
     times, t_start = [], time.perf_counter()
@@ -198,15 +431,55 @@ def cpu_baseline_c2(dims, budget_s=20.0):
                                                              os.cpu_count())}
 
 
+def cpu_baseline_others(configs, budget_s=4.0):
+    """C3 and C5 on the host: a few runs each (bounded), in the unit of their configuration."""
+    out = {}
+    n = 25600000
+    p, g, m, v = configs.c3_inputs(n)
+    ws = configs.Workspace()
+    configs.c3_cpu(p, g, m, v, 1, ws=ws)
+    times, t_start, step = [], time.perf_counter(), 2
+    while len(times) < 2 or (time.perf_counter() - t_start < budget_s and len(times) < 10):
+        t0 = time.perf_counter()
+        configs.c3_cpu(p, g, m, v, step, ws=ws)
+        times.append(time.perf_counter() - t0)
+        step += 1
+    sec = float(np.median(times))
+    out["C3"] = {"value": round(716800000 / sec / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                 "sample": "full C3 step, %d runs, median %.3f s" % (len(times), sec)}
+    from oracle import flex_model as fm
+    n = 16 * 1024 * 1024
+    x, w, b = configs.c5_inputs(n)
+    tx, tw, tb, ty = (fm._SimTensor((n,)) for _ in range(4))
+    tx.host_write(x)
+    tw.host_write(w)
+    tb.host_write(b)
+    ws = configs.Workspace()
+    times, t_start = [], time.perf_counter()
+    while len(times) < 2 or (time.perf_counter() - t_start < budget_s and len(times) < 8):
+        t0 = time.perf_counter()
+        ty.kernel_write(lambda: configs.c5_cpu_float(tx.load(), tw.load(), tb.load(), ws=ws))
+        times.append(time.perf_counter() - t0)
+    sec = float(np.median(times))
+    out["C5"] = {"value": round(n / sec, 1), "unit": "flex16 elements/s", "cores": 1, "kind": "port",
+                 "sample": "one C5 iteration (dequantise, relu(x*w+b), quantise, max|mantissa|, exponent "
+                           "policy) of the NumPy flex model, %d runs, median %.3f s" % (len(times), sec)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--all", action="store_true", help="also time configs C1, C3, C4, C5")
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--blocks", type=int, default=5,
+                    help="timed blocks of --steps steps (the first gives the headline, all give the spread)")
+    ap.add_argument("--configs", default="c2,c3,c5", help="which of c2, c3, c5 to run (c2 always runs)")
+    ap.add_argument("--no-cold", action="store_true", help="skip the measurements with a displaced cache")
+    ap.add_argument("--all", action="store_true", help="also time the small configurations C1 and C4")
     ap.add_argument("--compiled", action="store_true",
-                    help="also time five user graphs on the interpreter and with kernels compiled "
-                         "at run time (needs hipcc unless the program cache already holds them)")
+                    help="also time five user graphs: default kernel choice, interpreter only, compiled "
+                         "(needs hipcc unless the program cache already holds them)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
                     help="also issue N device-to-device copies of x (205 520 896 bytes each): a "
@@ -217,78 +490,45 @@ def main():
               "exchange except for tiny statistics all-reduces, which are not part of this run.",
               file=sys.stderr)
         sys.exit(2)
+    args.blocks = max(1, args.blocks)
+    which = set(s.strip().lower() for s in args.configs.split(","))
 
     import ngraph_hip as ng
     import ngraph_hip.transformers as ngt
     from ngraph_hip.frontends import neon
     from oracle import configs
 
-    dims = (256, 56, 56, 64)
-    n_elems = int(np.prod(dims))
-    algorithmic_bytes = 3 * n_elems * 4                       # stats read + normalise read + write
-    t = ngt.make_transformer_factory("hipgpu")()
-    rt = t.runtime
-    f, x, gamma, beta = build_c2(ng, neon, t, dims)
-    x_np, gamma_np, beta_np = configs.c2_inputs(dims[0], n_elems // dims[0], seed=1)
-    t.initialize()
-    t.get_op_tensor_view(x)[...] = x_np.reshape(dims)        # inputs resident before timing
-    group = t.kernel_groups[f]
-    group()                                                    # binds buffers, first launch
-    rt.sync()
-
-    ms = time_steps(rt, group, args.steps, args.warmup)
-    value = algorithmic_bytes / (ms * 1e-3) / 1e9
-
-    # dominant kernel: HIP-event duration of every launch over the same number of steps
-    prof = group.profile(repeats=max(args.steps // 2, 5), inner=10)
-    per_kernel = []
-    for k, times in prof:
-        per_kernel.append({"kernel": "+".join(sum(k.describe(), [])) if hasattr(k, "describe") else
-                           type(k).__name__, "ms": float(np.mean(times)),
-                           "bytes": kernel_bytes(k) if hasattr(k, "specs") else
-                           # the moments kernel reads x once and writes 3 floats per row
-                           (k.rows * k.R * 4 + k.rows * 12 if hasattr(k, "rows") else 0)})
-    dom = max(per_kernel, key=lambda d: d["ms"])
-    achieved = dom["bytes"] / (dom["ms"] * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": dom["kernel"], "achieved": round(achieved, 1),
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": next((v for k, v in MEASURED_TRAFFIC.items() if dom["kernel"].startswith(k)), None),
-                "algorithmic_bytes_per_launch": dom["bytes"],
-                "avg_launch_ms": round(dom["ms"], 5)}
-
-    if args.copy_calibration:
-        y_view = t.get_op_tensor_view(f.computation_op.values[0])
-        x_view = t.get_op_tensor_view(x)
-        for _ in range(args.copy_calibration):
-            rt.memcpy_d2d(y_view.ptr, x_view.ptr, n_elems * 4)
-        rt.sync()
-        group()                                                # y holds the normalised output again
-        rt.sync()
-
-    # parity spot-check at full size through a size-independent property: normalised output
-    # has per-channel mean beta and variance gamma^2 * var / (var + eps)
-    y = t.get_op_tensor_view(f.computation_op.values[0]).get(None).reshape(dims[0], -1)
-    ch_mean = y.astype(np.float64).mean(axis=1)
-    ch_var = y.astype(np.float64).var(axis=1)
-    assert np.abs(ch_mean).max() < 1e-4 and np.abs(ch_var - 1).max() < 1e-3, (ch_mean, ch_var)
-
-    out = {"metric": "achieved HBM GB/s on fused elementwise/reduction graphs (batch-norm forward)",
+    c2, x_np, gamma_np, beta_np = bench_c2(ng, ngt, neon, configs, args, not args.no_cold, args.copy_calibration)
+    ms = c2["ms_per_step"]["median_ms"]
+    value = c2["algorithmic_bytes_per_step"] / (ms * 1e-3) / 1e9
+    out = {"metric": "achieved HBM GB/s on fused elementwise/reduction graphs (batch-norm forward); flex16 elem/s "
+                     "under configs.C5",
            "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
-           "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True,
+           "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
            "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-           "config": {"workload": "C2 batch-norm forward: x fp32 [256,56,56,64] ~N(0.5,2), stats over "
-                                  "H,W,N then normalise; algorithmic bytes 616562688 per step",
-                      "elements": n_elems, "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
-                      "elements_per_s": round(n_elems / (ms * 1e-3), 1),
-                      "kernels": per_kernel},
-           "roofline": roofline}
-    t.close()
+           "config": {"workload": c2["workload"], "elements": int(np.prod(C2_DIMS)),
+                      "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+                      "elements_per_s": c2["elements_per_s"], "kernels": c2["kernels"],
+                      "ms_per_step_blocks": c2["ms_per_step"],
+                      "value_is": "median over %d blocks of %d back-to-back steps each" % (args.blocks, args.steps)},
+           "roofline": c2["roofline"]}
+    if "cold_step" in c2:
+        out["config"]["cold_step"] = c2["cold_step"]
+    out["configs"] = {"C2": c2}
+    if "c3" in which:
+        out["configs"]["C3"] = bench_c3(ng, ngt, neon, configs, args, not args.no_cold)
+    if "c5" in which:
+        out["configs"]["C5"] = bench_c5(ng, ngt, neon, configs, args, not args.no_cold)
     if args.all:
-        out["other_configs"] = other_configs(ng, ngt, neon, configs, max(5, args.steps // 3), 2)
+        out["configs"].update(small_configs(ng, ngt, neon, configs, max(5, args.steps // 4), 2))
     if args.compiled:
-        out["compiled_at_run_time"] = compiled_vs_interpreted(ng, ngt, max(5, args.steps // 5), 2)
+        out["compiled_at_run_time"] = compiled_vs_interpreted(ng, ngt, max(5, args.steps // 20), 2)
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline_c2(dims)
+        out["cpu_baseline"] = cpu_baseline_c2(configs, x_np, gamma_np, beta_np)
+        others = cpu_baseline_others(configs)
+        for name, blk in others.items():
+            if name in out["configs"]:
+                out["configs"][name]["cpu_baseline"] = blk
     print(json.dumps(out))
 
 

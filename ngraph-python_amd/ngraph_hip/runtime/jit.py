@@ -11,15 +11,29 @@ same C++ tables the built-in ones are made from, compiled by hipcc into a *progr
 compiler flags) and handed to the library with `ngh_programs_load`.  The object files are
 kept, so a program is compiled once per machine, not once per process.
 
-Opt-in (`make_transformer_factory("hipgpu", jit=True)` or NGH_JIT=1): compiling takes seconds
-per program, which pays for kernels that run many times over large tensors and not for a test
-suite's thousands of one-shot graphs.
+Three modes (`make_transformer_factory("hipgpu", jit=...)`, default from NGH_JIT, else "auto"):
+
+  "auto"  stages over large tensors (at least `jit_auto_min_elements` elements) that no compiled
+          kernel covers are compiled by worker threads once the computation runs for the second
+          time, while it goes on running on the interpreter; the kernel group loads the
+          libraries when they are ready and the next launch finds them.  Program libraries
+          already in the cache are loaded when the computation is first run.  Without hipcc on
+          the machine the computation simply stays on the interpreter.
+  True    every stage of at least `jit_min_elements` elements is compiled before the first
+          launch (the reference's behaviour: it compiles a computation's kernels when the
+          transformer is initialised); a missing hipcc is an error.
+  False   interpreter and built-in programs only.
+
+Compiling takes seconds per program, which pays for kernels that run many times over large
+tensors and not for a test suite's thousands of one-shot graphs: hence the size threshold of
+the default mode.
 """
 from __future__ import print_function
 
 import hashlib
 import os
 import subprocess
+import threading
 
 from ngraph_hip.runtime import hiplib
 from ngraph_hip.runtime.programs import stage_programs, render
@@ -42,8 +56,25 @@ extern "C" int ngh_program_library(int abi, unsigned entry_bytes, unsigned args_
 """
 
 
-def enabled_by_default():
-    return os.environ.get("NGH_JIT", "0") not in ("", "0")
+def default_mode():
+    """The transformer's jit mode when none is given: NGH_JIT=0 -> False, NGH_JIT=1 -> True,
+    anything else (or unset) -> "auto"."""
+    v = os.environ.get("NGH_JIT", "auto").strip().lower()
+    if v in ("0", "false", "off", "no"):
+        return False
+    if v in ("1", "true", "on", "yes"):
+        return True
+    return "auto"
+
+
+def normalize_mode(jit):
+    if jit is None:
+        return default_mode()
+    if isinstance(jit, str):
+        if jit.lower() == "auto":
+            return "auto"
+        raise ValueError("jit must be True, False or 'auto', not %r" % (jit,))
+    return bool(jit)
 
 
 def cache_dir():
@@ -89,7 +120,7 @@ def compile_programs(programs, verbose=False):
     src = base + ".hip"
     with open(src, "w") as fh:
         fh.write(text)
-    tmp = "%s.%d.tmp" % (lib, os.getpid())
+    tmp = "%s.%d.%d.tmp" % (lib, os.getpid(), threading.get_ident())
     try:
         hipcc = find_hipcc()
     except RuntimeError:
@@ -137,3 +168,139 @@ def ensure_programs(runtime, kernels, name, min_elements=4096, verbose=False):
         finally:
             pool.close()
     return sum(runtime.programs_load(path) for path in paths)
+
+
+def library_path_of(programs):
+    """Where the program library of `programs` lives in the cache (whether or not it exists)."""
+    flags, _ = _flags()
+    text = source_text(programs)
+    key = hashlib.sha256((text + _sources_digest() + " ".join(flags)).encode("utf-8")).hexdigest()[:20]
+    return os.path.join(cache_dir(), "ngh_programs_" + key + ".so")
+
+
+_executor = None
+_executor_lock = threading.Lock()
+
+
+def _compile_executor():
+    """One small pool of compile workers for the whole process, however many computations ask:
+    each job is a hipcc run (itself several processes), so a pool per computation would
+    flood a machine that builds many graphs."""
+    global _executor
+    with _executor_lock:
+        if _executor is None:
+            from concurrent.futures import ThreadPoolExecutor
+            workers = max(1, min(4, (os.cpu_count() or 2) // 2))
+            _executor = ThreadPoolExecutor(max_workers=workers, thread_name_prefix="ngh-jit")
+        return _executor
+
+
+class BackgroundPrograms(object):
+    """The uncovered programs of a kernel group, compiled off the launch path.
+
+    Libraries the cache already holds are loaded at once.  The others are handed to the
+    process-wide compile workers by `start` (the kernel group calls it once the computation has
+    run `after_calls` times: a computation that runs once never pays for a compiler run); the
+    workers run hipcc and touch no device.  `poll`, called from the thread that owns the
+    runtime, loads what has been compiled since the last call and returns True once nothing is
+    outstanding.  A compiler that is missing or fails leaves the group on the interpreter; the
+    message is kept in `error`.  `cancel` withdraws the jobs that have not started."""
+
+    def __init__(self, runtime, programs, after_calls=2, verbose=False):
+        self.runtime = runtime
+        self.error = None
+        self.loaded = 0
+        self.verbose = verbose
+        self.after_calls = int(after_calls)
+        self.calls = 0
+        self._futures = None               # None: compilation not started yet
+        self._todo = []
+        for p in programs:
+            path = library_path_of([p])
+            if os.path.exists(path):
+                self.loaded += runtime.programs_load(path)
+            else:
+                self._todo.append(p)
+
+    @property
+    def started(self):
+        return self._futures is not None
+
+    def start(self):
+        if self._futures is None:
+            ex = _compile_executor()
+            self._futures = [ex.submit(compile_programs, [p], self.verbose) for p in self._todo]
+            self._todo = []
+
+    def poll(self):
+        """Called once per execution of the computation."""
+        if self._futures is None:
+            if not self._todo:
+                return True
+            self.calls += 1
+            if self.calls >= self.after_calls:
+                self.start()
+            return False
+        waiting = []
+        for f in self._futures:
+            if not f.done():
+                waiting.append(f)
+            elif not f.cancelled():
+                try:
+                    self.loaded += self.runtime.programs_load(f.result())
+                except Exception as e:       # no hipcc, or it failed: stay on the interpreter
+                    self.error = self.error or str(e)
+        self._futures = waiting
+        return not waiting
+
+    def wait(self, timeout=None):
+        from concurrent.futures import wait as wait_all
+        self.start()
+        wait_all(self._futures, timeout=timeout)
+        return self.poll()
+
+    def cancel(self):
+        self._todo = []
+        for f in self._futures or []:
+            f.cancel()
+
+
+def start_background(runtime, kernels, name, min_elements, after_calls=2, verbose=False):
+    """BackgroundPrograms for the stages of `kernels` (of at least min_elements elements) that run on
+    the interpreter today, or None when there are none."""
+    programs = uncovered_programs(kernels, name, min_elements)
+    if not programs:
+        return None
+    return BackgroundPrograms(runtime, programs, after_calls=after_calls, verbose=verbose)
+
+
+def precompile_graphs(builders, verbose=False):
+    """Compile, without a device, the program libraries of the graphs in `builders` into the
+    cache, so that a later process (on a machine with a GPU, perhaps without hipcc) finds them.
+    builders: iterable of (backend name, build, transformer keyword arguments) with build()
+    returning (results, inputs) of a computation.  Returns the libraries' paths."""
+    from multiprocessing.pool import ThreadPool
+    import ngraph_hip.transformers as ngt
+    todo = {}
+    for backend, build, kwargs in builders:
+        if backend not in ngt.transformer_choices():
+            continue
+        t = ngt.make_transformer_factory(backend, dry_run=True, jit=False, **kwargs)()
+        try:
+            built = build()
+            f = t.computation(built[0], *built[1])
+            t.initialize()
+            kernels = t.kernel_groups[f].kernels
+            for k in kernels:
+                k.bind_buffers()
+            for p in uncovered_programs(kernels, "graph", min_elements=t.jit_min_elements):
+                todo[p[0]] = p
+        finally:
+            t.close()
+    if not todo:
+        return []
+    pool = ThreadPool(max(1, min(8, os.cpu_count() or 2)))      # the work is in hipcc subprocesses
+    try:
+        return pool.map(lambda p: compile_programs([p], verbose=verbose), list(todo.values()))
+    finally:
+        pool.close()

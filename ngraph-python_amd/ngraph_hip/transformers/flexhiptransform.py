@@ -265,9 +265,12 @@ class FlexHipTransformer(HipTransformer):
     max_written_views = 4        # a kernel merges max|mantissa| for at most 4 flex results
 
     def __init__(self, fixed_point=False, flex_verbose=False, collect_flex_data=False,
-                 resident=False, **kwargs):
-        """resident=True keeps scales, statistics and the exponent policy on the device (no
-        host round trip per kernel); False follows the reference's per-kernel read-back."""
+                 resident=True, **kwargs):
+        """resident=True (the default) keeps scales, statistics and the exponent policy on the
+        device: no host round trip per kernel, a record is read back only when the host looks at
+        its tensor.  resident=False follows the reference's loop, which reads max|mantissa| back
+        and runs the policy on the host after every kernel (flexgputransform.py:347-366); both
+        modes leave the same state after every computation."""
         self.flex_manager = HipFlexManager(fixed_point=fixed_point, verbose=flex_verbose,
                                            resident=resident)
         kwargs.setdefault("fuse_moments", False)

@@ -840,13 +840,39 @@ class HipKernelGroup(object):
             if not k.buffers_bound:
                 k.bind_buffers()
         self.assign_cache_hints()
-        if self.transformer.jit:
+        mode = self.transformer.jit
+        if mode is True:
             # compile what would otherwise run on the interpreter (float_ew2.py:1553-1653: the
             # reference compiles every kernel of a computation at this point)
             from ngraph_hip.runtime import jit
             jit.ensure_programs(self.transformer.runtime, self.kernels, self.name,
                                 min_elements=self.transformer.jit_min_elements)
+        elif mode == "auto":
+            # the same for the stages over large tensors, off the launch path: the computation
+            # starts on the interpreter and picks the compiled kernels up when they are ready
+            from ngraph_hip.runtime import jit
+            self._programs = jit.start_background(self.transformer.runtime, self.kernels, self.name,
+                                                  min_elements=self.transformer.jit_auto_min_elements)
         self._bound = True
+
+    _programs = None
+
+    def wait_for_programs(self, timeout=None):
+        """Block until the kernels being compiled for this computation (jit="auto") are loaded;
+        returns the compiler's message if it failed, else None."""
+        if not self._bound:
+            self.bind()
+        if self._programs is None:
+            return None
+        self._programs.wait(timeout)
+        error = self._programs.error
+        self._programs = None
+        return error
+
+    def cancel_programs(self):
+        if self._programs is not None:
+            self._programs.cancel()
+            self._programs = None
 
     def assign_cache_hints(self):
         uses = [k.buffer_uses() for k in self.kernels]
@@ -878,6 +904,8 @@ class HipKernelGroup(object):
     def __call__(self):
         if not self._bound:
             self.bind()
+        if self._programs is not None and self._programs.poll():
+            self._programs = None
         for k in self.kernels:
             self.setup_kernel_execute(k)
             k.execute()
@@ -1438,16 +1466,20 @@ class HipTransformer(ComputationGraphTransformer):
     max_written_views = NGH_MAX_TENSORS      # results one fused kernel may write
 
     def __init__(self, device_id=0, fusion=True, dry_run=False, fuse_moments=None, rng_seed=0, jit=None,
-                 jit_min_elements=4096, **kwargs):
+                 jit_min_elements=4096, jit_auto_min_elements=1 << 22, **kwargs):
         """dry_run=True lowers graphs to kernel specs without a device (no results can be
         read back); it exists so the host-side lowering can be inspected and tested.
         rng_seed keys the random fills (ng.uniform / ng.normal): same seed, same numbers.
-        jit=True compiles, when a computation is first run, kernels for those of its stages
-        (of at least jit_min_elements elements) that the library has no compiled program for;
-        default: the NGH_JIT environment variable, else off."""
+        jit: how stages that the library has no compiled program for get one (the reference
+        compiles every kernel of a computation when it is initialised, float_ew2.py:1553-1653).
+        "auto" (the default unless NGH_JIT says otherwise): stages of at least
+        jit_auto_min_elements elements are compiled in the background and swapped in when
+        ready; True: every stage of at least jit_min_elements elements is compiled before the
+        first launch; False: never."""
         from ngraph_hip.runtime import jit as _jit
-        self.jit = _jit.enabled_by_default() if jit is None else bool(jit)
+        self.jit = _jit.normalize_mode(jit)
         self.jit_min_elements = int(jit_min_elements)
+        self.jit_auto_min_elements = int(jit_auto_min_elements)
         try:
             self.runtime = DryRunRuntime() if dry_run else HipRuntime(device_id)
         except HipLibraryError as e:
@@ -1541,6 +1573,9 @@ class HipTransformer(ComputationGraphTransformer):
         pass
 
     def close(self):
+        for group in getattr(self, "kernel_groups", {}).values():
+            if hasattr(group, "cancel_programs"):
+                group.cancel_programs()
         rt = getattr(self, "runtime", None)
         if rt is not None:
             try:

@@ -134,35 +134,10 @@ def inputs_for(placeholders, seed):
 
 def precompile(verbose=False):
     """Compile the program libraries of every case (no device needed); returns their paths."""
-    import os
-    from multiprocessing.pool import ThreadPool
     from ngraph_hip.runtime import jit
-    todo = {}
-
-    def collect(backend, build, **kwargs):
-        t = ngt.make_transformer_factory(backend, dry_run=True, **kwargs)()
-        try:
-            built = build()
-            f = t.computation(built[0], *built[1])
-            t.initialize()
-            kernels = t.kernel_groups[f].kernels
-            for k in kernels:
-                k.bind_buffers()
-            for p in jit.uncovered_programs(kernels, "case", min_elements=t.jit_min_elements):
-                todo[p[0]] = p
-        finally:
-            t.close()
-
-    for backend, cases in (("hipgpu", FP32_CASES), ("flexhip", [flex_case])):
-        if backend in ngt.transformer_choices():
-            for case in cases:
-                collect(backend, case)
+    builders = [("hipgpu", case, {}) for case in FP32_CASES] + [("flexhip", flex_case, {})]
     for seed in RANDOM_SEEDS:
         for views in (False, True):
-            collect("hipgpu", lambda: random_case(seed, views), jit_min_elements=1)
-    pool = ThreadPool(max(1, min(8, os.cpu_count() or 2)))      # the work is in hipcc subprocesses
-    try:
-        paths = pool.map(lambda p: jit.compile_programs([p], verbose=verbose), list(todo.values()))
-    finally:
-        pool.close()
-    return paths
+            builders.append(("hipgpu", lambda seed=seed, views=views: random_case(seed, views),
+                             {"jit_min_elements": 1}))
+    return jit.precompile_graphs(builders, verbose=verbose)

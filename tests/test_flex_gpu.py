@@ -39,9 +39,11 @@ NG_OPS = {
 }
 
 
-@pytest.fixture
-def flex_unfused():
-    ngt.set_transformer_factory(ngt.make_transformer_factory("flexhip", fusion=False))
+@pytest.fixture(params=[False, True], ids=["host-policy", "device-policy"])
+def flex_unfused(request):
+    """One kernel per op, as the vectors were recorded; under the reference's host-side exponent
+    management and under the device-resident one (the default)."""
+    ngt.set_transformer_factory(ngt.make_transformer_factory("flexhip", fusion=False, resident=request.param))
     yield
     ngt.set_transformer_factory(None)
 

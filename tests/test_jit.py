@@ -67,6 +67,13 @@ def test_program_library_compiles_and_checks_its_caller(tmp_path, monkeypatch):
         t.close()
 
 
+def test_every_case_compiles_for_gfx950():
+    """Every skeleton's generated source compiles (hipcc cross-compiles without a device).  The
+    libraries land in the program cache, where the GPU tests of this file find them."""
+    paths = jit_cases.precompile()
+    assert len(paths) >= 40 and all(os.path.exists(p) for p in paths)
+
+
 def test_missing_compiler_is_reported_as_such(tmp_path, monkeypatch):
     import build_ext
 
@@ -82,15 +89,81 @@ def test_missing_compiler_is_reported_as_such(tmp_path, monkeypatch):
         t.close()
 
 
-def test_jit_is_off_unless_asked_for(monkeypatch):
+def test_default_mode_compiles_large_stages_in_the_background(monkeypatch):
     monkeypatch.delenv("NGH_JIT", raising=False)
     t = ngt.make_transformer_factory("hipgpu", dry_run=True)()
-    assert not t.jit
+    assert t.jit == "auto"
     t.close()
-    monkeypatch.setenv("NGH_JIT", "1")
-    t = ngt.make_transformer_factory("hipgpu", dry_run=True)()
-    assert t.jit
+    for value, mode in (("1", True), ("0", False), ("auto", "auto")):
+        monkeypatch.setenv("NGH_JIT", value)
+        t = ngt.make_transformer_factory("hipgpu", dry_run=True)()
+        assert t.jit == mode and (t.jit is mode or mode == "auto")
+        t.close()
+    t = ngt.make_transformer_factory("hipgpu", dry_run=True, jit=False)()
+    assert t.jit is False
     t.close()
+    with pytest.raises(ValueError):
+        ngt.make_transformer_factory("hipgpu", dry_run=True, jit="sometimes")()
+
+
+def test_background_programs_load_when_ready_and_only_for_large_stages(tmp_path, monkeypatch):
+    """jit="auto": nothing is compiled for a small computation; for a large one the libraries are
+    compiled by a worker thread and loaded by the kernel group once they exist; a second
+    transformer finds them in the cache and loads them when its kernels are bound."""
+    monkeypatch.setenv("NGH_PROGRAM_CACHE", str(tmp_path))
+    results, inputs = jit_cases.case_elementwise()            # 512 x 1024 elements
+    t = ngt.make_transformer_factory("hipgpu", dry_run=True, jit="auto")()
+    try:
+        f = t.computation(results, *inputs)
+        t.initialize()
+        group = t.kernel_groups[f]
+        group.bind()
+        assert group._programs is None and not os.listdir(str(tmp_path))
+    finally:
+        t.close()
+    for expect_thread in (True, False):
+        t = ngt.make_transformer_factory("hipgpu", dry_run=True, jit="auto", jit_auto_min_elements=1 << 18)()
+        try:
+            results, inputs = jit_cases.case_elementwise()
+            f = t.computation(results, *inputs)
+            t.initialize()
+            group = t.kernel_groups[f]
+            group.bind()
+            assert (group._programs is not None) and not group._programs.started
+            assert bool(group._programs._todo) == expect_thread
+            group()                            # first run: nothing is compiled for it
+            if expect_thread:
+                assert not group._programs.started and not os.listdir(str(tmp_path))
+                group()                        # second run: the compile jobs start
+                assert group._programs.started
+            assert group.wait_for_programs(timeout=300) is None
+            assert group._programs is None
+            libs = [n for n in os.listdir(str(tmp_path)) if n.endswith(".so")]
+            assert len(libs) == 1 and t.runtime.program_libraries == [os.path.join(str(tmp_path), libs[0])]
+        finally:
+            t.close()
+
+
+def test_background_compilation_without_a_compiler_stays_on_the_interpreter(tmp_path, monkeypatch):
+    import build_ext
+
+    def no_hipcc():
+        raise RuntimeError("hipcc not found")
+    monkeypatch.setenv("NGH_PROGRAM_CACHE", str(tmp_path))
+    monkeypatch.setattr(build_ext, "find_hipcc", no_hipcc)
+    t = ngt.make_transformer_factory("hipgpu", dry_run=True, jit="auto", jit_auto_min_elements=1 << 18)()
+    try:
+        results, inputs = jit_cases.case_elementwise()
+        f = t.computation(results, *inputs)
+        t.initialize()
+        group = t.kernel_groups[f]
+        group()                                              # runs (here: records) its launches
+        error = group.wait_for_programs(timeout=60)
+        assert error is not None and "needs hipcc" in error
+        assert t.runtime.program_libraries == []
+        group()
+    finally:
+        t.close()
 
 
 def _run(backend, case, seed, **kwargs):
@@ -102,6 +175,32 @@ def _run(backend, case, seed, **kwargs):
         groups = getattr(t, "kernel_groups", None)
         names = [d for k in groups[f].kernels for ds in k.describe() for d in ds] if groups else []
         return out, names
+    finally:
+        t.close()
+
+
+@pytest.mark.gpu
+def test_auto_mode_swaps_compiled_kernels_in_without_changing_results(tmp_path, monkeypatch):
+    """The default mode on the device: the first call runs on the interpreter while hipcc works
+    (an empty cache, so this test does compile one program on the spot), later calls on the
+    compiled kernel, and both give the same bits."""
+    monkeypatch.setenv("NGH_PROGRAM_CACHE", str(tmp_path))
+    t = ngt.make_transformer_factory("hipgpu", jit="auto", jit_auto_min_elements=1 << 18)()
+    try:
+        results, inputs = jit_cases.case_elementwise()
+        f = t.computation(results, *inputs)
+        vals = jit_cases.inputs_for(inputs, 3)
+        group_names = lambda: [d for k in t.kernel_groups[f].kernels for ds in k.describe() for d in ds]
+        first = [np.array(r).copy() for r in f(*vals)]
+        before = group_names()
+        assert t.kernel_groups[f].wait_for_programs(timeout=300) is None
+        second = [np.array(r).copy() for r in f(*vals)]
+        after = group_names()
+        if default_kernel_choice():
+            assert any("interp" in d for d in before) or any("special:jit_" in d for d in before), before
+            assert all(d.startswith("special:jit_") for d in after), after
+        for a, b in zip(first, second):
+            np.testing.assert_array_equal(a, b)
     finally:
         t.close()
 
