@@ -471,7 +471,7 @@ __device__ __forceinline__ void red_emit(const KArgs& k, int slot, Acc a, long l
     } else {
         const size_t w = ((size_t)slot * n_seg + seg) * n_out + out;
         ws.val[w] = a.v;
-        ws.idx[w] = a.i;
+        if (k.ops[k.op_end - k.n_red + slot].opcode >= NGH_OP_RED_ARGMAX) ws.idx[w] = a.i;   // only argmax / argmin carry one
     }
 }
 
@@ -557,7 +557,11 @@ __global__ __launch_bounds__(kBlock) void red_col_interp_kernel(const KArgs k, u
         }
     }
     const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const unsigned tx = lane & (TX - 1), ry = lane / TX, rows_per_wave = 64 / TX;
+    // TX == kBlock: the whole workgroup lies along the columns (kBlock * V consecutive outputs per
+    // row step: the longest contiguous runs this layout allows) and every lane owns its outputs
+    const bool wide = TX == kBlock;
+    const unsigned tx = wide ? threadIdx.x : (lane & (TX - 1)), ry = wide ? 0 : lane / TX;
+    const unsigned rows_per_wave = wide ? 1 : 64 / TX;
     unsigned b = blockIdx.x;
     const unsigned seg = b % n_seg;  b /= n_seg;
     const unsigned bx = b % n_bx;    b /= n_bx;
@@ -566,11 +570,27 @@ __global__ __launch_bounds__(kBlock) void red_col_interp_kernel(const KArgs k, u
     const unsigned i2 = (bx * TX + tx) * V;
     const unsigned r_begin = seg * seg_rows;
     const unsigned r_end = min((unsigned)k.shape[0], r_begin + seg_rows);
+    const unsigned n_out = (unsigned)k.shape[1] * d2;
+    if (wide) {
+        if (i2 < d2) {
+            for (unsigned r = r_begin; r < r_end; ++r) run_ops<V, 2>(k, rf, ex, VecAt<V>{r, i1, i2});
+            for (int s = 0; s < k.n_red; ++s) {
+#pragma unroll
+                for (int v = 0; v < V; ++v) {
+                    Acc a;
+                    a.v = ex.getf(ex_accv(k, s, V, v));
+                    a.i = ex.geti(ex_acci(k, s, V, v));
+                    red_emit(k, s, a, 0, i1, i2 + v, i1 * d2 + i2 + v, n_out, seg, n_seg, ws);
+                }
+            }
+        }
+        stats_epilogue(k, ex);
+        return;
+    }
     if (i2 < d2)
         for (unsigned r = r_begin + wave * rows_per_wave + ry; r < r_end; r += kWaves * rows_per_wave)
             run_ops<V, 2>(k, rf, ex, VecAt<V>{r, i1, i2});
 
-    const unsigned n_out = (unsigned)k.shape[1] * d2;
     for (int s = 0; s < k.n_red; ++s) {
         const int opc = red_opcode(k, s);
 #pragma unroll
@@ -645,22 +665,39 @@ __device__ __forceinline__ void red_finish_coords(const KArgs& k, unsigned out, 
     }
 }
 
+// A workgroup takes 64 outputs (one per lane: partial results of consecutive outputs are
+// consecutive in the workspace) and its four wavefronts a quarter of the segments each, in
+// segment order; the quarters meet in shared memory and are merged in wavefront order.
 __global__ __launch_bounds__(kBlock) void red_finish_kernel(const KArgs k, unsigned n_out,
                                                             unsigned n_seg, int row_mode, RedWs ws) {
-    const unsigned out = blockIdx.x * kBlock + threadIdx.x;
-    if (out >= n_out) return;
-    long long o0, o1, o2;
-    red_finish_coords(k, out, row_mode, o0, o1, o2);
+    __shared__ Acc sh[kWaves][64];
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned out = blockIdx.x * 64 + lane;
+    const unsigned per_wave = (n_seg + kWaves - 1) / kWaves;
+    const unsigned g_begin = min(n_seg, wave * per_wave), g_end = min(n_seg, g_begin + per_wave);
+    long long o0 = 0, o1 = 0, o2 = 0;
+    if (out < n_out) red_finish_coords(k, out, row_mode, o0, o1, o2);
     for (int s = 0; s < k.n_red; ++s) {
         const int opc = red_opcode(k, s);
+        const bool with_index = opc >= NGH_OP_RED_ARGMAX;
         Acc a = acc_init(opc);
-        for (unsigned g = 0; g < n_seg; ++g) {
-            const size_t w = ((size_t)s * n_seg + g) * n_out + out;
-            Acc b; b.v = ws.val[w]; b.i = ws.idx[w];
-            a = acc_merge(opc, a, b);
+        if (out < n_out) {
+#pragma unroll 4
+            for (unsigned g = g_begin; g < g_end; ++g) {
+                const size_t w = ((size_t)s * n_seg + g) * n_out + out;
+                Acc b; b.v = ws.val[w]; b.i = with_index ? ws.idx[w] : 0;
+                a = acc_merge(opc, a, b);
+            }
         }
-        RedWs none{nullptr, nullptr};
-        red_emit(k, s, a, o0, o1, o2, out, n_out, 0, 1, none);
+        sh[wave][lane] = a;
+        __syncthreads();
+        if (wave == 0 && out < n_out) {
+            // (a wavefront that had no segments holds the reduction's identity)
+            for (int w = 1; w < kWaves; ++w) a = acc_merge(opc, a, sh[w][lane]);
+            RedWs none{nullptr, nullptr};
+            red_emit(k, s, a, o0, o1, o2, out, n_out, 0, 1, none);
+        }
+        __syncthreads();
     }
 }
 
@@ -674,9 +711,10 @@ __global__ __launch_bounds__(kBlock) void red_finish_wave_kernel(const KArgs k, 
     for (int s = 0; s < k.n_red; ++s) {
         const int opc = red_opcode(k, s);
         Acc a = acc_init(opc);
+        const bool with_index = opc >= NGH_OP_RED_ARGMAX;
         for (unsigned g = lane; g < n_seg; g += 64) {
             const size_t w = ((size_t)s * n_seg + g) * n_out + out;
-            Acc b; b.v = ws.val[w]; b.i = ws.idx[w];
+            Acc b; b.v = ws.val[w]; b.i = with_index ? ws.idx[w] : 0;
             a = acc_merge(opc, a, b);
         }
 #pragma unroll

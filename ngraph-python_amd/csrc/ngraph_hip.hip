@@ -117,7 +117,8 @@ struct ngh_context {
     unsigned    stat_ws_blocks = 0;  // capacity per statistics slot
     int         ew_blocks_per_cu = 64;
     int         force_interp = 0;    // never pick a specialised kernel
-    int         red_wgs_per_cu = 8;  // workgroups per CU a split reduction aims for
+    int         red_wgs_per_cu = 8;  // workgroups per CU a split reduction along the contiguous axis aims for
+    int         red_col_wgs_per_cu = 2;  // ... and one across it
     int         no_tiles = 0;        // never use the LDS-tiled elementwise skeleton
     int         flex_self_managed = 2;  // ngh_launch_fused_flex: 0 = prepare / kernel / update launches,
                                      // 1 = policy at the end of the kernel, 2 = statistics deferred to the next user
@@ -531,10 +532,17 @@ int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage,
         const long long col_chunks = (P.k.shape[2] + P.V - 1) / P.V;
         P.tx = 1;
         while (P.tx < 64 && (long long)P.tx < col_chunks) P.tx <<= 1;
+        // Column reductions run best on few, long-lived workgroups (measured with a cold cache on a
+        // 268 MB matrix: one or two per compute unit reach 6.2-6.7 TB/s, eight 4.8), each walking
+        // down its columns with several rows in flight.  With many columns the whole workgroup
+        // lies along them: kBlock * V consecutive outputs per row step, every lane its own outputs.
+        const long long col_target = (ctx ? ctx->cus * ctx->red_col_wgs_per_cu : 256 * 2);
+        const bool wide = col_chunks >= kBlock && R * n_out > kSmallReduction && R >= 64;
+        if (wide) P.tx = kBlock;
         P.n_bx = (unsigned)((col_chunks + P.tx - 1) / P.tx);
-        const long long rows_per_pass = (long long)kWaves * (64 / P.tx);
+        const long long rows_per_pass = wide ? 1 : (long long)kWaves * (64 / P.tx);
         const long long base_wgs = (long long)P.n_bx * P.k.shape[1];
-        long long seg = std::max<long long>(1, target_wgs / std::max<long long>(1, base_wgs));
+        long long seg = std::max<long long>(1, col_target / std::max<long long>(1, base_wgs));
         seg = std::min<long long>(seg, std::max<long long>(1, R / (rows_per_pass * 8)));
         seg = std::min<long long>(seg, 4096);
         // a small problem is bound by launches: a second one (the fold of the segments) costs more
@@ -847,11 +855,12 @@ int launch_interp(ngh_context* ctx, Plan& P) {
     HIP_TRY(hipGetLastError());
     if (k.n_stat_slots) NGH_TRY(stat_fold(ctx, k, red_blocks));
     if (P.n_seg > 1) {
-        if (P.n_seg >= 32)
+        // few outputs with many segments each: a wavefront per output; else 64 outputs a workgroup
+        if (P.n_seg >= 32 && P.n_out < 1024)
             hipLaunchKernelGGL(red_finish_wave_kernel, dim3((P.n_out + kWaves - 1) / kWaves), dim3(kBlock), 0, ctx->stream,
                                k, P.n_out, P.n_seg, P.family == F_RED_ROW ? 1 : 0, ws);
         else
-            hipLaunchKernelGGL(red_finish_kernel, dim3((P.n_out + kBlock - 1) / kBlock), dim3(kBlock), 0, ctx->stream,
+            hipLaunchKernelGGL(red_finish_kernel, dim3((P.n_out + 63) / 64), dim3(kBlock), 0, ctx->stream,
                                k, P.n_out, P.n_seg, P.family == F_RED_ROW ? 1 : 0, ws);
         HIP_TRY(hipGetLastError());
     }
@@ -927,6 +936,7 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->flex_lazy_blocks_per_cu = std::max(1, env_int("NGH_FLEX_LAZY_BLOCKS_PER_CU", 6));
     ctx->no_tiles = env_int("NGH_NO_TILES", 0);
     ctx->red_wgs_per_cu = std::max(1, env_int("NGH_RED_WGS_PER_CU", 8));
+    ctx->red_col_wgs_per_cu = std::max(1, env_int("NGH_RED_COL_WGS_PER_CU", 2));
     ctx->cache_policy = env_int("NGH_CACHE_POLICY", -1);
     ctx->stream_bytes = (long long)env_int("NGH_STREAM_MIB", 192) << 20;
     ctx->moments_wgs_per_cu = std::max(1, env_int("NGH_MOMENTS_WGS_PER_CU", 8));

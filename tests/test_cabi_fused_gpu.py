@@ -293,7 +293,9 @@ def test_every_binary_op(hip_runtime, name):
 
 @pytest.mark.parametrize("name", ["sum", "prod", "max", "min", "argmax", "argmin"])
 @pytest.mark.parametrize("shape,layout", [((64, 10), "row"), ((64, 10), "col"), ((5000, 3), "row"),
-                                          ((300, 700), "col"), ((1, 9), "row"), ((40000, 2), "col")])
+                                          ((300, 700), "col"), ((1, 9), "row"), ((40000, 2), "col"),
+                                          # many columns: the whole workgroup lies along them
+                                          ((300, 4096), "col"), ((37, 4100), "col"), ((2000, 1027), "col")])
 def test_every_reduction(hip_runtime, name, shape, layout):
     """Reduce axis 0 of an [R, A] view; 'row' = R contiguous in memory, 'col' = A contiguous."""
     rt = hip_runtime
@@ -333,7 +335,8 @@ def test_every_reduction(hip_runtime, name, shape, layout):
     out_d.free()
 
 
-@pytest.mark.parametrize("shape,layout", [((40000, 2), "col"), ((200704, 4), "row"), ((3000, 300), "col")])
+@pytest.mark.parametrize("shape,layout", [((40000, 2), "col"), ((200704, 4), "row"), ((3000, 300), "col"),
+                                          ((3000, 2048), "col")])
 def test_signed_sum_against_float64(hip_runtime, shape, layout):
     """A cancelling sum: error must stay within 1e-6 of sum(|x|), checked against float64."""
     rt = hip_runtime
@@ -354,6 +357,43 @@ def test_signed_sum_against_float64(hip_runtime, shape, layout):
     assert np.all(np.abs(out_d.get().astype(np.float64) - truth) <= bound)
     x_d.free()
     out_d.free()
+
+
+@pytest.mark.parametrize("R,A", [(512, 2048), (100, 4100), (64, 1024), (1500, 1027)])
+def test_column_reductions_with_elementwise_stores_over_many_columns(hip_runtime, R, A):
+    """z = tanh(x*y + 0.5) stored, max and argmax of z and sum of x*x down the columns, in one
+    stage over [R, A] with A contiguous: every lane of the workgroup owns its columns, rows are
+    split into segments, and the plan reports it (family 2)."""
+    from ngraph_hip.runtime.hiplib import plan_fused
+    rt = hip_runtime
+    rs = np.random.RandomState(R + A)
+    x, y = rs.normal(0, 1, (R, A)).astype(f32), rs.normal(0, 1, (R, A)).astype(f32)
+    x[R // 2] = x[R // 3]
+    y[R // 2] = y[R // 3]                                  # ties: the lowest index wins
+    x_d, y_d, z_d = rt.array(x), rt.array(y), rt.empty((R, A))
+    mx_d, am_d, ss_d = rt.empty((A,)), rt.empty((A,), NGH_I32), rt.empty((A,))
+    sb = FusedSpecBuilder([R, A])
+    tx, ty, tz = (sb.tensor(d.ptr, [A, 1]) for d in (x_d, y_d, z_d))
+    tmx, tss = sb.tensor(mx_d.ptr, [0, 1]), sb.tensor(ss_d.ptr, [0, 1])
+    tam = sb.tensor(am_d.ptr, [0, 1], NGH_I32)
+    rx, ry = sb.load(tx), sb.load(ty)
+    z = sb.unary("tanh", sb.binary("add", sb.binary("mul", rx, ry), sb.constant(0.5)))
+    sb.store(tz, z)
+    sq = sb.unary("sqr", rx)
+    sb.reduce("max", z, tmx)
+    sb.reduce("argmax", z, tam)
+    sb.reduce("sum", sq, tss)
+    spec = sb.build()
+    assert plan_fused(spec)["family"] == 2
+    rt.launch_fused(spec)
+    z_w = numpy_ops.unary("tanh", numpy_ops.binary("add", numpy_ops.binary("mul", x, y), f32(0.5)))
+    z_g = z_d.get()
+    np.testing.assert_allclose(z_g, z_w, rtol=RTOL, atol=ATOL)
+    np.testing.assert_array_equal(mx_d.get(), z_g.max(axis=0))
+    np.testing.assert_array_equal(am_d.get(), z_g.argmax(axis=0))
+    np.testing.assert_allclose(ss_d.get(), (x.astype(np.float64) ** 2).sum(axis=0), rtol=RTOL, atol=ATOL)
+    for d in (x_d, y_d, z_d, mx_d, am_d, ss_d):
+        d.free()
 
 
 # ------------------------------------------------------------------ one-pass moments
