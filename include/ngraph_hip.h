@@ -57,7 +57,13 @@ extern "C" {
 #define NGH_F16     3          /* IEEE half in memory, float in registers   */
 /* Integer storage: converted to float on load; a store converts toward zero and
  * saturates at the type's range (the device conversion the reference's generated
- * "(type)reg" assignment compiles to).  Values are exact up to 2^24.            */
+ * "(type)reg" assignment compiles to).  Registers are fp32, so integer values are exact up to
+ * 2^24 (the reference keeps int32 / uint32 operands in integer registers, float_ew2.py:615-641).
+ * Where an index could exceed that, the library keeps it an integer or refuses the spec with
+ * NGH_E_UNSUPPORTED instead of losing bits: argmax / argmin into NGH_I32 / NGH_U32 storage
+ * store the integer index itself (over more than 2^24 elements any other result type is
+ * refused); NGH_OP_TAKE from a table of more than 2^24 entries along the looked-up axis and
+ * NGH_OP_IOTA along an axis longer than 2^24 are refused.                              */
 #define NGH_U32     4          /* uint32                                    */
 #define NGH_I16     5          /* int16 (plain integers, no scale)          */
 #define NGH_I8      6          /* int8                                      */
@@ -268,6 +274,18 @@ int  ngh_moments_f32(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t
  * array: calls that overlap there (two contexts, two host threads) race.                   */
 int  ngh_moments_f32_noalloc(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t R, int64_t row_stride,
                              float* dev_mean, float* dev_var, float* dev_rstd, float eps, uint32_t x_cache_hint);
+
+/* ---- float -> flex16 converter: replaces `convert` (gpu/flex_conv.py:745-791,
+ *      _prepare_convert_kernel :734-740), which turns the raw fp32 (or fp16) output of a dense
+ *      kernel into a flex tensor.  dev_out[i] = (int16)trunc(dev_in[i] * scale), toward zero;
+ *      values outside the int16 range (undefined in the reference's cast) saturate at
+ *      -32768 / 32767, NaN gives 0.  in_dtype is NGH_F32 or NGH_F16.  max |mantissa| is merged
+ *      into *dev_stats with an atomic max when dev_stats is not NULL (as int32: -32768 counts
+ *      as 32768).  When dev_scale is not NULL the multiplier is 1 / *dev_scale instead of
+ *      `scale`: the destination tensor's scale read on the device, for exponent management
+ *      that lives there.                                                               */
+int  ngh_convert_to_flex16(ngh_context* ctx, int16_t* dev_out, const void* dev_in, int32_t in_dtype, int64_t n,
+                           float scale, const float* dev_scale, int32_t* dev_stats);
 
 /* How stage `stage` would be launched, without a device (host-side tooling and
  * tests): out8 = {kernel family (0 streaming, 1 reduce along the contiguous axis,

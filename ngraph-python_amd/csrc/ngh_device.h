@@ -65,6 +65,7 @@ struct KArgs {
                                     // the value is the number of compute units
     FlexLazySlot lazy[4];
     int          lazy_blocks_per_cu;
+    int          ordered_arrival;   // last-arrival hand-offs use release / acquire tickets
     KTensor   t[NGH_MAX_TENSORS];
     float     consts[NGH_MAX_CONSTS];
     ngh_op    ops[NGH_MAX_OPS];
@@ -203,9 +204,8 @@ __device__ __forceinline__ float rng_normal(unsigned b0, unsigned b1) {
 
 // the fill rule: int(value / scale) cut toward zero, clipped (tensor_ops.py:690-707)
 __device__ __forceinline__ int flex_quantize_trunc(float v) {
-    v = truncf(v);
-    v = fminf(fmaxf(v, -32768.0f), 32767.0f);
-    return (v != v) ? 0 : (int)v;
+    const float r = fminf(fmaxf(truncf(v), -32768.0f), 32767.0f);   // (fmaxf drops a NaN: tested on v below)
+    return (v != v) ? 0 : (int)r;
 }
 
 __device__ __forceinline__ int iabs(int x) { return x < 0 ? -x : x; }

@@ -194,7 +194,8 @@ constexpr int kFlexGroupMaxWords = 4 * kFlexGroups * kFlexPad;
 template <int NS>
 __device__ __forceinline__ void flex_epilogue(ngh_flex_state* const (&state)[4], const int (&in_place)[4],
                                               int count, unsigned* tickets, int* group_max,
-                                              const int (&fmax)[4], int (*lds)[4] /* [NS][waves] */) {
+                                              const int (&fmax)[4], int (*lds)[4] /* [NS][waves] */,
+                                              int ordered) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int m[NS];
 #pragma unroll
@@ -217,16 +218,25 @@ __device__ __forceinline__ void flex_epilogue(ngh_flex_state* const (&state)[4],
             dep |= (unsigned)__hip_atomic_fetch_max(group_max + (s * kFlexGroups + g) * kFlexPad, bm,
                                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+        // `ordered`: the two tickets are release operations and the last arrival issues an acquire
+        // fence, as the memory model asks of a hand-off between workgroups; else they are relaxed and ordered behind the maxima by a
+        // data dependency alone, which the hardware honours (see moments_kernel)
         unsigned one = 1u;
         asm volatile("" : "+v"(one) : "v"(dep));          // the ticket waits for the maxima
         const unsigned members = (gridDim.x - g + kFlexGroups - 1) / kFlexGroups;
-        const unsigned t = __hip_atomic_fetch_add(tickets + g * kFlexPad, one, __ATOMIC_RELAXED,
-                                                  __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned t = ordered ? __hip_atomic_fetch_add(tickets + g * kFlexPad, one, __ATOMIC_RELEASE,
+                                                            __HIP_MEMORY_SCOPE_AGENT)
+                                   : __hip_atomic_fetch_add(tickets + g * kFlexPad, one, __ATOMIC_RELAXED,
+                                                            __HIP_MEMORY_SCOPE_AGENT);
         if (t == members - 1) {
             __hip_atomic_store(tickets + g * kFlexPad, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const unsigned t2 = __hip_atomic_fetch_add(tickets + kFlexGroups * kFlexPad, 1u, __ATOMIC_RELAXED,
-                                                       __HIP_MEMORY_SCOPE_AGENT);
+            if (ordered) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // the group's maxima are in
+            const unsigned t2 = ordered ? __hip_atomic_fetch_add(tickets + kFlexGroups * kFlexPad, 1u, __ATOMIC_RELEASE,
+                                                                 __HIP_MEMORY_SCOPE_AGENT)
+                                        : __hip_atomic_fetch_add(tickets + kFlexGroups * kFlexPad, 1u, __ATOMIC_RELAXED,
+                                                                 __HIP_MEMORY_SCOPE_AGENT);
             if (t2 == groups - 1) {
+                if (ordered) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // every group's maxima are in
                 __hip_atomic_store(tickets + kFlexGroups * kFlexPad, 0u, __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
                 last = 1;

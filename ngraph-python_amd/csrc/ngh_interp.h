@@ -460,10 +460,13 @@ __device__ __forceinline__ void red_emit(const KArgs& k, int slot, Acc a, long l
         const KTensor& t = k.t[k.red_out[slot]];
         const long long off = o0 * t.s[0] + o1 * t.s[1] + o2 * t.s[2];
         const float sc = (t.dtype == NGH_FLEX16) ? 1.0f / tensor_scale(t) : 1.0f;
-        const float result = acc_result(k.ops[k.op_end - k.n_red + slot].opcode, a);
+        const int opc = k.ops[k.op_end - k.n_red + slot].opcode;
+        const float result = acc_result(opc, a);
         int fmax = 0;
         if (k.probe) {
             if (t.dtype == NGH_FLEX16) fmax = probe_bits(result);
+        } else if (opc >= NGH_OP_RED_ARGMAX && (t.dtype == NGH_I32 || t.dtype == NGH_U32)) {
+            reinterpret_cast<int*>(t.p)[off] = a.i;       // an index into integer storage: no trip through fp32
         } else {
             store1(t, off, result, sc, fmax);
         }

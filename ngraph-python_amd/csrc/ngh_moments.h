@@ -39,7 +39,7 @@ template <bool NT>
 __global__ __launch_bounds__(kMomBlock) void moments_kernel(
     const float* __restrict__ x, long long row_stride, unsigned R, unsigned R4, unsigned n_seg,
     unsigned seg_chunks, float2* __restrict__ partial, unsigned* __restrict__ row_tickets,
-    float* __restrict__ mean, float* __restrict__ var, float* __restrict__ rstd, float eps) {
+    float* __restrict__ mean, float* __restrict__ var, float* __restrict__ rstd, float eps, int ordered) {
     const unsigned row = blockIdx.x / n_seg;
     const unsigned seg = blockIdx.x - row * n_seg;
     const float* xr = x + (long long)row * row_stride;
@@ -82,19 +82,31 @@ __global__ __launch_bounds__(kMomBlock) void moments_kernel(
     if (threadIdx.x == 0) {
         float2 a = sh[0];
         for (int w = 1; w < kMomBlock / 64; ++w) { a.x += sh[w].x; a.y += sh[w].y; }
-        // Publish the partial and take a ticket with device-scope read-modify-write atomics
-        // only: they are performed at the device's point of coherence, and the ticket is
-        // issued after the exchange has returned (its increment depends on the returned
-        // value), so whoever draws the last ticket can read every partial of the row there.
-        // A release fence instead would write back the whole L2 once per workgroup.
         const unsigned long long bits =
             (unsigned long long)__float_as_uint(a.x) | ((unsigned long long)__float_as_uint(a.y) << 32);
-        const unsigned long long old = __hip_atomic_exchange(
-            reinterpret_cast<unsigned long long*>(partial) + blockIdx.x, bits, __ATOMIC_RELAXED,
-            __HIP_MEMORY_SCOPE_AGENT);
-        unsigned one = 1u;
-        asm volatile("" : "+v"(one) : "v"((unsigned)old));   // orders the ticket after the exchange
-        ticket = __hip_atomic_fetch_add(row_tickets + row, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (ordered) {
+            // By the memory model: the partial is stored, the ticket is a release read-modify-write
+            // at device scope, and whoever draws the last ticket issues an acquire fence: it has
+            // then acquired every earlier increment's release (a release sequence runs through
+            // the increments), so the partials of the row are visible to it.
+            __hip_atomic_store(reinterpret_cast<unsigned long long*>(partial) + blockIdx.x, bits, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+            ticket = __hip_atomic_fetch_add(row_tickets + row, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+            if (ticket == n_seg - 1) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // only the merger acquires
+        } else {
+            // Without fences, relying on the hardware: publish the partial and take the ticket
+            // with device-scope read-modify-write atomics only.  They are performed at the
+            // device's point of coherence, and the ticket is issued after the exchange has
+            // returned (its increment depends on the returned value), so whoever draws the last
+            // ticket can read every partial of the row there.  The language's memory model does
+            // not promise this ordering; gfx950 delivers it.
+            const unsigned long long old = __hip_atomic_exchange(
+                reinterpret_cast<unsigned long long*>(partial) + blockIdx.x, bits, __ATOMIC_RELAXED,
+                __HIP_MEMORY_SCOPE_AGENT);
+            unsigned one = 1u;
+            asm volatile("" : "+v"(one) : "v"((unsigned)old));   // orders the ticket after the exchange
+            ticket = __hip_atomic_fetch_add(row_tickets + row, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
     __syncthreads();
     if (ticket != n_seg - 1 || threadIdx.x >= 64) return;

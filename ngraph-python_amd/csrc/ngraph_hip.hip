@@ -19,6 +19,7 @@
 #include "ngh_table.h"
 #include "ngh_moments.h"
 #include "ngh_flex.h"
+#include "ngh_convert.h"
 
 using namespace ngh;
 
@@ -126,6 +127,9 @@ struct ngh_context {
                                      // loads, bit 1 = non-temporal stores in pre-built kernels
     long long   stream_bytes = 192ll << 20;  // hints act on stages touching at least this much memory
     int         moments_wgs_per_cu = 8;
+    int         ordered_arrival = 0; // last-arrival hand-offs: 1 = release tickets + acquire fence (what the memory
+                                     // model asks for; measured 2.6x slower on the moments kernel: a device-scope
+                                     // release per workgroup), 0 = relaxed tickets behind a data dependency
     int         flex_lazy_blocks_per_cu = 6;  // grid of a launch with deferred statistics
     char        name[256] = "";
     uint64_t    total_bytes = 0;
@@ -138,6 +142,7 @@ struct ngh_context {
 namespace {
 
 constexpr long long kMaxStageElems = 1LL << 33;
+constexpr unsigned kExactIntegers = 1u << 24;     // integers an fp32 register holds exactly
 constexpr long long kSmallReduction = 1LL << 19;   // elements: below this a reduction stays one launch
 constexpr int kFlexMaxLazyRecords = 4096;   // tables up to this size get pages and words for deferred statistics
 
@@ -210,9 +215,15 @@ int validate(const ngh_fused_spec* sp) {
                     return fail(NGH_E_INVALID, "op %d: bad TAKE", pc);
                 if (sp->tensors[t].take_extent == 0)
                     return fail(NGH_E_INVALID, "op %d: TAKE from tensor %d without take_extent", pc, t);
+                if (sp->tensors[t].take_extent > kExactIntegers)
+                    return fail(NGH_E_UNSUPPORTED, "op %d: TAKE along an axis of %u entries: indices travel in fp32 "
+                                "registers, exact up to 2^24", pc, sp->tensors[t].take_extent);
                 defined[o.dst] = true;
             } else if (opc == NGH_OP_IOTA) {
                 if (o.a >= NGH_MAX_AXES || !reg_ok(o.dst)) return fail(NGH_E_INVALID, "op %d: bad IOTA", pc);
+                if (sp->shape[o.a] > (long long)kExactIntegers)
+                    return fail(NGH_E_UNSUPPORTED, "op %d: IOTA along an axis of %lld: index values travel in fp32 "
+                                "registers, exact up to 2^24", pc, (long long)sp->shape[o.a]);
                 defined[o.dst] = true;
             } else if (is_unary(opc)) {
                 if (!need(o.a) || !reg_ok(o.dst)) return fail(NGH_E_INVALID, "op %d: unary operand undefined", pc);
@@ -227,6 +238,12 @@ int validate(const ngh_fused_spec* sp) {
                 const int ot = S.red_out[n_red_seen];
                 if (ot < 0 || ot >= sp->n_tensors) return fail(NGH_E_INVALID, "stage %d: red_out[%d]", s, n_red_seen);
                 const ngh_tensor& T = sp->tensors[ot];
+                // argmax / argmin store their index as an integer into integer storage; through any
+                // other storage type it passes through fp32
+                if ((opc == NGH_OP_RED_ARGMAX || opc == NGH_OP_RED_ARGMIN) && sp->shape[0] > (long long)kExactIntegers &&
+                    T.dtype != NGH_I32 && T.dtype != NGH_U32)
+                    return fail(NGH_E_UNSUPPORTED, "stage %d: argmax/argmin over %lld elements needs an int32 or "
+                                "uint32 result (fp32 is exact up to 2^24)", s, (long long)sp->shape[0]);
                 if (T.strides[0] != 0 && sp->shape[0] > 1)
                     return fail(NGH_E_INVALID, "stage %d: reduction output %d must have stride 0 on axis 0", s, ot);
                 for (int a = 1; a < NGH_MAX_AXES; ++a)
@@ -536,8 +553,11 @@ int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage,
         // 268 MB matrix: one or two per compute unit reach 6.2-6.7 TB/s, eight 4.8), each walking
         // down its columns with several rows in flight.  With many columns the whole workgroup
         // lies along them: kBlock * V consecutive outputs per row step, every lane its own outputs.
-        const long long col_target = (ctx ? ctx->cus * ctx->red_col_wgs_per_cu : 256 * 2);
-        const bool wide = col_chunks >= kBlock && R * n_out > kSmallReduction && R >= 64;
+        // (The interpreter is the opposite case: it hides its per-op cost behind many resident
+        // wavefronts, so a stage without a compiled program keeps the large grid.)
+        const bool compiled = !(ctx && ctx->force_interp) && !P.k.probe && match_special(F_RED_COL, P.V, P.k, 0) >= 0;
+        const long long col_target = compiled ? (ctx ? ctx->cus * ctx->red_col_wgs_per_cu : 256 * 2) : target_wgs;
+        const bool wide = compiled && col_chunks >= kBlock && R * n_out > kSmallReduction && R >= 64;
         if (wide) P.tx = kBlock;
         P.n_bx = (unsigned)((col_chunks + P.tx - 1) / P.tx);
         const long long rows_per_pass = wide ? 1 : (long long)kWaves * (64 / P.tx);
@@ -702,8 +722,7 @@ int ensure_tickets(ngh_context* ctx, size_t n) {
 // The last (length % 4) elements of a contiguous 1-D stage, one element per lane.
 // Point the stage's statistics slots at per-workgroup scratch for a launch of `blocks`
 // workgroups, and, after the launch, fold the scratch into each tensor's statistics word.
-int stat_scratch(ngh_context* ctx, KArgs& k, unsigned blocks) {
-    if (k.n_stat_slots == 0) return NGH_OK;
+int ensure_stat_ws(ngh_context* ctx, unsigned blocks) {
     if (blocks > ctx->stat_ws_blocks) {
         if (ctx->stat_ws) {
             HIP_TRY(hipStreamSynchronize(ctx->stream));
@@ -714,6 +733,12 @@ int stat_scratch(ngh_context* ctx, KArgs& k, unsigned blocks) {
         HIP_TRY(hipMalloc((void**)&ctx->stat_ws, (size_t)cap * 4 * sizeof(int)));
         ctx->stat_ws_blocks = cap;
     }
+    return NGH_OK;
+}
+
+int stat_scratch(ngh_context* ctx, KArgs& k, unsigned blocks) {
+    if (k.n_stat_slots == 0) return NGH_OK;
+    NGH_TRY(ensure_stat_ws(ctx, blocks));
     for (int s = 0; s < 4; ++s) k.stat_partial[s] = ctx->stat_ws + (size_t)s * ctx->stat_ws_blocks;
     return NGH_OK;
 }
@@ -940,6 +965,9 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->cache_policy = env_int("NGH_CACHE_POLICY", -1);
     ctx->stream_bytes = (long long)env_int("NGH_STREAM_MIB", 192) << 20;
     ctx->moments_wgs_per_cu = std::max(1, env_int("NGH_MOMENTS_WGS_PER_CU", 8));
+    ctx->ordered_arrival = env_int("NGH_ORDERED_ARRIVAL", 0);
+    // the relaxed variant leans on what gfx950 does; on anything else only the ordered one runs
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) ctx->ordered_arrival = 1;
     hipError_t e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev0);
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev1);
@@ -1253,10 +1281,12 @@ int launch_moments(ngh_context* ctx, const MomentsPlan& m, const float* dev_x, i
     const dim3 grid((unsigned)(rows * m.n_seg));
     if (stream_x)
         hipLaunchKernelGGL(moments_kernel<true>, grid, dim3(kMomBlock), 0, ctx->stream, dev_x, (long long)row_stride,
-                           (unsigned)R, m.R4, m.n_seg, m.seg_chunks, partial, tickets, dev_mean, dev_var, dev_rstd, eps);
+                           (unsigned)R, m.R4, m.n_seg, m.seg_chunks, partial, tickets, dev_mean, dev_var, dev_rstd, eps,
+                           ctx->ordered_arrival);
     else
         hipLaunchKernelGGL(moments_kernel<false>, grid, dim3(kMomBlock), 0, ctx->stream, dev_x, (long long)row_stride,
-                           (unsigned)R, m.R4, m.n_seg, m.seg_chunks, partial, tickets, dev_mean, dev_var, dev_rstd, eps);
+                           (unsigned)R, m.R4, m.n_seg, m.seg_chunks, partial, tickets, dev_mean, dev_var, dev_rstd, eps,
+                           ctx->ordered_arrival);
     HIP_TRY(hipGetLastError());
     return NGH_OK;
 }
@@ -1295,6 +1325,45 @@ int ngh_moments_f32_noalloc(ngh_context* ctx, const float* dev_x, int64_t rows, 
     HIP_TRY(hipGetLastError());
     return launch_moments(ctx, m, dev_x, rows, R, row_stride, partial, tickets, dev_mean, dev_var, dev_rstd, eps,
                           x_cache_hint);
+}
+
+int ngh_convert_to_flex16(ngh_context* ctx, int16_t* dev_out, const void* dev_in, int32_t in_dtype, int64_t n,
+                          float scale, const float* dev_scale, int32_t* dev_stats) {
+    if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
+    if (n < 0) return fail(NGH_E_INVALID, "n %lld", (long long)n);
+    if (in_dtype != NGH_F32 && in_dtype != NGH_F16) return fail(NGH_E_INVALID, "source dtype %d (NGH_F32 or NGH_F16)", in_dtype);
+    if (n == 0) return NGH_OK;
+    if (!dev_out || !dev_in) return fail(NGH_E_INVALID, "NULL device pointer");
+    if (((uintptr_t)dev_out) % 2 || ((uintptr_t)dev_in) % (in_dtype == NGH_F32 ? 4 : 2))
+        return fail(NGH_E_INVALID, "misaligned pointer");
+    if (dev_scale) {
+        int32_t id = 0;
+        FlexTable* T = flex_table_of(ctx, dev_scale, &id);
+        if (T) {                                  // a scale inside a record: bring the record up to date first
+            FlexSettleArgs a;
+            a.n = 0;
+            NGH_TRY(flex_settle_add(ctx, *T, id, a));
+            NGH_TRY(flex_settle_flush(ctx, a));
+        }
+    }
+    const bool vec = ((uintptr_t)dev_out) % 16 == 0 && ((uintptr_t)dev_in) % 16 == 0;
+    const unsigned long long work = vec ? (unsigned long long)n / 8 + 8 : (unsigned long long)n;
+    const unsigned blocks = (unsigned)std::max<unsigned long long>(
+        1, std::min<unsigned long long>((work + kCvtBlock - 1) / kCvtBlock, (unsigned long long)ctx->cus * ctx->ew_blocks_per_cu));
+    NGH_TRY(ensure_stat_ws(ctx, blocks));
+    int* partial = ctx->stat_ws;
+#define NGH_CVT_LAUNCH(SRC, VEC)                                                                                 \
+    hipLaunchKernelGGL((convert_flex16_kernel<SRC, VEC>), dim3(blocks), dim3(kCvtBlock), 0, ctx->stream, dev_out, \
+                       dev_in, (unsigned long long)n, scale, dev_scale, partial)
+    if (in_dtype == NGH_F32) { if (vec) NGH_CVT_LAUNCH(NGH_F32, true); else NGH_CVT_LAUNCH(NGH_F32, false); }
+    else                     { if (vec) NGH_CVT_LAUNCH(NGH_F16, true); else NGH_CVT_LAUNCH(NGH_F16, false); }
+#undef NGH_CVT_LAUNCH
+    HIP_TRY(hipGetLastError());
+    if (dev_stats) {
+        hipLaunchKernelGGL(stats_fold_kernel, dim3(1), dim3(256), 0, ctx->stream, partial, blocks, dev_stats);
+        HIP_TRY(hipGetLastError());
+    }
+    return NGH_OK;
 }
 
 int ngh_plan_fused(const ngh_fused_spec* spec, int32_t stage, int32_t* out8) {
@@ -1512,6 +1581,7 @@ static int try_self_managed_launch(ngh_context* ctx, const ngh_fused_spec* spec,
         NGH_TRY(flex_settle_ids(ctx, dev, slot_id, P.k.n_stat_slots));
         NGH_TRY(ensure_tickets(ctx, (size_t)kFlexTicketWords + kFlexGroupMaxWords));
         P.k.flex_count = count;
+        P.k.ordered_arrival = ctx->ordered_arrival;
         P.k.tickets = ctx->tickets;
         P.k.group_max = (int*)(ctx->tickets + kFlexTicketWords);
     }

@@ -112,6 +112,7 @@ _SYMBOLS = {
                         ctypes.c_uint32],
     "ngh_moments_f32_noalloc": [_vp, _vp, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, _vp, _vp, _vp,
                                 ctypes.c_float, ctypes.c_uint32],
+    "ngh_convert_to_flex16": [_vp, _vp, _vp, _i32, ctypes.c_int64, ctypes.c_float, _vp, _vp],
     "ngh_plan_fused": [ctypes.POINTER(ngh_fused_spec), _i32, ctypes.POINTER(ctypes.c_int32)],
     "ngh_stats_alloc": [_vp, _i32, ctypes.POINTER(_vp)],
     "ngh_stats_reset": [_vp, _vp, _i32],
@@ -324,6 +325,14 @@ class HipRuntime(object):
                                                           int(row_stride), ctypes.c_void_p(mean),
                                                           ctypes.c_void_p(var), ctypes.c_void_p(rstd or None),
                                                           float(eps), int(x_cache_hint)))
+
+    def convert_to_flex16(self, out, src, src_dtype, n, scale=1.0, dev_scale=None, dev_stats=None):
+        """out[i] = (int16)trunc(src[i] * scale), saturating; max|mantissa| merged into dev_stats
+        (flex_conv.py:745-791).  With dev_scale the multiplier is 1 / *dev_scale."""
+        _check(self.lib, self.lib.ngh_convert_to_flex16(self.ctx, ctypes.c_void_p(out), ctypes.c_void_p(src),
+                                                        int(src_dtype), int(n), float(scale),
+                                                        ctypes.c_void_p(dev_scale or None),
+                                                        ctypes.c_void_p(dev_stats or None)))
 
     # -- flex statistics ---------------------------------------------------
     def stats_alloc(self, n):

@@ -335,6 +335,33 @@ def test_every_reduction(hip_runtime, name, shape, layout):
     out_d.free()
 
 
+@pytest.mark.parametrize("name", ["argmax", "argmin"])
+def test_arg_reduction_index_beyond_2_to_24_is_exact(hip_runtime, name):
+    """An index above 2^24 reaches int32 storage as the integer it is (no trip through an fp32
+    register, which would round it to an even number); the same reduction into fp32 is refused."""
+    from ngraph_hip.runtime.hiplib import HipLibraryError
+    rt = hip_runtime
+    R = (1 << 24) + 1025
+    x = np.zeros((R, 1), f32)
+    where = [(1 << 24) + 1001]                    # odd, above 2^24: not an fp32 number
+    x[where[0], 0] = 5.0 if name == "argmax" else -5.0
+    x_d = rt.array(x)
+    out_d, out_f = rt.empty((1,), NGH_I32), rt.empty((1,))
+    for layout in ([1, 1], [1, R]):               # as a column and as a row
+        rt.memset32(out_d.ptr, 0, 1)
+        sb = FusedSpecBuilder([R, 1])
+        sb.reduce(name, sb.load(sb.tensor(x_d.ptr, layout)), sb.tensor(out_d.ptr, [0, 1], NGH_I32))
+        rt.launch_fused(sb.build())
+        assert out_d.get().tolist() == where
+    sb = FusedSpecBuilder([R, 1])
+    sb.reduce(name, sb.load(sb.tensor(x_d.ptr, [1, 1])), sb.tensor(out_f.ptr, [0, 1]))
+    with pytest.raises(HipLibraryError) as e:
+        rt.launch_fused(sb.build())
+    assert e.value.code == -4
+    for d in (x_d, out_d, out_f):
+        d.free()
+
+
 @pytest.mark.parametrize("shape,layout", [((40000, 2), "col"), ((200704, 4), "row"), ((3000, 300), "col"),
                                           ((3000, 2048), "col")])
 def test_signed_sum_against_float64(hip_runtime, shape, layout):
@@ -426,6 +453,34 @@ def test_moments_rows(hip_runtime, rows, R, pad):
     assert not out_d.get()[2].any()
     for d in (x_d, out_d):
         d.free()
+
+
+def test_moments_hand_off_with_and_without_release_acquire_tickets(monkeypatch):
+    """The last workgroup of a row merges the row's segments.  By default the hand-off is a
+    relaxed ticket ordered behind the partial sums by a data dependency (what gfx950 honours);
+    NGH_ORDERED_ARRIVAL=1 selects release tickets and an acquire fence in the merger (what the
+    memory model asks for, at 2.6 times the kernel's duration).  Same sums in the same order:
+    identical results."""
+    from ngraph_hip.runtime.hiplib import HipRuntime
+    rs = np.random.RandomState(21)
+    x = rs.normal(3.0, 2.0, (300, 50000)).astype(f32)
+    seen = []
+    for ordered in ("0", "1"):
+        monkeypatch.setenv("NGH_ORDERED_ARRIVAL", ordered)
+        rt = HipRuntime(0)
+        try:
+            x_d, out_d = rt.array(x), rt.empty((3, 300))
+            for _ in range(3):                       # the arrival counters must be left at zero each time
+                rt.memset32(out_d.ptr, 0, 900)
+                rt.moments_f32(x_d.ptr, 300, 50000, 50000, out_d.ptr, out_d.ptr + 1200, out_d.ptr + 2400, 1e-5)
+                seen.append(out_d.get())
+        finally:
+            rt.close()
+    x64 = x.astype(np.float64)
+    np.testing.assert_allclose(seen[0][0], x64.mean(axis=1), rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(seen[0][1], x64.var(axis=1), rtol=RTOL, atol=ATOL)
+    for other in seen[1:]:
+        np.testing.assert_array_equal(other, seen[0])
 
 
 # ------------------------------------------------------------------ tiled skeleton (transposed views)
@@ -751,3 +806,50 @@ def test_flex_ids_past_the_end_of_the_table_are_rejected(hip_runtime):
         rt.sync()
     finally:
         rt.free(table)
+
+
+@pytest.mark.parametrize("src", ["f32", "f16"])
+@pytest.mark.parametrize("n,offset", [(1 << 20, 0), (100003, 0), (4099, 1), (5, 0), (1 << 22, 0)])
+def test_truncating_converter_to_flex16(hip_runtime, src, n, offset):
+    """ngh_convert_to_flex16 against the statement of the reference's `convert` kernel
+    (gpu/flex_conv.py:745-791): mantissa = (short)(value * scale), i.e. truncation toward zero,
+    max |mantissa| merged into the statistics word.  Outside the int16 range, where that cast
+    is undefined, the library saturates; NaN gives 0.  `offset` starts the views off the
+    16-byte boundary (the scalar path)."""
+    from ngraph_hip.runtime.hiplib import NGH_FLEX16, NGH_F16
+    rt = hip_runtime
+    rs = np.random.RandomState(n + offset)
+    np_src = np.float32 if src == "f32" else np.float16
+    dec = 9
+    values = rs.normal(0, 8, n + offset).astype(np_src)
+    values[offset:offset + 5] = np.array([1.999, -1.999, 63.99, -64.0, 0.0009765625], np_src)[:min(5, n)]
+    if n > 100:
+        values[offset + 50:offset + 54] = [70.0, -70.0, np.inf, -np.inf]      # beyond int16 at dec 9: saturate
+        values[offset + 60] = np.nan
+    src_d = rt.array(values, NGH_F32 if src == "f32" else NGH_F16)
+    out_d = rt.empty((n + offset,), NGH_FLEX16)
+    rt.memset16(out_d.ptr, 0x7777, n + offset)
+    stats = rt.stats_alloc(1)
+    itemsize = values.dtype.itemsize
+    rt.convert_to_flex16(out_d.ptr + 2 * offset, src_d.ptr + itemsize * offset, NGH_F32 if src == "f32" else NGH_F16,
+                         n, scale=float(2 ** dec), dev_stats=stats)
+    got = out_d.get()
+    with np.errstate(all="ignore"):
+        scaled = values[offset:].astype(np.float32) * np.float32(2 ** dec)           # cvt(value) * scale in fp32
+        want = np.clip(np.trunc(np.where(np.isnan(scaled), 0, scaled)), -32768, 32767).astype(np.int16)
+    np.testing.assert_array_equal(got[offset:], want)
+    assert (got[:offset] == 0x7777).all()                                           # nothing before the view
+    assert rt.stats_read(stats, 1)[0] == int(np.abs(want.astype(np.int32)).max())
+    # truncation, not rounding: 1.999 * 512 = 1023.49 -> 1023 and -1.999 -> -1023, 63.99 * 512 = 32762.9 -> 32762
+    if n >= 5:
+        first = (np.array([1.999, -1.999, 63.99], np_src).astype(np.float32) * 512).astype(np.float64)
+        assert got[offset:offset + 3].tolist() == np.clip(np.trunc(first), -32768, 32767).astype(int).tolist()
+    # the multiplier read from a device word (the tensor's scale 2**-dec) gives the same mantissas
+    scale_d = rt.array(np.array([2.0 ** -dec], np.float32))
+    rt.memset16(out_d.ptr, 0, n + offset)
+    rt.convert_to_flex16(out_d.ptr + 2 * offset, src_d.ptr + itemsize * offset, NGH_F32 if src == "f32" else NGH_F16,
+                         n, scale=123.0, dev_scale=scale_d.ptr)
+    np.testing.assert_array_equal(out_d.get()[offset:], want)
+    for d in (src_d, out_d, scale_d):
+        d.free()
+    rt.free(stats)

@@ -241,17 +241,23 @@ def test_flex_learning_rules_prebuilt_equals_interpreter(rule, resident, monkeyp
 # the tensor, or until something else needs the record.  Whatever it does, records, mantissas
 # and consumers must see exactly what the launch-by-launch policy of the host gives.
 
-_POLICY_MODES = [("host", None, None), ("three-launches", "0", None), ("end-of-kernel", "1", None),
-                 ("deferred", "2", None), ("deferred-small-grid", "2", "1")]
+# (name, NGH_FLEX_SELF_MANAGED, NGH_FLEX_LAZY_BLOCKS_PER_CU, NGH_ORDERED_ARRIVAL); the end-of-kernel
+# policy hands over between workgroups with relaxed tickets (default) or release tickets and an acquire fence
+_POLICY_MODES = [("host", None, None, None), ("three-launches", "0", None, None), ("end-of-kernel", "1", None, None),
+                 ("end-of-kernel-release-acquire-tickets", "1", None, "1"),
+                 ("deferred", "2", None, None), ("deferred-small-grid", "2", "1", None)]
 
 
 def _entry_state(entry):
     return (entry.dec, entry.next_dec, entry.last_maxabs, tuple(entry.history))
 
 
-def _with_policy_mode(monkeypatch, mode, grid):
+def _with_policy_mode(monkeypatch, mode, grid, ordered=None):
     monkeypatch.delenv("NGH_FLEX_SELF_MANAGED", raising=False)
     monkeypatch.delenv("NGH_FLEX_LAZY_BLOCKS_PER_CU", raising=False)
+    monkeypatch.delenv("NGH_ORDERED_ARRIVAL", raising=False)
+    if ordered is not None:
+        monkeypatch.setenv("NGH_ORDERED_ARRIVAL", ordered)
     if mode is not None:
         monkeypatch.setenv("NGH_FLEX_SELF_MANAGED", mode)
     if grid is not None:
@@ -263,8 +269,8 @@ def test_device_only_iterations_agree_across_policy_modes(n, monkeypatch):
     x0, w, b = configs.c5_inputs(n, seed=11)
     x0 = (x0 * 30.0).astype(np.float32)           # saturates at the first exponent: the policy has to move
     seen = {}
-    for name, mode, grid in _POLICY_MODES:
-        _with_policy_mode(monkeypatch, mode, grid)
+    for name, mode, grid, ordered in _POLICY_MODES:
+        _with_policy_mode(monkeypatch, mode, grid, ordered)
         t = ngt.make_transformer_factory("flexhip", resident=name != "host")()
         try:
             f, _, _ = _c5_graph(t, n)
@@ -300,8 +306,8 @@ def test_consumer_of_a_tensor_with_unfolded_statistics(monkeypatch):
     n = 1 << 18
     x0, w, b = configs.c5_inputs(n, seed=12)
     seen = {}
-    for name, mode, grid in _POLICY_MODES:
-        _with_policy_mode(monkeypatch, mode, grid)
+    for name, mode, grid, ordered in _POLICY_MODES:
+        _with_policy_mode(monkeypatch, mode, grid, ordered)
         t = ngt.make_transformer_factory("flexhip", resident=name != "host")()
         try:
             P = ng.make_axis(n, name="P")
@@ -336,8 +342,8 @@ def test_in_place_rule_iterated_on_the_device_agrees_across_policy_modes(monkeyp
     p0 = rs.normal(0, 0.1, n).astype(np.float32)
     g = rs.normal(0, 0.05, n).astype(np.float32)
     seen = {}
-    for name, mode, grid in _POLICY_MODES:
-        _with_policy_mode(monkeypatch, mode, grid)
+    for name, mode, grid, ordered in _POLICY_MODES:
+        _with_policy_mode(monkeypatch, mode, grid, ordered)
         t = ngt.make_transformer_factory("flexhip", resident=name != "host")()
         try:
             P = ng.make_axis(n, name="P")

@@ -244,3 +244,36 @@ def test_iteration_spaces_that_wrap_are_refused(shape):
     sp.shape[0], sp.shape[1] = 4, 4
     sp.tensors[0].strides[0] = 1 << 61
     assert lib.ngh_validate_fused(ctypes.byref(sp)) != 0
+
+
+def test_indices_beyond_fp32_exactness_are_refused_not_rounded():
+    """Registers are fp32 (integers exact to 2^24; the reference keeps int32 operands in integer
+    registers, float_ew2.py:615-641).  Where an index could exceed that, the spec is refused:
+    a lookup in a table longer than 2^24 along the looked-up axis, an index value along an axis
+    longer than 2^24, an argmax over more than 2^24 elements into anything but int32 / uint32."""
+    lib = load_library()
+    big = (1 << 24) + 8
+
+    def rc(sb):
+        return lib.ngh_validate_fused(ctypes.byref(sb.build()))
+
+    for extent, want in ((1 << 24, 0), (big, -4)):
+        sb = FusedSpecBuilder([64, 8])
+        idx = sb.load(sb.tensor(FAKE, [1, 0], NGH_I32))
+        table = sb.tensor(FAKE + (1 << 30), [8, 1], take_extent=extent)
+        sb.store(sb.tensor(FAKE + (2 << 30), [8, 1]), sb.take(table, idx, 0))
+        assert rc(sb) == want, lib.ngh_last_error()
+    for n, want in ((1 << 24, 0), (big, -4)):
+        sb = FusedSpecBuilder([n])
+        sb.store(sb.tensor(FAKE, [1]), sb.iota(0))
+        assert rc(sb) == want, lib.ngh_last_error()
+        assert want == 0 or b"2^24" in lib.ngh_last_error()
+    for dtype, want in ((NGH_I32, 0), (hiplib.NGH_U32, 0), (NGH_F32, -4), (hiplib.NGH_I16, -4)):
+        sb = FusedSpecBuilder([big, 4])
+        x = sb.load(sb.tensor(FAKE, [4, 1]))
+        sb.reduce("argmax", x, sb.tensor(FAKE + (1 << 32), [0, 1], dtype))
+        assert rc(sb) == want, (dtype, lib.ngh_last_error())
+    # a sum over as many elements is fine in any type
+    sb = FusedSpecBuilder([big, 4])
+    sb.reduce("sum", sb.load(sb.tensor(FAKE, [4, 1])), sb.tensor(FAKE + (1 << 32), [0, 1]))
+    assert rc(sb) == 0
