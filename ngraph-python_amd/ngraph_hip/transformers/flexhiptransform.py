@@ -28,7 +28,7 @@ from ngraph_hip.op_graph import op_graph as og
 from ngraph_hip.runtime.hiplib import NGH_FLEX16, NGH_SPEC_PROBE
 from ngraph_hip.transformers.hiptransform import (HipTransformer, HipDeviceTensor,
                                                   HipDeviceBufferStorage, HipKernelGroup,
-                                                  FusedKernel, CopyKernel)
+                                                  FusedKernel, CopyKernel, _td)
 from ngraph_hip.transformers.passes.passes import PeepholeGraphPass
 
 
@@ -200,8 +200,8 @@ class FlexCopyKernel(CopyKernel):
 
     def bind_buffers(self):
         t = self.transformer
-        src_buf = t.op_tensors[self.op.args[0].forwarded.tensor_description().base]
-        dst_buf = t.op_tensors[self.op.tensor_description().base]
+        src_buf = t.op_tensors[_td(self.op.args[0].forwarded).base]
+        dst_buf = t.op_tensors[_td(self.op).base]
         dst_buf.flex_entry = src_buf.flex_entry
         super(FlexCopyKernel, self).bind_buffers()
 

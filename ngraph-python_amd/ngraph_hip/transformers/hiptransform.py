@@ -35,8 +35,8 @@ from ngraph_hip.runtime.hiplib import (HipRuntime, DryRunRuntime, HipLibraryErro
                                        NGH_CACHE_STREAM_STORE)
 from ngraph_hip.transformers.base import (ComputationGraphTransformer, DeviceBufferStorage,
                                           DeviceTensor, UnsupportedTransformerException)
-from ngraph_hip.transformers.passes.passes import (SimplePrune, TensorSizeFold, PeepholeGraphPass,
-                                                   ReductionLayoutPass, ConstantFoldPass)
+from ngraph_hip.transformers.passes.passes import SimplePrune, PeepholeGraphPass
+from ngraph_hip.transformers.passes.hippasses import TensorSizeFold, ReductionLayoutPass, ConstantFoldPass
 
 # op class -> kernel op name (gputransform.py:129-275)
 _UNARY_NAMES = OrderedDict([
@@ -55,6 +55,19 @@ _REDUCTION_NAMES = OrderedDict([
     (og.Sum, "sum"), (og.Prod, "prod"), (og.Max, "max"), (og.Min, "min"),
     (og.Argmax, "argmax"), (og.Argmin, "argmin"),
 ])
+
+
+def _td(op):
+    """The tensor description of `op` in this backend's conventions: strides and offset in
+    elements, one stride per axis.  The graph front of this repository describes tensors that
+    way itself (`_adapt_td` is the identity); the plug-in for the real package, whose
+    descriptions hold byte strides and nested strides for flattened axes
+    (ngraph/op_graph/axes.py:1174-1232), replaces `_adapt_td`."""
+    return _adapt_td(op.tensor_description())
+
+
+def _adapt_td(td):
+    return td
 
 
 def _lookup(table, op):
@@ -159,6 +172,11 @@ class HipDeviceTensor(DeviceTensor):
         pass
 
     @property
+    def view(self):
+        """The view's description with strides and offset in elements (see _td)."""
+        return _adapt_td(self.tensor_description)
+
+    @property
     def np_dtype(self):
         d = self.tensor_description.dtype
         return d if isinstance(d, np.dtype) else np.dtype(np.int16)
@@ -173,19 +191,19 @@ class HipDeviceTensor(DeviceTensor):
 
     @property
     def ptr(self):
-        return self.device_buffer.ptr + self.tensor_description.offset * self.itemsize
+        return self.device_buffer.ptr + self.view.offset * self.itemsize
 
     @property
     def shape(self):
-        return self.tensor_description.shape
+        return self.view.shape
 
     @property
     def element_strides(self):
-        return self.tensor_description.full_strides
+        return self.view.full_strides
 
     def _read_raw(self):
         """The view's elements as a C-contiguous host array of the storage dtype."""
-        td, rt = self.tensor_description, self.transformer.runtime
+        td, rt = self.view, self.transformer.runtime
         out = np.empty(td.shape, dtype=self.np_dtype)
         if out.size == 0:
             return out
@@ -203,7 +221,7 @@ class HipDeviceTensor(DeviceTensor):
         return out
 
     def _write_raw(self, host):
-        td, rt = self.tensor_description, self.transformer.runtime
+        td, rt = self.view, self.transformer.runtime
         host = np.ascontiguousarray(np.broadcast_to(host, td.shape), dtype=self.np_dtype)
         if host.size == 0:
             return
@@ -362,7 +380,7 @@ class FusedKernel(HipKernel):
             prod = _producer(arg)
             if prod in value_reg:
                 return value_reg[prod]
-            td = arg.tensor_description()
+            td = _td(arg)
             key = _view_key(td)
             if key in value_reg:
                 return value_reg[key]
@@ -378,12 +396,12 @@ class FusedKernel(HipKernel):
             if isinstance(op, og.AssignOp):
                 target, val = op.args[0].forwarded, op.args[1].forwarded
                 r = operand_reg(val)
-                td = target.tensor_description()
+                td = _td(target)
                 program.append(("store", slot(td), r))
                 value_reg[_view_key(td)] = r
                 continue
             if isinstance(op, og.Fill):
-                td = op.args[0].forwarded.tensor_description()
+                td = _td(op.args[0].forwarded)
                 r = new_reg()
                 program.append(("const", r, float(op.scalar)))
                 program.append((self.fill_store, slot(td), r))
@@ -413,7 +431,7 @@ class FusedKernel(HipKernel):
                 # gputransform.py:197-199: ("take", x=idx, y=lut, axis=lut_axis)
                 lut, idx = op.args[0].forwarded, op.args[1].forwarded
                 x = operand_reg(idx)
-                lut_td = lut.tensor_description()
+                lut_td = _td(lut)
                 table = slot(lut_td)
                 out_axis = op.axes[op.lut_axis]
                 take_axes.append(out_axis)
@@ -432,7 +450,7 @@ class FusedKernel(HipKernel):
                         program.append(("assign", r, x))
                 else:
                     # reductions end the stage: collected here, emitted after every elementwise op
-                    reductions_at_end.append(("reduce", name, x, slot(op.tensor_description())))
+                    reductions_at_end.append(("reduce", name, x, slot(_td(op))))
                     red_slots.append(op)
                     continue
             elif name in og_unary_names:
@@ -445,7 +463,7 @@ class FusedKernel(HipKernel):
                 program.append((name, r, x, y))
             value_reg[op] = r
             if op in self.store_ops:
-                program.append(("store", slot(op.tensor_description()), r))
+                program.append(("store", slot(_td(op)), r))
 
         program.extend(reductions_at_end)
 
@@ -632,8 +650,8 @@ class CopyKernel(HipKernel):
 
     def bind_buffers(self):
         t = self.transformer
-        src_td = self.op.args[0].forwarded.tensor_description()
-        dst_td = self.op.tensor_description()
+        src_td = _td(self.op.args[0].forwarded)
+        dst_td = _td(self.op)
         self.src = t.get_tensor_description_tensor_view(src_td)
         self.dst = t.get_tensor_description_tensor_view(dst_td)
         self.shape = dst_td.shape
@@ -643,8 +661,8 @@ class CopyKernel(HipKernel):
         super(CopyKernel, self).bind_buffers()
 
     def buffer_uses(self):
-        return [(self.op.args[0].forwarded.tensor_description().base, True, False),
-                (self.op.tensor_description().base, False, True)]
+        return [(_td(self.op.args[0].forwarded).base, True, False),
+                (_td(self.op).base, False, True)]
 
     def describe(self):
         return [["copy_strided"]]
@@ -726,7 +744,7 @@ class MomentsFusionPass(PeepholeGraphPass):
 
     @staticmethod
     def _same_tensor(a, b):
-        ta, tb = a.tensor_description(), b.tensor_description()
+        ta, tb = _td(a), _td(b)
         return ta.base is tb.base and ta.parameter_key == tb.parameter_key and ta.axes == tb.axes
 
     def do_pass(self, ops, **kwargs):
@@ -778,7 +796,7 @@ class MomentsFusionPass(PeepholeGraphPass):
         x2, red2 = inner
         if not red2.is_equal_set(red_axes) or not self._same_tensor(x, x2):
             return
-        if x.dtype != np.dtype(np.float32) or moments_layout(x.tensor_description(), red_axes) is None:
+        if x.dtype != np.dtype(np.float32) or moments_layout(_td(x), red_axes) is None:
             return
         mom = MomentsOp(x, red_axes)
         mean_view = og.slice_along_axis(mom, mom.k_axis, 0)
@@ -797,21 +815,21 @@ class MomentsKernel(HipKernel):
 
     def bind_buffers(self):
         t = self.transformer
-        x_td = self.op.args[0].forwarded.tensor_description()
+        x_td = _td(self.op.args[0].forwarded)
         layout = moments_layout(x_td, self.op.reduction_axes)
         if layout is None:
             raise og_unsupported("MomentsOp operand lost its row layout")
         self.rows, self.R, self.row_stride = layout
         self.x = t.get_tensor_description_tensor_view(x_td)
-        self.out = t.get_tensor_description_tensor_view(self.op.tensor_description())
+        self.out = t.get_tensor_description_tensor_view(_td(self.op))
         super(MomentsKernel, self).bind_buffers()
 
     def buffer_uses(self):
-        return [(self.op.args[0].forwarded.tensor_description().base, True, False),
-                (self.op.tensor_description().base, False, True)]
+        return [(_td(self.op.args[0].forwarded).base, True, False),
+                (_td(self.op).base, False, True)]
 
     def set_cache_hints(self, hint_of):
-        self.x_cache_hint = hint_of(self.op.args[0].forwarded.tensor_description().base, True, False)
+        self.x_cache_hint = hint_of(_td(self.op.args[0].forwarded).base, True, False)
 
     def execute(self):
         out, eps = self.out.ptr, self.op.epsilon
@@ -1086,7 +1104,7 @@ class FusionPlanner(object):
             for op in list(g.ops):
                 if not plain(op) or iteration_axes(op).size <= self.small_tensor:
                     continue
-                base = op.tensor_description().base
+                base = _td(op).base
                 if base in returned:
                     continue
                 inside = set(groups[gi].ops)
@@ -1142,7 +1160,7 @@ class FusionPlanner(object):
             inside = set(g.ops)
             targets, ok = set(), True
             for op in g.ops:
-                base = op.tensor_description().base
+                base = _td(op).base
                 if base in returned:
                     ok = False
                     break
@@ -1202,14 +1220,14 @@ class FusionPlanner(object):
 
     @staticmethod
     def _outside_operands(chain):
-        inside = set(o.tensor_description().base for o in chain)
+        inside = set(_td(o).base for o in chain)
         out = []
         for o in chain:
             for a in o.args:
                 a = a.forwarded
                 if _scalar_constant_value(a) is not None:
                     continue
-                td = a.tensor_description()
+                td = _td(a)
                 if td.base not in inside:
                     out.append(td)
         return out
@@ -1220,7 +1238,7 @@ class FusionPlanner(object):
         for g in groups[first:last + 1]:
             for o in g.ops:
                 if isinstance(o, (og.AssignOp, og.Fill)) and \
-                        o.args[0].forwarded.tensor_description().base in bases:
+                        _td(o.args[0].forwarded).base in bases:
                     return True
         return False
 
@@ -1249,19 +1267,19 @@ class _Group(object):
     def _operand_views(self, op):
         reads, writes = [], []
         if isinstance(op, og.AssignOp):
-            writes.append(op.args[0].forwarded.tensor_description())
+            writes.append(_td(op.args[0].forwarded))
             srcs = [op.args[1]]
         elif isinstance(op, og.Fill):
-            writes.append(op.args[0].forwarded.tensor_description())
+            writes.append(_td(op.args[0].forwarded))
             srcs = []
         else:
-            writes.append(op.tensor_description())
+            writes.append(_td(op))
             srcs = list(op.args)
         for a in srcs:
             a = a.forwarded
             if _scalar_constant_value(a) is not None:
                 continue
-            reads.append(a.tensor_description())
+            reads.append(_td(a))
         return reads, writes
 
     def _account(self, op):
@@ -1286,7 +1304,7 @@ class _Group(object):
         produced = set()
         for op in ops:
             if op.is_tensor_op and not isinstance(op, (og.AssignOp, og.Fill)):
-                produced.add(op.tensor_description().base)
+                produced.add(_td(op).base)
         views, written = set(), set()
         for op in ops:
             reads, writes = self._operand_views(op)
@@ -1296,10 +1314,10 @@ class _Group(object):
             if isinstance(op, (og.AssignOp, og.Fill)):
                 written.update(_view_key(td) for td in writes)
             else:
-                base = op.tensor_description().base
+                base = _td(op).base
                 if base in returned or isinstance(op, og.ReductionOp) or \
                         any(u not in inside for u in readers.get(base, ())):
-                    written.add(_view_key(op.tensor_description()))
+                    written.add(_view_key(_td(op)))
         self.n_written_views = len(written)
         return len(views | written)
 
@@ -1371,7 +1389,7 @@ class _Group(object):
         axis, in one common axis order?  (The kernels reduce over a single axis.)"""
         ops = self.ops + [red_op]
         inside = set(ops)
-        produced = set(op.tensor_description().base for op in ops
+        produced = set(_td(op).base for op in ops
                        if op.is_tensor_op and not isinstance(op, (og.AssignOp, og.Fill)))
         tds = []
         for op in ops:
@@ -1383,9 +1401,9 @@ class _Group(object):
                 tds.extend(writes)
             elif not (isinstance(op, og.ReductionOp) and op.reduction_axes.size > 1):
                 # (a reduction over axes of length 1 is an elementwise assignment)
-                base = op.tensor_description().base
+                base = _td(op).base
                 if base in returned or any(u not in inside for u in readers.get(base, ())):
-                    tds.append(op.tensor_description())
+                    tds.append(_td(op))
         red = [a for a in red_op.reduction_axes if a.length != 1]
         if len(red) < 2:
             return True
@@ -1419,7 +1437,7 @@ class _Group(object):
                 if _scalar_constant_value(a) is not None:
                     continue
                 prod = _producer(a)
-                key = prod if prod in index and index[prod] < i else _view_key(a.tensor_description())
+                key = prod if prod in index and index[prod] < i else _view_key(_td(a))
                 born.setdefault(key, index[prod] if key is prod else i)
                 last[key] = i
             born.setdefault(op, i)
@@ -1444,7 +1462,7 @@ class _Group(object):
         for op in self.ops:
             if not op.is_tensor_op or isinstance(op, (og.AssignOp, og.Fill)):
                 continue
-            base = op.tensor_description().base
+            base = _td(op).base
             users = readers.get(base, ())
             if op in self.never_store:
                 continue
@@ -1533,12 +1551,12 @@ class HipTransformer(ComputationGraphTransformer):
                 for a in srcs:
                     a = a.forwarded
                     if a.is_tensor_op:
-                        readers.setdefault(a.tensor_description().base, set()).add(op)
+                        readers.setdefault(_td(a).base, set()).add(op)
         for comp in self.computations:
             for v in comp.computation_op.values:
                 v = v.forwarded
                 if v.is_tensor_op:
-                    returned.add(v.tensor_description().base)
+                    returned.add(_td(v).base)
         return readers, returned
 
     def transform_ordered_ops(self, computation, ordered_ops, name):

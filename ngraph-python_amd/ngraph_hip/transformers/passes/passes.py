@@ -1,15 +1,14 @@
-"""Graph passes run before lowering.
-
-Counterparts of ngraph/transformers/passes/passes.py for the op set of this
-path: the pass driver (passes.py:35-120), `replace_op` with axes repair, and
-the `SimplePrune` algebra (passes.py:499-628) that changes which ops reach the
-kernels (x*1, x*0, x*-1, x+0, constant sum/prod, log(exp x), -const).
+"""Graph passes run before lowering: the part that ngraph/transformers/passes/passes.py
+provides in the reference -- the pass driver (passes.py:35-120), `replace_op` with axes
+repair, and the `SimplePrune` algebra (passes.py:499-628) that changes which ops reach the
+kernels (x*1, x*0, x*-1, x+0, constant sum/prod, log(exp x), -const).  The passes that are
+this backend's own live in hippasses.py.
 """
 from __future__ import division
 import numpy as np
 
 from ngraph_hip.op_graph.op_graph import (
-    Op, NegativeOp, Multiply, Add, Sum, Prod, LogOp, ExpOp, Divide, TensorSizeOp, ContiguousOp,
+    Op, NegativeOp, Multiply, Add, Sum, Prod, LogOp, ExpOp, Divide, ContiguousOp,
     BroadcastOp, constant, negative, broadcast, axes_with_order, as_op, TensorOp)
 
 
@@ -126,82 +125,3 @@ class SimplePrune(PeepholeGraphPass):
             elif isinstance(x, ExpOp):
                 exp_x, = self.op_args(x)
                 self.replace_op(op, exp_x)
-
-
-class TensorSizeFold(PeepholeGraphPass):
-    """TensorSizeOp is known at transform time: make it a constant.
-
-    The reference backends fill a scalar tensor with `reduction_axes.size`
-    (gputransform.py:444-447, cputransform.py:759-761); a constant gives the
-    same value and lets it travel as a kernel argument.
-    """
-
-    def visit(self, op, *args):
-        if isinstance(op, TensorSizeOp):
-            self.replace_op(op, constant(float(op.reduction_axes.size)))
-
-
-def axes_merge_to_one(td, axes):
-    """Can `axes` of the view `td` be walked as ONE strided dimension?"""
-    dims = [(a.length, td.full_strides[td.axes.index(a)]) for a in axes if a.length != 1]
-    dims.sort(key=lambda d: -d[1])
-    for (n0, s0), (n1, s1) in zip(dims[:-1], dims[1:]):
-        if s0 != s1 * n1:
-            return False
-    return True
-
-
-class ReductionLayoutPass(PeepholeGraphPass):
-    """Reductions need their reduced axes to form one strided axis.
-
-    When they do not, the operand is first copied into (reduced..., kept...)
-    order; this is the layout conversion the reference inserts as a
-    DimshuffleOp for the same reason (gpulayout.py:861-979,
-    layout_common.py:347-378).
-    """
-
-    def visit(self, op, *args):
-        from ngraph_hip.op_graph.op_graph import ReductionOp
-        if not isinstance(op, ReductionOp) or len(op.reduction_axes) < 2:
-            return
-        x, = args
-        if axes_merge_to_one(x.tensor_description(), op.reduction_axes):
-            return
-        order = op.reduction_axes + (x.axes - op.reduction_axes)
-        new_x = ContiguousOp(axes_with_order(x, order))
-        self.replace_op(op, type(op)(new_x, reduction_axes=op.reduction_axes, dtype=op.dtype))
-
-
-class ConstantFoldPass(PeepholeGraphPass):
-    """Elementwise ops on scalar constants are evaluated at transform time.
-
-    Such subgraphs ((1 - beta_1), lr * 2, ...) would otherwise each cost a kernel launch per
-    call.  The value is computed in float32 with the NumPy ufunc of the same name, which is
-    what the per-op CPU path does with the same operands (cputransform.py:512-761).
-    """
-
-    _UNARY = {"NegativeOp": np.negative, "AbsoluteOp": np.abs, "SqrtOp": np.sqrt, "ExpOp": np.exp,
-              "LogOp": np.log, "ReciprocalOp": np.reciprocal, "SquareOp": np.square,
-              "TanhOp": np.tanh, "SignOp": np.sign, "SinOp": np.sin, "CosOp": np.cos}
-    _BINARY = {"Add": np.add, "Subtract": np.subtract, "Multiply": np.multiply,
-               "Divide": np.divide, "Power": np.power, "Maximum": np.maximum,
-               "Minimum": np.minimum, "FloorDivide": np.floor_divide, "Mod": np.mod}
-
-    def visit(self, op, *args):
-        name = type(op).__name__
-        if name not in self._UNARY and name not in self._BINARY:
-            return
-        if op.dtype != np.dtype(np.float32):
-            return
-        if name in self._UNARY and len(args) == 1:
-            c = _scalar_const(args[0])
-            if c is not None:
-                with np.errstate(all="ignore"):
-                    val = self._UNARY[name](np.float32(c), dtype=np.float32)
-                self.replace_op(op, constant(float(val), op.axes))
-        elif name in self._BINARY and len(args) == 2:
-            cx, cy = _scalar_const(args[0]), _scalar_const(args[1])
-            if cx is not None and cy is not None:
-                with np.errstate(all="ignore"):
-                    val = self._BINARY[name](np.float32(cx), np.float32(cy), dtype=np.float32)
-                self.replace_op(op, constant(float(val), op.axes))
