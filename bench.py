@@ -34,7 +34,9 @@ DISPLACE_BYTES = 512 << 20      # a device copy of this size between launches em
 # WRITE_SIZE (each scaled by a device copy of known size) -- not measured by this run.  A figure
 # is only reported for the very kernel and shape it was recorded on.
 RECORDED_TRAFFIC = {
-    ("C2", "special:batchnorm_k1/nt-stores", 51380224): (411176158, "profiles/c2_batchnorm_pmc_traffic.md"),
+    ("C2", "special:batchnorm_k1/nt-stores", 51380224): (411167839, "profiles/c2_c3_c5_pmc_traffic.md"),
+    ("C3", "special:adam_k1/nt-loads", 25600000): (716818595, "profiles/c2_c3_c5_pmc_traffic.md"),
+    ("C5", "special:flex_relu_fma_k0", 16777216): (134547767, "profiles/c2_c3_c5_pmc_traffic.md"),
 }
 
 
@@ -449,10 +451,18 @@ def compiled_vs_interpreted(ng, ngt, steps, warmup, An=8192, Bn=8192):
                 group()
                 t.runtime.sync()
                 ms = float(np.median(step_blocks(t.runtime, group, steps, warmup, 3)))
+                nbytes = passes * An * Bn * 4
                 row[label] = {
-                    "ms_per_step": round(ms, 5), "GB/s": round(passes * An * Bn * 4 / (ms * 1e-3) / 1e9, 1),
-                    "frac_of_hbm_peak": round(passes * An * Bn * 4 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                    "ms_per_step": round(ms, 5), "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                    "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                     "kernels": [d for k in group.kernels for ds in k.describe() for d in ds]}
+                if label != "interpreted":
+                    # one step per event pair with the cache emptied by a 512 MiB read before it
+                    d = Displacer(t.runtime)
+                    cold = max(cold_step_ms(group, t.runtime, d, 9) - event_pair_overhead_ms(t.runtime), 1e-6)
+                    d.free()
+                    row[label]["cold_step"] = {"ms": round(cold, 5), "GB/s": round(nbytes / (cold * 1e-3) / 1e9, 1),
+                                               "frac_of_hbm_peak": round(nbytes / (cold * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
             finally:
                 t.close()
         out[name] = row

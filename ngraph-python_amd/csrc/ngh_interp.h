@@ -685,11 +685,22 @@ __global__ __launch_bounds__(kBlock) void red_finish_kernel(const KArgs k, unsig
         const bool with_index = opc >= NGH_OP_RED_ARGMAX;
         Acc a = acc_init(opc);
         if (out < n_out) {
-#pragma unroll 4
-            for (unsigned g = g_begin; g < g_end; ++g) {
-                const size_t w = ((size_t)s * n_seg + g) * n_out + out;
-                Acc b; b.v = ws.val[w]; b.i = with_index ? ws.idx[w] : 0;
-                a = acc_merge(opc, a, b);
+            // eight partial results are asked for before the first is merged: the loads are
+            // independent, the merges are not, and one round trip per segment is what this
+            // kernel's time would otherwise consist of
+            constexpr int kBatch = 8;
+            for (unsigned g0 = g_begin; g0 < g_end; g0 += kBatch) {
+                Acc b[kBatch];
+#pragma unroll
+                for (int j = 0; j < kBatch; ++j) {
+                    const unsigned g = min(g0 + j, g_end - 1);          // (a repeated load, merged only once)
+                    const size_t w = ((size_t)s * n_seg + g) * n_out + out;
+                    b[j].v = ws.val[w];
+                    b[j].i = with_index ? ws.idx[w] : 0;
+                }
+#pragma unroll
+                for (int j = 0; j < kBatch; ++j)
+                    if (g0 + j < g_end) a = acc_merge(opc, a, b[j]);
             }
         }
         sh[wave][lane] = a;
