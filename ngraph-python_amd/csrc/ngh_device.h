@@ -518,7 +518,17 @@ __global__ __launch_bounds__(256) void stats_fold_kernel(const int* __restrict__
                                                          int* __restrict__ word) {
     __shared__ int sh[4];
     int m = 0;
-    for (unsigned i = threadIdx.x; i < n; i += 256) m = max(m, partial[i]);
+    // eight loads at a time: one workgroup folds up to tens of thousands of partial maxima, and a
+    // load per round trip would make this tiny kernel take longer than the kernel it follows
+    unsigned i = threadIdx.x;
+    for (; i + 7 * 256 < n; i += 8 * 256) {
+        int v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = partial[i + j * 256];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) m = max(m, v[j]);
+    }
+    for (; i < n; i += 256) m = max(m, partial[i]);
 #pragma unroll
     for (int s = 32; s > 0; s >>= 1) m = max(m, __shfl_xor(m, s, 64));
     if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = m;

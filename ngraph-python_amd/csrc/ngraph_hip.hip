@@ -958,7 +958,8 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->ew_blocks_per_cu = std::max(1, env_int("NGH_EW_BLOCKS_PER_CU", 64));
     ctx->force_interp = env_int("NGH_FORCE_INTERP", 0);
     ctx->flex_self_managed = env_int("NGH_FLEX_SELF_MANAGED", 2);
-    ctx->flex_lazy_blocks_per_cu = std::max(1, env_int("NGH_FLEX_LAZY_BLOCKS_PER_CU", 6));
+    ctx->flex_lazy_blocks_per_cu = env_int("NGH_FLEX_LAZY_BLOCKS_PER_CU", 6);
+    if (ctx->flex_lazy_blocks_per_cu == 0) ctx->flex_lazy_blocks_per_cu = 1;
     ctx->no_tiles = env_int("NGH_NO_TILES", 0);
     ctx->red_wgs_per_cu = std::max(1, env_int("NGH_RED_WGS_PER_CU", 8));
     ctx->red_col_wgs_per_cu = std::max(1, env_int("NGH_RED_COL_WGS_PER_CU", 2));
