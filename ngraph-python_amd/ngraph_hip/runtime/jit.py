@@ -118,9 +118,13 @@ def compile_programs(programs, verbose=False):
     if os.path.exists(lib):
         return lib
     src = base + ".hip"
-    with open(src, "w") as fh:
+    unique = "%d.%d.tmp" % (os.getpid(), threading.get_ident())
+    # (the source goes into place whole as well: another thread or process compiling the same
+    # programs may be reading it)
+    with open(src + "." + unique, "w") as fh:
         fh.write(text)
-    tmp = "%s.%d.%d.tmp" % (lib, os.getpid(), threading.get_ident())
+    os.replace(src + "." + unique, src)
+    tmp = "%s.%s" % (lib, unique)
     try:
         hipcc = find_hipcc()
     except RuntimeError:
@@ -132,6 +136,8 @@ def compile_programs(programs, verbose=False):
         print(" ".join(cmd))
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, universal_newlines=True)
     if proc.returncode != 0:
+        if os.path.exists(tmp):
+            os.remove(tmp)
         raise RuntimeError("hipcc failed on %s:\n%s" % (src, proc.stdout))
     os.replace(tmp, lib)          # atomic: another process may be compiling the same programs
     return lib
