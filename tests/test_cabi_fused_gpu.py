@@ -265,6 +265,85 @@ def test_every_unary_op(hip_runtime, name):
     y_d.free()
 
 
+def _ulps(got, want):
+    """Distance between two float32 arrays in units of the float32 spacing at `want`."""
+    with np.errstate(all="ignore"):
+        spacing = np.spacing(np.abs(want).astype(f32))
+        d = np.abs(got.astype(np.float64) - want.astype(np.float64)) / spacing
+    d[(got == want) | (np.isnan(got) & np.isnan(want))] = 0
+    return d
+
+
+_TRANSCENDENTAL_RANGES = {
+    # name: (float64 function, sampler of n float32 arguments)
+    "exp": (np.exp, lambda rs, n: rs.uniform(-104, 89, n)),
+    "exp2": (np.exp2, lambda rs, n: rs.uniform(-150, 128, n)),
+    "log": (np.log, lambda rs, n: np.exp(rs.uniform(np.log(1e-45), np.log(3e38), n))),
+    "log2": (np.log2, lambda rs, n: np.exp(rs.uniform(np.log(1e-45), np.log(3e38), n))),
+    "tanh": (np.tanh, lambda rs, n: np.concatenate([rs.uniform(-12, 12, n // 2), rs.normal(0, 1e-3, n - n // 2)])),
+    "sin": (np.sin, lambda rs, n: np.concatenate([rs.uniform(-100, 100, n // 2), rs.uniform(-1e6, 1e6, n - n // 2)])),
+    "cos": (np.cos, lambda rs, n: np.concatenate([rs.uniform(-100, 100, n // 2), rs.uniform(-1e6, 1e6, n - n // 2)])),
+    "sqrt": (np.sqrt, lambda rs, n: np.exp(rs.uniform(np.log(1e-45), np.log(3e38), n))),
+    "rcp": (lambda v: 1.0 / v, lambda rs, n: np.exp(rs.uniform(np.log(1e-38), np.log(3e38), n)) * rs.choice([-1, 1], n)),
+}
+
+
+@pytest.mark.parametrize("name", sorted(_TRANSCENDENTAL_RANGES))
+def test_transcendental_ops_within_2_ulp(hip_runtime, name):
+    """A million arguments over each function's whole float32 range, denormal results included:
+    the kernel's result is within 2 units in the last place of the correctly rounded one
+    (float64 NumPy, rounded), and within 4 of the oracle's float32 NumPy result, which is itself
+    up to 3 away from the correctly rounded value (exp2, log) on the build machine."""
+    rt = hip_runtime
+    truth_fn, sample = _TRANSCENDENTAL_RANGES[name]
+    x = sample(np.random.RandomState(5), 1 << 20).astype(f32)
+    with np.errstate(all="ignore"):
+        truth = truth_fn(x.astype(np.float64)).astype(f32)
+    want = numpy_ops.unary(name, x)
+    x_d, y_d = rt.array(x), rt.empty(x.shape)
+    sb = FusedSpecBuilder(x.shape)
+    tx, ty = sb.tensor(x_d.ptr, [1]), sb.tensor(y_d.ptr, [1])
+    sb.store(ty, sb.unary(name, sb.load(tx)))
+    rt.launch_fused(sb.build())
+    got = y_d.get()
+    x_d.free()
+    y_d.free()
+    d_truth, d_oracle = _ulps(got, truth), _ulps(got, want)
+    assert np.isfinite(d_truth).all() and np.isfinite(d_oracle).all()      # same infinities, same NaNs
+    worst = int(np.argmax(d_truth))
+    assert d_truth.max() <= 2, (name, x[worst], got[worst], truth[worst])
+    worst = int(np.argmax(d_oracle))
+    assert d_oracle.max() <= 4, (name, x[worst], got[worst], want[worst])
+
+
+def test_sigmoid_and_pow_within_ulps_of_the_oracle(hip_runtime):
+    """sig is the composite 1 / (1 + exp(-x)) on both sides (op_graph.py:4183-4197): the kernel's
+    exp is within 1 ulp of exact and NumPy's within 2, which the division carries into at most 4
+    ulp between the two results; pow stays within 2."""
+    rt = hip_runtime
+    rs = np.random.RandomState(6)
+    n = 1 << 20
+    x = rs.uniform(-87, 87, n).astype(f32)
+    want = numpy_ops.unary("sig", x)
+    x_d, y_d = rt.array(x), rt.empty(x.shape)
+    sb = FusedSpecBuilder(x.shape)
+    tx, ty = sb.tensor(x_d.ptr, [1]), sb.tensor(y_d.ptr, [1])
+    sb.store(ty, sb.unary("sig", sb.load(tx)))
+    rt.launch_fused(sb.build())
+    assert _ulps(y_d.get(), want).max() <= 4
+    base = np.exp(rs.uniform(np.log(1e-3), np.log(1e3), n)).astype(f32)
+    expo = rs.uniform(-8, 8, n).astype(f32)
+    want = numpy_ops.binary("pow", base, expo)
+    b_d, e_d = rt.array(base), rt.array(expo)
+    sb = FusedSpecBuilder(x.shape)
+    tb, te, ty = sb.tensor(b_d.ptr, [1]), sb.tensor(e_d.ptr, [1]), sb.tensor(y_d.ptr, [1])
+    sb.store(ty, sb.binary("pow", sb.load(tb), sb.load(te)))
+    rt.launch_fused(sb.build())
+    assert _ulps(y_d.get(), want).max() <= 2
+    for d in (x_d, y_d, b_d, e_d):
+        d.free()
+
+
 @pytest.mark.parametrize("name", [n for n in BINARY_OPS])
 def test_every_binary_op(hip_runtime, name):
     rt = hip_runtime
