@@ -370,6 +370,63 @@ def test_every_binary_op(hip_runtime, name):
         d.free()
 
 
+_SPECIAL = np.array([0.0, -0.0, 1.0, -1.0, 0.5, -0.5, 2.0, -2.0, 3.0, -3.0, 2.5, -2.5, 1e-38, -1e-38, 1e-45, 3e38,
+                     -3e38, 88.0, -88.0, 104.0, -104.0, 1e6, np.inf, -np.inf, np.nan], dtype=f32)
+
+
+def _assert_same_special(got, want, what, zero_sign=True):
+    """NaN where the oracle has NaN, the same infinities, the same sign of zero; finite values to
+    the tolerance of the ordinary tests."""
+    np.testing.assert_array_equal(np.isnan(got), np.isnan(want), err_msg=what + ": NaN pattern")
+    ok = ~np.isnan(want)
+    inf = ok & np.isinf(want)
+    np.testing.assert_array_equal(got[inf], want[inf], err_msg=what + ": infinities")
+    zero = ok & (want == 0)
+    np.testing.assert_array_equal(got[zero], want[zero], err_msg=what + ": zeros")
+    if zero_sign:
+        np.testing.assert_array_equal(np.signbit(got[zero]), np.signbit(want[zero]), err_msg=what + ": sign of zero")
+    fin = ok & ~inf & ~zero
+    np.testing.assert_allclose(got[fin], want[fin], rtol=RTOL, atol=0, err_msg=what)
+
+
+@pytest.mark.parametrize("name", [n for n in UNARY_OPS])
+def test_unary_ops_on_special_values(hip_runtime, name):
+    """Zeros of both signs, denormals, values that overflow exp, infinities and NaN go through
+    every unary op like through the oracle's NumPy call (cputransform.py:512-761)."""
+    rt = hip_runtime
+    x = np.tile(_SPECIAL, 11)[:256 + 7]                   # a vector body and a scalar tail
+    want = numpy_ops.unary(name, x)
+    x_d, y_d = rt.array(x), rt.empty(x.shape)
+    sb = FusedSpecBuilder(x.shape)
+    tx, ty = sb.tensor(x_d.ptr, [1]), sb.tensor(y_d.ptr, [1])
+    sb.store(ty, sb.unary(name, sb.load(tx)))
+    rt.launch_fused(sb.build())
+    got = y_d.get()
+    x_d.free()
+    y_d.free()
+    _assert_same_special(got, want, name)
+
+
+@pytest.mark.parametrize("name", [n for n in BINARY_OPS])
+def test_binary_ops_on_special_values(hip_runtime, name):
+    """Every pair of the special values through every binary op: division and remainder by zero,
+    NaN in comparisons, minimum / maximum with NaN, powers of zero and of negative numbers."""
+    rt = hip_runtime
+    x, y = (a.ravel().copy() for a in np.meshgrid(_SPECIAL, _SPECIAL, indexing="ij"))
+    want = numpy_ops.binary(name, x, y)
+    x_d, y_d, z_d = rt.array(x), rt.array(y), rt.empty(x.shape)
+    sb = FusedSpecBuilder(x.shape)
+    tx, ty, tz = sb.tensor(x_d.ptr, [1]), sb.tensor(y_d.ptr, [1]), sb.tensor(z_d.ptr, [1])
+    sb.store(tz, sb.binary(name, sb.load(tx), sb.load(ty)))
+    rt.launch_fused(sb.build())
+    got = z_d.get()
+    for d in (x_d, y_d, z_d):
+        d.free()
+    # maximum(+0, -0): NumPy's vector loop returns the second operand and its scalar loop (the
+    # last few elements of an array) the first, so the sign of that zero is not compared
+    _assert_same_special(got, want, name, zero_sign=name not in ("minimum", "maximum"))
+
+
 @pytest.mark.parametrize("name", ["sum", "prod", "max", "min", "argmax", "argmin"])
 @pytest.mark.parametrize("shape,layout", [((64, 10), "row"), ((64, 10), "col"), ((5000, 3), "row"),
                                           ((300, 700), "col"), ((1, 9), "row"), ((40000, 2), "col"),
@@ -412,6 +469,49 @@ def test_every_reduction(hip_runtime, name, shape, layout):
         np.testing.assert_allclose(got, want, rtol=1e-5 if name != "prod" else 1e-4, atol=1e-5)
     x_d.free()
     out_d.free()
+
+
+@pytest.mark.parametrize("layout", ["row", "col"])
+@pytest.mark.parametrize("name", ["sum", "prod", "max", "min", "argmax", "argmin"])
+def test_reductions_over_nan_and_infinities(hip_runtime, name, layout):
+    """Columns holding a NaN, infinities of one sign, of both signs, or only finite values:
+    np.sum / prod / max / min give NaN for a column with a NaN (and sum for +inf with -inf),
+    np.argmax / argmin the position of the first NaN (cputransform.py:521-527, 670-676)."""
+    rt = hip_runtime
+    R, A = 700, 12
+    rs = np.random.RandomState(21)
+    logical = rs.uniform(0.5, 1.5, (R, A)).astype(f32)
+    logical[300, 1] = np.nan
+    logical[5, 2] = np.nan
+    logical[650, 2] = np.nan
+    logical[100, 3] = np.inf
+    logical[101, 4] = -np.inf
+    logical[10, 5] = np.inf
+    logical[600, 5] = -np.inf
+    logical[0, 6] = np.nan
+    logical[R - 1, 7] = np.nan
+    logical[200, 8] = np.inf
+    logical[400, 8] = np.nan
+    logical[50, 9] = np.inf
+    logical[60, 9] = np.inf
+    want = numpy_ops.reduce(name, logical, 0)
+    store, strides = (np.ascontiguousarray(logical.T), [1, R]) if layout == "row" else (logical, [A, 1])
+    x_d = rt.array(store)
+    is_arg = name.startswith("arg")
+    out_d = rt.empty((A,), NGH_I32 if is_arg else NGH_F32)
+    sb = FusedSpecBuilder([R, A])
+    tx = sb.tensor(x_d.ptr, strides)
+    to = sb.tensor(out_d.ptr, [0, 1], NGH_I32 if is_arg else NGH_F32)
+    sb.reduce(name, sb.load(tx), to)
+    rt.launch_fused(sb.build())
+    got = out_d.get()
+    x_d.free()
+    out_d.free()
+    if is_arg:
+        np.testing.assert_array_equal(got, want)
+    else:
+        np.testing.assert_array_equal(np.isnan(got), np.isnan(want))
+        np.testing.assert_allclose(got[~np.isnan(want)], want[~np.isnan(want)], rtol=1e-4)
 
 
 @pytest.mark.parametrize("name", ["argmax", "argmin"])
