@@ -4,6 +4,5 @@
 from the private `autoflex.gpu` package (ngraph/flex/__init__.py:1-4): the
 manager, the per-tensor entry and the 16-bit flex dtype.
 """
-from ngraph_hip.flex.base import Flex, flex16, FlexEntry, FlexManager  # noqa: F401
+from ngraph_hip.flex.base import Flex, flex16, FlexEntry, FlexManager, flex_gpu_transformer_name  # noqa: F401
 from ngraph_hip.flex.hipflex import HipFlexManager, HipFlexEntry, HipFlex, hipflex16  # noqa: F401
-from ngraph_hip.flex.names import flex_gpu_transformer_name  # noqa: F401

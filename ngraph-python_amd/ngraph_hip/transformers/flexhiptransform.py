@@ -23,7 +23,7 @@ from __future__ import division
 import numpy as np
 
 from ngraph_hip.flex import HipFlexManager, hipflex16, HipFlex
-from ngraph_hip.flex.names import flex_gpu_transformer_name
+from ngraph_hip.flex.base import flex_gpu_transformer_name
 from ngraph_hip.op_graph import op_graph as og
 from ngraph_hip.runtime.hiplib import NGH_FLEX16, NGH_SPEC_PROBE
 from ngraph_hip.transformers.hiptransform import (HipTransformer, HipDeviceTensor,
