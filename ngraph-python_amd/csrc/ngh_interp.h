@@ -619,10 +619,11 @@ __global__ __launch_bounds__(kBlock) void red_col_interp_kernel(const KArgs k, u
 }
 
 // ---------------------------------------------------------------------------
-// Reduction along kernel axis 2 for short rows (at most 64 chunks of V): a row
-// takes TR lanes (a power of two), a workgroup 256 / TR rows, and a butterfly
-// inside the TR lanes finishes the row -- no LDS, no idle wavefronts where
-// one workgroup per row would leave most of its 256 threads without work.
+// Reduction along kernel axis 2 for short rows: a row takes TR lanes (a power of
+// two, at most a wavefront; a lane takes every TR-th chunk of V), a workgroup
+// 256 / TR rows, and a butterfly inside the TR lanes finishes the row -- no LDS,
+// no barrier, no idle wavefronts where one workgroup per row would leave most of
+// its 256 threads without work.
 // ---------------------------------------------------------------------------
 template <int V>
 __global__ __launch_bounds__(kBlock) void red_rows_small_interp_kernel(const KArgs k, unsigned n_out, unsigned TR) {
@@ -640,7 +641,8 @@ __global__ __launch_bounds__(kBlock) void red_rows_small_interp_kernel(const KAr
     const unsigned d1 = (unsigned)k.shape[1];
     const unsigned i0 = out / d1, i1 = out - i0 * d1;
     const unsigned chunks = (unsigned)(k.shape[2] / V);
-    if (out < n_out && pos < chunks) run_ops<V, 1>(k, rf, ex, VecAt<V>{i0, i1, (long long)pos * V});
+    if (out < n_out)
+        for (unsigned c = pos; c < chunks; c += TR) run_ops<V, 1>(k, rf, ex, VecAt<V>{i0, i1, (long long)c * V});
     RedWs none{nullptr, nullptr};
     for (int s = 0; s < k.n_red; ++s) {
         const int opc = red_opcode(k, s);

@@ -141,4 +141,57 @@ __global__ __launch_bounds__(kMomBlock) void moments_kernel(
     }
 }
 
+// Many short rows (layer normalisation: tens of thousands of rows of a few thousand elements):
+// L lanes per row (a power of two up to a wavefront), 256 / L rows per workgroup.  Same sums
+// around the same pivot as above, folded by a butterfly inside the L lanes: no partial sums in
+// memory, no tickets, no barrier.
+template <bool NT>
+__global__ __launch_bounds__(kMomBlock) void moments_rows_kernel(
+    const float* __restrict__ x, long long row_stride, unsigned R, unsigned R4, unsigned rows, unsigned L,
+    float* __restrict__ mean, float* __restrict__ var, float* __restrict__ rstd, float eps) {
+    const unsigned row = blockIdx.x * (kMomBlock / L) + threadIdx.x / L;
+    const unsigned pos = threadIdx.x & (L - 1);
+    const bool live = row < rows;                       // (idle lanes still take part in the butterfly)
+    const float* xr = x + (long long)(live ? row : 0) * row_stride;
+    const float pivot = xr[0];
+    const float4* x4 = reinterpret_cast<const float4*>(xr);
+    float s1[kMomUnroll], s2[kMomUnroll];
+#pragma unroll
+    for (int u = 0; u < kMomUnroll; ++u) s1[u] = s2[u] = 0.0f;
+    // (a lane's last turn may hold fewer than kMomUnroll chunks: the missing ones count as the
+    // pivot, which adds nothing -- every lane of a row leaves the loop in the same turn)
+    for (unsigned c = pos; live && c < R4; c += kMomUnroll * L) {
+        float4 v[kMomUnroll];
+#pragma unroll
+        for (int u = 0; u < kMomUnroll; ++u)
+            v[u] = (c + u * L < R4) ? mom_load<NT>(x4 + c + u * L) : make_float4(pivot, pivot, pivot, pivot);
+#pragma unroll
+        for (int u = 0; u < kMomUnroll; ++u) {
+            const float a = v[u].x - pivot, b = v[u].y - pivot, cc = v[u].z - pivot, d = v[u].w - pivot;
+            s1[u] += (a + b) + (cc + d);
+            s2[u] += (a * a + b * b) + (cc * cc + d * d);
+        }
+    }
+    if (live)
+        for (unsigned i = R4 * 4 + pos; i < R; i += L) {     // elements past the last whole float4
+            const float a = xr[i] - pivot;
+            s1[0] += a;
+            s2[0] += a * a;
+        }
+    float t1 = (s1[0] + s1[1]) + (s1[2] + s1[3]);
+    float t2 = (s2[0] + s2[1]) + (s2[2] + s2[3]);
+    for (unsigned m = L >> 1; m > 0; m >>= 1) {
+        t1 += __shfl_xor(t1, (int)m, 64);
+        t2 += __shfl_xor(t2, (int)m, 64);
+    }
+    if (live && pos == 0) {
+        const float inv = 1.0f / (float)R;
+        const float d = t1 * inv;
+        const float v = fmaxf(t2 * inv - d * d, 0.0f);
+        mean[row] = pivot + d;
+        var[row] = v;
+        if (rstd) rstd[row] = 1.0f / sqrtf(v + eps);
+    }
+}
+
 }  // namespace ngh

@@ -120,6 +120,7 @@ struct ngh_context {
     int         force_interp = 0;    // never pick a specialised kernel
     int         red_wgs_per_cu = 8;  // workgroups per CU a split reduction along the contiguous axis aims for
     int         red_col_wgs_per_cu = 2;  // ... and one across it
+    int         row_wave_chunks = 0;     // rows of up to this many chunks are reduced by one wavefront each
     int         no_tiles = 0;        // never use the LDS-tiled elementwise skeleton
     int         flex_self_managed = 2;  // ngh_launch_fused_flex: 0 = prepare / kernel / update launches,
                                      // 1 = policy at the end of the kernel, 2 = statistics deferred to the next user
@@ -265,6 +266,7 @@ int validate(const ngh_fused_spec* sp) {
 // planner
 // ---------------------------------------------------------------------------
 enum Family { F_EW = 0, F_RED_ROW, F_RED_COL, F_EW_TILED };
+constexpr int kRowWaveChunks = 512;
 
 struct Plan {
     Family   family = F_EW;
@@ -584,6 +586,23 @@ int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage,
             P.small_rows = true;
             P.tx = 1;
             while ((long long)P.tx < chunks) P.tx <<= 1;
+            // with rows enough to fill the chip several times over, a lane takes up to four chunks
+            // of its row (all in flight at once) and a quarter of the wavefronts do the work
+            const long long lanes_wanted = (ctx ? ctx->cus : 256) * 2048LL * 4;
+            for (int shrink = 0; shrink < 2 && P.tx > 1 && (long long)n_out * (P.tx / 2) >= lanes_wanted; ++shrink)
+                P.tx >>= 1;
+            P.n_seg = 1;
+            P.seg_len = (unsigned)chunks;
+            return NGH_OK;
+        }
+        // rows of a few thousand elements, and enough of them to fill the chip that way: a
+        // wavefront per row, every lane several chunks, the same butterfly -- a workgroup per
+        // row would spend its time on the barrier and the launch of a workgroup per kilobyte
+        const long long wave_chunks = ctx ? ctx->row_wave_chunks : kRowWaveChunks;
+        const long long cus = ctx ? ctx->cus : 256;
+        if (chunks <= wave_chunks && (long long)n_out >= cus * 4 * kWaves) {
+            P.small_rows = true;
+            P.tx = 64;
             P.n_seg = 1;
             P.seg_len = (unsigned)chunks;
             return NGH_OK;
@@ -963,6 +982,7 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->no_tiles = env_int("NGH_NO_TILES", 0);
     ctx->red_wgs_per_cu = std::max(1, env_int("NGH_RED_WGS_PER_CU", 8));
     ctx->red_col_wgs_per_cu = std::max(1, env_int("NGH_RED_COL_WGS_PER_CU", 2));
+    ctx->row_wave_chunks = std::max(0, env_int("NGH_ROW_WAVE_CHUNKS", kRowWaveChunks));
     ctx->cache_policy = env_int("NGH_CACHE_POLICY", -1);
     ctx->stream_bytes = (long long)env_int("NGH_STREAM_MIB", 192) << 20;
     ctx->moments_wgs_per_cu = std::max(1, env_int("NGH_MOMENTS_WGS_PER_CU", 8));
@@ -1254,7 +1274,11 @@ int ngh_programs_count(int32_t* built_in, int32_t* loaded) {
 namespace {
 // How ngh_moments_f32 splits rows into segments: enough workgroups to fill the chip, but at
 // least 4 unrolled sweeps per segment.
-struct MomentsPlan { unsigned R4, seg_chunks, n_seg; };
+struct MomentsPlan {
+    unsigned R4, seg_chunks, n_seg;
+    bool per_wave;       // many short rows: `lanes` lanes per row, no partial sums (moments_rows_kernel)
+    unsigned lanes;
+};
 
 int plan_moments(const ngh_context* ctx, const float* dev_x, int64_t rows, int64_t R, int64_t row_stride,
                  const float* dev_mean, const float* dev_var, MomentsPlan& m) {
@@ -1265,6 +1289,13 @@ int plan_moments(const ngh_context* ctx, const float* dev_x, int64_t rows, int64
         return fail(NGH_E_UNSUPPORTED, "rows must start on 16-byte boundaries");
     if (rows >= (1LL << 24) || R >= (1LL << 32)) return fail(NGH_E_UNSUPPORTED, "extent too large");
     m.R4 = (unsigned)(R / 4);
+    m.per_wave = (long long)m.R4 <= ctx->row_wave_chunks * 2 && rows >= (long long)ctx->cus * 4 * (kMomBlock / 64);
+    // a lane per chunk of the row, up to a wavefront; with rows enough to fill the chip several
+    // times over, a quarter of that (each lane then has four chunks in flight)
+    m.lanes = 1;
+    while (m.lanes < 64 && m.lanes < m.R4) m.lanes <<= 1;
+    for (int shrink = 0; shrink < 2 && m.lanes > 1 && rows * (long long)(m.lanes / 2) >= (long long)ctx->cus * 2048 * 4; ++shrink)
+        m.lanes >>= 1;
     long long seg = std::max<long long>(1, (long long)ctx->cus * ctx->moments_wgs_per_cu / rows);
     seg = std::min<long long>(seg, std::max<long long>(1, m.R4 / (kMomBlock * kMomUnroll * 2)));
     seg = std::min<long long>(seg, 4096);
@@ -1279,6 +1310,20 @@ int launch_moments(ngh_context* ctx, const MomentsPlan& m, const float* dev_x, i
     const bool stream_x = ctx->cache_policy >= 0
                               ? (ctx->cache_policy & 1)
                               : ((x_cache_hint & NGH_CACHE_STREAM_LOAD) && rows * R * 4 >= ctx->stream_bytes);
+    if (m.per_wave) {
+        const unsigned rows_per_wg = kMomBlock / m.lanes;
+        const dim3 row_grid((unsigned)((rows + rows_per_wg - 1) / rows_per_wg));
+        if (stream_x)
+            hipLaunchKernelGGL(moments_rows_kernel<true>, row_grid, dim3(kMomBlock), 0, ctx->stream, dev_x,
+                               (long long)row_stride, (unsigned)R, m.R4, (unsigned)rows, m.lanes, dev_mean, dev_var,
+                               dev_rstd, eps);
+        else
+            hipLaunchKernelGGL(moments_rows_kernel<false>, row_grid, dim3(kMomBlock), 0, ctx->stream, dev_x,
+                               (long long)row_stride, (unsigned)R, m.R4, (unsigned)rows, m.lanes, dev_mean, dev_var,
+                               dev_rstd, eps);
+        HIP_TRY(hipGetLastError());
+        return NGH_OK;
+    }
     const dim3 grid((unsigned)(rows * m.n_seg));
     if (stream_x)
         hipLaunchKernelGGL(moments_kernel<true>, grid, dim3(kMomBlock), 0, ctx->stream, dev_x, (long long)row_stride,
@@ -1299,8 +1344,10 @@ int ngh_moments_f32(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t 
     MomentsPlan m;
     NGH_TRY(plan_moments(ctx, dev_x, rows, R, row_stride, dev_mean, dev_var, m));
     if (rows == 0) return NGH_OK;
-    NGH_TRY(ensure_ws(ctx, (size_t)rows * m.n_seg * sizeof(float2)));
-    NGH_TRY(ensure_tickets(ctx, (size_t)rows));
+    if (!m.per_wave) {
+        NGH_TRY(ensure_ws(ctx, (size_t)rows * m.n_seg * sizeof(float2)));
+        NGH_TRY(ensure_tickets(ctx, (size_t)rows));
+    }
     return launch_moments(ctx, m, dev_x, rows, R, row_stride, (float2*)ctx->ws, ctx->tickets, dev_mean, dev_var,
                           dev_rstd, eps, x_cache_hint);
 }
@@ -1311,6 +1358,9 @@ int ngh_moments_f32_noalloc(ngh_context* ctx, const float* dev_x, int64_t rows, 
     MomentsPlan m;
     NGH_TRY(plan_moments(ctx, dev_x, rows, R, row_stride, dev_mean, dev_var, m));
     if (rows == 0) return NGH_OK;
+    if (m.per_wave)            // a wavefront per row: no scratch at all
+        return launch_moments(ctx, m, dev_x, rows, R, row_stride, nullptr, nullptr, dev_mean, dev_var, dev_rstd, eps,
+                              x_cache_hint);
     if ((size_t)rows > kNoAllocRows || (size_t)rows * m.n_seg > kNoAllocPartials)
         return fail(NGH_E_UNSUPPORTED, "ngh_moments_f32_noalloc: %lld rows in %u segments each exceed the fixed scratch "
                     "(%zu rows, %zu partial sums); use ngh_moments_f32", (long long)rows, m.n_seg, kNoAllocRows,

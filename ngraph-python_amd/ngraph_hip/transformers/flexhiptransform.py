@@ -263,6 +263,7 @@ class FlexHipTransformer(HipTransformer):
     atol_precision_multiplier = 8
     kernel_group_class = FlexHipKernelGroup
     max_written_views = 4        # a kernel merges max|mantissa| for at most 4 flex results
+    split_reductions = False     # an intermediate result would be rounded to flex16 on its way
 
     def __init__(self, fixed_point=False, flex_verbose=False, collect_flex_data=False,
                  resident=True, **kwargs):

@@ -1482,6 +1482,7 @@ class HipTransformer(ComputationGraphTransformer):
 
     kernel_group_class = HipKernelGroup
     max_written_views = NGH_MAX_TENSORS      # results one fused kernel may write
+    split_reductions = True                  # ReductionLayoutPass: reduce group by group of axes, no copy
 
     def __init__(self, device_id=0, fusion=True, dry_run=False, fuse_moments=None, rng_seed=0, jit=None,
                  jit_min_elements=4096, jit_auto_min_elements=1 << 22, **kwargs):
@@ -1510,7 +1511,7 @@ class HipTransformer(ComputationGraphTransformer):
         self.graph_passes = [SimplePrune(), TensorSizeFold(), ConstantFoldPass(), SimplePrune()]
         if fusion if fuse_moments is None else fuse_moments:
             self.graph_passes.append(MomentsFusionPass())
-        self.graph_passes.append(ReductionLayoutPass())
+        self.graph_passes.append(ReductionLayoutPass(split=self.split_reductions))
 
     # -- dtype mapping ---------------------------------------------------------------------
     def ngh_dtype(self, dtype):

@@ -2,7 +2,8 @@
 
 * TensorSizeFold      TensorSizeOp becomes a constant;
 * ConstantFoldPass    elementwise ops on scalar constants are evaluated at transform time;
-* ReductionLayoutPass a reduction whose reduced axes do not form one strided axis gets a copy
+* ReductionLayoutPass a reduction whose reduced axes do not form one strided axis is taken in
+                      steps over groups of axes that do, or (argmax / argmin, flex) gets a copy
                       of its operand in (reduced..., kept...) order -- where the reference
                       inserts a DimshuffleOp (gpulayout.py:861-979, layout_common.py:347-378).
 
@@ -56,14 +57,42 @@ def axes_merge_to_one(td, axes):
     return True
 
 
+def strided_axis_groups(td, axes):
+    """`axes` of the view `td` partitioned into groups that can each be walked as one strided
+    dimension (outermost group first)."""
+    dims = sorted(((td.full_strides[td.axes.index(a)], a) for a in axes if a.length != 1), key=lambda d: -d[0])
+    groups = []
+    for stride, axis in dims:
+        if groups and groups[-1][1] == stride * axis.length:
+            groups[-1][0].append(axis)
+            groups[-1][1] = stride
+        else:
+            groups.append([[axis], stride])
+    groups = [g[0] for g in groups]
+    unit = [a for a in axes if a.length == 1]
+    if unit:
+        groups = ([groups[0] + unit] + groups[1:]) if groups else [unit]
+    return groups
+
+
 class ReductionLayoutPass(PeepholeGraphPass):
     """Reductions need their reduced axes to form one strided axis.
 
-    When they do not, the operand is first copied into (reduced..., kept...)
-    order; this is the layout conversion the reference inserts as a
-    DimshuffleOp for the same reason (gpulayout.py:861-979,
-    layout_common.py:347-378).
+    When they do not, the reference copies the operand into (reduced..., kept...) order with a
+    DimshuffleOp (gpulayout.py:861-979, layout_common.py:347-378): a full extra read and write
+    of the operand.  With `split`, a sum, product, maximum or minimum is instead taken group by
+    group of axes that do form one strided axis, the largest group first -- sum over (N, HW) of
+    an [N, C, HW] tensor becomes sum over N of (sum over HW): one pass over the operand and a
+    small second reduction, no copy.  The result is the same reduction in another association
+    order; argmax / argmin (whose results are positions in the original axis), and storage
+    types that round every stored intermediate (`split=False`), keep the copy.
     """
+
+    _SPLITTABLE = ("Sum", "Prod", "Max", "Min")
+
+    def __init__(self, split=True, **kwargs):
+        super(ReductionLayoutPass, self).__init__(**kwargs)
+        self.split = split
 
     def visit(self, op, *args):
         if not isinstance(op, ReductionOp) or len(op.reduction_axes) < 2:
@@ -71,6 +100,15 @@ class ReductionLayoutPass(PeepholeGraphPass):
         x, = args
         if axes_merge_to_one(_td(x), op.reduction_axes):
             return
+        if self.split and type(op).__name__ in self._SPLITTABLE:
+            groups = strided_axis_groups(_td(x), op.reduction_axes)
+            if len(groups) > 1:
+                first = max(groups, key=lambda g: int(np.prod([a.length for a in g])))
+                rest = [a for a in op.reduction_axes if a not in first]
+                inner = type(op)(x, reduction_axes=first, dtype=op.dtype)
+                # (the outer reduction is visited in the next sweep and split again if need be)
+                self.replace_op(op, type(op)(inner, reduction_axes=rest, dtype=op.dtype))
+                return
         order = op.reduction_axes + (x.axes - op.reduction_axes)
         new_x = ContiguousOp(axes_with_order(x, order))
         self.replace_op(op, type(op)(new_x, reduction_axes=op.reduction_axes, dtype=op.dtype))

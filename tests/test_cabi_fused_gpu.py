@@ -431,7 +431,10 @@ def test_binary_ops_on_special_values(hip_runtime, name):
 @pytest.mark.parametrize("shape,layout", [((64, 10), "row"), ((64, 10), "col"), ((5000, 3), "row"),
                                           ((300, 700), "col"), ((1, 9), "row"), ((40000, 2), "col"),
                                           # many columns: the whole workgroup lies along them
-                                          ((300, 4096), "col"), ((37, 4100), "col"), ((2000, 1027), "col")])
+                                          ((300, 4096), "col"), ((37, 4100), "col"), ((2000, 1027), "col"),
+                                          # thousands of rows of a few hundred chunks: a wavefront per row
+                                          ((1024, 4200), "row"), ((300, 5000), "row"), ((401, 4100), "row"),
+                                          ((2048, 4096), "row")])
 def test_every_reduction(hip_runtime, name, shape, layout):
     """Reduce axis 0 of an [R, A] view; 'row' = R contiguous in memory, 'col' = A contiguous."""
     rt = hip_runtime
@@ -604,10 +607,13 @@ def test_column_reductions_with_elementwise_stores_over_many_columns(hip_runtime
 
 # ------------------------------------------------------------------ one-pass moments
 @pytest.mark.parametrize("rows,R,pad", [(1, 1, 3), (3, 2, 2), (5, 7, 1), (4, 1024, 0), (256, 3136, 0),
-                                        (2, 1000003, 1), (700, 260, 0), (1, 4, 0)])
+                                        (2, 1000003, 1), (700, 260, 0), (1, 4, 0),
+                                        # many short rows: a wavefront per row
+                                        (4096, 1024, 0), (5000, 1027, 1), (70000, 3, 1), (4100, 4096, 0),
+                                        (4100, 4100, 0)])
 def test_moments_rows(hip_runtime, rows, R, pad):
     """ngh_moments_f32 against float64 row statistics; rows of every length class (shorter than
-    a vector, ragged tails, many segments), with a row stride wider than the row.  Launched
+    a vector, ragged tails, many segments, thousands of short rows), with a row stride wider than the row.  Launched
     twice: the second launch checks that the arrival counters were left at zero."""
     rt = hip_runtime
     rs = np.random.RandomState(rows * 7 + R)

@@ -160,6 +160,45 @@ def test_reduction_out_axes_and_noncontiguous(backend):
         np.testing.assert_allclose(f(xv), xv.sum(axis=(1, 3)), rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("ng_fn,np_fn", [(ng.sum, np.sum), (ng.prod, np.prod), (ng.max, np.max), (ng.min, np.min)])
+def test_reduction_over_axes_that_are_not_adjacent(backend, ng_fn, np_fn):
+    """[N, C, H, W] reduced over N, H and W keeping C (the batch-norm statistics of the N-major
+    layout), over N and W, and over C and W: the reduced axes form two strided groups."""
+    ax = axes(N=6, C=5, H=7, W=9)
+    x = ng.placeholder(ax)
+    xv = rng.uniform(0.8, 1.25, ax)
+    keep = [(ax[1:2], (0, 2, 3)), (ax[1:3], (0, 3)), (ax[0:1] + ax[2:3], (1, 3))]
+    with executor([ng_fn(x, out_axes=out) for out, _ in keep], x) as f:
+        got = f(xv)
+    for g, (_, reduced) in zip(got, keep):
+        np.testing.assert_allclose(g, np_fn(xv, axis=reduced), rtol=1e-5, atol=1e-6)
+
+
+def _kernels_lowered_for(results, placeholders, backend="hipgpu"):
+    t = ngt.make_transformer_factory(backend, dry_run=True, jit=False)()
+    try:
+        f = t.computation(results, *placeholders)
+        t.initialize()
+        return [type(k).__name__ for k in t.kernel_groups[f].kernels]
+    finally:
+        t.close()
+
+
+def test_split_reductions_need_no_copy_of_the_operand():
+    """Sum / prod / max / min over axes in two strided groups are taken group by group (one
+    pass over the operand, then a small reduction); argmax, whose result is a position along the
+    original axes, and flex tensors, which would round the intermediate, copy the operand into
+    (reduced, kept) order first, as the reference does (layout_common.py:347-378)."""
+    ax = axes(N=6, C=5, H=7, W=9)
+    x = ng.placeholder(ax)
+    keep_c = ax[1:2]
+    for fn in (ng.sum, ng.prod, ng.max, ng.min):
+        assert "CopyKernel" not in _kernels_lowered_for([fn(x, out_axes=keep_c)], [x]), fn.__name__
+    flat = ng.flatten_at(ng.axes_with_order(x, ax[0:1] + ax[2:4] + ax[1:2]), 3)
+    assert "CopyKernel" in _kernels_lowered_for([ng.argmax(flat, out_axes=flat.axes[1:])], [x])
+    assert "FlexCopyKernel" in _kernels_lowered_for([ng.sum(x, out_axes=keep_c)], [x], backend="flexhip")
+
+
 def test_argmax_argmin_first_index_wins(backend):
     ax = axes(C=7, N=9)
     x = ng.placeholder(ax)

@@ -36,7 +36,9 @@ def test_noalloc_moments_equal_the_allocating_entry_point(hip_runtime):
     rs = np.random.RandomState(11)
     # first call: many segments per row; second: smaller, other segmenting, rows not a power of two;
     # third: more rows than compute units (one segment each), R not a multiple of 4
-    for rows, R in ((256, 100352), (37, 4100), (3000, 515)):
+    # then many short rows, which a wavefront each reduces without any scratch (whole float4s
+    # only, a ragged end, rows shorter than a float4, the longest rows that go this way)
+    for rows, R in ((256, 100352), (37, 4100), (3000, 515), (8192, 64), (4500, 1027), (5000, 3), (4096, 4096)):
         x = rs.normal(0.5, 2.0, (rows, R)).astype(f32)
         want, got = _both(rt, x)
         assert not np.isnan(got).any()
@@ -51,8 +53,10 @@ def test_noalloc_moments_reject_what_the_fixed_scratch_cannot_hold(hip_runtime):
     rt = hip_runtime
     x_d, o_d = rt.empty((16,)), rt.empty((3,))
     with pytest.raises(HipLibraryError) as e:
-        # 70000 rows: more arrival counters than the array has (nothing is launched)
-        rt.moments_f32_noalloc(x_d.ptr, 70000, 4, 0, o_d.ptr, o_d.ptr, None, 0.0)
+        # 70000 rows of 8192 elements: more arrival counters than the array has (nothing is
+        # launched; rows of up to 4096 elements would take the wavefront-per-row kernel, which
+        # needs no scratch and has no such limit)
+        rt.moments_f32_noalloc(x_d.ptr, 70000, 8192, 0, o_d.ptr, o_d.ptr, None, 0.0)
     assert e.value.code == -4 and "scratch" in str(e.value)
     x_d.free()
     o_d.free()
