@@ -561,6 +561,15 @@ int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage,
         const long long col_target = compiled ? (ctx ? ctx->cus * ctx->red_col_wgs_per_cu : 256 * 2) : target_wgs;
         const bool wide = compiled && col_chunks >= kBlock && R * n_out > kSmallReduction && R >= 64;
         if (wide) P.tx = kBlock;
+        if (R * n_out <= kSmallReduction) {
+            // A small problem is bound by latency: every row a lane walks down is a round trip
+            // that depends on the one before.  Narrower column groups put more lanes on each
+            // column (64 / TX rows per wavefront at once) while the workgroups still fit the chip.
+            const long long cus = ctx ? ctx->cus : 256;
+            while (P.tx > 4 && R > (long long)kWaves * (64 / P.tx) &&
+                   ((col_chunks + P.tx / 2 - 1) / (P.tx / 2)) * P.k.shape[1] <= cus * 2)
+                P.tx >>= 1;
+        }
         P.n_bx = (unsigned)((col_chunks + P.tx - 1) / P.tx);
         const long long rows_per_pass = wide ? 1 : (long long)kWaves * (64 / P.tx);
         const long long base_wgs = (long long)P.n_bx * P.k.shape[1];
