@@ -21,6 +21,7 @@ __global__ __launch_bounds__(kCopyBlock) void fill_kernel(T* p, T value, size_t 
 
 struct CopyArgs {
     int       rank;
+    int       diagonal;   // transpose kernels: deal the tiles along diagonals (see copy_diagonal)
     unsigned  total;
     long long shape[kCopyMaxRank];
     long long ds[kCopyMaxRank];   // destination element strides
@@ -52,6 +53,19 @@ __global__ __launch_bounds__(kCopyBlock) void copy_nd_kernel(T* dst, const T* sr
 // both the global read and the global write are coalesced.
 constexpr int kCopyTile = 64;
 
+// When both strided strides are multiples of 4 KiB, tiles are dealt along diagonals: consecutive
+// workgroups differ in both tile coordinates.  The tiles of one tile row then start a multiple of
+// a large power of two apart on the strided side and fall on the same few memory channels; in
+// row-major order the workgroups resident at one time would all read (or all write) through
+// those few channels (8192 x 8192 fp32: 131 us row-major, 102 us along diagonals).  With other
+// strides row-major order is the faster one by a few per cent.
+__device__ __forceinline__ unsigned copy_diagonal(unsigned row, unsigned col, unsigned n_rows, int diagonal) {
+    return diagonal ? (row + col) % n_rows : row;
+}
+inline int copy_wants_diagonal(long long stride_a, long long stride_b, int itemsize) {
+    return (stride_a * itemsize) % 4096 == 0 && (stride_b * itemsize) % 4096 == 0;
+}
+
 template <typename T>
 __global__ __launch_bounds__(kCopyBlock) void copy_tr_kernel(T* dst, const T* src, const CopyArgs a,
                                                              unsigned tiles_r, unsigned tiles_c) {
@@ -60,7 +74,7 @@ __global__ __launch_bounds__(kCopyBlock) void copy_tr_kernel(T* dst, const T* sr
     const unsigned R = (unsigned)a.shape[r_ax], C = (unsigned)a.shape[c_ax];
     unsigned b = blockIdx.x;
     const unsigned tc = b % tiles_c; b /= tiles_c;
-    const unsigned tr = b % tiles_r; b /= tiles_r;
+    const unsigned tr = copy_diagonal(b % tiles_r, tc, tiles_r, a.diagonal); b /= tiles_r;
     long long so = 0, dof = 0;
     for (int ax = r_ax - 1; ax >= 0; --ax) {
         const unsigned d = (unsigned)a.shape[ax];
@@ -108,14 +122,20 @@ __global__ __launch_bounds__(kCopyBlock) void copy_vec_kernel(T* dst, const T* s
 // consecutive source rows-elements (float4 along the source-contiguous axis), scatters them
 // into the padded tile, and after the barrier gathers four tile elements that are consecutive
 // along the destination-contiguous axis.  Needs R, C and the strides to be multiples of 4.
+// TILE x TILE elements per workgroup: 64 (contiguous runs of 256 bytes on both sides) or 128
+// (512 bytes, 65 KiB of LDS) for matrices with enough tiles of that size to fill the chip.
+template <int TILE>
 __global__ __launch_bounds__(kCopyBlock) void copy_tr4_kernel(uint32_t* dst, const uint32_t* src, const CopyArgs a,
                                                               unsigned tiles_r, unsigned tiles_c) {
-    __shared__ uint32_t tile[kCopyTile][kCopyTile + 1];     // [c_local][r_local]
+    constexpr int kChunks = TILE / 4;                      // float4 chunks along a tile edge
+    constexpr int kLines = kCopyBlock / kChunks;           // tile lines the workgroup covers per turn
+    constexpr int kTurns = TILE / kLines;
+    __shared__ uint32_t tile[TILE][TILE + 1];              // [c_local][r_local]
     const int r_ax = a.rank - 2, c_ax = a.rank - 1;
     const unsigned R = (unsigned)a.shape[r_ax], C = (unsigned)a.shape[c_ax];
     unsigned b = blockIdx.x;
     const unsigned tc = b % tiles_c; b /= tiles_c;
-    const unsigned tr = b % tiles_r; b /= tiles_r;
+    const unsigned tr = copy_diagonal(b % tiles_r, tc, tiles_r, a.diagonal); b /= tiles_r;
     long long so = 0, dof = 0;
     for (int ax = r_ax - 1; ax >= 0; --ax) {
         const unsigned d = (unsigned)a.shape[ax];
@@ -124,24 +144,24 @@ __global__ __launch_bounds__(kCopyBlock) void copy_tr4_kernel(uint32_t* dst, con
         so += (long long)i * a.ss[ax];
         dof += (long long)i * a.ds[ax];
     }
-    const unsigned cx = threadIdx.x & 15, j = threadIdx.x >> 4;     // 16 chunks of 4 x 16 lines
-    uint4 v[4];
+    const unsigned cx = threadIdx.x % kChunks, j = threadIdx.x / kChunks;
+    uint4 v[kTurns];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const unsigned c = tc * kCopyTile + j + 16 * i, r = tr * kCopyTile + cx * 4;
+    for (int i = 0; i < kTurns; ++i) {
+        const unsigned c = tc * TILE + j + kLines * i, r = tr * TILE + cx * 4;
         v[i] = make_uint4(0, 0, 0, 0);
         if (r < R && c < C) v[i] = *reinterpret_cast<const uint4*>(src + so + (long long)c * a.ss[c_ax] + r);
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        uint32_t* row = tile[j + 16 * i] + cx * 4;
+    for (int i = 0; i < kTurns; ++i) {
+        uint32_t* row = tile[j + kLines * i] + cx * 4;
         row[0] = v[i].x; row[1] = v[i].y; row[2] = v[i].z; row[3] = v[i].w;
     }
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const unsigned rl = j + 16 * i;
-        const unsigned r = tr * kCopyTile + rl, c = tc * kCopyTile + cx * 4;
+    for (int i = 0; i < kTurns; ++i) {
+        const unsigned rl = j + kLines * i;
+        const unsigned r = tr * TILE + rl, c = tc * TILE + cx * 4;
         if (r < R && c < C) {
             const uint4 w = make_uint4(tile[cx * 4][rl], tile[cx * 4 + 1][rl], tile[cx * 4 + 2][rl], tile[cx * 4 + 3][rl]);
             *reinterpret_cast<uint4*>(dst + dof + (long long)r * a.ds[r_ax] + c) = w;
@@ -159,7 +179,8 @@ inline bool copy_aligned(const void* dst, const void* src, const CopyArgs& a, in
 }
 
 template <typename T>
-inline hipError_t launch_copy_t(hipStream_t stream, int cus, void* dst, const void* src, const CopyArgs& a) {
+inline hipError_t launch_copy_t(hipStream_t stream, int cus, void* dst, const void* src, const CopyArgs& plain) {
+    const CopyArgs& a = plain;
     constexpr int V = 16 / (int)sizeof(T);
     const int last = a.rank - 1;
     if (a.rank >= 1 && a.ss[last] == 1 && a.ds[last] == 1 && a.shape[last] % V == 0 &&
@@ -179,13 +200,23 @@ inline hipError_t launch_copy_t(hipStream_t stream, int cus, void* dst, const vo
         unsigned long long blocks = (unsigned long long)tiles_r * tiles_c;
         for (int ax = 0; ax < a.rank - 2; ++ax) blocks *= (unsigned long long)a.shape[ax];
         if (blocks < (1ULL << 31)) {
+            CopyArgs a = plain;
+            a.diagonal = copy_wants_diagonal(a.ss[a.rank - 1], a.ds[a.rank - 2], (int)sizeof(T));
             if constexpr (sizeof(T) == 4) {
                 // 16-byte accesses: the source is read along r, the destination written along c
                 if (a.shape[a.rank - 2] % 4 == 0 && a.shape[a.rank - 1] % 4 == 0 &&
                     a.ss[a.rank - 1] % 4 == 0 && a.ds[a.rank - 2] % 4 == 0 &&
                     copy_aligned(dst, src, a, a.rank - 2, a.rank - 1, 4)) {
-                    hipLaunchKernelGGL(copy_tr4_kernel, dim3((unsigned)blocks), dim3(kCopyBlock), 0, stream,
-                                       (uint32_t*)dst, (const uint32_t*)src, a, tiles_r, tiles_c);
+                    const unsigned big_r = (unsigned)((a.shape[a.rank - 2] + 127) / 128);
+                    const unsigned big_c = (unsigned)((a.shape[a.rank - 1] + 127) / 128);
+                    const unsigned long long big_blocks = blocks / ((unsigned long long)tiles_r * tiles_c) * big_r * big_c;
+                    // (measured: 8192 x 8192 102 -> 95 us, 16384 x 4096 108 -> 102 us; strides off the 4 KiB grid lose a few per cent)
+                    if (a.diagonal && big_blocks >= (unsigned long long)cus * 8)
+                        hipLaunchKernelGGL(copy_tr4_kernel<128>, dim3((unsigned)big_blocks), dim3(kCopyBlock), 0, stream,
+                                           (uint32_t*)dst, (const uint32_t*)src, a, big_r, big_c);
+                    else
+                        hipLaunchKernelGGL(copy_tr4_kernel<64>, dim3((unsigned)blocks), dim3(kCopyBlock), 0, stream,
+                                           (uint32_t*)dst, (const uint32_t*)src, a, tiles_r, tiles_c);
                     return hipGetLastError();
                 }
             }

@@ -51,6 +51,7 @@ struct KArgs {
     int       iota_map[3];   // kernel axis holding spec axis k (for NGH_OP_IOTA)
     int       n_stat_slots;
     int       n_staged;      // tiled skeleton: operands staged through LDS tiles
+    int       tile_diagonal; // tiled skeleton: deal the tiles along diagonals (strides that are multiples of 4 KiB)
     unsigned  rng_seed, rng_counter;   // NGH_OP_RNG_*
     int       probe;         // NGH_SPEC_PROBE: record max|value| bits instead of storing
     int*      stat_ptr[4];   // device word of each per-thread accumulator

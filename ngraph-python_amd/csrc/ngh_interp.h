@@ -397,7 +397,11 @@ __global__ __launch_bounds__(kBlock) void ew_tiled_interp_kernel(const KArgs k, 
     for (unsigned tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const unsigned tb = tile % tiles_b;
         const unsigned r = tile / tiles_b;
-        const unsigned ta = r % tiles_a;
+        // With strides that are multiples of 4 KiB, tiles are dealt along diagonals (consecutive
+        // workgroups differ in both tile coordinates): the tiles of one tile row then start a
+        // multiple of a large power of two apart on the transposed operand, on the same few memory
+        // channels, and in row-major order all resident workgroups would go through those at once.
+        const unsigned ta = k.tile_diagonal ? (r % tiles_a + tb) % tiles_a : r % tiles_a;
         const unsigned i0 = r / tiles_a;
         const unsigned a0 = ta * kTile, b0 = tb * kTile;
         // stage in: lanes along axis 1

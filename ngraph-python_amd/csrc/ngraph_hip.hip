@@ -471,6 +471,12 @@ int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage,
                         kt.t[t].stage_slot = n_staged++;
                 }
                 kt.n_staged = n_staged;
+                kt.tile_diagonal = 1;
+                for (int t = 0; t < sp.n_tensors; ++t) {
+                    if (!used[t]) continue;
+                    const long long strided = kt.t[t].stage_slot >= 0 ? kt.t[t].s[2] : kt.t[t].s[1];
+                    if ((strided * itemsize_of(kt.t[t].dtype)) % 4096 != 0) kt.tile_diagonal = 0;
+                }
                 // small problems take 16 x 16 tiles: four times the workgroups, one element per lane
                 int tile = kTile;
                 if (kt.shape[0] * ((kt.shape[1] + 31) / 32) * ((kt.shape[2] + 31) / 32) < 4LL * (ctx ? ctx->cus : 256))

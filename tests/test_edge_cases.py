@@ -172,6 +172,26 @@ def test_strided_copy_all_permutations(hip_runtime, shape, itemsize):
 
 
 @gpu
+@pytest.mark.parametrize("rows,cols", [(8192, 4096), (8000, 4000), (4100, 2052)])
+def test_transposes_whose_strides_are_multiples_of_4_kib(hip_runtime, rows, cols):
+    """Transposes between buffers whose row pitch is a multiple of 4 KiB take the tiles along
+    diagonals (and 128 x 128 tiles when there are enough of them); sub-views leave ragged tiles at
+    the edges and must not touch what lies outside them."""
+    rt = hip_runtime
+    src = np.arange(8192 * 4096, dtype=np.float32).reshape(8192, 4096)
+    s_d = rt.array(src)
+    d_d = rt.empty((4096, 8192))
+    rt.memset32(d_d.ptr, 0x7fc00000, 4096 * 8192)
+    # dst[c, r] = src[r, c] for r < rows, c < cols
+    rt.copy_strided(d_d.ptr, s_d.ptr, (cols, rows), (8192, 1), (1, 4096), 4)
+    got = d_d.get()
+    np.testing.assert_array_equal(got[:cols, :rows], src[:rows, :cols].T)
+    assert np.isnan(got[cols:, :]).all() and np.isnan(got[:, rows:]).all()
+    s_d.free()
+    d_d.free()
+
+
+@gpu
 def test_strided_copy_argument_checks(hip_runtime):
     from ngraph_hip.runtime import HipLibraryError
     rt = hip_runtime
