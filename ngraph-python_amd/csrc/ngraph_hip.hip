@@ -121,6 +121,7 @@ struct ngh_context {
     int         red_wgs_per_cu = 8;  // workgroups per CU a split reduction along the contiguous axis aims for
     int         red_col_wgs_per_cu = 2;  // ... and one across it
     int         row_wave_chunks = 0;     // rows of up to this many chunks are reduced by one wavefront each
+    int         tile4 = 1;               // tiled elementwise programs may take 64 x 64 tiles with 16-byte accesses
     int         no_tiles = 0;        // never use the LDS-tiled elementwise skeleton
     int         flex_self_managed = 2;  // ngh_launch_fused_flex: 0 = prepare / kernel / update launches,
                                      // 1 = policy at the end of the kernel, 2 = statistics deferred to the next user
@@ -804,12 +805,47 @@ int launch_tail(ngh_context* ctx, const Plan& P) {
     return stat_fold(ctx, kt, 1);
 }
 
+// Can the tiled stage move four elements per access on every operand (ew_tiled4_static_kernel)?
+bool tile4_ok(const KArgs& k, unsigned used_mask) {
+    if (k.shape[1] % 4 || k.shape[2] % 4) return false;
+    for (int t = 0; t < k.n_tensors; ++t) {
+        if (!(used_mask & (1u << t))) continue;
+        const KTensor& T = k.t[t];
+        if (T.stage_slot >= 0) {                       // contiguous along kernel axis 1
+            if (((uintptr_t)T.p) % 16 || T.s[0] % 4 || T.s[2] % 4) return false;
+        } else if (T.s[2] != 0) {                      // must be contiguous along kernel axis 2
+            if (T.s[2] != 1 || ((uintptr_t)T.p) % 16 || T.s[0] % 4 || T.s[1] % 4) return false;
+        }
+    }
+    return true;
+}
+
+// A compiled tiled stage takes 64 x 64 tiles when every operand allows 16-byte accesses and
+// there are tiles of that size enough to fill the chip.
+bool wants_tile4(const ngh_context* ctx, const Plan& P, long long& ta4, long long& tb4, long long& n4) {
+    ta4 = (P.k.shape[1] + kTile4 - 1) / kTile4;
+    tb4 = (P.k.shape[2] + kTile4 - 1) / kTile4;
+    n4 = P.k.shape[0] * ta4 * tb4;
+    return P.family == F_EW_TILED && P.special >= 0 && !P.k.probe && ctx->tile4 && P.tile == kTile &&
+           n4 >= 4LL * ctx->cus && tile4_ok(P.k, P.load_mask | P.store_mask);
+}
+
 int launch_interp(ngh_context* ctx, Plan& P) {
     if (P.family == F_EW_TILED) {
         if (P.n_tiles == 0) return NGH_OK;
         const unsigned blocks = std::min<unsigned>(P.n_tiles, (unsigned)(ctx->cus * ctx->ew_blocks_per_cu));
         NGH_TRY(stat_scratch(ctx, P.k, blocks));
         if (P.special >= 0 && !P.k.probe) {
+            // a compiled program takes 64 x 64 tiles with 16-byte accesses where every operand
+            // allows them and there are tiles of that size enough to fill the chip
+            long long ta4, tb4, n4;
+            if (wants_tile4(ctx, P, ta4, tb4, n4)) {
+                const unsigned blocks4 = (unsigned)std::min<long long>(n4, (long long)ctx->cus * ctx->ew_blocks_per_cu);
+                NGH_TRY(stat_scratch(ctx, P.k, blocks4));
+                HIP_TRY(launch_special_tiled(P.special, ctx->stream, blocks4, P.k, (unsigned)ta4, (unsigned)tb4,
+                                             (unsigned)n4, kTile4));
+                return stat_fold(ctx, P.k, blocks4);
+            }
             HIP_TRY(launch_special_tiled(P.special, ctx->stream, blocks, P.k, P.tiles_a, P.tiles_b, P.n_tiles, P.tile));
             return stat_fold(ctx, P.k, blocks);
         }
@@ -998,6 +1034,7 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->red_wgs_per_cu = std::max(1, env_int("NGH_RED_WGS_PER_CU", 8));
     ctx->red_col_wgs_per_cu = std::max(1, env_int("NGH_RED_COL_WGS_PER_CU", 2));
     ctx->row_wave_chunks = std::max(0, env_int("NGH_ROW_WAVE_CHUNKS", kRowWaveChunks));
+    ctx->tile4 = env_int("NGH_TILE4", 1);
     ctx->cache_policy = env_int("NGH_CACHE_POLICY", -1);
     ctx->stream_bytes = (long long)env_int("NGH_STREAM_MIB", 192) << 20;
     ctx->moments_wgs_per_cu = std::max(1, env_int("NGH_MOMENTS_WGS_PER_CU", 8));
@@ -1246,6 +1283,8 @@ int ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec, int32_t sta
     if (!ctx->force_interp)
         P.special = match_special(P.family, P.V, P.k, P.tail);
     describe(P, name128, 128);
+    long long ta4, tb4, n4;
+    if (wants_tile4(ctx, P, ta4, tb4, n4)) strncat(name128, "/tiles64", 127 - strlen(name128));
     if (P.special >= 0 && P.family == F_EW) {
         static const char* const suffix[4] = {"", "/nt-loads", "/nt-stores", "/nt-loads-stores"};
         const int cp = stage_cache_policy(ctx, *spec, spec->stages[stage]);

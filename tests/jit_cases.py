@@ -41,6 +41,18 @@ def case_transposed_operand():
     return [ng.sigmoid(ng.axes_with_order(xs, [A, B]) * x) + y], [xs, x, y]
 
 
+def case_transposed_operands_large():
+    # enough 64 x 64 tiles for the compiled tiled program to take 16-byte accesses, with ragged
+    # tiles at both edges (2052 = 32 * 64 + 4); a transposed fp32 operand, a transposed fp16
+    # operand, and a result assigned through a transposed view of a variable
+    A, B = ng.make_axis(2052, name="A"), ng.make_axis(2056, name="B")
+    xs, hs = ng.placeholder([B, A]), ng.placeholder([B, A], dtype=np.float16)
+    y = ng.placeholder([A, B])
+    v = ng.variable([B, A], initial_value=0)
+    z = ng.tanh(ng.axes_with_order(xs, [A, B]) * y) + ng.axes_with_order(hs, [A, B])
+    return [ng.sequential([ng.assign(ng.axes_with_order(v, [A, B]), z * 0.5), z]), v * 1.0], [xs, hs, y]
+
+
 def case_softmax():
     A, B = _ab()
     x = ng.placeholder([A, B])
@@ -100,7 +112,7 @@ def case_lookup_table():
 
 
 FP32_CASES = [case_elementwise, case_column_reduction_with_store, case_row_reduction_with_store,
-              case_transposed_operand, case_softmax, case_mixed_storage_types, case_ragged,
+              case_transposed_operand, case_transposed_operands_large, case_softmax, case_mixed_storage_types, case_ragged,
               case_misaligned_slices, case_short_rows, case_dropout, case_lookup_table]
 
 

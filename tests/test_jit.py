@@ -222,6 +222,8 @@ def test_compiled_programs_agree_with_the_interpreter(case):
     if default_kernel_choice():
         # every stage large enough to be worth a compiled kernel has one now
         assert not any("interp" in n for n in names if "tail" not in n), names
+        if case is jit_cases.case_transposed_operands_large:
+            assert any(n.endswith("/tiles64") for n in names), names
 
 
 @pytest.mark.gpu
