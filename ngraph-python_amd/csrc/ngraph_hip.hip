@@ -616,7 +616,8 @@ int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage,
         // row would spend its time on the barrier and the launch of a workgroup per kilobyte
         const long long wave_chunks = ctx ? ctx->row_wave_chunks : kRowWaveChunks;
         const long long cus = ctx ? ctx->cus : 256;
-        if (chunks <= wave_chunks && (long long)n_out >= cus * 4 * kWaves) {
+        // (with one element per chunk the same row lengths qualify)
+        if (chunks <= wave_chunks * (P.V == 1 ? 4 : 1) && (long long)n_out >= cus * 4 * kWaves) {
             P.small_rows = true;
             P.tx = 64;
             P.n_seg = 1;
