@@ -469,6 +469,81 @@ def compiled_vs_interpreted(ng, ngt, steps, warmup, An=8192, Bn=8192):
     return out
 
 
+# ------------------------------------------------------------------------------------- shapes
+def shape_survey_cases(ng):
+    """(name, results, inputs, algorithmic bytes) of graphs over 64-270 MB tensors in the layouts
+    and extents that everyday graphs have: broadcasts, transposed operands, reductions along,
+    across and over several axes, many short rows, odd extents."""
+    def ax(n, name):
+        return ng.make_axis(n, name=name)
+    A, B = ax(8192, "A"), ax(8192, "B")
+    x, y = ng.placeholder([A, B]), ng.placeholder([A, B])
+    row_vec, col_vec = ng.placeholder([B]), ng.placeholder([A])
+    full = 8192 * 8192 * 4
+    yield "x + b[B] (operand broadcast along rows)", [x + row_vec], [x, row_vec], 2 * full
+    yield "x * c[A] (operand broadcast along the contiguous axis)", [x * col_vec], [x, col_vec], 2 * full
+    xt = ng.placeholder([B, A])
+    yield "tanh(transposed x) * y", [ng.tanh(ng.axes_with_order(xt, [A, B])) * y], [xt, y], 3 * full
+    yield "sum across the contiguous axis [8192,8192]", [ng.sum(x, out_axes=[B])], [x], full
+    yield "sum along the contiguous axis [8192,8192]", [ng.sum(x, out_axes=[A])], [x], full
+    N, C, HW = ax(64, "N"), ax(256, "C"), ax(3136, "HW")
+    v = ng.placeholder([N, C, HW])
+    nchw = 64 * 256 * 3136 * 4
+    yield "[N,C,HW] sum over N and HW", [ng.sum(v, out_axes=[C])], [v], nchw
+    yield "[N,C,HW] sum over C", [ng.sum(v, out_axes=[N, HW])], [v], nchw
+    yield "[N,C,HW] sum over HW", [ng.sum(v, out_axes=[N, C])], [v], nchw
+    gamma, beta = ng.placeholder([C]), ng.placeholder([C])
+    mean, var = ng.mean(v, out_axes=[C]), ng.variance(v, out_axes=[C])
+    yield ("[N,C,HW] batch norm (two-pass statistics over N and HW, normalise; 4 passes)",
+           [gamma * ((v - mean) * ng.reciprocal(ng.sqrt(var + 1e-5))) + beta], [v, gamma, beta], 4 * nchw)
+    for rows, k in ((131072, 256), (32768, 1024), (32768, 1000), (32768, 1001), (8192, 4096)):
+        R, K = ax(rows, "R%d" % k), ax(k, "K%d" % k)
+        w = ng.placeholder([R, K])
+        mu, vv = ng.mean(w, out_axes=[R]), ng.variance(w, out_axes=[R])
+        yield ("layer norm of rows [%d,%d] (one-pass statistics, normalise; 3 passes)" % (rows, k),
+               [(w - mu) * ng.reciprocal(ng.sqrt(vv + 1e-5))], [w], 3 * rows * k * 4)
+        e = ng.exp(w - ng.max(w, out_axes=[R]))
+        yield ("softmax of rows [%d,%d] (maximum, sum of exponentials, normalise; 4 passes)" % (rows, k),
+               [e / ng.sum(e, out_axes=[R])], [w], 4 * rows * k * 4)
+    O1, O2 = ax(8191, "O1"), ax(8191, "O2")
+    o, o2 = ng.placeholder([O1, O2]), ng.placeholder([O1, O2])
+    odd = 8191 * 8191 * 4
+    yield "tanh(x * y) [8191,8191]", [ng.tanh(o * o2)], [o, o2], 3 * odd
+    yield "sum along the contiguous axis [8191,8191]", [ng.sum(o, out_axes=[O1])], [o], odd
+    yield "sum across the contiguous axis [8191,8191]", [ng.sum(o, out_axes=[O2])], [o], odd
+
+
+def shape_survey(ng, ngt, steps, warmup):
+    """The graphs of shape_survey_cases with the transformer's default kernel choice (programs
+    compiled at run time loaded before timing): ms per step, algorithmic GB/s, and each
+    kernel's duration from HIP events."""
+    out = {}
+    for name, results, inputs, nbytes in shape_survey_cases(ng):
+        t = ngt.make_transformer_factory("hipgpu")()
+        try:
+            f = t.computation(results, *inputs)
+            values = [np.random.RandomState(i).uniform(0.5, 1.5, p.axes.lengths).astype(np.float32)
+                      for i, p in enumerate(inputs)]
+            f(*values)
+            group = t.kernel_groups[f]
+            f(*values)                                   # the second run starts the compile workers
+            error = group.wait_for_programs()
+            group()
+            t.runtime.sync()
+            ms = float(np.median(step_blocks(t.runtime, group, steps, warmup, 3)))
+            kernels = [("+".join(d for ds in k.describe() for d in ds), round(float(np.median(times)) * 1e3, 1))
+                       for k, times in group.profile(repeats=3, inner=10)]
+            out[name] = {"ms_per_step": round(ms, 5), "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                         "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                         "algorithmic_bytes_per_step": int(nbytes),
+                         "kernels_us": kernels}
+            if error:
+                out[name]["compiler"] = error
+        finally:
+            t.close()
+    return out
+
+
 # ------------------------------------------------------------------------------------- CPU baseline
 def cpu_baseline_c2(configs, x, gamma, beta, budget_s=20.0):
     ws = configs.Workspace()
@@ -534,6 +609,9 @@ def main():
     ap.add_argument("--compiled", action="store_true",
                     help="also time five user graphs: default kernel choice, interpreter only, compiled "
                          "(needs hipcc unless the program cache already holds them)")
+    ap.add_argument("--shapes", action="store_true",
+                    help="also time a survey of everyday layouts and extents (broadcasts, transposed operands, "
+                         "reductions over one and several axes, many short rows, odd extents)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
                     help="also issue N device-to-device copies of x (205 520 896 bytes each): a "
@@ -575,6 +653,8 @@ def main():
         out["configs"]["C5"] = bench_c5(ng, ngt, neon, configs, args, not args.no_cold)
     if args.all:
         out["configs"].update(small_configs(ng, ngt, neon, configs, max(5, args.steps // 4), 2))
+    if args.shapes:
+        out["shapes"] = shape_survey(ng, ngt, max(5, args.steps // 10), 2)
     if args.compiled:
         out["compiled_at_run_time"] = compiled_vs_interpreted(ng, ngt, max(5, args.steps // 20), 2)
     if not args.no_cpu:
