@@ -566,7 +566,10 @@ int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage,
         // wavefronts, so a stage without a compiled program keeps the large grid.)
         const bool compiled = !(ctx && ctx->force_interp) && !P.k.probe && match_special(F_RED_COL, P.V, P.k, 0) >= 0;
         const long long col_target = compiled ? (ctx ? ctx->cus * ctx->red_col_wgs_per_cu : 256 * 2) : target_wgs;
-        const bool wide = compiled && col_chunks >= kBlock && R * n_out > kSmallReduction && R >= 64;
+        // (... unless the last of those workgroups per row would be mostly idle lanes)
+        const long long wide_blocks = (col_chunks + kBlock - 1) / kBlock;
+        const bool wide = compiled && col_chunks >= kBlock && R * n_out > kSmallReduction && R >= 64 &&
+                          col_chunks * 10 >= wide_blocks * kBlock * 9;
         if (wide) P.tx = kBlock;
         if (R * n_out <= kSmallReduction) {
             // A small problem is bound by latency: every row a lane walks down is a round trip
