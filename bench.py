@@ -654,9 +654,9 @@ def main():
     if args.all:
         out["configs"].update(small_configs(ng, ngt, neon, configs, max(5, args.steps // 4), 2))
     if args.shapes:
-        out["shapes"] = shape_survey(ng, ngt, max(5, args.steps // 10), 2)
+        out["shapes"] = shape_survey(ng, ngt, max(20, args.steps // 4), 2)
     if args.compiled:
-        out["compiled_at_run_time"] = compiled_vs_interpreted(ng, ngt, max(5, args.steps // 20), 2)
+        out["compiled_at_run_time"] = compiled_vs_interpreted(ng, ngt, max(20, args.steps // 4), 2)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_c2(configs, x_np, gamma_np, beta_np)
         others = cpu_baseline_others(configs)
