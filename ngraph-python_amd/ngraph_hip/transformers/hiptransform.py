@@ -796,8 +796,10 @@ class MomentsFusionPass(PeepholeGraphPass):
         x2, red2 = inner
         if not red2.is_equal_set(red_axes) or not self._same_tensor(x, x2):
             return
-        if x.dtype != np.dtype(np.float32) or moments_layout(_td(x), red_axes) is None:
+        if x.dtype != np.dtype(np.float32):
             return
+        if moments_layout(_td(x), red_axes) is None:
+            return self._visit_two_level(op, m, x, red_axes)
         mom = MomentsOp(x, red_axes)
         mean_view = og.slice_along_axis(mom, mom.k_axis, 0)
         var_view = og.slice_along_axis(mom, mom.k_axis, 1)
@@ -805,6 +807,40 @@ class MomentsFusionPass(PeepholeGraphPass):
         self.var_views[var_view] = mom
         self.replace_op(op, var_view)
         self.replace_op(self._strip(m), mean_view)
+
+    def _visit_two_level(self, op, m, x, red_axes):
+        """The reduced axes do not form one run of contiguous rows, but some of them do (sum over
+        N, H and W of an [N, C, H, W] tensor: rows of H*W elements): one-pass moments of those
+        rows, then the rows' statistics are combined over the remaining axes, which is exact
+        for rows of equal length:  mean = E[mean_row],  var = E[var_row + (mean_row - mean)^2].
+        One read of x instead of two, and no copy of x into (reduced, kept) order."""
+        td = _td(x)
+        inner = [a for a in red_axes if a.length != 1 and td.full_strides[td.axes.index(a)] == 1]
+        if len(inner) != 1:
+            return
+        # grow the run of rows outwards while the next reduced axis continues it
+        run, stride = list(inner), inner[0].length
+        grown = True
+        while grown:
+            grown = False
+            for a in red_axes:
+                if a not in run and a.length != 1 and td.full_strides[td.axes.index(a)] == stride:
+                    run.append(a)
+                    stride *= a.length
+                    grown = True
+        outer = [a for a in red_axes if a not in run]
+        R = int(np.prod([a.length for a in run]))
+        if not outer or R < 64 or moments_layout(td, og.make_axes(run)) is None:
+            return
+        mom = MomentsOp(x, og.make_axes(run))
+        row_mean = og.slice_along_axis(mom, mom.k_axis, 0)
+        row_var = og.slice_along_axis(mom, mom.k_axis, 1)
+        n_rows = float(np.prod([a.length for a in outer]))
+        mean = og.sum(row_mean, reduction_axes=outer) / n_rows
+        var = og.sum(row_var + og.square(row_mean - mean), reduction_axes=outer) / n_rows
+        self.moments.append((x, red_axes, mean, var))
+        self.replace_op(op, var)
+        self.replace_op(self._strip(m), mean)
 
 
 class MomentsKernel(HipKernel):

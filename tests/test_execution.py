@@ -220,6 +220,37 @@ def test_mean_variance(backend):
     np.testing.assert_allclose(v, xv.var(axis=(1, 2)), rtol=1e-5, atol=1e-6)
 
 
+def test_mean_variance_over_axes_in_two_groups(backend):
+    """Batch-norm statistics of an [N, C, H, W] tensor: mean and variance over N, H and W, then
+    the normalisation.  The HIP transformer takes one-pass moments of the H*W rows and combines
+    them over N (mean of the rows' means; mean of the rows' variances plus the squared distance
+    of their means), which is exact for rows of equal length."""
+    ax = axes(N=6, C=5, H=16, W=8)
+    x = ng.placeholder(ax)
+    gamma, beta = ng.placeholder(ax[1:2]), ng.placeholder(ax[1:2])
+    xv = rng.normal(0.5, 2, ax)
+    gv, bv = rng.uniform(0.5, 1.5, ax[1:2]), rng.uniform(0.5, 1.5, ax[1:2])
+    m = ng.mean(x, out_axes=ax[1:2])
+    v = ng.variance(x, out_axes=ax[1:2])
+    y = gamma * ((x - m) * ng.reciprocal(ng.sqrt(v + 1e-5))) + beta
+    with executor([m, v, y], x, gamma, beta) as f:
+        m_g, v_g, y_g = f(xv, gv, bv)
+    x64 = xv.astype(np.float64)
+    m64, v64 = x64.mean(axis=(0, 2, 3)), x64.var(axis=(0, 2, 3))
+    np.testing.assert_allclose(m_g, m64, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(v_g, v64, rtol=1e-5, atol=1e-6)
+    y64 = gv[None, :, None, None] * ((x64 - m64[None, :, None, None]) / np.sqrt(v64 + 1e-5)[None, :, None, None]) \
+        + bv[None, :, None, None]
+    np.testing.assert_allclose(y_g, y64, rtol=1e-5, atol=1e-5)
+
+
+def test_two_group_statistics_take_one_pass_moments():
+    ax = axes(N=6, C=5, H=16, W=8)
+    x = ng.placeholder(ax)
+    kernels = _kernels_lowered_for([ng.mean(x, out_axes=ax[1:2]), ng.variance(x, out_axes=ax[1:2])], [x])
+    assert kernels[0] == "MomentsKernel" and "CopyKernel" not in kernels, kernels
+
+
 def test_4d_elementwise_and_sums(backend):
     """Shapes of tests/transformer_dependent/test_kernel_generator.py:43-131."""
     for shape in [(64, 10, 28, 32), (3, 16, 16, 4), (7, 15, 19, 5), (3, 5, 7, 2)]:
