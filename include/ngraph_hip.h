@@ -258,7 +258,8 @@ int  ngh_programs_count(int32_t* built_in, int32_t* loaded);
 /* Per-row mean and (biased) variance of a [rows, R] fp32 matrix with contiguous rows in ONE
  * read of x (x_cache_hint: NGH_CACHE_* bits for x): fuses the reductions behind ng.mean + ng.variance
  * (op_graph.py:4007-4009, 4252-4266), the statistics of batch normalisation
- * (frontends/neon/layer.py:1242-1245).  row_stride in elements, multiple of 4.
+ * (frontends/neon/layer.py:1242-1245).  row_stride in elements (any: rows need not start on
+ * 16-byte boundaries).
  * dev_rstd, when not NULL, also receives 1/sqrt(var + eps), the factor of layer.py:1255.  */
 int  ngh_moments_f32(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t R, int64_t row_stride,
                      float* dev_mean, float* dev_var, float* dev_rstd, float eps, uint32_t x_cache_hint);

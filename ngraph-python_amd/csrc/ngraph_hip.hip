@@ -1343,8 +1343,7 @@ int plan_moments(const ngh_context* ctx, const float* dev_x, int64_t rows, int64
     if (rows < 0 || R <= 0) return fail(NGH_E_INVALID, "rows %lld, R %lld", (long long)rows, (long long)R);
     if (rows == 0) return NGH_OK;
     if (!dev_x || !dev_mean || !dev_var) return fail(NGH_E_INVALID, "NULL device pointer");
-    if (((uintptr_t)dev_x) % 16 || row_stride % 4)
-        return fail(NGH_E_UNSUPPORTED, "rows must start on 16-byte boundaries");
+    if (((uintptr_t)dev_x) % 4) return fail(NGH_E_INVALID, "x is not aligned to its element size");
     if (rows >= (1LL << 24) || R >= (1LL << 32)) return fail(NGH_E_UNSUPPORTED, "extent too large");
     m.R4 = (unsigned)(R / 4);
     m.per_wave = (long long)m.R4 <= ctx->row_wave_chunks * 2 && rows >= (long long)ctx->cus * 4 * (kMomBlock / 64);

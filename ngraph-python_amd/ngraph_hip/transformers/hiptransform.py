@@ -709,8 +709,6 @@ def moments_layout(td, reduction_axes):
     R = int(np.prod([n for n, _ in red], dtype=np.int64))
     rows = int(np.prod([n for n, _ in kept], dtype=np.int64)) if kept else 1
     row_stride = kept[-1][1] if kept else R
-    if row_stride % 4 or td.offset % 4:
-        return None
     return rows, R, row_stride
 
 

@@ -640,6 +640,28 @@ def test_moments_rows(hip_runtime, rows, R, pad):
         d.free()
 
 
+@pytest.mark.parametrize("rows,R,stride,first", [(256, 3137, 3139, 1), (5000, 1001, 1001, 3), (37, 100003, 100005, 2),
+                                                 (4100, 4095, 4097, 1), (70000, 5, 7, 1)])
+def test_moments_of_rows_off_16_byte_boundaries(hip_runtime, rows, R, stride, first):
+    """Rows that start at any float: odd row pitch, a view that begins a few elements into its
+    buffer.  Both kernels (segments of long rows, a group of lanes per short row) read them with
+    unaligned 16-byte loads; results against float64."""
+    rt = hip_runtime
+    rs = np.random.RandomState(rows + R)
+    host = rs.normal(-1.0, 3.0, first + rows * stride).astype(f32)
+    x_d = rt.array(host)
+    out_d = rt.empty((3, rows))
+    rt.memset32(out_d.ptr, 0x7fc00000, 3 * rows)
+    rt.moments_f32(x_d.ptr + 4 * first, rows, R, stride, out_d.ptr, out_d.ptr + 4 * rows, out_d.ptr + 8 * rows, 1e-5)
+    mean, var, rstd = out_d.get()
+    view = np.lib.stride_tricks.as_strided(host[first:], (rows, R), (4 * stride, 4)).astype(np.float64)
+    np.testing.assert_allclose(mean, view.mean(axis=1), rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(var, view.var(axis=1), rtol=1e-4, atol=1e-5)
+    np.testing.assert_array_equal(rstd, (f32(1) / np.sqrt(var + f32(1e-5))).astype(f32))
+    for d in (x_d, out_d):
+        d.free()
+
+
 def test_moments_hand_off_with_and_without_release_acquire_tickets(monkeypatch):
     """The last workgroup of a row merges the row's segments.  By default the hand-off is a
     relaxed ticket ordered behind the partial sums by a data dependency (what gfx950 honours);
