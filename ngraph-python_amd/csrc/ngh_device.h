@@ -50,6 +50,7 @@ struct KArgs {
     int       red_axis;      // kernel axis the reductions run along (0 or 2), -1 = none
     int       iota_map[3];   // kernel axis holding spec axis k (for NGH_OP_IOTA)
     int       n_stat_slots;
+    int       n_store_stat_slots;   // the first of them belong to tensors a STORE op writes, the rest to reduction results
     int       n_staged;      // tiled skeleton: operands staged through LDS tiles
     int       tile_diagonal; // tiled skeleton: deal the tiles along diagonals (strides that are multiples of 4 KiB)
     unsigned  rng_seed, rng_counter;   // NGH_OP_RNG_*

@@ -457,9 +457,18 @@ struct RedWs {
     int*   idx;
 };
 
+// max|mantissa| of the flex results a thread has emitted, by statistics slot
+struct RedStats {
+    int m[4] = {0, 0, 0, 0};
+    __device__ __forceinline__ void note(int slot, int v) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) m[s] = (s == slot) ? max(m[s], v) : m[s];
+    }
+};
+
 __device__ __forceinline__ void red_emit(const KArgs& k, int slot, Acc a, long long o0, long long o1,
                                          long long o2, unsigned out, unsigned n_out, unsigned seg,
-                                         unsigned n_seg, RedWs ws) {
+                                         unsigned n_seg, RedWs ws, RedStats& stats) {
     if (n_seg == 1) {
         const KTensor& t = k.t[k.red_out[slot]];
         const long long off = o0 * t.s[0] + o1 * t.s[1] + o2 * t.s[2];
@@ -474,12 +483,27 @@ __device__ __forceinline__ void red_emit(const KArgs& k, int slot, Acc a, long l
         } else {
             store1(t, off, result, sc, fmax);
         }
-        if (t.stats != nullptr && fmax > 0) atomicMax(t.stats, fmax);
+        // One statistics word per tensor and a result per workgroup or lane: thousands of
+        // read-modify-writes on one address would run one after the other (8192 of them took
+        // 250 us).  A result with a statistics slot is merged through the workgroup's partial
+        // maximum like the results of STORE ops; without one (more flex results than slots),
+        // a result that does not exceed what is there already (read at device scope) adds nothing.
+        if (t.stat_slot >= 0) stats.note(t.stat_slot, fmax);
+        else if (t.stats != nullptr && fmax > 0 &&
+                 fmax > __hip_atomic_load(t.stats, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+            atomicMax(t.stats, fmax);
     } else {
         const size_t w = ((size_t)slot * n_seg + seg) * n_out + out;
         ws.val[w] = a.v;
         if (k.ops[k.op_end - k.n_red + slot].opcode >= NGH_OP_RED_ARGMAX) ws.idx[w] = a.i;   // only argmax / argmin carry one
     }
+}
+
+// The interpreter kernels keep statistics per thread in `ex`: add what the thread emitted.
+__device__ __forceinline__ void red_stats_to_extra(const KArgs& k, Extra& ex, const RedStats& stats) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+        if (s >= k.n_store_stat_slots && s < k.n_stat_slots) ex.seti(ex_stat(s), max(ex.geti(ex_stat(s)), stats.m[s]));
 }
 
 // The reduction ops of a stage are its last n_red ops, slot k = k-th of them.
@@ -528,14 +552,16 @@ __global__ __launch_bounds__(kBlock) void red_row_interp_kernel(const KArgs k, u
         if (lane == 0) sh[s][wave] = a;
     }
     __syncthreads();
+    RedStats emitted;
     if (threadIdx.x == 0) {
         for (int s = 0; s < k.n_red; ++s) {
             const int opc = red_opcode(k, s);
             Acc a = sh[s][0];
             for (int w = 1; w < kWaves; ++w) a = acc_merge(opc, a, sh[s][w]);
-            red_emit(k, s, a, i0, i1, 0, out, n_out, seg, n_seg, ws);
+            red_emit(k, s, a, i0, i1, 0, out, n_out, seg, n_seg, ws, emitted);
         }
     }
+    red_stats_to_extra(k, ex, emitted);
     stats_epilogue(k, ex);
 }
 
@@ -578,6 +604,7 @@ __global__ __launch_bounds__(kBlock) void red_col_interp_kernel(const KArgs k, u
     const unsigned r_begin = seg * seg_rows;
     const unsigned r_end = min((unsigned)k.shape[0], r_begin + seg_rows);
     const unsigned n_out = (unsigned)k.shape[1] * d2;
+    RedStats emitted;
     if (wide) {
         if (i2 < d2) {
             for (unsigned r = r_begin; r < r_end; ++r) run_ops<V, 2>(k, rf, ex, VecAt<V>{r, i1, i2});
@@ -587,10 +614,11 @@ __global__ __launch_bounds__(kBlock) void red_col_interp_kernel(const KArgs k, u
                     Acc a;
                     a.v = ex.getf(ex_accv(k, s, V, v));
                     a.i = ex.geti(ex_acci(k, s, V, v));
-                    red_emit(k, s, a, 0, i1, i2 + v, i1 * d2 + i2 + v, n_out, seg, n_seg, ws);
+                    red_emit(k, s, a, 0, i1, i2 + v, i1 * d2 + i2 + v, n_out, seg, n_seg, ws, emitted);
                 }
             }
         }
+        red_stats_to_extra(k, ex, emitted);
         stats_epilogue(k, ex);
         return;
     }
@@ -614,11 +642,12 @@ __global__ __launch_bounds__(kBlock) void red_col_interp_kernel(const KArgs k, u
             for (int v = 0; v < V; ++v) {
                 Acc a = sh[0][lane][v];
                 for (int w = 1; w < kWaves; ++w) a = acc_merge(opc, a, sh[w][lane][v]);
-                red_emit(k, s, a, 0, i1, i2 + v, i1 * d2 + i2 + v, n_out, seg, n_seg, ws);
+                red_emit(k, s, a, 0, i1, i2 + v, i1 * d2 + i2 + v, n_out, seg, n_seg, ws, emitted);
             }
         }
         __syncthreads();
     }
+    red_stats_to_extra(k, ex, emitted);
     stats_epilogue(k, ex);
 }
 
@@ -648,15 +677,26 @@ __global__ __launch_bounds__(kBlock) void red_rows_small_interp_kernel(const KAr
     if (out < n_out)
         for (unsigned c = pos; c < chunks; c += TR) run_ops<V, 1>(k, rf, ex, VecAt<V>{i0, i1, (long long)c * V});
     RedWs none{nullptr, nullptr};
+    RedStats emitted;
     for (int s = 0; s < k.n_red; ++s) {
         const int opc = red_opcode(k, s);
         Acc a;
         a.v = ex.getf(ex_accv(k, s));
         a.i = ex.geti(ex_acci(k, s));
         for (unsigned m = TR >> 1; m > 0; m >>= 1) a = acc_merge(opc, a, acc_shfl_xor(a, (int)m));
-        if (pos == 0 && out < n_out) red_emit(k, s, a, i0, i1, 0, out, n_out, 0, 1, none);
+        if (pos == 0 && out < n_out) red_emit(k, s, a, i0, i1, 0, out, n_out, 0, 1, none, emitted);
     }
+    red_stats_to_extra(k, ex, emitted);
     stats_epilogue(k, ex);
+}
+
+// The merge kernels of split reductions: the workgroup's maximum of what it emitted goes to the
+// slot's per-workgroup partial (whole workgroup calls).
+__device__ __forceinline__ void red_stats_flush(const KArgs& k, const RedStats& stats) {
+    __shared__ int flush_lds[4][kWaves];
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+        if (s >= k.n_store_stat_slots && s < k.n_stat_slots) block_stat_max(stats.m[s], k.stat_partial[s], flush_lds[s]);
 }
 
 // Second pass of a split reduction: merges an output's segments (in a fixed order) and
@@ -686,6 +726,7 @@ __global__ __launch_bounds__(kBlock) void red_finish_kernel(const KArgs k, unsig
     const unsigned g_begin = min(n_seg, wave * per_wave), g_end = min(n_seg, g_begin + per_wave);
     long long o0 = 0, o1 = 0, o2 = 0;
     if (out < n_out) red_finish_coords(k, out, row_mode, o0, o1, o2);
+    RedStats emitted;
     for (int s = 0; s < k.n_red; ++s) {
         const int opc = red_opcode(k, s);
         const bool with_index = opc >= NGH_OP_RED_ARGMAX;
@@ -715,20 +756,21 @@ __global__ __launch_bounds__(kBlock) void red_finish_kernel(const KArgs k, unsig
             // (a wavefront that had no segments holds the reduction's identity)
             for (int w = 1; w < kWaves; ++w) a = acc_merge(opc, a, sh[w][lane]);
             RedWs none{nullptr, nullptr};
-            red_emit(k, s, a, o0, o1, o2, out, n_out, 0, 1, none);
+            red_emit(k, s, a, o0, o1, o2, out, n_out, 0, 1, none, emitted);
         }
         __syncthreads();
     }
+    red_stats_flush(k, emitted);
 }
 
 __global__ __launch_bounds__(kBlock) void red_finish_wave_kernel(const KArgs k, unsigned n_out,
                                                                  unsigned n_seg, int row_mode, RedWs ws) {
     const unsigned lane = threadIdx.x & 63;
     const unsigned out = blockIdx.x * kWaves + (threadIdx.x >> 6);
-    if (out >= n_out) return;
-    long long o0, o1, o2;
-    red_finish_coords(k, out, row_mode, o0, o1, o2);
-    for (int s = 0; s < k.n_red; ++s) {
+    RedStats emitted;
+    long long o0 = 0, o1 = 0, o2 = 0;
+    if (out < n_out) red_finish_coords(k, out, row_mode, o0, o1, o2);
+    for (int s = 0; s < k.n_red && out < n_out; ++s) {
         const int opc = red_opcode(k, s);
         Acc a = acc_init(opc);
         const bool with_index = opc >= NGH_OP_RED_ARGMAX;
@@ -741,9 +783,10 @@ __global__ __launch_bounds__(kBlock) void red_finish_wave_kernel(const KArgs k, 
         for (int m = 32; m > 0; m >>= 1) a = acc_merge(opc, a, acc_shfl_xor(a, m));
         if (lane == 0) {
             RedWs none{nullptr, nullptr};
-            red_emit(k, s, a, o0, o1, o2, out, n_out, 0, 1, none);
+            red_emit(k, s, a, o0, o1, o2, out, n_out, 0, 1, none, emitted);
         }
     }
+    red_stats_flush(k, emitted);
 }
 
 }  // namespace ngh

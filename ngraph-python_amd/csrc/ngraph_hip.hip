@@ -338,6 +338,19 @@ void fill_kargs(const ngh_fused_spec& sp, const ngh_stage& S, const int perm[3],
             k.n_stat_slots = 5;      // more flex results with statistics than slots: plan_stage rejects
         }
     }
+    // flex results of the stage's reductions take the statistics slots the stores left (their
+    // max|mantissa| then travels through per-workgroup partial maxima like a store's, instead
+    // of one atomic per result on the tensor's statistics word)
+    k.n_store_stat_slots = std::min(k.n_stat_slots, 4);
+    for (int r = 0; r < S.n_reductions && k.n_stat_slots < 4; ++r) {
+        const int t = S.red_out[r];
+        if (t < 0 || t >= sp.n_tensors) continue;
+        KTensor& K = k.t[t];
+        if (K.dtype == NGH_FLEX16 && K.stats != nullptr && K.stat_slot < 0) {
+            K.stat_slot = k.n_stat_slots;
+            k.stat_ptr[k.n_stat_slots++] = K.stats;
+        }
+    }
     memcpy(k.consts, sp.consts, sizeof(k.consts));
     memcpy(k.ops, sp.ops, sizeof(k.ops));
 }
@@ -782,8 +795,8 @@ int stat_scratch(ngh_context* ctx, KArgs& k, unsigned blocks) {
     return NGH_OK;
 }
 
-int stat_fold(ngh_context* ctx, const KArgs& k, unsigned blocks) {
-    for (int s = 0; s < k.n_stat_slots; ++s) {
+int stat_fold(ngh_context* ctx, const KArgs& k, unsigned blocks, int first = 0, int last = 4) {
+    for (int s = first; s < k.n_stat_slots && s < last; ++s) {
         if (k.stat_ptr[s] == nullptr) continue;
         hipLaunchKernelGGL(stats_fold_kernel, dim3(1), dim3(256), 0, ctx->stream, k.stat_partial[s], blocks,
                            k.stat_ptr[s]);
@@ -914,6 +927,11 @@ int launch_interp(ngh_context* ctx, Plan& P) {
         ws.val = (float*)ctx->ws;
         ws.idx = (int*)ctx->ws + n;
     }
+    // the merge kernel of a split reduction: few outputs with many segments each take a wavefront
+    // per output; else 64 outputs a workgroup.  It emits the results, so the statistics of flex
+    // results come from its workgroups (the partial arrays hold the larger of the two grids).
+    const bool finish_by_wave = P.n_seg >= 32 && P.n_out < 1024;
+    const unsigned finish_blocks = P.n_seg > 1 ? (finish_by_wave ? (P.n_out + kWaves - 1) / kWaves : (P.n_out + 63) / 64) : 0;
     unsigned red_blocks = 0;
     if (P.special >= 0 && !k.probe) {
         // a pre-built reduction: same grid and workspace as the interpreter's kernel
@@ -922,21 +940,21 @@ int launch_interp(ngh_context* ctx, Plan& P) {
         red_blocks = small ? (P.n_out + rows_per_wg - 1) / rows_per_wg
                    : P.family == F_RED_ROW ? P.n_out * P.n_seg
                                            : (unsigned)((unsigned long long)P.n_bx * (unsigned)k.shape[1] * P.n_seg);
-        NGH_TRY(stat_scratch(ctx, k, red_blocks));
+        NGH_TRY(stat_scratch(ctx, k, std::max(red_blocks, finish_blocks)));
         // (a row reduction takes no TX unless its rows are short: TX lanes per row then)
         HIP_TRY(launch_special_red(P.special, ctx->stream, red_blocks, k, P.family == F_RED_ROW ? P.n_out : P.n_bx,
                                    P.n_seg, P.seg_len, P.family == F_RED_ROW && !small ? 0u : P.tx, ws, P.cache_policy));
     } else if (P.family == F_RED_ROW && P.small_rows) {
         const unsigned rows_per_wg = kBlock / P.tx;
         red_blocks = (P.n_out + rows_per_wg - 1) / rows_per_wg;
-        NGH_TRY(stat_scratch(ctx, k, red_blocks));
+        NGH_TRY(stat_scratch(ctx, k, std::max(red_blocks, finish_blocks)));
         if (V == 4)
             hipLaunchKernelGGL(red_rows_small_interp_kernel<4>, dim3(red_blocks), dim3(kBlock), lds, ctx->stream, k, P.n_out, P.tx);
         else
             hipLaunchKernelGGL(red_rows_small_interp_kernel<1>, dim3(red_blocks), dim3(kBlock), lds, ctx->stream, k, P.n_out, P.tx);
     } else if (P.family == F_RED_ROW) {
         const unsigned blocks = red_blocks = P.n_out * P.n_seg;
-        NGH_TRY(stat_scratch(ctx, k, blocks));
+        NGH_TRY(stat_scratch(ctx, k, std::max(blocks, finish_blocks)));
         if (V == 4)
             hipLaunchKernelGGL(red_row_interp_kernel<4>, dim3(blocks), dim3(kBlock), lds, ctx->stream, k, P.n_out, P.n_seg, P.seg_len, ws);
         else
@@ -945,23 +963,23 @@ int launch_interp(ngh_context* ctx, Plan& P) {
         const unsigned long long blocks = (unsigned long long)P.n_bx * (unsigned)k.shape[1] * P.n_seg;
         if (blocks >= (1ULL << 31)) return fail(NGH_E_UNSUPPORTED, "reduction grid too large");
         red_blocks = (unsigned)blocks;
-        NGH_TRY(stat_scratch(ctx, k, red_blocks));
+        NGH_TRY(stat_scratch(ctx, k, std::max(red_blocks, finish_blocks)));
         if (V == 4)
             hipLaunchKernelGGL(red_col_interp_kernel<4>, dim3(red_blocks), dim3(kBlock), interp_lds_bytes(k, 4, 4), ctx->stream, k, P.n_bx, P.n_seg, P.seg_len, P.tx, ws);
         else
             hipLaunchKernelGGL(red_col_interp_kernel<1>, dim3(red_blocks), dim3(kBlock), lds, ctx->stream, k, P.n_bx, P.n_seg, P.seg_len, P.tx, ws);
     }
     HIP_TRY(hipGetLastError());
-    if (k.n_stat_slots) NGH_TRY(stat_fold(ctx, k, red_blocks));
+    if (k.n_stat_slots) NGH_TRY(stat_fold(ctx, k, red_blocks, 0, P.n_seg > 1 ? k.n_store_stat_slots : 4));
     if (P.n_seg > 1) {
-        // few outputs with many segments each: a wavefront per output; else 64 outputs a workgroup
-        if (P.n_seg >= 32 && P.n_out < 1024)
-            hipLaunchKernelGGL(red_finish_wave_kernel, dim3((P.n_out + kWaves - 1) / kWaves), dim3(kBlock), 0, ctx->stream,
+        if (finish_by_wave)
+            hipLaunchKernelGGL(red_finish_wave_kernel, dim3(finish_blocks), dim3(kBlock), 0, ctx->stream,
                                k, P.n_out, P.n_seg, P.family == F_RED_ROW ? 1 : 0, ws);
         else
-            hipLaunchKernelGGL(red_finish_kernel, dim3((P.n_out + 63) / 64), dim3(kBlock), 0, ctx->stream,
+            hipLaunchKernelGGL(red_finish_kernel, dim3(finish_blocks), dim3(kBlock), 0, ctx->stream,
                                k, P.n_out, P.n_seg, P.family == F_RED_ROW ? 1 : 0, ws);
         HIP_TRY(hipGetLastError());
+        if (k.n_stat_slots > k.n_store_stat_slots) NGH_TRY(stat_fold(ctx, k, finish_blocks, k.n_store_stat_slots, 4));
     }
     return NGH_OK;
 }
