@@ -125,6 +125,7 @@ struct ngh_context {
     int         no_tiles = 0;        // never use the LDS-tiled elementwise skeleton
     int         flex_self_managed = 2;  // ngh_launch_fused_flex: 0 = prepare / kernel / update launches,
                                      // 1 = policy at the end of the kernel, 2 = statistics deferred to the next user
+                                     // for stages up to stream_bytes and 1 beyond, 3 = always deferred
     int         cache_policy = -1;   // -1: from the operands' cache hints; 0..3 forces bit 0 = non-temporal
                                      // loads, bit 1 = non-temporal stores in pre-built kernels
     long long   stream_bytes = 192ll << 20;  // hints act on stages touching at least this much memory
@@ -1237,6 +1238,21 @@ int ngh_validate_fused(const ngh_fused_spec* spec) { return validate(spec); }
 // MI355X): below `stream_bytes` everything is left cacheable.  Above it, loads stream when
 // every full-size operand read is marked as read by this kernel only, and stores stream
 // when every operand written is marked as not read again soon.
+// Bytes of the operands a stage touches (every operand once).
+static long long stage_bytes(const ngh_fused_spec& sp, const ngh_stage& S) {
+    bool loads[NGH_MAX_TENSORS], stores[NGH_MAX_TENSORS];
+    stage_tensors(sp, S, loads, stores);
+    long long bytes = 0;
+    for (int t = 0; t < sp.n_tensors; ++t) {
+        if (!loads[t] && !stores[t]) continue;
+        long long n = 1;
+        for (int a = 0; a < sp.rank; ++a)
+            if (sp.tensors[t].strides[a] != 0) n *= sp.shape[a];
+        bytes += n * itemsize_of(sp.tensors[t].dtype);
+    }
+    return bytes;
+}
+
 static int stage_cache_policy(const ngh_context* ctx, const ngh_fused_spec& sp, const ngh_stage& S) {
     if (ctx->cache_policy >= 0) return ctx->cache_policy & 3;
     bool loads[NGH_MAX_TENSORS], stores[NGH_MAX_TENSORS];
@@ -1677,6 +1693,12 @@ static int try_self_managed_launch(ngh_context* ctx, const ngh_fused_spec* spec,
         stage_tensors(*spec, spec->stages[0], loads, stores);
         for (int t = 0; T && t < P.k.n_tensors; ++t)
             if (P.k.t[t].stat_slot >= 0 && loads[t] && !P.k.flex_in_place[P.k.t[t].stat_slot]) T = nullptr;
+        // Deferring pays while the operands fit the last-level cache: the kernel then runs on few
+        // long-lived workgroups (each pays the prologue), which streams operands of that size as
+        // fast as a large grid does.  Beyond it the large grid is faster by more than the policy
+        // step at the end of the kernel costs (x*y+x over flex16 tensors: 16 M elements 18.8 us
+        // deferred / 22.1 us not, 32 M 37.3 / 38.4, 48 M 56.8 / 52.8, 64 M 75.3 / 69.2).
+        if (T && ctx->flex_self_managed == 2 && stage_bytes(*spec, spec->stages[0]) > ctx->stream_bytes) T = nullptr;
     }
     if (T) {
         // deferred statistics: everything the kernel merely reads must be in its plain form
