@@ -243,17 +243,29 @@ def test_flex_learning_rules_prebuilt_equals_interpreter(rule, resident, monkeyp
 
 # (name, NGH_FLEX_SELF_MANAGED, NGH_FLEX_LAZY_BLOCKS_PER_CU, NGH_ORDERED_ARRIVAL); the end-of-kernel
 # policy hands over between workgroups with relaxed tickets (default) or release tickets and an acquire fence
-_POLICY_MODES = [("host", None, None, None), ("three-launches", "0", None, None), ("end-of-kernel", "1", None, None),
-                 ("end-of-kernel-release-acquire-tickets", "1", None, "1"),
-                 ("deferred", "2", None, None), ("deferred-small-grid", "2", "1", None)]
+# (name, NGH_FLEX_SELF_MANAGED, NGH_FLEX_LAZY_BLOCKS_PER_CU, NGH_ORDERED_ARRIVAL, NGH_STREAM_MIB); the last one
+# lowers the size from which a stage takes the policy step at its end instead of deferring it, so
+# that stages of both kinds follow each other on the same tensors
+_AMBIENT_STREAM_MIB = os.environ.get("NGH_STREAM_MIB")
+_POLICY_MODES = [("host", None, None, None, None), ("three-launches", "0", None, None, None),
+                 ("end-of-kernel", "1", None, None, None),
+                 ("end-of-kernel-release-acquire-tickets", "1", None, "1", None),
+                 ("deferred", "2", None, None, None), ("deferred-small-grid", "2", "1", None, None),
+                 ("mixed-by-size", "2", None, None, "1")]
 
 
 def _entry_state(entry):
     return (entry.dec, entry.next_dec, entry.last_maxabs, tuple(entry.history))
 
 
-def _with_policy_mode(monkeypatch, mode, grid, ordered=None):
+def _with_policy_mode(monkeypatch, mode, grid, ordered=None, stream_mib=None):
     monkeypatch.delenv("NGH_FLEX_SELF_MANAGED", raising=False)
+    if stream_mib is not None:
+        monkeypatch.setenv("NGH_STREAM_MIB", stream_mib)
+    elif _AMBIENT_STREAM_MIB is None:
+        monkeypatch.delenv("NGH_STREAM_MIB", raising=False)
+    else:
+        monkeypatch.setenv("NGH_STREAM_MIB", _AMBIENT_STREAM_MIB)
     monkeypatch.delenv("NGH_FLEX_LAZY_BLOCKS_PER_CU", raising=False)
     monkeypatch.delenv("NGH_ORDERED_ARRIVAL", raising=False)
     if ordered is not None:
@@ -269,8 +281,8 @@ def test_device_only_iterations_agree_across_policy_modes(n, monkeypatch):
     x0, w, b = configs.c5_inputs(n, seed=11)
     x0 = (x0 * 30.0).astype(np.float32)           # saturates at the first exponent: the policy has to move
     seen = {}
-    for name, mode, grid, ordered in _POLICY_MODES:
-        _with_policy_mode(monkeypatch, mode, grid, ordered)
+    for name, mode, grid, ordered, stream_mib in _POLICY_MODES:
+        _with_policy_mode(monkeypatch, mode, grid, ordered, stream_mib)
         t = ngt.make_transformer_factory("flexhip", resident=name != "host")()
         try:
             f, _, _ = _c5_graph(t, n)
@@ -284,6 +296,8 @@ def test_device_only_iterations_agree_across_policy_modes(n, monkeypatch):
                         assert t.runtime.flex_unsettled() == 1    # y's record, and only that
                     else:           # a forced kernel choice may or may not take the one-launch path
                         assert t.runtime.flex_unsettled() in (0, 1)
+                elif name == "mixed-by-size":
+                    assert t.runtime.flex_unsettled() in (0, 1)
                 elif name != "host":
                     assert t.runtime.flex_unsettled() == 0
                 if it in (2, 6):                    # look twice: after a few launches, and at the end
@@ -306,8 +320,8 @@ def test_consumer_of_a_tensor_with_unfolded_statistics(monkeypatch):
     n = 1 << 18
     x0, w, b = configs.c5_inputs(n, seed=12)
     seen = {}
-    for name, mode, grid, ordered in _POLICY_MODES:
-        _with_policy_mode(monkeypatch, mode, grid, ordered)
+    for name, mode, grid, ordered, stream_mib in _POLICY_MODES:
+        _with_policy_mode(monkeypatch, mode, grid, ordered, stream_mib)
         t = ngt.make_transformer_factory("flexhip", resident=name != "host")()
         try:
             P = ng.make_axis(n, name="P")
@@ -342,8 +356,8 @@ def test_in_place_rule_iterated_on_the_device_agrees_across_policy_modes(monkeyp
     p0 = rs.normal(0, 0.1, n).astype(np.float32)
     g = rs.normal(0, 0.05, n).astype(np.float32)
     seen = {}
-    for name, mode, grid, ordered in _POLICY_MODES:
-        _with_policy_mode(monkeypatch, mode, grid, ordered)
+    for name, mode, grid, ordered, stream_mib in _POLICY_MODES:
+        _with_policy_mode(monkeypatch, mode, grid, ordered, stream_mib)
         t = ngt.make_transformer_factory("flexhip", resident=name != "host")()
         try:
             P = ng.make_axis(n, name="P")
