@@ -53,6 +53,7 @@ struct KArgs {
     int       n_store_stat_slots;   // the first of them belong to tensors a STORE op writes, the rest to reduction results
     int       n_staged;      // tiled skeleton: operands staged through LDS tiles
     int       tile_diagonal; // tiled skeleton: deal the tiles along diagonals (strides that are multiples of 4 KiB)
+    int       ragged;        // rows along kernel axis 2 are not whole aligned vectors: a row's last chunk is short
     unsigned  rng_seed, rng_counter;   // NGH_OP_RNG_*
     int       probe;         // NGH_SPEC_PROBE: record max|value| bits instead of storing
     int*      stat_ptr[4];   // device word of each per-thread accumulator

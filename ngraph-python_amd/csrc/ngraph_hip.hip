@@ -123,6 +123,7 @@ struct ngh_context {
     int         row_wave_chunks = 0;     // rows of up to this many chunks are reduced by one wavefront each
     int         tile4 = 1;               // tiled elementwise programs may take 64 x 64 tiles with 16-byte accesses
     int         no_tiles = 0;        // never use the LDS-tiled elementwise skeleton
+    int         no_ragged = 0;       // never run compiled programs 4-wide over rows that are not whole aligned vectors
     int         flex_self_managed = 2;  // ngh_launch_fused_flex: 0 = prepare / kernel / update launches,
                                      // 1 = policy at the end of the kernel, 2 = statistics deferred to the next user
                                      // for stages up to stream_bytes and 1 beyond, 3 = always deferred
@@ -376,6 +377,21 @@ bool vec_ok(const KArgs& k, const bool* used, int V, bool any_type = false) {
 
 bool vec4_ok(const KArgs& k, const bool* used) { return vec_ok(k, used, 4); }
 
+// Can the stage move 4 elements per lane along kernel axis 2 although vec_ok says no -- rows whose
+// length is not a multiple of 4, or that do not start on 16-byte boundaries?  The compiled
+// programs can (program_ragged_ok has the conditions on the program), given unit strides.
+bool ragged_rows_ok(const KArgs& k, const bool* used) {
+    if (k.shape[2] < 8) return false;
+    int dtypes[NGH_MAX_TENSORS];
+    unsigned char bcast[NGH_MAX_TENSORS];
+    for (int t = 0; t < NGH_MAX_TENSORS; ++t) {
+        dtypes[t] = t < k.n_tensors ? k.t[t].dtype : NGH_F32;
+        bcast[t] = (t < k.n_tensors && k.t[t].s[2] == 0) ? 1 : 0;
+        if (t < k.n_tensors && used[t] && k.t[t].s[2] != 0 && k.t[t].s[2] != 1) return false;
+    }
+    return program_ragged_ok(4, k.ops + k.op_begin, k.op_end - k.op_begin, dtypes, bcast);
+}
+
 constexpr size_t kInterpLdsPreferred = 64 * 1024;   // keeps >= 2 workgroups per CU
 constexpr size_t kInterpLdsMax = 128 * 1024;
 constexpr size_t kInterpLdsWide = 40 * 1024;        // budget when widening the interpreter's vectors
@@ -399,16 +415,23 @@ int gather_width(const KArgs& k) {
     return interp_lds_bytes(k, 4) <= kInterpLdsPreferred ? 4 : 1;
 }
 
-int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan& P);
+int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan& P, bool allow_ragged);
 
 int plan_stage(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan& P) {
-    NGH_TRY(plan_stage_impl(ctx, sp, stage, P));
+    NGH_TRY(plan_stage_impl(ctx, sp, stage, P, !(ctx && (ctx->force_interp || ctx->no_ragged))));
+    // Ragged rows are a mode of the compiled programs only: a stage without one (yet) is planned
+    // again for the interpreter.  (Without a context the plan says what a program should be
+    // compiled for.)
+    if (P.k.ragged && ctx && (P.k.probe || match_special(P.family, P.V, P.k, 0) < 0)) {
+        P = Plan();
+        NGH_TRY(plan_stage_impl(ctx, sp, stage, P, false));
+    }
     if (P.k.n_stat_slots > 4)
         return fail(NGH_E_UNSUPPORTED, "stage %d stores more than 4 flex16 tensors with statistics", stage);
     return NGH_OK;
 }
 
-int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan& P) {
+int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage, Plan& P, bool allow_ragged) {
     const ngh_stage& S = sp.stages[stage];
     bool loads[NGH_MAX_TENSORS], stores[NGH_MAX_TENSORS], used[NGH_MAX_TENSORS];
     stage_tensors(sp, S, loads, stores);
@@ -451,6 +474,10 @@ int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage,
                 if (vec_ok(P.k, used, V)) { P.V = V; P.tail = n % V; break; }
                 P.k.shape[2] = n;
             }
+        }
+        if (allow_ragged && P.V == 1 && P.tail == 0 && P.k.shape[0] * P.k.shape[1] > 1 && ragged_rows_ok(P.k, used)) {
+            P.V = 4;
+            P.k.ragged = 1;
         }
         bool plain_stores = true;     // a truncating store writes memory directly, never through a tile
         for (int pc = S.op_begin; pc < S.op_end; ++pc) plain_stores = plain_stores && sp.ops[pc].opcode != NGH_OP_STORE_TRUNC;
@@ -521,7 +548,7 @@ int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage,
         if (P.tail == 0 && P.V >= 4)
             if (P.V < 8 && vec_ok(P.k, used, 8, true) && interp_lds_bytes(P.k, 8) <= kInterpLdsWide) P.Vi = 8;
         const long long rows = P.k.shape[0] * P.k.shape[1];
-        const long long cpr = P.k.shape[2] / P.V;
+        const long long cpr = (P.k.shape[2] + (P.k.ragged ? P.V - 1 : 0)) / P.V;
         if (rows * cpr >= (1LL << 32) || rows >= (1LL << 32))
             return fail(NGH_E_UNSUPPORTED, "stage has %lld chunks; split the launch", rows * cpr);
         P.chunks_per_row = (unsigned)cpr;
@@ -612,8 +639,12 @@ int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage,
         for (int a = 0; a < 3; ++a) P.perm[a] = perm[a];
         P.family = F_RED_ROW;
         P.V = (r_contig && vec4_ok(P.k, used)) ? 4 : 1;
+        if (allow_ragged && P.V == 1 && r_contig && ragged_rows_ok(P.k, used)) {
+            P.V = 4;
+            P.k.ragged = 1;
+        }
         P.n_out = (unsigned)n_out;
-        const long long chunks = R / P.V;
+        const long long chunks = (R + (P.k.ragged ? P.V - 1 : 0)) / P.V;
         if (chunks <= 64) {
             // short rows: TR lanes per row, several rows per workgroup, no segments
             P.small_rows = true;
@@ -876,6 +907,7 @@ int launch_interp(ngh_context* ctx, Plan& P) {
         HIP_TRY(hipGetLastError());
         return stat_fold(ctx, P.k, blocks);
     }
+    if (P.k.ragged && P.special < 0) return fail(NGH_E_RUNTIME, "a stage planned for ragged rows has no compiled program");
     int V = (P.family == F_EW) ? P.Vi : P.V;
     size_t lds = interp_lds_bytes(P.k, V);
     while (lds > kInterpLdsPreferred && V > 1 && P.family == F_EW) {
@@ -1054,6 +1086,7 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->flex_lazy_blocks_per_cu = env_int("NGH_FLEX_LAZY_BLOCKS_PER_CU", 6);
     if (ctx->flex_lazy_blocks_per_cu == 0) ctx->flex_lazy_blocks_per_cu = 1;
     ctx->no_tiles = env_int("NGH_NO_TILES", 0);
+    ctx->no_ragged = env_int("NGH_NO_RAGGED", 0);
     ctx->red_wgs_per_cu = std::max(1, env_int("NGH_RED_WGS_PER_CU", 8));
     ctx->red_col_wgs_per_cu = std::max(1, env_int("NGH_RED_COL_WGS_PER_CU", 2));
     ctx->row_wave_chunks = std::max(0, env_int("NGH_ROW_WAVE_CHUNKS", kRowWaveChunks));
@@ -1323,6 +1356,7 @@ int ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec, int32_t sta
     describe(P, name128, 128);
     long long ta4, tb4, n4;
     if (wants_tile4(ctx, P, ta4, tb4, n4)) strncat(name128, "/tiles64", 127 - strlen(name128));
+    if (P.k.ragged) strncat(name128, "/ragged", 127 - strlen(name128));
     if (P.special >= 0 && P.family == F_EW) {
         static const char* const suffix[4] = {"", "/nt-loads", "/nt-stores", "/nt-loads-stores"};
         const int cp = stage_cache_policy(ctx, *spec, spec->stages[stage]);
@@ -1514,6 +1548,11 @@ int ngh_plan_fused(const ngh_fused_spec* spec, int32_t stage, int32_t* out8) {
     if (stage < 0 || stage >= spec->n_stages) return fail(NGH_E_INVALID, "stage %d", stage);
     Plan P;
     NGH_TRY(plan_stage(nullptr, *spec, stage, P));
+    if (P.k.ragged && env_int("NGH_NO_RAGGED", 0)) {
+        // (no context here to carry the knob: the plan a program gets compiled for follows it too)
+        P = Plan();
+        NGH_TRY(plan_stage_impl(nullptr, *spec, stage, P, false));
+    }
     out8[0] = (int)P.family; out8[1] = P.V;
     out8[2] = P.perm[0]; out8[3] = P.perm[1]; out8[4] = P.perm[2];
     out8[5] = (int)P.tail;

@@ -74,6 +74,23 @@ def case_ragged():
     return [ng.exp(-ng.square(x)) * y + 1.0, ng.sum(x * y + 1.0, out_axes=[A])], [x, y]
 
 
+def case_ragged_long_rows():
+    # rows of 4099 elements: 4 elements per lane with a short last chunk per row, a workgroup per
+    # row segment in the elementwise pass and per row in the reductions
+    A, B = ng.make_axis(37, name="A"), ng.make_axis(4099, name="B")
+    x, y = ng.placeholder([A, B]), ng.placeholder([A, B])
+    return [ng.tanh(x * y) + x, ng.sum(x * y + 1.0, out_axes=[A]), ng.max(x - y, out_axes=[A]),
+            ng.argmax(x + y, out_axes=[A])], [x, y]
+
+
+def case_ragged_many_rows():
+    # a softmax over many rows of 1001: a wavefront per row in the reductions
+    C, N = ng.make_axis(1001, name="C"), ng.make_axis(4200, name="N")
+    x = ng.placeholder([N, C])
+    e = ng.exp(x - ng.max(x, out_axes=[N]))
+    return [e / ng.sum(e, out_axes=[N])], [x]
+
+
 def case_misaligned_slices():
     # windows that start one element into rows of odd length: no vector access, so the
     # compiled program takes one element per lane with the operands' own strides
@@ -113,7 +130,7 @@ def case_lookup_table():
 
 FP32_CASES = [case_elementwise, case_column_reduction_with_store, case_row_reduction_with_store,
               case_transposed_operand, case_transposed_operands_large, case_softmax, case_mixed_storage_types, case_ragged,
-              case_misaligned_slices, case_short_rows, case_dropout, case_lookup_table]
+              case_ragged_long_rows, case_ragged_many_rows, case_misaligned_slices, case_short_rows, case_dropout, case_lookup_table]
 
 
 def flex_case():

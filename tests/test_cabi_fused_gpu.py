@@ -434,7 +434,12 @@ def test_binary_ops_on_special_values(hip_runtime, name):
                                           ((300, 4096), "col"), ((37, 4100), "col"), ((2000, 1027), "col"),
                                           # thousands of rows of a few hundred chunks: a wavefront per row
                                           ((1024, 4200), "row"), ((300, 5000), "row"), ((401, 4100), "row"),
-                                          ((2048, 4096), "row")])
+                                          ((2048, 4096), "row"),
+                                          # rows that are not whole float4s: 4 elements per lane all the same,
+                                          # a short last chunk per row (several rows per workgroup, a wavefront
+                                          # per row, a workgroup per row, several workgroups per row)
+                                          ((77, 300), "row"), ((1001, 4200), "row"), ((4099, 40), "row"),
+                                          ((20003, 5), "row")])
 def test_every_reduction(hip_runtime, name, shape, layout):
     """Reduce axis 0 of an [R, A] view; 'row' = R contiguous in memory, 'col' = A contiguous."""
     rt = hip_runtime
@@ -466,6 +471,8 @@ def test_every_reduction(hip_runtime, name, shape, layout):
     spec = sb.build()
     rt.launch_fused(spec)
     got = out_d.get()
+    if layout == "row" and R % 4 and R >= 8 and name == "sum" and default_kernel_choice():
+        assert rt.describe_fused(spec, 0).endswith("/ragged")
     if is_arg:
         np.testing.assert_array_equal(got, want)
     else:

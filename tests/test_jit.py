@@ -212,8 +212,15 @@ def test_compiled_programs_agree_with_the_interpreter(case):
     want, _ = _run("cpu", case, 5)
     interp, names_interp = _run("hipgpu", case, 5, jit=False)
     compiled, names = _run("hipgpu", case, 5, jit=True)
+    # Same bits as the interpreter -- except where the compiled program runs 4 elements per lane
+    # over rows that are not whole aligned vectors (the interpreter takes those one element per
+    # lane): a reduction then adds up in another order.
+    ragged = any("/ragged" in n for n in names)
     for a, b, w in zip(interp, compiled, want):
-        np.testing.assert_array_equal(a, b)
+        if ragged:
+            np.testing.assert_allclose(a, b, rtol=2e-6, atol=1e-6)
+        else:
+            np.testing.assert_array_equal(a, b)
         if case is jit_cases.case_dropout:
             # the oracle draws from NumPy's generator: only the distribution is comparable
             assert abs(np.count_nonzero(compiled[0]) / compiled[0].size - 0.75) < 0.01
@@ -222,6 +229,9 @@ def test_compiled_programs_agree_with_the_interpreter(case):
     if default_kernel_choice():
         # every stage large enough to be worth a compiled kernel has one now
         assert not any("interp" in n for n in names if "tail" not in n), names
+        if case in (jit_cases.case_ragged, jit_cases.case_ragged_long_rows, jit_cases.case_ragged_many_rows,
+                    jit_cases.case_misaligned_slices):
+            assert any(n.endswith("/ragged") for n in names), names
         if case is jit_cases.case_transposed_operands_large:
             assert any(n.endswith("/tiles64") for n in names), names
 
@@ -235,11 +245,17 @@ def test_random_graphs_compiled_agree_with_the_interpreter(seed, views):
         try:
             results, inputs, values = jit_cases.random_case(seed, views)
             f = t.computation(results, *inputs)
-            return [np.array(r).copy() for r in f(*values)]
+            out = [np.array(r).copy() for r in f(*values)]
+            return out, [d for k in t.kernel_groups[f].kernels for ds in k.describe() for d in ds]
         finally:
             t.close()
-    for a, b in zip(run(jit=False), run(jit=True, jit_min_elements=1)):
-        np.testing.assert_array_equal(a, b)
+    (interp, _), (compiled, names) = run(jit=False), run(jit=True, jit_min_elements=1)
+    ragged = any("/ragged" in n for n in names)       # (see the test above)
+    for a, b in zip(interp, compiled):
+        if ragged:
+            np.testing.assert_allclose(a, b, rtol=1e-5, atol=1e-5)
+        else:
+            np.testing.assert_array_equal(a, b)
 
 
 @pytest.mark.gpu
