@@ -294,6 +294,16 @@ int  ngh_convert_to_flex16(ngh_context* ctx, int16_t* dev_out, const void* dev_i
  * index of the matching pre-built specialisation or -1, reduction segments}.     */
 int  ngh_plan_fused(const ngh_fused_spec* spec, int32_t stage, int32_t* out8);
 
+/* Would ngh_launch_fused run every stage of the spec in ONE kernel -- the way the reference's
+ * compound kernels run their stages one after the other inside one launch, a reduction's result
+ * reaching the next stage without a trip through a second launch (float_ew2.py:1135-1483,
+ * stage loop :1268-1321)?  Possible for a "row chain": rows (spec axis 0, the reduced one) of up
+ * to 2048 elements, fp32 operands with unit stride along the row or broadcast along it, at
+ * least one reduction stage.  out4 = {1 if the spec qualifies, index of the compiled chain
+ * program or -1 (without one the stages are launched one by one), lanes per row, stages}.
+ * No device needed (host-side tooling and tests).                                          */
+int  ngh_plan_chain(const ngh_fused_spec* spec, int32_t* out4);
+
 /* ---- flex statistics: the int32 device words FlexPtrDescription binds
  *      (float_ew2.py:363-374); replaces the manager's allocate/readback
  *      (flexgputransform.py:143-150, 361-366)                                */

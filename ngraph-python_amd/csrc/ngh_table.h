@@ -82,10 +82,35 @@ inline int match_special(int family, int V, const KArgs& k, long long /*tail*/) 
     return -1;
 }
 
+// A chain (family 4) whose stages are the programs of `ks` (argument blocks of the spec's stages
+// in row order: kernel axis 2 = the reduced axis; families[i] = 1 for a stage with reductions,
+// 0 for an elementwise one), or -1.
+inline int match_chain(const KArgs* ks, const int* families, int n) {
+    auto matches = [&](const StaticEntry& e) {
+        if (e.family != 4 || e.chain_len != n) return false;
+        for (int i = 0; i < n; ++i)
+            if (!entry_matches(e.chain[i], families[i], 4, ks[i])) return false;
+        return true;
+    };
+    for (int i = 0; i < kStaticCount; ++i)
+        if (matches(kStaticTable[i])) return i;
+    LoadedPrograms& L = loaded_programs();
+    const int count = L.count.load(std::memory_order_acquire);
+    for (int i = 0; i < count; ++i)
+        if (matches(L.entries[i])) return kStaticCount + i;
+    return -1;
+}
+
 // Same program (what match_special compares), whatever the name.
 inline bool same_program(const StaticEntry& a, const StaticEntry& b) {
     if (a.family != b.family || a.V != b.V || a.n_ops != b.n_ops || a.n_tensors != b.n_tensors || a.n_red != b.n_red)
         return false;
+    if (a.family == 4) {
+        if (a.chain_len != b.chain_len) return false;
+        for (int i = 0; i < a.chain_len; ++i)
+            if (!same_program(a.chain[i], b.chain[i])) return false;
+        return true;
+    }
     for (int r = 0; r < a.n_red; ++r) if (a.red_out[r] != b.red_out[r]) return false;
     for (int j = 0; j < a.n_ops; ++j)
         if (a.ops[j].opcode != b.ops[j].opcode || a.ops[j].dst != b.ops[j].dst || a.ops[j].a != b.ops[j].a ||
@@ -135,6 +160,12 @@ inline hipError_t launch_special_tiled(int i, hipStream_t stream, unsigned block
 inline hipError_t launch_special_red(int i, hipStream_t stream, unsigned blocks, const KArgs& k, unsigned n_first,
                                      unsigned n_seg, unsigned seg_len, unsigned TX, RedWs ws, int cache_policy) {
     special_entry(i).launch_red(stream, blocks, k, n_first, n_seg, seg_len, TX, ws, cache_policy);
+    return hipGetLastError();
+}
+
+inline hipError_t launch_special_chain(int i, hipStream_t stream, unsigned blocks, const KArgs& k, unsigned n_out,
+                                       unsigned TR, int cache_policy) {
+    special_entry(i).launch_chain(stream, blocks, k, n_out, TR, cache_policy);
     return hipGetLastError();
 }
 

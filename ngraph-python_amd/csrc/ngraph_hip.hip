@@ -123,6 +123,7 @@ struct ngh_context {
     int         row_wave_chunks = 0;     // rows of up to this many chunks are reduced by one wavefront each
     int         tile4 = 1;               // tiled elementwise programs may take 64 x 64 tiles with 16-byte accesses
     int         no_tiles = 0;        // never use the LDS-tiled elementwise skeleton
+    int         no_chain = 0;        // never run the stages of a spec as one row-chain kernel
     int         no_ragged = 0;       // never run compiled programs 4-wide over rows that are not whole aligned vectors
     int         flex_self_managed = 2;  // ngh_launch_fused_flex: 0 = prepare / kernel / update launches,
                                      // 1 = policy at the end of the kernel, 2 = statistics deferred to the next user
@@ -1087,6 +1088,7 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     if (ctx->flex_lazy_blocks_per_cu == 0) ctx->flex_lazy_blocks_per_cu = 1;
     ctx->no_tiles = env_int("NGH_NO_TILES", 0);
     ctx->no_ragged = env_int("NGH_NO_RAGGED", 0);
+    ctx->no_chain = env_int("NGH_NO_CHAIN", 0);
     ctx->red_wgs_per_cu = std::max(1, env_int("NGH_RED_WGS_PER_CU", 8));
     ctx->red_col_wgs_per_cu = std::max(1, env_int("NGH_RED_COL_WGS_PER_CU", 2));
     ctx->row_wave_chunks = std::max(0, env_int("NGH_ROW_WAVE_CHUNKS", kRowWaveChunks));
@@ -1314,10 +1316,76 @@ static int stage_cache_policy(const ngh_context* ctx, const ngh_fused_spec& sp, 
     return ((any_load && all_load) ? 1 : 0) | ((any_store && all_store) ? 2 : 0);
 }
 
+// ---------------------------------------------------------------------------
+// Row chains: every stage of a spec in one kernel (row_chain_static_kernel).  Possible when the
+// spec's rows -- spec axis 0, the axis its reduction stages reduce -- are short enough for a group
+// of lanes of one wavefront each, and every stage can run over ragged rows (fp32 operands with
+// unit stride along the row, or broadcast along it).
+// ---------------------------------------------------------------------------
+struct ChainPlan {
+    int      n = 0;                       // stages (the spec's non-empty ones)
+    int      stage_of[NGH_MAX_STAGES];
+    int      families[NGH_MAX_STAGES];
+    KArgs    k[NGH_MAX_STAGES];
+    unsigned n_out = 0, TR = 64;
+    int      special = -1;
+};
+
+// Could the spec run as a row chain (whether or not a compiled chain exists)?
+bool plan_row_chain(const ngh_context* ctx, const ngh_fused_spec& sp, ChainPlan& C) {
+    if (sp.flags & NGH_SPEC_PROBE) return false;
+    const long long wave_chunks = ctx ? ctx->row_wave_chunks : kRowWaveChunks;
+    const long long R = sp.shape[0], n_out = sp.shape[1] * sp.shape[2];
+    const long long chunks = (R + 3) / 4;
+    if (R < 8 || chunks > wave_chunks || chunks > 64 * kChainAhead || n_out < 1 || n_out >= (1LL << 31)) return false;
+    bool any_red = false;
+    const int perm[3] = {1, 2, 0};
+    for (int s = 0; s < sp.n_stages; ++s) {
+        const ngh_stage& S = sp.stages[s];
+        if (S.op_end == S.op_begin) continue;
+        if (C.n == NGH_MAX_STAGES) return false;
+        KArgs& k = C.k[C.n];
+        fill_kargs(sp, S, perm, k);
+        bool loads[NGH_MAX_TENSORS], stores[NGH_MAX_TENSORS], used[NGH_MAX_TENSORS];
+        stage_tensors(sp, S, loads, stores);
+        for (int t = 0; t < NGH_MAX_TENSORS; ++t) used[t] = loads[t] || stores[t];
+        if (k.n_stat_slots != 0 || k.probe || !ragged_rows_ok(k, used) ||
+            !program_loads_hoistable(k.ops + k.op_begin, k.op_end - k.op_begin))
+            return false;
+        for (int r = 0; r < S.n_reductions; ++r) {
+            const ngh_tensor& T = sp.tensors[S.red_out[r]];
+            if (T.strides[0] != 0 || (T.dtype != NGH_F32 && T.dtype != NGH_I32 && T.dtype != NGH_U32)) return false;
+        }
+        any_red = any_red || S.n_reductions > 0;
+        C.stage_of[C.n] = s;
+        C.families[C.n] = S.n_reductions > 0 ? 1 : 0;
+        ++C.n;
+    }
+    if (C.n < 2 || !any_red) return false;
+    C.n_out = (unsigned)n_out;
+    C.TR = 1;
+    while ((long long)C.TR < chunks && C.TR < 64) C.TR <<= 1;
+    // (rows enough to fill the chip several times over: a lane takes up to four chunks of its row)
+    const long long lanes_wanted = (ctx ? ctx->cus : 256) * 2048LL * 4;
+    for (int shrink = 0; shrink < 2 && chunks <= 64 && C.TR > 1 && n_out * (C.TR / 2) >= lanes_wanted; ++shrink)
+        C.TR >>= 1;
+    return true;
+}
+
 int ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec) {
     if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
     NGH_TRY(validate(spec));
     NGH_TRY(flex_settle_spec(ctx, *spec));
+    if (spec->n_stages > 1 && !ctx->force_interp && !ctx->no_chain && !ctx->no_ragged) {
+        ChainPlan C;
+        if (plan_row_chain(ctx, *spec, C) && (C.special = match_chain(C.k, C.families, C.n)) >= 0) {
+            const unsigned rows_per_wg = kBlock / C.TR;
+            const unsigned blocks = (C.n_out + rows_per_wg - 1) / rows_per_wg;
+            const int cp = stage_cache_policy(ctx, *spec, spec->stages[C.stage_of[C.n - 1]]) & kCpNtStore;
+            HIP_TRY(launch_special_chain(C.special, ctx->stream, blocks, C.k[C.n - 1], C.n_out, C.TR, cp));
+            return NGH_OK;
+        }
+    }
     for (int s = 0; s < spec->n_stages; ++s) {
         if (spec->stages[s].op_end == spec->stages[s].op_begin) continue;
         Plan P;
@@ -1349,6 +1417,14 @@ int ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec, int32_t sta
     if (!ctx || !name128) return fail(NGH_E_INVALID, "NULL argument");
     NGH_TRY(validate(spec));
     if (stage < 0 || stage >= spec->n_stages) return fail(NGH_E_INVALID, "stage %d", stage);
+    if (spec->n_stages > 1 && !ctx->force_interp && !ctx->no_chain && !ctx->no_ragged) {
+        ChainPlan C;
+        if (plan_row_chain(ctx, *spec, C) && (C.special = match_chain(C.k, C.families, C.n)) >= 0) {
+            const int cp = stage_cache_policy(ctx, *spec, spec->stages[C.stage_of[C.n - 1]]) & kCpNtStore;
+            snprintf(name128, 128, "special:%s/chain-of-%d%s", special_name(C.special), C.n, cp ? "/nt-stores" : "");
+            return NGH_OK;
+        }
+    }
     Plan P;
     NGH_TRY(plan_stage(ctx, *spec, stage, P));
     if (!ctx->force_interp)
@@ -1558,6 +1634,19 @@ int ngh_plan_fused(const ngh_fused_spec* spec, int32_t stage, int32_t* out8) {
     out8[5] = (int)P.tail;
     out8[6] = match_special(P.family, P.V, P.k, P.tail);
     out8[7] = (int)P.n_seg;
+    return NGH_OK;
+}
+
+int ngh_plan_chain(const ngh_fused_spec* spec, int32_t* out4) {
+    if (!out4) return fail(NGH_E_INVALID, "out4 is NULL");
+    NGH_TRY(validate(spec));
+    ChainPlan C;
+    const bool ok = spec->n_stages > 1 && !env_int("NGH_NO_CHAIN", 0) && !env_int("NGH_NO_RAGGED", 0) &&
+                    plan_row_chain(nullptr, *spec, C);
+    out4[0] = ok ? 1 : 0;
+    out4[1] = ok ? match_chain(C.k, C.families, C.n) : -1;
+    out4[2] = ok ? (int)C.TR : 0;
+    out4[3] = ok ? C.n : 0;
     return NGH_OK;
 }
 

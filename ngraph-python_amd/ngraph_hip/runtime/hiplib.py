@@ -114,6 +114,7 @@ _SYMBOLS = {
                                 ctypes.c_float, ctypes.c_uint32],
     "ngh_convert_to_flex16": [_vp, _vp, _vp, _i32, ctypes.c_int64, ctypes.c_float, _vp, _vp],
     "ngh_plan_fused": [ctypes.POINTER(ngh_fused_spec), _i32, ctypes.POINTER(ctypes.c_int32)],
+    "ngh_plan_chain": [ctypes.POINTER(ngh_fused_spec), ctypes.POINTER(ctypes.c_int32)],
     "ngh_stats_alloc": [_vp, _i32, ctypes.POINTER(_vp)],
     "ngh_stats_reset": [_vp, _vp, _i32],
     "ngh_stats_read": [_vp, _vp, _i32, _vp],
@@ -166,6 +167,14 @@ def plan_fused(spec, stage=0):
     _check(lib, lib.ngh_plan_fused(ctypes.byref(spec), int(stage), out))
     return {"family": out[0], "V": out[1], "perm": (out[2], out[3], out[4]), "tail": out[5],
             "special": out[6], "segments": out[7]}
+
+
+def plan_chain(spec):
+    """Would the library run every stage of `spec` in one kernel (a row chain)?"""
+    lib = load_library()
+    out = (ctypes.c_int32 * 4)()
+    _check(lib, lib.ngh_plan_chain(ctypes.byref(spec), out))
+    return {"eligible": bool(out[0]), "special": out[1], "lanes_per_row": out[2], "stages": out[3]}
 
 
 def exported_symbols():

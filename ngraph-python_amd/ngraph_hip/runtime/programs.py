@@ -18,8 +18,16 @@ def stage_programs(kernels, name, seen=None, min_elements=4096, vector_only=Fals
     programs = []
     seen = set() if seen is None else seen
     k_index = 0
+    # (a run of kernels that has settled which of them merge stands for those kernels)
+    kernels = [u for k in kernels for u in (k.kernels if hasattr(k, "members") and hasattr(k, "kernels") else [k])]
     for kernel in kernels:
         for spec in getattr(kernel, "specs", [])[:1]:
+            if spec.n_stages > 1:
+                chain = _chain_program(spec, "%s_k%d" % (name, k_index), seen, min_elements)
+                if chain is not None:
+                    if chain:
+                        programs.append(chain)
+                    continue          # (its stages get no programs of their own)
             for stage in range(spec.n_stages):
                 plan = hiplib.plan_fused(spec, stage)
                 st = spec.stages[stage]
@@ -82,37 +90,91 @@ def stage_programs(kernels, name, seen=None, min_elements=4096, vector_only=Fals
     return programs
 
 
+def _chain_program(spec, name, seen, min_elements):
+    """The record of a spec whose stages run as one row-chain kernel (family 4: its second field
+    holds the records of the stages, which are programs over rows along spec axis 0, 4 elements
+    per lane); None when the spec is no chain, () when the chain is recorded already or too
+    small to be worth a kernel."""
+    plan = hiplib.plan_chain(spec)
+    if not plan["eligible"]:
+        return None
+    if spec.shape[0] * spec.shape[1] * spec.shape[2] < min_elements:
+        return ()
+    dtypes = [spec.tensors[i].dtype for i in range(spec.n_tensors)]
+    bcast = [1 if spec.tensors[i].strides[0] == 0 else 0 for i in range(spec.n_tensors)]
+    members = []
+    for stage in range(spec.n_stages):
+        st = spec.stages[stage]
+        if st.op_end == st.op_begin:
+            continue
+        ops = [(o.opcode, o.dst, o.a, o.b) for o in spec.ops[st.op_begin:st.op_end]]
+        red_out = [st.red_out[r] for r in range(st.n_reductions)]
+        stored = set(o[1] for o in ops if o[0] == hiplib.OPCODES["store"])
+        loaded = set(o[2] for o in ops if o[0] == hiplib.OPCODES["load"])
+        members.append(("%s_s%d" % (name, stage), ops, dtypes, bcast, [-1] * spec.n_tensors, 0, spec.n_regs, 4,
+                        1 if red_out else 0, red_out, [-1] * spec.n_tensors,
+                        [1 if i in loaded else 0 for i in range(spec.n_tensors)],
+                        [1 if i in stored else 0 for i in range(spec.n_tensors)], -1))
+    key = ("chain",) + tuple((tuple(m[1]), tuple(m[2]), tuple(m[3]), m[8], tuple(m[9])) for m in members)
+    if key in seen:
+        return ()
+    seen.add(key)
+    return (name, members, dtypes, bcast, [], 0, spec.n_regs, 4, 4, [], [], [], [], plan["special"])
+
+
+def _render_struct(lines, struct, record):
+    name, ops, dtypes, bcast, stat_slot, n_slots, n_regs, V, family, red_out, staged, loaded, stored, _ = record
+    lines.append("struct %s {  // %s" % (struct, name))
+    lines.append("    static constexpr int V = %d, n_ops = %d, n_regs = %d, n_tensors = %d, "
+                 "n_stat_slots = %d, family = %d, n_red = %d;"
+                 % (V, len(ops), max(n_regs, 1), len(dtypes), n_slots, family, len(red_out)))
+    lines.append("    static constexpr int red_out[%d] = {%s};"
+                 % (max(len(red_out), 1), ", ".join(map(str, red_out or [0]))))
+    lines.append("    static constexpr ngh_op ops[%d] = {%s};"
+                 % (len(ops), ", ".join("{%d,%d,%d,%d}" % o for o in ops)))
+    lines.append("    static constexpr int dtypes[%d] = {%s};" % (len(dtypes), ", ".join(map(str, dtypes))))
+    lines.append("    static constexpr unsigned char bcast[%d] = {%s};" % (len(bcast), ", ".join(map(str, bcast))))
+    lines.append("    static constexpr int stat_slot[%d] = {%s};" % (len(stat_slot), ", ".join(map(str, stat_slot))))
+    lines.append("    static constexpr int n_staged = %d;" % sum(1 for x in staged if x >= 0))
+    lines.append("    static constexpr signed char staged[%d] = {%s};" % (len(staged), ", ".join(map(str, staged))))
+    lines.append("    static constexpr unsigned char loaded[%d] = {%s};" % (len(loaded), ", ".join(map(str, loaded))))
+    lines.append("    static constexpr unsigned char stored[%d] = {%s};" % (len(stored), ", ".join(map(str, stored))))
+    lines.append("};")
+
+
+_ENTRY = ('{{"{1}", {0}::family, {0}::V, {0}::n_ops, {0}::ops, {0}::n_tensors, {0}::dtypes, '
+          '{0}::bcast, {0}::n_red, {0}::red_out, {2}}},')
+
+
 def render(programs, header, prefix="SP", table="kStaticTable", count="kStaticCount"):
     """C++ text: one `struct <prefix>n` per record, the entry table and its length."""
     lines = list(header)
-    for i, (name, ops, dtypes, bcast, stat_slot, n_slots, n_regs, V, family, red_out, staged, loaded,
-            stored, _) in enumerate(programs):
-        lines.append("struct %s%d {  // %s" % (prefix, i, name))
-        lines.append("    static constexpr int V = %d, n_ops = %d, n_regs = %d, n_tensors = %d, "
-                     "n_stat_slots = %d, family = %d, n_red = %d;"
-                     % (V, len(ops), max(n_regs, 1), len(dtypes), n_slots, family, len(red_out)))
-        lines.append("    static constexpr int red_out[%d] = {%s};"
-                     % (max(len(red_out), 1), ", ".join(map(str, red_out or [0]))))
-        lines.append("    static constexpr ngh_op ops[%d] = {%s};"
-                     % (len(ops), ", ".join("{%d,%d,%d,%d}" % o for o in ops)))
-        lines.append("    static constexpr int dtypes[%d] = {%s};" % (len(dtypes), ", ".join(map(str, dtypes))))
-        lines.append("    static constexpr unsigned char bcast[%d] = {%s};" % (len(bcast), ", ".join(map(str, bcast))))
-        lines.append("    static constexpr int stat_slot[%d] = {%s};" % (len(stat_slot), ", ".join(map(str, stat_slot))))
-        lines.append("    static constexpr int n_staged = %d;" % sum(1 for x in staged if x >= 0))
-        lines.append("    static constexpr signed char staged[%d] = {%s};" % (len(staged), ", ".join(map(str, staged))))
-        lines.append("    static constexpr unsigned char loaded[%d] = {%s};" % (len(loaded), ", ".join(map(str, loaded))))
-        lines.append("    static constexpr unsigned char stored[%d] = {%s};" % (len(stored), ", ".join(map(str, stored))))
-        lines.append("};")
+    for i, p in enumerate(programs):
+        if p[8] == 4:
+            # a chain: the structs of its stages and the array of their entries (no launchers)
+            for j, member in enumerate(p[1]):
+                _render_struct(lines, "%s%d_%d" % (prefix, i, j), member)
+            lines.append("static const StaticEntry %s%d_stages[] = {" % (prefix, i))
+            for j, member in enumerate(p[1]):
+                lines.append("    " + _ENTRY.format("%s%d_%d" % (prefix, i, j), member[0],
+                                                    "nullptr, nullptr, nullptr, nullptr"))
+            lines.append("};")
+        else:
+            _render_struct(lines, prefix + str(i), p)
     lines.append("static const StaticEntry %s[] = {" % table)
     for i, p in enumerate(programs):
+        if p[8] == 4:
+            stages = ", ".join("%s%d_%d" % (prefix, i, j) for j in range(len(p[1])))
+            lines.append('    {"%s", 4, 4, 0, nullptr, 0, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr, '
+                         '%d, %s%d_stages, &launch_static_chain<%s>},' % (p[0], len(p[1]), prefix, i, stages))
+            continue
         if p[8] == 0:
             launch = "&launch_static<{0}>, nullptr, {0}::staged, nullptr".format(prefix + str(i))
         elif p[8] == 3:
             launch = "nullptr, nullptr, {0}::staged, &launch_static_tiled<{0}>".format(prefix + str(i))
         else:
             launch = "nullptr, &launch_static_red<{0}>, {0}::staged, nullptr".format(prefix + str(i))
-        lines.append('    {{"{1}", {0}::family, {0}::V, {0}::n_ops, {0}::ops, {0}::n_tensors, {0}::dtypes, '
-                     '{0}::bcast, {0}::n_red, {0}::red_out, {2}}},'.format(prefix + str(i), p[0], launch))
+        lines.append("    " + _ENTRY.format(prefix + str(i), p[0], launch))
     if not programs:
         lines.append('    {"none", 0, 4, 0, nullptr, 0, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr},')
     lines.append("};")

@@ -27,6 +27,7 @@ import numpy as np
 
 from ngraph_hip.op_graph import op_graph as og
 from ngraph_hip.op_graph.op_graph import Op, OrderedSet
+from ngraph_hip.runtime import hiplib
 from ngraph_hip.runtime.hiplib import (HipRuntime, DryRunRuntime, HipLibraryError, FusedSpecBuilder, NGH_F32,
                                        NGH_FLEX16, NGH_I32, NGH_F16, NGH_U32, NGH_I16, NGH_I8, NGH_U8,
                                        NGH_MAX_TENSORS,
@@ -305,6 +306,50 @@ class _Dim(object):
         self.length, self.strides, self.tag, self.named = int(length), list(strides), tag, named
 
 
+def _emit_program(sb, program, inner):
+    """Append `program` (tuples over symbolic registers, FusedKernel._collect) to the spec builder
+    as the ops of its current stage; returns the operand slots it reads and writes."""
+    reg_map = {}
+
+    def reg(sym):
+        if sym not in reg_map:
+            reg_map[sym] = sb.reg()
+        return reg_map[sym]
+
+    written, read = set(), set()
+    for ins in program:
+        kind = ins[0]
+        if kind == "const":
+            sb.constant(ins[2], reg(ins[1]))
+        elif kind == "load":
+            sb.load(ins[2], reg(ins[1]))
+            read.add(ins[2])
+        elif kind in ("store", "store_trunc"):
+            sb.store(ins[1], reg(ins[2]), truncate=(kind == "store_trunc"))
+            written.add(ins[1])
+        elif kind == "iota":
+            axis = [i for i, d in enumerate(inner) if d.named == ins[2].name]
+            if not axis:
+                raise og_unsupported("one-hot axis was merged away")
+            sb.iota(axis[0], reg(ins[1]))
+        elif kind == "rng":
+            sb.rng(ins[2], ins[3], reg(ins[1]))
+        elif kind == "take":
+            axis = [i for i, d in enumerate(inner) if d.named == ins[4].name]
+            if not axis:
+                raise og_unsupported("lookup axis was merged away or looped on the host")
+            sb.take(ins[3], reg(ins[2]), axis[0], reg(ins[1]))
+            read.add(ins[3])
+        elif kind == "reduce":
+            sb.reduce(ins[1], reg(ins[2]), ins[3])
+            written.add(ins[3])
+        elif len(ins) == 3:
+            sb.unary(kind, reg(ins[2]), reg(ins[1]))
+        else:
+            sb.binary(kind, reg(ins[2]), reg(ins[3]), reg(ins[1]))
+    return read, written
+
+
 class FusedKernel(HipKernel):
     """A compound elementwise / reduction kernel = one ngh_fused_spec per outer index.
 
@@ -337,7 +382,10 @@ class FusedKernel(HipKernel):
             self._lower()
         super(FusedKernel, self).bind_buffers()
 
-    def _lower(self):
+    def _collect(self):
+        """Pass 1 of the lowering: the operands (views) the group touches and its program over
+        symbolic registers; returns (operands, program, it_axes, red_axes, onehot_axes,
+        take_axes, take_strides)."""
         t = self.transformer
         ops = self.ops
         first = ops[0]
@@ -466,6 +514,10 @@ class FusedKernel(HipKernel):
                 program.append(("store", slot(_td(op)), r))
 
         program.extend(reductions_at_end)
+        return operands, program, it_axes, red_axes, onehot_axes, take_axes, take_strides
+
+    def _lower(self):
+        operands, program, it_axes, red_axes, onehot_axes, take_axes, take_strides = self._collect()
 
         # ---- pass 2: dims = iteration axes with every operand's stride -----------------------
         def strides_over(td, axes):
@@ -564,44 +616,7 @@ class FusedKernel(HipKernel):
             slot = sb.tensor(view.ptr + offsets[s] * view.itemsize, strides, dtype,
                              take_extent=self.take_extents.get(s, 0))
             assert slot == s
-        reg_map = {}
-
-        def reg(sym):
-            if sym not in reg_map:
-                reg_map[sym] = sb.reg()
-            return reg_map[sym]
-
-        written, read = set(), set()
-        for ins in program:
-            kind = ins[0]
-            if kind == "const":
-                sb.constant(ins[2], reg(ins[1]))
-            elif kind == "load":
-                sb.load(ins[2], reg(ins[1]))
-                read.add(ins[2])
-            elif kind in ("store", "store_trunc"):
-                sb.store(ins[1], reg(ins[2]), truncate=(kind == "store_trunc"))
-                written.add(ins[1])
-            elif kind == "iota":
-                axis = [i for i, d in enumerate(inner) if d.named == ins[2].name]
-                if not axis:
-                    raise og_unsupported("one-hot axis was merged away")
-                sb.iota(axis[0], reg(ins[1]))
-            elif kind == "rng":
-                sb.rng(ins[2], ins[3], reg(ins[1]))
-            elif kind == "take":
-                axis = [i for i, d in enumerate(inner) if d.named == ins[4].name]
-                if not axis:
-                    raise og_unsupported("lookup axis was merged away or looped on the host")
-                sb.take(ins[3], reg(ins[2]), axis[0], reg(ins[1]))
-                read.add(ins[3])
-            elif kind == "reduce":
-                sb.reduce(ins[1], reg(ins[2]), ins[3])
-                written.add(ins[3])
-            elif len(ins) == 3:
-                sb.unary(kind, reg(ins[2]), reg(ins[1]))
-            else:
-                sb.binary(kind, reg(ins[2]), reg(ins[3]), reg(ins[1]))
+        read, written = _emit_program(sb, program, inner)
         spec = sb.build()
         index = len(self.specs)
         spec.rng_seed = (t.rng_seed * 0x9E3779B1 + index * 0x85EBCA77 + self.kernel_number) & 0xFFFFFFFF
@@ -876,6 +891,185 @@ class MomentsKernel(HipKernel):
         return [["moments_f32"]]
 
 
+class ChainKernel(HipKernel):
+    """Consecutive fused kernels over the same rows, merged: the STAGES of one spec.
+
+    Reductions along the rows whose results the next kernels read back, elementwise passes over
+    the same rows -- the maximum, the sum of exponentials and the normalised result of a softmax
+    -- which the library runs in one kernel when it can (ngh_plan_chain; the reference's
+    compound kernels run their stages inside one launch the same way, float_ew2.py:1135-1483).
+    The operand then crosses the memory interface once instead of once per kernel.
+    """
+
+    def __init__(self, transformer, members, spec, uses):
+        super(ChainKernel, self).__init__(transformer)
+        self.members = list(members)
+        self.name = self.members[0].name
+        self.ops = [op for m in self.members for op in m.ops]
+        self.specs = [spec]
+        self.spec_uses = [uses]
+        self.buffers_bound = True
+
+    @classmethod
+    def merged(cls, transformer, members):
+        """The ChainKernel of `members`, or None when they do not form a row chain."""
+        t = transformer
+        parts = [m._collect() for m in members]
+        red_axes, all_axes = None, None
+        for operands, program, it_axes, r_axes, onehot_axes, take_axes, _ in parts:
+            if onehot_axes or take_axes or any(ins[0] in ("iota", "rng", "take", "store_trunc") for ins in program):
+                return None
+            # (axes compare by name: a window of an axis is another iteration space)
+            extents = lambda axes: set((a.name, a.length) for a in axes)
+            if all_axes is None:
+                all_axes = it_axes
+            elif extents(it_axes) != extents(all_axes):
+                return None
+            if any(ins[0] == "reduce" for ins in program):
+                if red_axes is None:
+                    red_axes = r_axes
+                elif extents(r_axes) != extents(red_axes):
+                    return None
+            for td in operands:
+                if not extents(td.axes) <= extents(all_axes):
+                    return None
+        if red_axes is None or not extents(red_axes) <= extents(all_axes):
+            return None
+        order = list(red_axes) + [a for a in all_axes if a not in red_axes]
+
+        def walk(td):
+            return [td.full_strides[td.axes.index(axis)] if axis in td.axes else 0 for axis in order]
+
+        # one operand table for all stages; a view is known by the memory it walks over the chain's
+        # axes (a reduction's result, and the same tensor broadcast along the row for the next
+        # stage, are one operand)
+        union, slot_of, programs = [], {}, []
+        for operands, program, _, _, _, _, _ in parts:
+            local = []
+            for td in operands:
+                key = (td.base, td.dtype, td.offset, tuple(walk(td)))
+                if key not in slot_of:
+                    slot_of[key] = len(union)
+                    union.append(td)
+                local.append(slot_of[key])
+            remapped = []
+            for ins in program:
+                if ins[0] == "load":
+                    ins = (ins[0], ins[1], local[ins[2]])
+                elif ins[0] == "store":
+                    ins = (ins[0], local[ins[1]], ins[2])
+                elif ins[0] == "reduce":
+                    ins = (ins[0], ins[1], ins[2], local[ins[3]])
+                remapped.append(ins)
+            programs.append(remapped)
+        if len(union) > NGH_MAX_TENSORS:
+            return None
+        # what a stage writes, every stage must see through that one view
+        written = set(ins[1] for prog in programs for ins in prog if ins[0] == "store")
+        written |= set(ins[3] for prog in programs for ins in prog if ins[0] == "reduce")
+        for s in written:
+            if any(td.base is union[s].base and td is not union[s] for td in union):
+                return None
+        walks = [walk(td) for td in union]
+        dims = []
+        for j, axis in enumerate(order):
+            dims.append(_Dim(axis.length, [w[j] for w in walks], "red" if axis in red_axes else None))
+        if any(d.length == 0 for d in dims):
+            return None
+        dims = FusedKernel._coalesce(dims, True)
+        if len([d for d in dims if d.tag == "red"]) != 1 or len(dims) > 3:
+            return None          # (the reduced axes do not walk as one, or axes are left to a host loop)
+        outer, inner = FusedKernel._split_outer(dims, True)
+        sb = FusedSpecBuilder([d.length for d in inner] or [1])
+        for s, td in enumerate(union):
+            view = t.get_tensor_description_tensor_view(td)
+            sb.tensor(view.ptr, [d.strides[s] for d in inner] or [0], t.ngh_dtype(td.dtype))
+        read, written = set(), set()
+        try:
+            for prog in programs:
+                r, w = _emit_program(sb, prog, inner)
+                read |= r
+                written |= w
+                sb.end_stage()
+            spec = sb.build()
+        except ValueError:           # more ops, constants or live values than one spec holds
+            return None
+        if not hiplib.plan_chain(spec)["eligible"]:
+            return None
+        t.runtime.validate_fused(spec)
+        return cls(t, members, spec, [(td.base, s in read, s in written) for s, td in enumerate(union)])
+
+    def buffer_uses(self):
+        return list(self.spec_uses[0])
+
+    def set_cache_hints(self, hint_of):
+        for s, (base, is_read, is_written) in enumerate(self.spec_uses[0]):
+            self.specs[0].tensors[s].cache_hint = hint_of(base, is_read, is_written)
+
+    def execute(self):
+        self.transformer.runtime.launch_fused(self.specs[0])
+
+    def describe(self):
+        rt = self.transformer.runtime
+        return [[rt.describe_fused(spec, s) for s in range(spec.n_stages)] for spec in self.specs]
+
+
+class KernelRun(HipKernel):
+    """A run of consecutive fused kernels that may merge into ChainKernels.  Which do is decided
+    when the buffers are bound (a spec needs addresses): greedily, the longest runs the library
+    accepts as a row chain; a member that merges with no neighbour stays as it is.  The kernel
+    group then takes the resulting kernels in this one's place (HipKernelGroup.bind)."""
+
+    max_stages = 6               # NGH_MAX_STAGES
+
+    def __init__(self, transformer, members):
+        super(KernelRun, self).__init__(transformer)
+        self.members = list(members)
+        self.name = self.members[0].name
+        self.kernels = []
+
+    def bind_buffers(self):
+        if not self.buffers_bound:
+            self.kernels = []
+            a, n = 0, len(self.members)
+            while a < n:
+                merged = None
+                for b in range(min(n, a + self.max_stages), a + 1, -1):
+                    merged = ChainKernel.merged(self.transformer, self.members[a:b])
+                    if merged is not None:
+                        break
+                if merged is None:
+                    self.members[a].bind_buffers()
+                    self.kernels.append(self.members[a])
+                    a += 1
+                else:
+                    self.kernels.append(merged)
+                    a = b
+        super(KernelRun, self).bind_buffers()
+
+    @property
+    def ops(self):
+        return [op for m in self.members for op in m.ops]
+
+    @property
+    def specs(self):
+        return [spec for k in self.kernels for spec in k.specs]
+
+    def buffer_uses(self):
+        return [u for k in self.kernels for u in k.buffer_uses()]
+
+    def set_cache_hints(self, hint_of):
+        for k in self.kernels:
+            k.set_cache_hints(hint_of)
+
+    def execute(self):
+        for k in self.kernels:
+            k.execute()
+
+    def describe(self):
+        return [d for k in self.kernels for d in k.describe()]
+
+
 class HipKernelGroup(object):
     """The kernels of one computation and the loop that runs them (gputransform.py:348-522)."""
 
@@ -891,6 +1085,8 @@ class HipKernelGroup(object):
         for k in self.kernels:
             if not k.buffers_bound:
                 k.bind_buffers()
+        # (a run of kernels has settled which of them merge: its kernels take its place)
+        self.kernels = [u for k in self.kernels for u in (k.kernels if isinstance(k, KernelRun) else [k])]
         self.assign_cache_hints()
         mode = self.transformer.jit
         if mode is True:
@@ -1517,6 +1713,7 @@ class HipTransformer(ComputationGraphTransformer):
     kernel_group_class = HipKernelGroup
     max_written_views = NGH_MAX_TENSORS      # results one fused kernel may write
     split_reductions = True                  # ReductionLayoutPass: reduce group by group of axes, no copy
+    chain_kernels = True                     # consecutive kernels over the same rows run as stages of one spec
 
     def __init__(self, device_id=0, fusion=True, dry_run=False, fuse_moments=None, rng_seed=0, jit=None,
                  jit_min_elements=4096, jit_auto_min_elements=1 << 22, **kwargs):
@@ -1609,9 +1806,32 @@ class HipTransformer(ComputationGraphTransformer):
                     group.kernels.append(MomentsKernel(self, op))
                 else:
                     raise ValueError("Unhandled op: {}".format(op))
+        if self.chain_kernels and self.fusion:
+            group.kernels = self._chained(group.kernels)
         self.kernel_groups[computation] = group
         computation.executor = group
         return name
+
+    def _chained(self, kernels):
+        """Runs of consecutive fused kernels with a reduction among them become KernelRuns."""
+        out, run = [], []
+
+        def flush():
+            if len(run) >= 2 and any(isinstance(op, og.ReductionOp) and op.reduction_axes.size > 1
+                                     for k in run for op in k.ops):
+                out.append(KernelRun(self, run))
+            else:
+                out.extend(run)
+            del run[:]
+
+        for k in kernels:
+            if type(k) is FusedKernel:
+                run.append(k)
+            else:
+                flush()
+                out.append(k)
+        flush()
+        return out
 
     def make_fused_kernel(self, ops, store_ops, name):
         return FusedKernel(self, ops, store_ops, name)

@@ -28,4 +28,4 @@ def default_kernel_choice():
     would pick (then tests still check results, but not which kernel produced them)."""
     import os
     return not any(os.environ.get(k) for k in ("NGH_FORCE_INTERP", "NGH_NO_TILES", "NGH_CACHE_POLICY", "NGH_TILE4",
-                                                  "NGH_ROW_WAVE_CHUNKS", "NGH_STREAM_MIB", "NGH_NO_RAGGED"))
+                                                  "NGH_ROW_WAVE_CHUNKS", "NGH_STREAM_MIB", "NGH_NO_RAGGED", "NGH_NO_CHAIN"))

@@ -84,11 +84,28 @@ def case_ragged_long_rows():
 
 
 def case_ragged_many_rows():
-    # a softmax over many rows of 1001: a wavefront per row in the reductions
+    # many rows of 1001: a wavefront per row
+    C, N = ng.make_axis(1001, name="C"), ng.make_axis(4200, name="N")
+    x = ng.placeholder([N, C])
+    return [ng.sum(ng.exp(x) * 0.5, out_axes=[N])], [x]
+
+
+def case_softmax_ragged_rows():
+    # a softmax over many rows of 1001: its three kernels become the stages of one row chain
     C, N = ng.make_axis(1001, name="C"), ng.make_axis(4200, name="N")
     x = ng.placeholder([N, C])
     e = ng.exp(x - ng.max(x, out_axes=[N]))
     return [e / ng.sum(e, out_axes=[N])], [x]
+
+
+def case_row_chain_with_stored_intermediate():
+    # log-softmax and the row norms of the same tensor: two results, reductions of different
+    # kinds, an intermediate that is stored by one stage and read back by the next
+    C, N = ng.make_axis(300, name="C"), ng.make_axis(5000, name="N")
+    x = ng.placeholder([N, C])
+    shifted = x - ng.max(x, out_axes=[N])
+    logp = shifted - ng.log(ng.sum(ng.exp(shifted), out_axes=[N]))
+    return [logp, ng.sqrt(ng.sum(logp * logp, out_axes=[N])), shifted], [x]
 
 
 def case_misaligned_slices():
@@ -130,7 +147,8 @@ def case_lookup_table():
 
 FP32_CASES = [case_elementwise, case_column_reduction_with_store, case_row_reduction_with_store,
               case_transposed_operand, case_transposed_operands_large, case_softmax, case_mixed_storage_types, case_ragged,
-              case_ragged_long_rows, case_ragged_many_rows, case_misaligned_slices, case_short_rows, case_dropout, case_lookup_table]
+              case_ragged_long_rows, case_ragged_many_rows, case_softmax_ragged_rows,
+              case_row_chain_with_stored_intermediate, case_misaligned_slices, case_short_rows, case_dropout, case_lookup_table]
 
 
 def flex_case():

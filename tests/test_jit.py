@@ -214,8 +214,8 @@ def test_compiled_programs_agree_with_the_interpreter(case):
     compiled, names = _run("hipgpu", case, 5, jit=True)
     # Same bits as the interpreter -- except where the compiled program runs 4 elements per lane
     # over rows that are not whole aligned vectors (the interpreter takes those one element per
-    # lane): a reduction then adds up in another order.
-    ragged = any("/ragged" in n for n in names)
+    # lane), or several stages as one row-chain kernel: a reduction then adds up in another order.
+    ragged = any("/ragged" in n or "/chain-of-" in n for n in names)
     for a, b, w in zip(interp, compiled, want):
         if ragged:
             np.testing.assert_allclose(a, b, rtol=2e-6, atol=1e-6)
@@ -232,6 +232,9 @@ def test_compiled_programs_agree_with_the_interpreter(case):
         if case in (jit_cases.case_ragged, jit_cases.case_ragged_long_rows, jit_cases.case_ragged_many_rows,
                     jit_cases.case_misaligned_slices):
             assert any(n.endswith("/ragged") for n in names), names
+        if case in (jit_cases.case_softmax, jit_cases.case_softmax_ragged_rows, jit_cases.case_short_rows,
+                    jit_cases.case_row_chain_with_stored_intermediate):
+            assert any("/chain-of-" in n for n in names), names
         if case is jit_cases.case_transposed_operands_large:
             assert any(n.endswith("/tiles64") for n in names), names
 
@@ -250,7 +253,7 @@ def test_random_graphs_compiled_agree_with_the_interpreter(seed, views):
         finally:
             t.close()
     (interp, _), (compiled, names) = run(jit=False), run(jit=True, jit_min_elements=1)
-    ragged = any("/ragged" in n for n in names)       # (see the test above)
+    ragged = any("/ragged" in n or "/chain-of-" in n for n in names)       # (see the test above)
     for a, b in zip(interp, compiled):
         if ragged:
             np.testing.assert_allclose(a, b, rtol=1e-5, atol=1e-5)
@@ -285,13 +288,13 @@ def test_compiled_flex_program_agrees_with_the_interpreter(resident):
 @pytest.mark.gpu
 def test_loading_a_program_library_twice_adds_nothing():
     from ngraph_hip.runtime import HipRuntime
-    t, kernels = _dry_kernels(jit_cases.case_softmax)
+    t, kernels = _dry_kernels(jit_cases.case_ragged_long_rows)
     try:
         # (earlier tests of this process may have loaded these very programs)
         built_in = hiplib.programs_count()[0]
         programs = [p for p in jit.uncovered_programs(kernels, "case", include_covered=True)
                     if not 0 <= p[-1] < built_in]
-        assert len(programs) == 2
+        assert len(programs) == 3
         paths = [jit.compile_programs([p]) for p in programs]
         path = paths[0]
     finally:
