@@ -298,7 +298,7 @@ int  ngh_plan_fused(const ngh_fused_spec* spec, int32_t stage, int32_t* out8);
  * compound kernels run their stages one after the other inside one launch, a reduction's result
  * reaching the next stage without a trip through a second launch (float_ew2.py:1135-1483,
  * stage loop :1268-1321)?  Possible for a "row chain": rows (spec axis 0, the reduced one) of up
- * to 2048 elements, fp32 operands with unit stride along the row or broadcast along it, at
+ * to 8192 elements, fp32 operands with unit stride along the row or broadcast along it, at
  * least one reduction stage.  out4 = {1 if the spec qualifies, index of the compiled chain
  * program or -1 (without one the stages are launched one by one), lanes per row, stages}.
  * No device needed (host-side tooling and tests).                                          */

@@ -154,6 +154,9 @@ def collect():
         if backend not in ngt.transformer_choices():
             continue
         t = ngt.make_transformer_factory(backend, dry_run=True)()
+        # (the patterns stand for tensors of any size: their kernels stay separate programs here,
+        # whether or not the small stand-ins would merge into a row chain)
+        t.chain_kernels = False
         f = build(t)
         t.initialize()
         kernels = t.kernel_groups[f].kernels

@@ -1337,7 +1337,10 @@ bool plan_row_chain(const ngh_context* ctx, const ngh_fused_spec& sp, ChainPlan&
     const long long wave_chunks = ctx ? ctx->row_wave_chunks : kRowWaveChunks;
     const long long R = sp.shape[0], n_out = sp.shape[1] * sp.shape[2];
     const long long chunks = (R + 3) / 4;
-    if (R < 8 || chunks > wave_chunks || chunks > 64 * kChainAhead || n_out < 1 || n_out >= (1LL << 31)) return false;
+    // (a group of lanes or a wavefront per row as far as the row reductions use them, beyond
+    // that a workgroup per row while a lane's kChainAhead chunks cover the row)
+    if (R < 8 || wave_chunks <= 0 || chunks > (long long)kBlock * kChainAhead || n_out < 1 || n_out >= (1LL << 31))
+        return false;
     bool any_red = false;
     const int perm[3] = {1, 2, 0};
     for (int s = 0; s < sp.n_stages; ++s) {
@@ -1365,6 +1368,7 @@ bool plan_row_chain(const ngh_context* ctx, const ngh_fused_spec& sp, ChainPlan&
     C.n_out = (unsigned)n_out;
     C.TR = 1;
     while ((long long)C.TR < chunks && C.TR < 64) C.TR <<= 1;
+    if (chunks > 64 * kChainAhead || chunks > wave_chunks) C.TR = kBlock;
     // (rows enough to fill the chip several times over: a lane takes up to four chunks of its row)
     const long long lanes_wanted = (ctx ? ctx->cus : 256) * 2048LL * 4;
     for (int shrink = 0; shrink < 2 && chunks <= 64 && C.TR > 1 && n_out * (C.TR / 2) >= lanes_wanted; ++shrink)

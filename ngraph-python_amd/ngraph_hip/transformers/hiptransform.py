@@ -1354,8 +1354,11 @@ class FusionPlanner(object):
                 for hi in targets:
                     h = groups[hi]
                     have = set(_view_key(td) for o in h.ops for td in h._operand_views(o)[0])
+                    # (large next to the result itself: the per-row maxima of 131072 rows of 256
+                    # elements are many, and still 1/256 of a pass)
+                    large = max(self.small_tensor, iteration_axes(op).size // 16)
                     extra_large = [td for td in leaves
-                                   if _view_key(td) not in have and _memory_elements(td) > self.small_tensor]
+                                   if _view_key(td) not in have and _memory_elements(td) > large]
                     if len(extra_large) > 1:
                         break
                     # the repeated ops are private to the kernel: whoever else needs them has them

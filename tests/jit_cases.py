@@ -75,9 +75,9 @@ def case_ragged():
 
 
 def case_ragged_long_rows():
-    # rows of 4099 elements: 4 elements per lane with a short last chunk per row, a workgroup per
-    # row segment in the elementwise pass and per row in the reductions
-    A, B = ng.make_axis(37, name="A"), ng.make_axis(4099, name="B")
+    # rows of 9001 elements (too long for a row chain): 4 elements per lane with a short last
+    # chunk per row, a workgroup per row segment in the elementwise pass and per row in the reductions
+    A, B = ng.make_axis(37, name="A"), ng.make_axis(9001, name="B")
     x, y = ng.placeholder([A, B]), ng.placeholder([A, B])
     return [ng.tanh(x * y) + x, ng.sum(x * y + 1.0, out_axes=[A]), ng.max(x - y, out_axes=[A]),
             ng.argmax(x + y, out_axes=[A])], [x, y]
@@ -96,6 +96,15 @@ def case_softmax_ragged_rows():
     x = ng.placeholder([N, C])
     e = ng.exp(x - ng.max(x, out_axes=[N]))
     return [e / ng.sum(e, out_axes=[N])], [x]
+
+
+def case_softmax_long_rows():
+    # rows of 4099 and of 8192 elements: a workgroup per row in the chain kernel
+    C, N, C2 = ng.make_axis(4099, name="C"), ng.make_axis(300, name="N"), ng.make_axis(8192, name="C2")
+    x, x2 = ng.placeholder([N, C]), ng.placeholder([N, C2])
+    e = ng.exp(x - ng.max(x, out_axes=[N]))
+    e2 = ng.exp(x2 - ng.max(x2, out_axes=[N]))
+    return [e / ng.sum(e, out_axes=[N]), e2 / ng.sum(e2, out_axes=[N]), ng.argmax(x2, out_axes=[N])], [x, x2]
 
 
 def case_row_chain_with_stored_intermediate():
@@ -147,7 +156,7 @@ def case_lookup_table():
 
 FP32_CASES = [case_elementwise, case_column_reduction_with_store, case_row_reduction_with_store,
               case_transposed_operand, case_transposed_operands_large, case_softmax, case_mixed_storage_types, case_ragged,
-              case_ragged_long_rows, case_ragged_many_rows, case_softmax_ragged_rows,
+              case_ragged_long_rows, case_ragged_many_rows, case_softmax_ragged_rows, case_softmax_long_rows,
               case_row_chain_with_stored_intermediate, case_misaligned_slices, case_short_rows, case_dropout, case_lookup_table]
 
 

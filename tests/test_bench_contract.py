@@ -67,6 +67,6 @@ def test_user_graphs_of_the_compiled_leg_have_no_built_in_programs():
             for k in kernels:
                 k.bind_buffers()
             assert jit.uncovered_programs(kernels, name), name
-            assert passes >= 2
+            assert min(passes.values() if isinstance(passes, dict) else [passes]) >= 2
         finally:
             t.close()

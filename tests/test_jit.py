@@ -233,7 +233,7 @@ def test_compiled_programs_agree_with_the_interpreter(case):
                     jit_cases.case_misaligned_slices):
             assert any(n.endswith("/ragged") for n in names), names
         if case in (jit_cases.case_softmax, jit_cases.case_softmax_ragged_rows, jit_cases.case_short_rows,
-                    jit_cases.case_row_chain_with_stored_intermediate):
+                    jit_cases.case_softmax_long_rows, jit_cases.case_row_chain_with_stored_intermediate):
             assert any("/chain-of-" in n for n in names), names
         if case is jit_cases.case_transposed_operands_large:
             assert any(n.endswith("/tiles64") for n in names), names
@@ -314,3 +314,153 @@ def test_loading_a_program_library_twice_adds_nothing():
             rt.programs_load(hiplib.library_path())
     finally:
         rt.close()
+
+
+# ---------------------------------------------------------------------------------- row chains
+def _softmax_spec(px, pm, ps, py, R, rows, row_stride=None, x_dtype=hiplib.NGH_F32, only=None):
+    """max / sum of exponentials / normalise over the rows of an [rows, R] tensor as three stages
+    (only: just that one of them)."""
+    stride = R if row_stride is None else row_stride
+    sb = hiplib.FusedSpecBuilder([R, rows])
+    tx, ty = sb.tensor(px, [1, stride], x_dtype), sb.tensor(py, [1, stride])
+    tm, ts = sb.tensor(pm, [0, 1]), sb.tensor(ps, [0, 1])
+    if only in (None, 0):
+        sb.reduce("max", sb.load(tx), tm)
+        sb.end_stage()
+    if only in (None, 1):
+        sb.reduce("sum", sb.unary("exp", sb.binary("sub", sb.load(tx), sb.load(tm))), ts)
+        sb.end_stage()
+    if only in (None, 2):
+        e = sb.unary("exp", sb.binary("sub", sb.load(tx), sb.load(tm)))
+        sb.store(ty, sb.binary("div", e, sb.load(ts)))
+    return sb.build()
+
+
+def test_which_specs_are_row_chains():
+    """ngh_plan_chain without a device: rows of 8 to 8192 fp32 elements with unit stride, at least
+    one reduction stage, more than one stage."""
+    ok = lambda spec: hiplib.plan_chain(spec)["eligible"]
+    assert ok(_softmax_spec(4096, 8192, 12288, 16384, 1001, 300))
+    assert hiplib.plan_chain(_softmax_spec(4096, 8192, 12288, 16384, 1001, 300))["lanes_per_row"] == 64
+    assert hiplib.plan_chain(_softmax_spec(4096, 8192, 12288, 16384, 100, 300))["lanes_per_row"] == 32
+    assert hiplib.plan_chain(_softmax_spec(4096, 8192, 12288, 16384, 5000, 300))["lanes_per_row"] == 256
+    assert ok(_softmax_spec(4100, 8192, 12288, 16388, 1000, 300, row_stride=1003))      # any 4-byte-aligned start
+    assert not ok(_softmax_spec(4096, 8192, 12288, 16384, 7, 300))
+    assert not ok(_softmax_spec(4096, 8192, 12288, 16384, 8193, 300))
+    assert not ok(_softmax_spec(4096, 8192, 12288, 16384, 1000, 300, x_dtype=hiplib.NGH_FLEX16))
+    # rows that are strided in memory
+    sb = hiplib.FusedSpecBuilder([64, 300])
+    tx, tm, ty = sb.tensor(4096, [300, 1]), sb.tensor(8192, [0, 1]), sb.tensor(16384, [300, 1])
+    sb.reduce("max", sb.load(tx), tm)
+    sb.end_stage()
+    sb.store(ty, sb.binary("sub", sb.load(tx), sb.load(tm)))
+    assert not ok(sb.build())
+    # one stage, and stages without a reduction
+    sb = hiplib.FusedSpecBuilder([64, 300])
+    sb.reduce("max", sb.load(sb.tensor(4096, [1, 64])), sb.tensor(8192, [0, 1]))
+    assert not ok(sb.build())
+    sb = hiplib.FusedSpecBuilder([64, 300])
+    tx, ty, tz = sb.tensor(4096, [1, 64]), sb.tensor(16384, [1, 64]), sb.tensor(65536, [1, 64])
+    sb.store(ty, sb.unary("exp", sb.load(tx)))
+    sb.end_stage()
+    sb.store(tz, sb.unary("tanh", sb.load(tx)))
+    assert not ok(sb.build())
+
+
+def _fenced_chain_spec(px, pi, pt, py, pn, R, rows):
+    sb = hiplib.FusedSpecBuilder([R, rows])
+    tx, ti = sb.tensor(px, [1, R]), sb.tensor(pi, [0, 1], hiplib.NGH_I32)
+    tt, ty, tn = sb.tensor(pt, [1, R]), sb.tensor(py, [1, R]), sb.tensor(pn, [0, 1])
+    sb.reduce("argmax", sb.load(tx), ti)
+    sb.end_stage()
+    # t = x * 2 + position of the row's maximum; n = sum(t * t)
+    t = sb.binary("add", sb.binary("mul", sb.load(tx), sb.constant(2.0)), sb.load(ti))
+    sb.store(tt, t)
+    sb.reduce("sum", sb.binary("mul", t, t), tn)
+    sb.end_stage()
+    # y = t / sqrt(n), t read back from memory
+    sb.store(ty, sb.binary("div", sb.load(tt), sb.unary("sqrt", sb.load(tn))))
+    return sb.build()
+
+
+def test_row_chain_specs_compile_for_gfx950():
+    """(also leaves their program libraries in the cache for the device tests below)"""
+    for spec in (_softmax_spec(4096, 8192, 12288, 16384, 1001, 300),
+                 _fenced_chain_spec(4096, 8192, 12288, 16384, 20480, 777, 3000)):
+        programs = jit.uncovered_programs([_SpecHolder(spec)], "chain", min_elements=1, include_covered=True)
+        assert len(programs) == 1 and programs[0][8] == 4
+        assert os.path.exists(jit.compile_programs(programs))
+
+
+class _SpecHolder(object):
+    def __init__(self, spec):
+        self.specs = [spec]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,R,stride", [(300, 1001, None), (5000, 100, None), (2000, 16, None), (64, 8192, None),
+                                           (70, 4099, None), (301, 1000, 1003), (1, 9, None)])
+def test_row_chain_through_the_c_abi(hip_runtime, rows, R, stride, monkeypatch):
+    """A three-stage softmax spec: launched as one chain kernel it gives what its stages give when
+    launched one by one, and what NumPy gives."""
+    rt = hip_runtime
+    stride = R if stride is None else stride
+    rs = np.random.RandomState(rows + R)
+    x = rs.normal(0, 3, (rows, stride)).astype(np.float32)
+    x_d = rt.array(x)
+    outs = {}
+    for chained in (True, False):
+        m_d, s_d, y_d = rt.empty((rows,)), rt.empty((rows,)), rt.empty((rows, stride))
+        rt.memset32(y_d.ptr, 0x7fc00000, rows * stride)
+        spec = _softmax_spec(x_d.ptr, m_d.ptr, s_d.ptr, y_d.ptr, R, rows, row_stride=stride)
+        jit.ensure_programs(rt, [_SpecHolder(spec)], "softmax_chain", min_elements=1)
+        if chained:
+            if default_kernel_choice():
+                assert "/chain-of-3" in rt.describe_fused(spec, 0)
+            rt.launch_fused(spec)
+        else:
+            # the same stages, each a spec of its own
+            for stage in range(3):
+                one = _softmax_spec(x_d.ptr, m_d.ptr, s_d.ptr, y_d.ptr, R, rows, row_stride=stride, only=stage)
+                assert "chain" not in rt.describe_fused(one, 0)
+                rt.launch_fused(one)
+        outs[chained] = (m_d.get(), s_d.get(), y_d.get())
+        for d in (m_d, s_d, y_d):
+            d.free()
+    x_d.free()
+    x64 = x[:, :R].astype(np.float64)
+    e = np.exp(x64 - x64.max(axis=1, keepdims=True))
+    for m, s, y in outs.values():
+        np.testing.assert_array_equal(m, x[:, :R].max(axis=1))
+        np.testing.assert_allclose(s, e.sum(axis=1), rtol=1e-5)
+        np.testing.assert_allclose(y[:, :R], e / e.sum(axis=1, keepdims=True), rtol=1e-5, atol=1e-6)
+        assert np.isnan(y[:, R:]).all()                  # the gap between rows is not written
+    np.testing.assert_allclose(outs[True][2][:, :R], outs[False][2][:, :R], rtol=2e-6, atol=1e-7)
+
+
+@pytest.mark.gpu
+def test_row_chain_with_results_that_go_through_memory(hip_runtime):
+    """What the stages of a chain cannot hand on in registers goes through memory behind a fence:
+    the position of the maximum (kept as int32) read back by the next stage, and a tensor that
+    one stage stores and the next loads."""
+    rt = hip_runtime
+    rows, R = 3000, 777
+    rs = np.random.RandomState(5)
+    x = rs.normal(0, 1, (rows, R)).astype(np.float32)
+    x_d, i_d, t_d, y_d, n_d = rt.array(x), rt.empty((rows,), hiplib.NGH_I32), rt.empty((rows, R)), rt.empty((rows, R)), \
+        rt.empty((rows,))
+    spec = _fenced_chain_spec(x_d.ptr, i_d.ptr, t_d.ptr, y_d.ptr, n_d.ptr, R, rows)
+    assert hiplib.plan_chain(spec)["eligible"]
+    jit.ensure_programs(rt, [_SpecHolder(spec)], "fenced_chain", min_elements=1)
+    if default_kernel_choice():
+        assert "/chain-of-3" in rt.describe_fused(spec, 0)
+    rt.launch_fused(spec)
+    pos = x.argmax(axis=1)
+    np.testing.assert_array_equal(i_d.get(), pos)
+    t_want = x.astype(np.float64) * 2.0 + pos[:, None]
+    n_want = (t_want * t_want).sum(axis=1)
+    np.testing.assert_allclose(t_d.get(), t_want, rtol=1e-6)
+    np.testing.assert_allclose(n_d.get(), n_want, rtol=1e-5)
+    np.testing.assert_allclose(y_d.get(), t_want / np.sqrt(n_want)[:, None], rtol=1e-5, atol=1e-7)
+    for d in (x_d, i_d, t_d, y_d, n_d):
+        d.free()
