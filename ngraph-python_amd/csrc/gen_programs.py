@@ -114,6 +114,17 @@ def pattern_lstm_bias_gradient(t):
     return t.computation(ng.sum(gates, out_axes=[G]), gates_st)
 
 
+def pattern_softmax_rows(t):
+    N, C = _axes(N=4096, C=1000)
+    x = ng.placeholder([N, C])
+    return t.computation(ng.softmax(x, normalization_axes=ng.make_axes([C])), x)
+
+
+# patterns whose kernels merge into one row chain (rows of up to 8192 elements along the
+# contiguous axis): the chain is built in, so that these run as one launch without run-time
+# compilation, whatever their size
+CHAINS = ("softmax_rows",)
+
 PATTERNS = [
     ("c1_tanh_sigmoid", "hipgpu", pattern_c1),
     ("adam", "hipgpu", pattern_adam),
@@ -144,6 +155,7 @@ PATTERNS = [
     # the planner orders ops of large tensors differently (nothing above 65536 elements is
     # materialised early), which gives the cell a second program
     ("lstm_cell_large", "hipgpu", lambda t: pattern_lstm_cell(t, 2048, 512)),
+    ("softmax_rows", "hipgpu", pattern_softmax_rows),
 ]
 
 
@@ -156,7 +168,7 @@ def collect():
         t = ngt.make_transformer_factory(backend, dry_run=True)()
         # (the patterns stand for tensors of any size: their kernels stay separate programs here,
         # whether or not the small stand-ins would merge into a row chain)
-        t.chain_kernels = False
+        t.chain_kernels = name in CHAINS
         f = build(t)
         t.initialize()
         kernels = t.kernel_groups[f].kernels

@@ -88,8 +88,11 @@ inline int match_special(int family, int V, const KArgs& k, long long /*tail*/) 
 inline int match_chain(const KArgs* ks, const int* families, int n) {
     auto matches = [&](const StaticEntry& e) {
         if (e.family != 4 || e.chain_len != n) return false;
-        for (int i = 0; i < n; ++i)
+        for (int i = 0; i < n; ++i) {
             if (!entry_matches(e.chain[i], families[i], 4, ks[i])) return false;
+            for (int t = 0; t < ks[i].n_tensors; ++t)
+                if ((e.chain[i].rowshared[t] != 0) != (ks[i].t[t].s[0] == 0 && ks[i].t[t].s[1] == 0)) return false;
+        }
         return true;
     };
     for (int i = 0; i < kStaticCount; ++i)
@@ -107,8 +110,11 @@ inline bool same_program(const StaticEntry& a, const StaticEntry& b) {
         return false;
     if (a.family == 4) {
         if (a.chain_len != b.chain_len) return false;
-        for (int i = 0; i < a.chain_len; ++i)
+        for (int i = 0; i < a.chain_len; ++i) {
             if (!same_program(a.chain[i], b.chain[i])) return false;
+            for (int t = 0; t < a.chain[i].n_tensors; ++t)
+                if ((a.chain[i].rowshared[t] != 0) != (b.chain[i].rowshared[t] != 0)) return false;
+        }
         return true;
     }
     for (int r = 0; r < a.n_red; ++r) if (a.red_out[r] != b.red_out[r]) return false;

@@ -102,6 +102,9 @@ def _chain_program(spec, name, seen, min_elements):
         return ()
     dtypes = [spec.tensors[i].dtype for i in range(spec.n_tensors)]
     bcast = [1 if spec.tensors[i].strides[0] == 0 else 0 for i in range(spec.n_tensors)]
+    # (the same for every row: a layer norm's gain and bias)
+    rowshared = [1 if spec.tensors[i].strides[1] == 0 and spec.tensors[i].strides[2] == 0 else 0
+                 for i in range(spec.n_tensors)]
     members = []
     for stage in range(spec.n_stages):
         st = spec.stages[stage]
@@ -114,8 +117,8 @@ def _chain_program(spec, name, seen, min_elements):
         members.append(("%s_s%d" % (name, stage), ops, dtypes, bcast, [-1] * spec.n_tensors, 0, spec.n_regs, 4,
                         1 if red_out else 0, red_out, [-1] * spec.n_tensors,
                         [1 if i in loaded else 0 for i in range(spec.n_tensors)],
-                        [1 if i in stored else 0 for i in range(spec.n_tensors)], -1))
-    key = ("chain",) + tuple((tuple(m[1]), tuple(m[2]), tuple(m[3]), m[8], tuple(m[9])) for m in members)
+                        [1 if i in stored else 0 for i in range(spec.n_tensors)], -1, rowshared))
+    key = ("chain", tuple(rowshared)) + tuple((tuple(m[1]), tuple(m[2]), tuple(m[3]), m[8], tuple(m[9])) for m in members)
     if key in seen:
         return ()
     seen.add(key)
@@ -123,7 +126,8 @@ def _chain_program(spec, name, seen, min_elements):
 
 
 def _render_struct(lines, struct, record):
-    name, ops, dtypes, bcast, stat_slot, n_slots, n_regs, V, family, red_out, staged, loaded, stored, _ = record
+    name, ops, dtypes, bcast, stat_slot, n_slots, n_regs, V, family, red_out, staged, loaded, stored, _ = record[:14]
+    rowshared = record[14] if len(record) > 14 else [0] * len(dtypes)
     lines.append("struct %s {  // %s" % (struct, name))
     lines.append("    static constexpr int V = %d, n_ops = %d, n_regs = %d, n_tensors = %d, "
                  "n_stat_slots = %d, family = %d, n_red = %d;"
@@ -139,6 +143,7 @@ def _render_struct(lines, struct, record):
     lines.append("    static constexpr signed char staged[%d] = {%s};" % (len(staged), ", ".join(map(str, staged))))
     lines.append("    static constexpr unsigned char loaded[%d] = {%s};" % (len(loaded), ", ".join(map(str, loaded))))
     lines.append("    static constexpr unsigned char stored[%d] = {%s};" % (len(stored), ", ".join(map(str, stored))))
+    lines.append("    static constexpr unsigned char rowshared[%d] = {%s};" % (len(rowshared), ", ".join(map(str, rowshared))))
     lines.append("};")
 
 
@@ -157,7 +162,8 @@ def render(programs, header, prefix="SP", table="kStaticTable", count="kStaticCo
             lines.append("static const StaticEntry %s%d_stages[] = {" % (prefix, i))
             for j, member in enumerate(p[1]):
                 lines.append("    " + _ENTRY.format("%s%d_%d" % (prefix, i, j), member[0],
-                                                    "nullptr, nullptr, nullptr, nullptr"))
+                                                    "nullptr, nullptr, nullptr, nullptr, 0, nullptr, "
+                                                    "%s%d_%d::rowshared" % (prefix, i, j)))
             lines.append("};")
         else:
             _render_struct(lines, prefix + str(i), p)
@@ -166,7 +172,7 @@ def render(programs, header, prefix="SP", table="kStaticTable", count="kStaticCo
         if p[8] == 4:
             stages = ", ".join("%s%d_%d" % (prefix, i, j) for j in range(len(p[1])))
             lines.append('    {"%s", 4, 4, 0, nullptr, 0, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr, '
-                         '%d, %s%d_stages, &launch_static_chain<%s>},' % (p[0], len(p[1]), prefix, i, stages))
+                         '%d, %s%d_stages, nullptr, &launch_static_chain<%s>},' % (p[0], len(p[1]), prefix, i, stages))
             continue
         if p[8] == 0:
             launch = "&launch_static<{0}>, nullptr, {0}::staged, nullptr".format(prefix + str(i))
