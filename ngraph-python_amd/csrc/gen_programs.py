@@ -120,10 +120,17 @@ def pattern_softmax_rows(t):
     return t.computation(ng.softmax(x, normalization_axes=ng.make_axes([C])), x)
 
 
+def pattern_log_softmax_rows(t):
+    N, C = _axes(N=4096, C=1000)
+    x = ng.placeholder([N, C])
+    shifted = x - ng.max(x, out_axes=[N])
+    return t.computation(shifted - ng.log(ng.sum(ng.exp(shifted), out_axes=[N])), x)
+
+
 # patterns whose kernels merge into one row chain (rows of up to 8192 elements along the
 # contiguous axis): the chain is built in, so that these run as one launch without run-time
 # compilation, whatever their size
-CHAINS = ("softmax_rows",)
+CHAINS = ("softmax_rows", "log_softmax_rows")
 
 PATTERNS = [
     ("c1_tanh_sigmoid", "hipgpu", pattern_c1),
@@ -156,6 +163,7 @@ PATTERNS = [
     # materialised early), which gives the cell a second program
     ("lstm_cell_large", "hipgpu", lambda t: pattern_lstm_cell(t, 2048, 512)),
     ("softmax_rows", "hipgpu", pattern_softmax_rows),
+    ("log_softmax_rows", "hipgpu", pattern_log_softmax_rows),
 ]
 
 

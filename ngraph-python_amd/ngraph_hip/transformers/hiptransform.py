@@ -1373,6 +1373,7 @@ class FusionPlanner(object):
         return groups
 
     cheap_ops = ("add", "sub", "mul", "div", "neg", "abs", "sqrt", "rcp", "sqr", "minimum", "maximum", "assign")
+    costly_ops = ("log", "exp", "safelog", "log2", "exp2")
 
     def _absorb_small_groups(self, groups, readers, returned):
         """A kernel over a few elements (per-channel factors between two passes over a big tensor)
@@ -1388,8 +1389,12 @@ class FusionPlanner(object):
         for gi, g in enumerate(groups):
             if not g.fusable or len(g.ops) > self.max_recompute_ops or \
                     g.axes.size > self.small_tensor or \
-                    not all(kernel_op_name(o) in self.cheap_ops for o in g.ops):
+                    not all(kernel_op_name(o) in self.cheap_ops + self.costly_ops for o in g.ops):
                 continue
+            # (a logarithm or exponential per row: repeated by a kernel with at least 64 elements
+            # a row, it is one such op per 4-element chunk at most, and none where the kernels
+            # merge into a row chain, whose stages compute a row's values once)
+            costly = any(kernel_op_name(o) in self.costly_ops for o in g.ops)
             inside = set(g.ops)
             targets, ok = set(), True
             for op in g.ops:
@@ -1403,7 +1408,8 @@ class FusionPlanner(object):
                     for hi in holders.get(u, (-1,)):
                         if hi <= gi or hi in gone or not groups[hi].fusable or \
                                 not g.axes.is_sub_set(groups[hi].axes) or \
-                                groups[hi].axes.size <= self.small_tensor:
+                                groups[hi].axes.size <= self.small_tensor or \
+                                (costly and groups[hi].axes.size < 64 * g.axes.size):
                             ok = False
                             break
                         targets.add(hi)
