@@ -339,6 +339,8 @@ def _softmax_spec(px, pm, ps, py, R, rows, row_stride=None, x_dtype=hiplib.NGH_F
 def test_which_specs_are_row_chains():
     """ngh_plan_chain without a device: rows of 8 to 8192 fp32 elements with unit stride, at least
     one reduction stage, more than one stage."""
+    if not default_kernel_choice():
+        pytest.skip("a kernel-choice knob of the library is set")
     ok = lambda spec: hiplib.plan_chain(spec)["eligible"]
     assert ok(_softmax_spec(4096, 8192, 12288, 16384, 1001, 300))
     assert hiplib.plan_chain(_softmax_spec(4096, 8192, 12288, 16384, 1001, 300))["lanes_per_row"] == 64
@@ -388,8 +390,9 @@ def test_row_chain_specs_compile_for_gfx950():
     for spec in (_softmax_spec(4096, 8192, 12288, 16384, 1001, 300),
                  _fenced_chain_spec(4096, 8192, 12288, 16384, 20480, 777, 3000)):
         programs = jit.uncovered_programs([_SpecHolder(spec)], "chain", min_elements=1, include_covered=True)
-        assert len(programs) == 1 and programs[0][8] == 4
-        assert os.path.exists(jit.compile_programs(programs))
+        if default_kernel_choice():
+            assert len(programs) == 1 and programs[0][8] == 4
+        assert not programs or os.path.exists(jit.compile_programs(programs))
 
 
 class _SpecHolder(object):
@@ -450,7 +453,7 @@ def test_row_chain_with_results_that_go_through_memory(hip_runtime):
     x_d, i_d, t_d, y_d, n_d = rt.array(x), rt.empty((rows,), hiplib.NGH_I32), rt.empty((rows, R)), rt.empty((rows, R)), \
         rt.empty((rows,))
     spec = _fenced_chain_spec(x_d.ptr, i_d.ptr, t_d.ptr, y_d.ptr, n_d.ptr, R, rows)
-    assert hiplib.plan_chain(spec)["eligible"]
+    assert hiplib.plan_chain(spec)["eligible"] or not default_kernel_choice()
     jit.ensure_programs(rt, [_SpecHolder(spec)], "fenced_chain", min_elements=1)
     if default_kernel_choice():
         assert "/chain-of-3" in rt.describe_fused(spec, 0)
