@@ -899,6 +899,10 @@ class ChainKernel(HipKernel):
     -- which the library runs in one kernel when it can (ngh_plan_chain; the reference's
     compound kernels run their stages inside one launch the same way, float_ew2.py:1135-1483).
     The operand then crosses the memory interface once instead of once per kernel.
+
+    Chains are compiled programs: while the library has none for this spec (none built in, the
+    run-time compiler not done yet, or switched off) the members run one by one as they would
+    have alone, with the programs they match by themselves.
     """
 
     def __init__(self, transformer, members, spec, uses):
@@ -908,7 +912,16 @@ class ChainKernel(HipKernel):
         self.ops = [op for m in self.members for op in m.ops]
         self.specs = [spec]
         self.spec_uses = [uses]
+        for m in self.members:
+            m.bind_buffers()
         self.buffers_bound = True
+        self.ready = False
+        self.programs_changed()
+
+    def programs_changed(self):
+        """Called when compiled programs may have been added to the library's table."""
+        if not self.ready:
+            self.ready = hiplib.plan_chain(self.specs[0])["special"] >= 0
 
     @classmethod
     def merged(cls, transformer, members):
@@ -1003,13 +1016,37 @@ class ChainKernel(HipKernel):
         return list(self.spec_uses[0])
 
     def set_cache_hints(self, hint_of):
+        whole = {}
         for s, (base, is_read, is_written) in enumerate(self.spec_uses[0]):
-            self.specs[0].tensors[s].cache_hint = hint_of(base, is_read, is_written)
+            self.specs[0].tensors[s].cache_hint = whole[base] = hint_of(base, is_read, is_written)
+        # the members, for as long as they run by themselves: what one of them streams past the
+        # cache another must not want to find there
+        readers = {}
+        for m in self.members:
+            for base, is_read, _ in m.buffer_uses():
+                if is_read:
+                    readers[base] = readers.get(base, 0) + 1
+
+        def member_hint(base, is_read, is_written):
+            hint = whole.get(base, 0)
+            if readers.get(base, 0) > 1:
+                hint &= ~NGH_CACHE_STREAM_LOAD
+            if readers.get(base, 0) > 0:
+                hint &= ~NGH_CACHE_STREAM_STORE
+            return hint
+        for m in self.members:
+            m.set_cache_hints(member_hint)
 
     def execute(self):
-        self.transformer.runtime.launch_fused(self.specs[0])
+        if self.ready:
+            self.transformer.runtime.launch_fused(self.specs[0])
+        else:
+            for m in self.members:
+                m.execute()
 
     def describe(self):
+        if not self.ready:
+            return [d for m in self.members for d in m.describe()]
         rt = self.transformer.runtime
         return [[rt.describe_fused(spec, s) for s in range(spec.n_stages)] for spec in self.specs]
 
@@ -1095,6 +1132,7 @@ class HipKernelGroup(object):
             from ngraph_hip.runtime import jit
             jit.ensure_programs(self.transformer.runtime, self.kernels, self.name,
                                 min_elements=self.transformer.jit_min_elements)
+            self.programs_changed()
         elif mode == "auto":
             # the same for the stages over large tensors, off the launch path: the computation
             # starts on the interpreter and picks the compiled kernels up when they are ready
@@ -1104,6 +1142,11 @@ class HipKernelGroup(object):
         self._bound = True
 
     _programs = None
+
+    def programs_changed(self):
+        for k in self.kernels:
+            if hasattr(k, "programs_changed"):
+                k.programs_changed()
 
     def wait_for_programs(self, timeout=None):
         """Block until the kernels being compiled for this computation (jit="auto") are loaded;
@@ -1115,6 +1158,7 @@ class HipKernelGroup(object):
         self._programs.wait(timeout)
         error = self._programs.error
         self._programs = None
+        self.programs_changed()
         return error
 
     def cancel_programs(self):
@@ -1154,6 +1198,7 @@ class HipKernelGroup(object):
             self.bind()
         if self._programs is not None and self._programs.poll():
             self._programs = None
+            self.programs_changed()
         for k in self.kernels:
             self.setup_kernel_execute(k)
             k.execute()

@@ -467,3 +467,33 @@ def test_row_chain_with_results_that_go_through_memory(hip_runtime):
     np.testing.assert_allclose(y_d.get(), t_want / np.sqrt(n_want)[:, None], rtol=1e-5, atol=1e-7)
     for d in (x_d, i_d, t_d, y_d, n_d):
         d.free()
+
+
+@pytest.mark.gpu
+def test_chained_kernels_run_by_themselves_until_the_chain_is_compiled():
+    """Without a compiled chain (run-time compilation off, no such chain built in) the merged
+    kernels keep running one by one, with the programs they match by themselves; with
+    compilation on the same graph is one launch.  Same results either way."""
+    def run(**kwargs):
+        t = ngt.make_transformer_factory("hipgpu", **kwargs)()
+        try:
+            C, N = ng.make_axis(700, name="C"), ng.make_axis(3000, name="N")
+            x = ng.placeholder([N, C])
+            e = ng.exp((x - ng.max(x, out_axes=[N])) * 0.5)
+            f = t.computation(e / ng.sum(e, out_axes=[N]), x)
+            xv = np.random.RandomState(2).normal(0, 2, (3000, 700)).astype(np.float32)
+            out = np.array(f(xv)).copy()
+            names = [d for k in t.kernel_groups[f].kernels for ds in k.describe() for d in ds]
+            return out, names, xv
+        finally:
+            t.close()
+    alone, names_alone, xv = run(jit=False)
+    chained, names_chained, _ = run(jit=True, jit_min_elements=1)
+    if default_kernel_choice():
+        assert not any("/chain-of-" in n for n in names_alone), names_alone
+        assert "special:max_along_k0" in names_alone[0], names_alone        # the built-in row maximum
+        assert len(names_chained) == 3 and all("/chain-of-3" in n for n in names_chained), names_chained
+    e = np.exp((xv.astype(np.float64) - xv.max(axis=1, keepdims=True)) * 0.5)
+    want = e / e.sum(axis=1, keepdims=True)
+    np.testing.assert_allclose(alone, want, rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(chained, want, rtol=1e-5, atol=1e-7)
