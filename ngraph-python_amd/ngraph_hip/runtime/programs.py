@@ -98,7 +98,9 @@ def _chain_program(spec, name, seen, min_elements):
     plan = hiplib.plan_chain(spec)
     if not plan["eligible"]:
         return None
-    if spec.shape[0] * spec.shape[1] * spec.shape[2] < min_elements:
+    # (a chain is worth a kernel sooner than a single stage is: it saves launches, not only time
+    # on the interpreter)
+    if spec.shape[0] * spec.shape[1] * spec.shape[2] < min_elements // 16:
         return ()
     dtypes = [spec.tensors[i].dtype for i in range(spec.n_tensors)]
     bcast = [1 if spec.tensors[i].strides[0] == 0 else 0 for i in range(spec.n_tensors)]
