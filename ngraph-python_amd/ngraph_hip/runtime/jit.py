@@ -273,13 +273,28 @@ class BackgroundPrograms(object):
             f.cancel()
 
 
-def start_background(runtime, kernels, name, min_elements, after_calls=2, verbose=False):
+def start_background(runtime, kernels, name, min_elements, after_calls=2, verbose=False, small_min_elements=None):
     """BackgroundPrograms for the stages of `kernels` (of at least min_elements elements) that run on
     the interpreter today, or None when there are none."""
     programs = uncovered_programs(kernels, name, min_elements)
+    if not programs and small_min_elements is None:
+        return None
+    if small_min_elements is not None and (programs or _has_large_stage(kernels, min_elements)):
+        # A computation over large tensors: its small stages (statistics combined between two
+        # passes, per-channel factors) are launches on the same critical path, several
+        # microseconds each on the interpreter, so they get programs too.
+        programs = uncovered_programs(kernels, name, small_min_elements)
     if not programs:
         return None
     return BackgroundPrograms(runtime, programs, after_calls=after_calls, verbose=verbose)
+
+
+def _has_large_stage(kernels, min_elements):
+    for k in kernels:
+        for spec in getattr(k, "specs", [])[:1]:
+            if spec.shape[0] * spec.shape[1] * spec.shape[2] >= min_elements:
+                return True
+    return False
 
 
 def precompile_graphs(builders, verbose=False):

@@ -1138,7 +1138,8 @@ class HipKernelGroup(object):
             # starts on the interpreter and picks the compiled kernels up when they are ready
             from ngraph_hip.runtime import jit
             self._programs = jit.start_background(self.transformer.runtime, self.kernels, self.name,
-                                                  min_elements=self.transformer.jit_auto_min_elements)
+                                                  min_elements=self.transformer.jit_auto_min_elements,
+                                                  small_min_elements=self.transformer.jit_min_elements)
         self._bound = True
 
     _programs = None
@@ -1453,7 +1454,7 @@ class FusionPlanner(object):
                     for hi in holders.get(u, (-1,)):
                         if hi <= gi or hi in gone or not groups[hi].fusable or \
                                 not g.axes.is_sub_set(groups[hi].axes) or \
-                                groups[hi].axes.size <= self.small_tensor or \
+                                groups[hi].axes.size < 16 * g.axes.size or \
                                 (costly and groups[hi].axes.size < 64 * g.axes.size):
                             ok = False
                             break
