@@ -107,6 +107,16 @@ def case_softmax_long_rows():
     return [e / ng.sum(e, out_axes=[N]), e2 / ng.sum(e2, out_axes=[N]), ng.argmax(x2, out_axes=[N])], [x, x2]
 
 
+def case_softmax_over_windows():
+    # rows inside a window of a larger tensor: two kept axes that do not merge into one, rows that
+    # start anywhere, a result written into a window as well
+    A, B, C = ng.make_axis(37, name="A"), ng.make_axis(60, name="B"), ng.make_axis(310, name="C")
+    x = ng.placeholder([A, B, C])
+    xs = ng.tensor_slice(x, [slice(None), slice(5, 55), slice(3, 303)])
+    e = ng.exp(xs - ng.max(xs, reduction_axes=xs.axes[2:]))
+    return [e / ng.sum(e, reduction_axes=xs.axes[2:]), ng.argmax(xs, reduction_axes=xs.axes[2:])], [x]
+
+
 def case_row_chain_with_stored_intermediate():
     # log-softmax and the row norms of the same tensor: two results, reductions of different
     # kinds, an intermediate that is stored by one stage and read back by the next
@@ -156,7 +166,7 @@ def case_lookup_table():
 
 FP32_CASES = [case_elementwise, case_column_reduction_with_store, case_row_reduction_with_store,
               case_transposed_operand, case_transposed_operands_large, case_softmax, case_mixed_storage_types, case_ragged,
-              case_ragged_long_rows, case_ragged_many_rows, case_softmax_ragged_rows, case_softmax_long_rows,
+              case_ragged_long_rows, case_ragged_many_rows, case_softmax_ragged_rows, case_softmax_long_rows, case_softmax_over_windows,
               case_row_chain_with_stored_intermediate, case_misaligned_slices, case_short_rows, case_dropout, case_lookup_table]
 
 
