@@ -860,6 +860,7 @@ class MomentsKernel(HipKernel):
     def __init__(self, transformer, op):
         super(MomentsKernel, self).__init__(transformer)
         self.op = op
+        self.name = "moments"
         self.x_cache_hint = 0
 
     def bind_buffers(self):
@@ -891,6 +892,20 @@ class MomentsKernel(HipKernel):
         return [["moments_f32"]]
 
 
+class _ChainScratch(object):
+    """An operand of a chain that is no tensor of the graph: one row of a statistics tensor, taken
+    over for an intermediate (what a tensor description tells the merge, and its address)."""
+
+    def __init__(self, base, ptr, axes, row):
+        self.base, self.ptr, self.axes, self.offset = base, ptr, og.make_axes(axes), ("row", row)
+        self.dtype = np.dtype(np.float32)
+        strides, step = [], 1
+        for a in reversed(list(axes)):
+            strides.insert(0, step)
+            step *= a.length
+        self.full_strides = tuple(strides)
+
+
 class ChainKernel(HipKernel):
     """Consecutive fused kernels over the same rows, merged: the STAGES of one spec.
 
@@ -909,7 +924,7 @@ class ChainKernel(HipKernel):
         super(ChainKernel, self).__init__(transformer)
         self.members = list(members)
         self.name = self.members[0].name
-        self.ops = [op for m in self.members for op in m.ops]
+        self.ops = [op for m in self.members for op in getattr(m, "ops", None) or [m.op]]
         self.specs = [spec]
         self.spec_uses = [uses]
         for m in self.members:
@@ -926,8 +941,90 @@ class ChainKernel(HipKernel):
     @classmethod
     def merged(cls, transformer, members):
         """The ChainKernel of `members`, or None when they do not form a row chain."""
-        t = transformer
-        parts = [m._collect() for m in members]
+        if isinstance(members[0], MomentsKernel):
+            parts = cls._parts_after_moments(transformer, members[0], members[1:])
+        elif any(isinstance(m, MomentsKernel) for m in members):
+            parts = None
+        else:
+            parts = [m._collect() for m in members]
+        return None if parts is None else cls._merge_parts(transformer, members, parts)
+
+    @staticmethod
+    def _parts_after_moments(t, moments, rest):
+        """Mean, variance and 1/sqrt(variance + eps) of rows, and the kernels that use them, as
+        stages: sum(x); sum((x - sum / n)^2); then the kernels, each load of a statistic replaced
+        by its value computed from the two sums -- the statements ng.mean and ng.variance stand
+        for (op_graph.py:4007-4009, 4252-4266).  The two sums go where the statistics would
+        have gone, which is why nothing outside `rest` may read those."""
+        if not rest or any(type(k) is not FusedKernel for k in rest):
+            return None
+        op = moments.op
+        mom_base = _td(op).base
+        readers, returned = t._usage_maps()
+        inside = set(o for k in rest for o in k.ops)
+        if mom_base in returned or any(u not in inside for u in readers.get(mom_base, ())):
+            return None
+        moments.bind_buffers()
+        x_td = _td(op.args[0].forwarded)
+        n = float(op.reduction_axes.size)
+        kept = [a for a in x_td.axes if a not in op.reduction_axes]
+        rows = moments.rows
+        sums = [_ChainScratch(mom_base, moments.out.ptr + i * rows * 4, kept, i) for i in range(2)]
+        parts = [([x_td, sums[0]], [("load", 0, 0), ("reduce", "sum", 0, 1)],
+                  x_td.axes, op.reduction_axes, [], [], {})]
+        need_var = False
+        later = []
+        for k in rest:
+            operands, program, it_axes, r_axes, onehot_axes, take_axes, take_strides = k._collect()
+            row_of = {}
+            for s, td in enumerate(operands):
+                if td.base is mom_base:
+                    view = t.get_tensor_description_tensor_view(td)
+                    row_of[s] = (view.ptr - moments.out.ptr) // (rows * 4)
+                    if row_of[s] not in (0, 1, 2) or (view.ptr - moments.out.ptr) % (rows * 4):
+                        return None
+            if any(ins[0] in ("store", "reduce") and ins[1 if ins[0] == "store" else 3] in row_of for ins in program):
+                return None
+            new_operands = [td for s, td in enumerate(operands) if s not in row_of]
+            slot_map = {s: i for i, s in enumerate(s for s in range(len(operands)) if s not in row_of)}
+            s0, s1 = len(new_operands), len(new_operands) + 1
+            new_operands += sums
+            next_reg = [1 + max([ins[1] for ins in program if ins[0] not in ("store", "store_trunc", "reduce")] + [0])]
+
+            def reg():
+                next_reg[0] += 1
+                return next_reg[0] - 1
+            new_program = []
+            for ins in program:
+                if ins[0] == "load" and ins[2] in row_of:
+                    row = row_of[ins[2]]
+                    total, count = reg(), reg()
+                    new_program += [("load", total, s0 if row == 0 else s1), ("const", count, n)]
+                    if row < 2:
+                        new_program.append(("div", ins[1], total, count))
+                    else:
+                        var, eps, shifted, root = reg(), reg(), reg(), reg()
+                        new_program += [("div", var, total, count), ("const", eps, float(op.epsilon)),
+                                        ("add", shifted, var, eps), ("sqrt", root, shifted), ("rcp", ins[1], root)]
+                    need_var = need_var or row > 0
+                elif ins[0] == "load":
+                    new_program.append((ins[0], ins[1], slot_map[ins[2]]))
+                elif ins[0] == "store":
+                    new_program.append((ins[0], slot_map[ins[1]], ins[2]))
+                elif ins[0] == "reduce":
+                    new_program.append((ins[0], ins[1], ins[2], slot_map[ins[3]]))
+                else:
+                    new_program.append(ins)
+            later.append((new_operands, new_program, it_axes, r_axes, onehot_axes, take_axes, take_strides))
+        if need_var:
+            parts.append(([x_td, sums[0], sums[1]],
+                          [("load", 0, 0), ("load", 1, 1), ("const", 2, n), ("div", 3, 1, 2), ("sub", 4, 0, 3),
+                           ("mul", 5, 4, 4), ("reduce", "sum", 5, 2)],
+                          x_td.axes, op.reduction_axes, [], [], {}))
+        return parts + later
+
+    @classmethod
+    def _merge_parts(cls, t, members, parts):
         red_axes, all_axes = None, None
         for operands, program, it_axes, r_axes, onehot_axes, take_axes, _ in parts:
             if onehot_axes or take_axes or any(ins[0] in ("iota", "rng", "take", "store_trunc") for ins in program):
@@ -981,8 +1078,10 @@ class ChainKernel(HipKernel):
         written = set(ins[1] for prog in programs for ins in prog if ins[0] == "store")
         written |= set(ins[3] for prog in programs for ins in prog if ins[0] == "reduce")
         for s in written:
-            if any(td.base is union[s].base and td is not union[s] for td in union):
-                return None
+            for td in union:
+                if td.base is union[s].base and td is not union[s] and \
+                        not (isinstance(td, _ChainScratch) and isinstance(union[s], _ChainScratch)):
+                    return None          # (two scratch operands are different rows of their tensor)
         walks = [walk(td) for td in union]
         dims = []
         for j, axis in enumerate(order):
@@ -995,8 +1094,8 @@ class ChainKernel(HipKernel):
         outer, inner = FusedKernel._split_outer(dims, True)
         sb = FusedSpecBuilder([d.length for d in inner] or [1])
         for s, td in enumerate(union):
-            view = t.get_tensor_description_tensor_view(td)
-            sb.tensor(view.ptr, [d.strides[s] for d in inner] or [0], t.ngh_dtype(td.dtype))
+            ptr = td.ptr if isinstance(td, _ChainScratch) else t.get_tensor_description_tensor_view(td).ptr
+            sb.tensor(ptr, [d.strides[s] for d in inner] or [0], t.ngh_dtype(td.dtype))
         read, written = set(), set()
         try:
             for prog in programs:
@@ -1086,11 +1185,11 @@ class KernelRun(HipKernel):
 
     @property
     def ops(self):
-        return [op for m in self.members for op in m.ops]
+        return [op for m in self.members for op in getattr(m, "ops", None) or [m.op]]
 
     @property
     def specs(self):
-        return [spec for k in self.kernels for spec in k.specs]
+        return [spec for k in self.kernels for spec in getattr(k, "specs", [])]
 
     def buffer_uses(self):
         return [u for k in self.kernels for u in k.buffer_uses()]
@@ -1872,8 +1971,9 @@ class HipTransformer(ComputationGraphTransformer):
         out, run = [], []
 
         def flush():
-            if len(run) >= 2 and any(isinstance(op, og.ReductionOp) and op.reduction_axes.size > 1
-                                     for k in run for op in k.ops):
+            if len(run) >= 2 and (isinstance(run[0], MomentsKernel) or
+                                  any(isinstance(op, og.ReductionOp) and op.reduction_axes.size > 1
+                                      for k in run for op in k.ops)):
                 out.append(KernelRun(self, run))
             else:
                 out.extend(run)
@@ -1881,6 +1981,10 @@ class HipTransformer(ComputationGraphTransformer):
 
         for k in kernels:
             if type(k) is FusedKernel:
+                run.append(k)
+            elif type(k) is MomentsKernel:
+                # (the statistics of rows and the kernels that use them may merge as well)
+                flush()
                 run.append(k)
             else:
                 flush()

@@ -179,6 +179,7 @@ def _kernels_lowered_for(results, placeholders, backend="hipgpu"):
     try:
         f = t.computation(results, *placeholders)
         t.initialize()
+        t.kernel_groups[f].bind()        # (runs of kernels settle which of them merge)
         return [type(k).__name__ for k in t.kernel_groups[f].kernels]
     finally:
         t.close()

@@ -498,3 +498,43 @@ def test_chained_kernels_run_by_themselves_until_the_chain_is_compiled():
     want = e / e.sum(axis=1, keepdims=True)
     np.testing.assert_allclose(alone, want, rtol=1e-5, atol=1e-7)
     np.testing.assert_allclose(chained, want, rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.gpu
+def test_row_statistics_and_their_consumer_merge_into_a_chain():
+    """mean / variance of rows (one MomentsOp in the graph) and the kernel that normalises with
+    them: one chain -- sum, sum of squared deviations, normalise -- when nothing else reads the
+    statistics; with the statistics returned as well, or without a compiled chain, the one-pass
+    moments kernel and the normalise kernel as before."""
+    def run(with_stats, **kwargs):
+        t = ngt.make_transformer_factory("hipgpu", **kwargs)()
+        try:
+            N, C = ng.make_axis(2500, name="N"), ng.make_axis(777, name="C")
+            x, g, b = ng.placeholder([N, C]), ng.placeholder([C]), ng.placeholder([C])
+            mean, var = ng.mean(x, out_axes=[N]), ng.variance(x, out_axes=[N])
+            y = g * ((x - mean) * ng.reciprocal(ng.sqrt(var + 1e-5))) + b
+            f = t.computation([y, mean, var] if with_stats else [y], x, g, b)
+            rs = np.random.RandomState(8)
+            xv = rs.normal(0.5, 2.0, (2500, 777)).astype(np.float32)
+            gv, bv = rs.uniform(0.5, 1.5, 777).astype(np.float32), rs.uniform(-1, 1, 777).astype(np.float32)
+            out = [np.array(r).copy() for r in f(xv, gv, bv)]
+            names = [d for k in t.kernel_groups[f].kernels for ds in k.describe() for d in ds]
+            return out, names, (xv, gv, bv)
+        finally:
+            t.close()
+    # (first without compilation: a program, once loaded, serves every transformer of the process)
+    alone, names_alone, _ = run(False, jit=False)
+    chained, names_chained, (xv, gv, bv) = run(False, jit=True, jit_min_elements=1)
+    with_stats, names_stats, _ = run(True, jit=True, jit_min_elements=1)
+    if default_kernel_choice():
+        assert all("/chain-of-3" in n for n in names_chained) and len(names_chained) == 3, names_chained
+        # (unless an earlier test of this process has loaded this very chain already)
+        assert names_alone[0] == "moments_f32" or all("/chain-of-3" in n for n in names_alone), names_alone
+        assert names_stats[0] == "moments_f32" and not any("chain" in n for n in names_stats), names_stats
+    x64 = xv.astype(np.float64)
+    m, v = x64.mean(axis=1, keepdims=True), x64.var(axis=1, keepdims=True)
+    want = gv * ((x64 - m) / np.sqrt(v + 1e-5)) + bv
+    for got in (chained[0], alone[0], with_stats[0]):
+        np.testing.assert_allclose(got, want, rtol=1e-5, atol=2e-6)
+    np.testing.assert_allclose(with_stats[1], m[:, 0], rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(with_stats[2], v[:, 0], rtol=1e-5, atol=1e-6)
