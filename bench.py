@@ -505,8 +505,11 @@ def shape_survey_cases(ng):
         R, K = ax(rows, "R%d" % k), ax(k, "K%d" % k)
         w = ng.placeholder([R, K])
         mu, vv = ng.mean(w, out_axes=[R]), ng.variance(w, out_axes=[R])
-        yield ("layer norm of rows [%d,%d] (one-pass statistics, normalise; 3 passes)" % (rows, k),
-               [(w - mu) * ng.reciprocal(ng.sqrt(vv + 1e-5))], [w], 3 * rows * k * 4)
+        # (as one row-chain kernel x is read once; else the one-pass moments kernel reads it, then
+        # the normalise kernel)
+        yield ("layer norm of rows [%d,%d] (statistics, normalise)" % (rows, k),
+               [(w - mu) * ng.reciprocal(ng.sqrt(vv + 1e-5))], [w],
+               {"chain": 2 * rows * k * 4, "kernels": 3 * rows * k * 4})
         e = ng.exp(w - ng.max(w, out_axes=[R]))
         # (as one row-chain kernel the operand is read once and the result written once; as three
         # kernels it is read three times)
@@ -542,8 +545,10 @@ def shape_survey(ng, ngt, steps, warmup):
                        for k, times in group.profile(repeats=3, inner=10)]
             if isinstance(nbytes, dict):
                 chained = any("/chain-of-" in d for d, _ in kernels)
+                passes = nbytes["kernels"] // (nbytes["chain"] // 2)
                 nbytes = nbytes["chain" if chained else "kernels"]
-                name += " (one row-chain kernel; 2 passes)" if chained else " (3 kernels; 4 passes)"
+                name += " (one row-chain kernel; 2 passes)" if chained else \
+                    " (%d kernels; %d passes)" % (len(kernels), passes)
             out[name] = {"ms_per_step": round(ms, 5), "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
                          "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                          "algorithmic_bytes_per_step": int(nbytes),
