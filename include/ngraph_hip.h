@@ -301,7 +301,10 @@ int  ngh_plan_fused(const ngh_fused_spec* spec, int32_t stage, int32_t* out8);
  * to 8192 elements, fp32 operands with unit stride along the row or broadcast along it, at
  * least one reduction stage.  out4 = {1 if the spec qualifies, index of the compiled chain
  * program or -1 (without one the stages are launched one by one), lanes per row, stages}.
- * No device needed (host-side tooling and tests).                                          */
+ * A stage of a row chain may also STORE one value per row: a value that does not vary along
+ * axis 0 (computed from operands with stride 0 there, such as earlier stages' results) into a
+ * tensor with stride 0 on axis 0; ngh_launch_fused refuses such a spec (NGH_E_UNSUPPORTED)
+ * unless it runs as a chain.  No device needed (host-side tooling and tests).              */
 int  ngh_plan_chain(const ngh_fused_spec* spec, int32_t* out4);
 
 /* ---- flex statistics: the int32 device words FlexPtrDescription binds

@@ -191,6 +191,7 @@ int validate(const ngh_fused_spec* sp) {
         if (S.n_reductions < 0 || S.n_reductions > NGH_MAX_REDUCTIONS)
             return fail(NGH_E_INVALID, "stage %d: n_reductions %d", s, S.n_reductions);
         bool defined[NGH_MAX_REGS] = {false};
+        bool along0[NGH_MAX_REGS] = {false};     // the value varies along axis 0
         int n_red_seen = 0;
         for (int pc = S.op_begin; pc < S.op_end; ++pc) {
             const ngh_op& o = sp->ops[pc];
@@ -202,18 +203,26 @@ int validate(const ngh_fused_spec* sp) {
             if (opc == NGH_OP_LOAD) {
                 if (o.a >= sp->n_tensors || !reg_ok(o.dst)) return fail(NGH_E_INVALID, "op %d: bad LOAD", pc);
                 defined[o.dst] = true;
+                along0[o.dst] = sp->shape[0] > 1 && sp->tensors[o.a].strides[0] != 0;
             } else if (opc == NGH_OP_STORE || opc == NGH_OP_STORE_TRUNC) {
                 if (o.dst >= sp->n_tensors || !need(o.a)) return fail(NGH_E_INVALID, "op %d: bad STORE", pc);
                 const ngh_tensor& T = sp->tensors[o.dst];
-                for (int a = 0; a < NGH_MAX_AXES; ++a)
-                    if (sp->shape[a] > 1 && T.strides[a] == 0)
-                        return fail(NGH_E_INVALID, "op %d: STORE to a tensor broadcast along axis %d", pc, a);
+                for (int a = 0; a < NGH_MAX_AXES; ++a) {
+                    if (sp->shape[a] <= 1 || T.strides[a] != 0) continue;
+                    // One value per row (axis 0 is the row, the axis reductions run along): allowed for a
+                    // value that is the same all along the row -- computed from operands broadcast along
+                    // it, such as the results of earlier stages' reductions.
+                    if (a == 0 && opc == NGH_OP_STORE && !along0[o.a]) continue;
+                    return fail(NGH_E_INVALID, "op %d: STORE to a tensor broadcast along axis %d", pc, a);
+                }
             } else if (opc == NGH_OP_CONST) {
                 if (o.a >= sp->n_consts || !reg_ok(o.dst)) return fail(NGH_E_INVALID, "op %d: bad CONST", pc);
                 defined[o.dst] = true;
+                along0[o.dst] = false;
             } else if (opc == NGH_OP_RNG_UNIFORM || opc == NGH_OP_RNG_NORMAL) {
                 if (!reg_ok(o.dst)) return fail(NGH_E_INVALID, "op %d: bad RNG destination", pc);
                 defined[o.dst] = true;
+                along0[o.dst] = true;
             } else if (opc == NGH_OP_TAKE) {
                 const int t = o.b & 15, axis = o.b >> 4;
                 if (t >= sp->n_tensors || axis >= sp->rank || !need(o.a) || !reg_ok(o.dst))
@@ -224,19 +233,23 @@ int validate(const ngh_fused_spec* sp) {
                     return fail(NGH_E_UNSUPPORTED, "op %d: TAKE along an axis of %u entries: indices travel in fp32 "
                                 "registers, exact up to 2^24", pc, sp->tensors[t].take_extent);
                 defined[o.dst] = true;
+                along0[o.dst] = true;
             } else if (opc == NGH_OP_IOTA) {
                 if (o.a >= NGH_MAX_AXES || !reg_ok(o.dst)) return fail(NGH_E_INVALID, "op %d: bad IOTA", pc);
                 if (sp->shape[o.a] > (long long)kExactIntegers)
                     return fail(NGH_E_UNSUPPORTED, "op %d: IOTA along an axis of %lld: index values travel in fp32 "
                                 "registers, exact up to 2^24", pc, (long long)sp->shape[o.a]);
                 defined[o.dst] = true;
+                along0[o.dst] = true;
             } else if (is_unary(opc)) {
                 if (!need(o.a) || !reg_ok(o.dst)) return fail(NGH_E_INVALID, "op %d: unary operand undefined", pc);
                 defined[o.dst] = true;
+                along0[o.dst] = along0[o.a];
             } else if (is_binary(opc)) {
                 if (!need(o.a) || !need(o.b) || !reg_ok(o.dst))
                     return fail(NGH_E_INVALID, "op %d: binary operand undefined", pc);
                 defined[o.dst] = true;
+                along0[o.dst] = along0[o.a] || along0[o.b];
             } else if (is_reduce(opc)) {
                 if (!need(o.a) || o.dst != n_red_seen || n_red_seen >= S.n_reductions)
                     return fail(NGH_E_INVALID, "op %d: reduction slot %d out of order", pc, o.dst);
@@ -381,7 +394,7 @@ bool vec4_ok(const KArgs& k, const bool* used) { return vec_ok(k, used, 4); }
 // Can the stage move 4 elements per lane along kernel axis 2 although vec_ok says no -- rows whose
 // length is not a multiple of 4, or that do not start on 16-byte boundaries?  The compiled
 // programs can (program_ragged_ok has the conditions on the program), given unit strides.
-bool ragged_rows_ok(const KArgs& k, const bool* used) {
+bool ragged_rows_ok(const KArgs& k, const bool* used, bool row_stores = false) {
     if (k.shape[2] < 8) return false;
     int dtypes[NGH_MAX_TENSORS];
     unsigned char bcast[NGH_MAX_TENSORS];
@@ -390,7 +403,7 @@ bool ragged_rows_ok(const KArgs& k, const bool* used) {
         bcast[t] = (t < k.n_tensors && k.t[t].s[2] == 0) ? 1 : 0;
         if (t < k.n_tensors && used[t] && k.t[t].s[2] != 0 && k.t[t].s[2] != 1) return false;
     }
-    return program_ragged_ok(4, k.ops + k.op_begin, k.op_end - k.op_begin, dtypes, bcast);
+    return program_ragged_ok(4, k.ops + k.op_begin, k.op_end - k.op_begin, dtypes, bcast, row_stores);
 }
 
 constexpr size_t kInterpLdsPreferred = 64 * 1024;   // keeps >= 2 workgroups per CU
@@ -439,6 +452,10 @@ int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage,
     for (int t = 0; t < NGH_MAX_TENSORS; ++t) used[t] = loads[t] || stores[t];
     long long total = sp.shape[0] * sp.shape[1] * sp.shape[2];
     if (total >= kMaxStageElems) return fail(NGH_E_UNSUPPORTED, "stage view of %lld elements exceeds 2^33", total);
+    for (int pc = S.op_begin; pc < S.op_end; ++pc)
+        if (sp.ops[pc].opcode == NGH_OP_STORE && sp.shape[0] > 1 && sp.tensors[sp.ops[pc].dst].strides[0] == 0)
+            return fail(NGH_E_UNSUPPORTED, "stage %d stores one value per row: only a row chain runs it "
+                        "(ngh_plan_chain tells whether the spec is one and has a compiled program)", stage);
 
     if (S.n_reductions == 0) {
         // fast axis = the one along which most memory traffic is contiguous: every
@@ -1352,7 +1369,7 @@ bool plan_row_chain(const ngh_context* ctx, const ngh_fused_spec& sp, ChainPlan&
         bool loads[NGH_MAX_TENSORS], stores[NGH_MAX_TENSORS], used[NGH_MAX_TENSORS];
         stage_tensors(sp, S, loads, stores);
         for (int t = 0; t < NGH_MAX_TENSORS; ++t) used[t] = loads[t] || stores[t];
-        if (k.n_stat_slots != 0 || k.probe || !ragged_rows_ok(k, used) ||
+        if (k.n_stat_slots != 0 || k.probe || !ragged_rows_ok(k, used, true) ||
             !program_loads_hoistable(k.ops + k.op_begin, k.op_end - k.op_begin))
             return false;
         for (int r = 0; r < S.n_reductions; ++r) {

@@ -954,22 +954,29 @@ class ChainKernel(HipKernel):
         """Mean, variance and 1/sqrt(variance + eps) of rows, and the kernels that use them, as
         stages: sum(x); sum((x - sum / n)^2); then the kernels, each load of a statistic replaced
         by its value computed from the two sums -- the statements ng.mean and ng.variance stand
-        for (op_graph.py:4007-4009, 4252-4266).  The two sums go where the statistics would
-        have gone, which is why nothing outside `rest` may read those."""
+        for (op_graph.py:4007-4009, 4252-4266).  When nothing outside `rest` reads the statistics
+        the two sums go where those would have gone; else the sums get memory of their own and
+        a stage in between writes the statistics out, one value per row."""
         if not rest or any(type(k) is not FusedKernel for k in rest):
             return None
         op = moments.op
         mom_base = _td(op).base
         readers, returned = t._usage_maps()
         inside = set(o for k in rest for o in k.ops)
-        if mom_base in returned or any(u not in inside for u in readers.get(mom_base, ())):
-            return None
+        private = mom_base not in returned and all(u in inside for u in readers.get(mom_base, ()))
         moments.bind_buffers()
         x_td = _td(op.args[0].forwarded)
         n = float(op.reduction_axes.size)
         kept = [a for a in x_td.axes if a not in op.reduction_axes]
         rows = moments.rows
-        sums = [_ChainScratch(mom_base, moments.out.ptr + i * rows * 4, kept, i) for i in range(2)]
+        stats = [_ChainScratch(mom_base, moments.out.ptr + i * rows * 4, kept, i) for i in range(3)]
+        if private:
+            sums = stats[:2]
+        else:
+            if getattr(moments, "chain_scratch", None) is None:
+                moments.chain_scratch = t.runtime.malloc(2 * rows * 4)       # (freed with the runtime)
+            own = object()
+            sums = [_ChainScratch(own, moments.chain_scratch + i * rows * 4, kept, i) for i in range(2)]
         parts = [([x_td, sums[0]], [("load", 0, 0), ("reduce", "sum", 0, 1)],
                   x_td.axes, op.reduction_axes, [], [], {})]
         need_var = False
@@ -1016,11 +1023,21 @@ class ChainKernel(HipKernel):
                 else:
                     new_program.append(ins)
             later.append((new_operands, new_program, it_axes, r_axes, onehot_axes, take_axes, take_strides))
-        if need_var:
+        if need_var or not private:
             parts.append(([x_td, sums[0], sums[1]],
                           [("load", 0, 0), ("load", 1, 1), ("const", 2, n), ("div", 3, 1, 2), ("sub", 4, 0, 3),
                            ("mul", 5, 4, 4), ("reduce", "sum", 5, 2)],
                           x_td.axes, op.reduction_axes, [], [], {}))
+        if not private:
+            # the statistics themselves, for their other readers
+            program = [("load", 0, 0), ("load", 1, 1), ("const", 2, n), ("div", 3, 0, 2), ("store", 2, 3),
+                       ("div", 4, 1, 2), ("store", 3, 4)]
+            operands = [sums[0], sums[1], stats[0], stats[1]]
+            if op.epsilon is not None:
+                program += [("const", 5, float(op.epsilon)), ("add", 6, 4, 5), ("sqrt", 7, 6), ("rcp", 8, 7),
+                            ("store", 4, 8)]
+                operands.append(stats[2])
+            parts.append((operands, program, x_td.axes, og.make_axes(()), [], [], {}))
         return parts + later
 
     @classmethod

@@ -503,9 +503,9 @@ def test_chained_kernels_run_by_themselves_until_the_chain_is_compiled():
 @pytest.mark.gpu
 def test_row_statistics_and_their_consumer_merge_into_a_chain():
     """mean / variance of rows (one MomentsOp in the graph) and the kernel that normalises with
-    them: one chain -- sum, sum of squared deviations, normalise -- when nothing else reads the
-    statistics; with the statistics returned as well, or without a compiled chain, the one-pass
-    moments kernel and the normalise kernel as before."""
+    them: one chain -- sum, sum of squared deviations, normalise; with the statistics returned
+    as well, a stage in between that writes them out, one value per row.  Without a compiled
+    chain: the one-pass moments kernel and the normalise kernel as before."""
     def run(with_stats, **kwargs):
         t = ngt.make_transformer_factory("hipgpu", **kwargs)()
         try:
@@ -530,7 +530,7 @@ def test_row_statistics_and_their_consumer_merge_into_a_chain():
         assert all("/chain-of-3" in n for n in names_chained) and len(names_chained) == 3, names_chained
         # (unless an earlier test of this process has loaded this very chain already)
         assert names_alone[0] == "moments_f32" or all("/chain-of-3" in n for n in names_alone), names_alone
-        assert names_stats[0] == "moments_f32" and not any("chain" in n for n in names_stats), names_stats
+        assert all("/chain-of-4" in n for n in names_stats) and len(names_stats) == 4, names_stats
     x64 = xv.astype(np.float64)
     m, v = x64.mean(axis=1, keepdims=True), x64.var(axis=1, keepdims=True)
     want = gv * ((x64 - m) / np.sqrt(v + 1e-5)) + bv
@@ -538,3 +538,42 @@ def test_row_statistics_and_their_consumer_merge_into_a_chain():
         np.testing.assert_allclose(got, want, rtol=1e-5, atol=2e-6)
     np.testing.assert_allclose(with_stats[1], m[:, 0], rtol=1e-5, atol=1e-6)
     np.testing.assert_allclose(with_stats[2], v[:, 0], rtol=1e-5, atol=1e-6)
+
+
+def _row_store_spec(px, ps, pm, R, rows, varying=False):
+    """sum of rows, then a stage that stores one value per row (the mean)."""
+    sb = hiplib.FusedSpecBuilder([R, rows])
+    tx, ts, tm = sb.tensor(px, [1, R]), sb.tensor(ps, [0, 1]), sb.tensor(pm, [0, 1])
+    sb.reduce("sum", sb.load(tx), ts)
+    sb.end_stage()
+    mean = sb.binary("div", sb.load(ts), sb.constant(float(R)))
+    sb.store(tm, sb.binary("add", mean, sb.load(tx)) if varying else mean)
+    return sb
+
+
+def test_one_value_per_row_may_be_stored_only_if_it_is_the_same_along_the_row():
+    from ngraph_hip.runtime.hiplib import DryRunRuntime
+    rt = DryRunRuntime()
+    rt.validate_fused(_row_store_spec(4096, 8192, 12288, 100, 50).build())
+    with pytest.raises(hiplib.HipLibraryError, match="broadcast along axis 0"):
+        rt.validate_fused(_row_store_spec(4096, 8192, 12288, 100, 50, varying=True).build())
+
+
+@pytest.mark.gpu
+def test_a_spec_that_stores_one_value_per_row_runs_as_a_chain_or_not_at_all(hip_runtime):
+    rt = hip_runtime
+    rows, R = 1500, 333
+    x = np.random.RandomState(3).normal(1.0, 2.0, (rows, R)).astype(np.float32)
+    x_d, s_d, m_d = rt.array(x), rt.empty((rows,)), rt.empty((rows,))
+    spec = _row_store_spec(x_d.ptr, s_d.ptr, m_d.ptr, R, rows).build()
+    if hiplib.plan_chain(spec)["special"] < 0:
+        with pytest.raises(hiplib.HipLibraryError, match="row chain"):
+            rt.launch_fused(spec)
+    if default_kernel_choice():
+        jit.ensure_programs(rt, [_SpecHolder(spec)], "row_store", min_elements=1)
+        assert "/chain-of-2" in rt.describe_fused(spec, 0)
+        rt.launch_fused(spec)
+        np.testing.assert_allclose(m_d.get(), x.astype(np.float64).mean(axis=1), rtol=1e-5, atol=1e-6)
+        np.testing.assert_allclose(s_d.get(), x.astype(np.float64).sum(axis=1), rtol=1e-5, atol=1e-4)
+    for d in (x_d, s_d, m_d):
+        d.free()
