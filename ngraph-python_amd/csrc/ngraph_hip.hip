@@ -1662,7 +1662,9 @@ int ngh_plan_chain(const ngh_fused_spec* spec, int32_t* out4) {
     if (!out4) return fail(NGH_E_INVALID, "out4 is NULL");
     NGH_TRY(validate(spec));
     ChainPlan C;
+    // (no context here: the knobs a context would carry are read from the environment, as it does)
     const bool ok = spec->n_stages > 1 && !env_int("NGH_NO_CHAIN", 0) && !env_int("NGH_NO_RAGGED", 0) &&
+                    !env_int("NGH_FORCE_INTERP", 0) && env_int("NGH_ROW_WAVE_CHUNKS", kRowWaveChunks) > 0 &&
                     plan_row_chain(nullptr, *spec, C);
     out4[0] = ok ? 1 : 0;
     out4[1] = ok ? match_chain(C.k, C.families, C.n) : -1;
