@@ -190,7 +190,8 @@ def test_cache_policy_does_not_change_results(policy, monkeypatch):
         f = t.computation([y, xmean, xvar], x)
         out.extend(np.array(a) for a in f(x_np.reshape(dims)))
         assert not check_names or \
-            any("special:batchnorm" in d for k in t.kernel_groups[f].kernels for ds in k.describe() for d in ds)
+            any("special:batchnorm" in d or "/chain-of-" in d     # (rows this short merge into a row chain once one is compiled)
+                for k in t.kernel_groups[f].kernels for ds in k.describe() for d in ds)
         t.close()
         return out
 
