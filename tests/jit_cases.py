@@ -117,6 +117,15 @@ def case_softmax_over_windows():
     return [e / ng.sum(e, reduction_axes=xs.axes[2:]), ng.argmax(xs, reduction_axes=xs.axes[2:])], [x]
 
 
+def case_softmax_forward_and_backward():
+    # a softmax and the derivative of a loss through it: five kernels over the same rows, one chain
+    C, N = ng.make_axis(500, name="C"), ng.make_axis(3000, name="N")
+    x, tgt = ng.placeholder([N, C]), ng.placeholder([N, C])
+    e = ng.exp(x - ng.max(x, out_axes=[N]))
+    y = e / ng.sum(e, out_axes=[N])
+    return [y, ng.deriv(ng.sum(y * tgt, out_axes=()), x)], [x, tgt]
+
+
 def case_row_chain_with_stored_intermediate():
     # log-softmax and the row norms of the same tensor: two results, reductions of different
     # kinds, an intermediate that is stored by one stage and read back by the next
@@ -167,6 +176,7 @@ def case_lookup_table():
 FP32_CASES = [case_elementwise, case_column_reduction_with_store, case_row_reduction_with_store,
               case_transposed_operand, case_transposed_operands_large, case_softmax, case_mixed_storage_types, case_ragged,
               case_ragged_long_rows, case_ragged_many_rows, case_softmax_ragged_rows, case_softmax_long_rows, case_softmax_over_windows,
+              case_softmax_forward_and_backward,
               case_row_chain_with_stored_intermediate, case_misaligned_slices, case_short_rows, case_dropout, case_lookup_table]
 
 

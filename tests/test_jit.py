@@ -234,6 +234,7 @@ def test_compiled_programs_agree_with_the_interpreter(case):
             assert any(n.endswith("/ragged") for n in names), names
         if case in (jit_cases.case_softmax, jit_cases.case_softmax_ragged_rows, jit_cases.case_short_rows,
                     jit_cases.case_softmax_long_rows, jit_cases.case_softmax_over_windows,
+                    jit_cases.case_softmax_forward_and_backward,
                     jit_cases.case_row_chain_with_stored_intermediate):
             assert any("/chain-of-" in n for n in names), names
         if case is jit_cases.case_transposed_operands_large:
