@@ -283,7 +283,7 @@ int validate(const ngh_fused_spec* sp) {
 // planner
 // ---------------------------------------------------------------------------
 enum Family { F_EW = 0, F_RED_ROW, F_RED_COL, F_EW_TILED };
-constexpr int kRowWaveChunks = 512;
+constexpr int kRowWaveChunks = 1024;
 
 struct Plan {
     Family   family = F_EW;
@@ -1511,7 +1511,7 @@ int plan_moments(const ngh_context* ctx, const float* dev_x, int64_t rows, int64
     if (((uintptr_t)dev_x) % 4) return fail(NGH_E_INVALID, "x is not aligned to its element size");
     if (rows >= (1LL << 24) || R >= (1LL << 32)) return fail(NGH_E_UNSUPPORTED, "extent too large");
     m.R4 = (unsigned)(R / 4);
-    m.per_wave = (long long)m.R4 <= ctx->row_wave_chunks * 2 && rows >= (long long)ctx->cus * 4 * (kMomBlock / 64);
+    m.per_wave = (long long)m.R4 <= ctx->row_wave_chunks && rows >= (long long)ctx->cus * 4 * (kMomBlock / 64);
     // a lane per chunk of the row, up to a wavefront; with rows enough to fill the chip several
     // times over, a quarter of that (each lane then has four chunks in flight)
     m.lanes = 1;
