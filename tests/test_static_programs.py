@@ -145,3 +145,31 @@ def test_cache_hints_batchnorm_keeps_x_cacheable_and_streams_y():
     assert reads == [0]                                           # x: two readers, stays cacheable
     assert writes == [hiplib.NGH_CACHE_STREAM_STORE]              # y: a result nobody here reads
     t.close()
+
+
+def test_cache_hints_of_a_row_chain_and_of_its_members():
+    """A softmax merged into one chain: the chain is the only reader of x (its loads may stream)
+    and nothing reads y again (its stores may stream); the three kernels it consists of, which
+    run by themselves until the chain is compiled, read x one after the other, so none of them
+    may stream it past the cache, and only the last writes a result nobody reads."""
+    t = ngt.make_transformer_factory("hipgpu", dry_run=True, jit=False)()
+    N, C = ng.make_axis(4096, name="N"), ng.make_axis(1000, name="C")
+    x = ng.placeholder([N, C])
+    e = ng.exp((x - ng.max(x, out_axes=[N])) * 0.5)
+    f = t.computation(e / ng.sum(e, out_axes=[N]), x)
+    t.initialize()
+    group = t.kernel_groups[f]
+    group.bind()
+    assert [type(k).__name__ for k in group.kernels] == ["ChainKernel"]
+    chain = group.kernels[0]
+    big = _hints(group)
+    assert sorted(big) == [(False, True, hiplib.NGH_CACHE_STREAM_STORE), (True, False, hiplib.NGH_CACHE_STREAM_LOAD)]
+    member_hints = []
+    for m in chain.members:
+        for spec, uses in zip(m.specs, m.spec_uses):
+            for s, (base, is_read, is_written) in enumerate(uses):
+                if int(np.prod(base.shape or (1,))) > 65536:
+                    member_hints.append((is_read, is_written, spec.tensors[s].cache_hint))
+    assert member_hints == [(True, False, 0), (True, False, 0), (True, False, 0),
+                            (False, True, hiplib.NGH_CACHE_STREAM_STORE)]
+    t.close()
