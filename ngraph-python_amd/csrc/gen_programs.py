@@ -127,10 +127,29 @@ def pattern_log_softmax_rows(t):
     return t.computation(shifted - ng.log(ng.sum(ng.exp(shifted), out_axes=[N])), x)
 
 
+def pattern_batchnorm_short_rows(t):
+    # (the same statements as pattern_batchnorm: with rows of up to 8192 elements the statistics
+    # and the normalise kernel merge into one row chain that also writes the statistics out)
+    return pattern_batchnorm(t)
+
+
+def _layer_norm_pattern(affine):
+    def build(t):
+        N, C = _axes(N=4096, C=1000)
+        x = ng.placeholder([N, C])
+        mean, var = ng.mean(x, out_axes=[N]), ng.variance(x, out_axes=[N])
+        y = (x - mean) * ng.reciprocal(ng.sqrt(var + 1e-5))
+        if affine:
+            g, b = ng.placeholder([C]), ng.placeholder([C])
+            return t.computation(g * y + b, x, g, b)
+        return t.computation(y, x)
+    return build
+
+
 # patterns whose kernels merge into one row chain (rows of up to 8192 elements along the
 # contiguous axis): the chain is built in, so that these run as one launch without run-time
 # compilation, whatever their size
-CHAINS = ("softmax_rows", "log_softmax_rows")
+CHAINS = ("softmax_rows", "log_softmax_rows", "batchnorm_short_rows", "layer_norm_rows", "layer_norm_affine_rows")
 
 PATTERNS = [
     ("c1_tanh_sigmoid", "hipgpu", pattern_c1),
@@ -164,6 +183,9 @@ PATTERNS = [
     ("lstm_cell_large", "hipgpu", lambda t: pattern_lstm_cell(t, 2048, 512)),
     ("softmax_rows", "hipgpu", pattern_softmax_rows),
     ("log_softmax_rows", "hipgpu", pattern_log_softmax_rows),
+    ("batchnorm_short_rows", "hipgpu", pattern_batchnorm_short_rows),
+    ("layer_norm_rows", "hipgpu", _layer_norm_pattern(False)),
+    ("layer_norm_affine_rows", "hipgpu", _layer_norm_pattern(True)),
 ]
 
 

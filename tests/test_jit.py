@@ -578,3 +578,46 @@ def test_a_spec_that_stores_one_value_per_row_runs_as_a_chain_or_not_at_all(hip_
         np.testing.assert_allclose(s_d.get(), x.astype(np.float64).sum(axis=1), rtol=1e-5, atol=1e-4)
     for d in (x_d, s_d, m_d):
         d.free()
+
+
+@pytest.mark.gpu
+def test_normalisations_over_short_rows_run_as_built_in_chains():
+    """Batch normalisation as the neon front writes it, layer normalisation and (log-)softmax over
+    rows of up to 8192 elements: one launch each from chains built into the library, without
+    run-time compilation."""
+    from ngraph_hip.frontends import neon
+    rs = np.random.RandomState(4)
+    t = ngt.make_transformer_factory("hipgpu", jit=False)()
+    try:
+        C, H, W, N = (ng.make_axis(n, name=k) for k, n in zip("CHWN", (48, 9, 9, 32)))
+        x = ng.placeholder([C, H, W, N])
+        gv, bv = rs.uniform(0.5, 1.5, 48).astype(np.float32), rs.uniform(-1, 1, 48).astype(np.float32)
+        gamma, beta = ng.variable([C], initial_value=gv), ng.variable([C], initial_value=bv)
+        y, mean, var = neon.batch_norm_train(x, gamma, beta, out_axes=[C])
+        bn = t.computation([y, mean, var], x)
+        R, K = ng.make_axis(700, name="R"), ng.make_axis(1500, name="K")
+        w = ng.placeholder([R, K])
+        mu, vv = ng.mean(w, out_axes=[R]), ng.variance(w, out_axes=[R])
+        ln = t.computation((w - mu) * ng.reciprocal(ng.sqrt(vv + 1e-5)), w)
+        sm = t.computation(ng.softmax(w, normalization_axes=ng.make_axes([K])), w)
+        xv = rs.normal(0.5, 2.0, (48, 9, 9, 32)).astype(np.float32)
+        wv = rs.normal(0.0, 3.0, (700, 1500)).astype(np.float32)
+        y_, mean_, var_ = [np.array(a) for a in bn(xv)]
+        ln_, sm_ = np.array(ln(wv)), np.array(sm(wv))
+        if default_kernel_choice():
+            for f, name, stages in ((bn, "batchnorm_short_rows_k0", 4), (ln, "layer_norm_rows_k0", 3), (sm, "softmax_rows_k0", 3)):
+                names = [d for k in t.kernel_groups[f].kernels for ds in k.describe() for d in ds]
+                assert names == ["special:%s/chain-of-%d" % (name, stages)] * stages, names
+    finally:
+        t.close()
+    x64 = xv.astype(np.float64).reshape(48, -1)
+    m, v = x64.mean(axis=1), x64.var(axis=1)
+    np.testing.assert_allclose(mean_, m, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(var_, v, rtol=1e-5, atol=1e-6)
+    want = gv[:, None] * (x64 - m[:, None]) / np.sqrt(v[:, None] + 1e-5) + bv[:, None]
+    np.testing.assert_allclose(y_.reshape(48, -1), want, rtol=1e-5, atol=2e-6)
+    w64 = wv.astype(np.float64)
+    np.testing.assert_allclose(ln_, (w64 - w64.mean(axis=1, keepdims=True)) / np.sqrt(w64.var(axis=1, keepdims=True) + 1e-5),
+                               rtol=1e-5, atol=2e-6)
+    e = np.exp(w64 - w64.max(axis=1, keepdims=True))
+    np.testing.assert_allclose(sm_, e / e.sum(axis=1, keepdims=True), rtol=1e-5, atol=1e-7)
