@@ -124,6 +124,7 @@ struct ngh_context {
     int         tile4 = 1;               // tiled elementwise programs may take 64 x 64 tiles with 16-byte accesses
     int         no_tiles = 0;        // never use the LDS-tiled elementwise skeleton
     int         no_chain = 0;        // never run the stages of a spec as one row-chain kernel
+    int         wide_min_rows = 2;   // column reductions: rows from which a whole workgroup lies along the columns
     int         no_ragged = 0;       // never run compiled programs 4-wide over rows that are not whole aligned vectors
     int         flex_self_managed = 2;  // ngh_launch_fused_flex: 0 = prepare / kernel / update launches,
                                      // 1 = policy at the end of the kernel, 2 = statistics deferred to the next user
@@ -627,7 +628,7 @@ int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage,
         const long long col_target = compiled ? (ctx ? ctx->cus * ctx->red_col_wgs_per_cu : 256 * 2) : target_wgs;
         // (... unless the last of those workgroups per row would be mostly idle lanes)
         const long long wide_blocks = (col_chunks + kBlock - 1) / kBlock;
-        const bool wide = compiled && col_chunks >= kBlock && R * n_out > kSmallReduction && R >= 64 &&
+        const bool wide = compiled && col_chunks >= kBlock && R * n_out > kSmallReduction && R >= (ctx ? ctx->wide_min_rows : 2) &&
                           col_chunks * 10 >= wide_blocks * kBlock * 9;
         if (wide) P.tx = kBlock;
         if (R * n_out <= kSmallReduction) {
@@ -1106,6 +1107,7 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->no_tiles = env_int("NGH_NO_TILES", 0);
     ctx->no_ragged = env_int("NGH_NO_RAGGED", 0);
     ctx->no_chain = env_int("NGH_NO_CHAIN", 0);
+    ctx->wide_min_rows = std::max(1, env_int("NGH_WIDE_MIN_ROWS", 2));
     ctx->red_wgs_per_cu = std::max(1, env_int("NGH_RED_WGS_PER_CU", 8));
     ctx->red_col_wgs_per_cu = std::max(1, env_int("NGH_RED_COL_WGS_PER_CU", 2));
     ctx->row_wave_chunks = std::max(0, env_int("NGH_ROW_WAVE_CHUNKS", kRowWaveChunks));
