@@ -1517,11 +1517,14 @@ class FusionPlanner(object):
                     h = groups[hi]
                     have = set(_view_key(td) for o in h.ops for td in h._operand_views(o)[0])
                     # (large next to the result itself: the per-row maxima of 131072 rows of 256
-                    # elements are many, and still 1/256 of a pass)
-                    large = max(self.small_tensor, iteration_axes(op).size // 16)
+                    # elements are many, and still 1/256 of a pass; what counts is what the kernel
+                    # would read on top of what it reads anyway: one more pass at most, a little over
+                    # it with the maxima of ten-element columns)
+                    size = iteration_axes(op).size
+                    large = max(self.small_tensor, size // 16)
                     extra_large = [td for td in leaves
                                    if _view_key(td) not in have and _memory_elements(td) > large]
-                    if len(extra_large) > 1:
+                    if len(extra_large) > 1 and sum(_memory_elements(td) for td in extra_large) > size + size // 4:
                         break
                     # the repeated ops are private to the kernel: whoever else needs them has them
                     new = _Group.rebuilt(h, chain, readers, returned, h.private)
