@@ -386,9 +386,7 @@ class FusedKernel(HipKernel):
         """Pass 1 of the lowering: the operands (views) the group touches and its program over
         symbolic registers; returns (operands, program, it_axes, red_axes, onehot_axes,
         take_axes, take_strides)."""
-        t = self.transformer
         ops = self.ops
-        first = ops[0]
         reductions = [op for op in ops if isinstance(op, og.ReductionOp) and op.reduction_axes.size > 1]
         # (a kernel may carry a few ops over a subset of its axes, absorbed from a smaller kernel:
         # they are simply repeated along the missing axes)
@@ -1108,7 +1106,7 @@ class ChainKernel(HipKernel):
         dims = FusedKernel._coalesce(dims, True)
         if len([d for d in dims if d.tag == "red"]) != 1 or len(dims) > 3:
             return None          # (the reduced axes do not walk as one, or axes are left to a host loop)
-        outer, inner = FusedKernel._split_outer(dims, True)
+        _, inner = FusedKernel._split_outer(dims, True)
         sb = FusedSpecBuilder([d.length for d in inner] or [1])
         for s, td in enumerate(union):
             ptr = td.ptr if isinstance(td, _ChainScratch) else t.get_tensor_description_tensor_view(td).ptr
