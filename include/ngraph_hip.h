@@ -232,6 +232,12 @@ int  ngh_copy_strided(ngh_context* ctx, void* dev_dst, const void* dev_src,
 /* ---- compound kernels: replaces CudaSourceFile.add_kernel + compile +
  *      prepared_async_call (float_ew2.py:1553-1653, gputransform.py:343-345) */
 int  ngh_validate_fused(const ngh_fused_spec* spec);
+/* Stages run in order and each stage sees what the stages before it wrote, also when two
+ * operand slots name overlapping memory (an in-place update through a second view): a spec
+ * with such slots, one of them written, is never run as one row-chain kernel, whose stages
+ * keep operands in registers; it is launched stage by stage.  Within ONE stage the reference's
+ * rule holds (float_ew2.py:685-790: a buffer is one register per kernel): an element written
+ * through one slot must not be read through another slot at a different position.          */
 int  ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec);
 /* Which pre-built kernel family ngh_launch_fused picks for stage `stage`
  * of `spec` (diagnostics and tests): writes a NUL-terminated name.          */

@@ -1350,6 +1350,24 @@ struct ChainPlan {
     int      special = -1;
 };
 
+// Do the byte ranges two operands span in the spec's iteration space intersect?
+static bool tensors_overlap(const ngh_fused_spec& sp, const ngh_tensor& A, const ngh_tensor& B) {
+    auto range = [&](const ngh_tensor& T, unsigned long long& lo, unsigned long long& hi) {
+        long long below = 0, above = 0;
+        for (int a = 0; a < sp.rank; ++a) {
+            const long long reach = (long long)T.strides[a] * (long long)(sp.shape[a] > 0 ? sp.shape[a] - 1 : 0);
+            (reach < 0 ? below : above) += reach;
+        }
+        const long long item = itemsize_of(T.dtype);
+        lo = (unsigned long long)T.dev + (unsigned long long)(below * item);
+        hi = (unsigned long long)T.dev + (unsigned long long)((above + 1) * item);
+    };
+    unsigned long long alo, ahi, blo, bhi;
+    range(A, alo, ahi);
+    range(B, blo, bhi);
+    return alo < bhi && blo < ahi;
+}
+
 // Could the spec run as a row chain (whether or not a compiled chain exists)?
 bool plan_row_chain(const ngh_context* ctx, const ngh_fused_spec& sp, ChainPlan& C) {
     if (sp.flags & NGH_SPEC_PROBE) return false;
@@ -1384,6 +1402,28 @@ bool plan_row_chain(const ngh_context* ctx, const ngh_fused_spec& sp, ChainPlan&
         ++C.n;
     }
     if (C.n < 2 || !any_red) return false;
+    // The chain keeps operands in registers from stage to stage and hands reduction results
+    // over without going through memory: two operand slots over the same memory, one of them
+    // written by a stage, would see each other's writes when the stages are launched one by
+    // one and not inside the chain.  Such a spec runs stage by stage.
+    {
+        bool written[NGH_MAX_TENSORS] = {}, used[NGH_MAX_TENSORS] = {};
+        for (int i = 0; i < C.n; ++i) {
+            bool loads[NGH_MAX_TENSORS], stores[NGH_MAX_TENSORS];
+            const ngh_stage& S = sp.stages[C.stage_of[i]];
+            stage_tensors(sp, S, loads, stores);
+            for (int r = 0; r < S.n_reductions; ++r) stores[S.red_out[r]] = true;
+            for (int t = 0; t < sp.n_tensors; ++t) {
+                written[t] = written[t] || stores[t];
+                used[t] = used[t] || loads[t] || stores[t];
+            }
+        }
+        for (int t = 0; t < sp.n_tensors; ++t) {
+            if (!written[t]) continue;
+            for (int u = 0; u < sp.n_tensors; ++u)
+                if (u != t && used[u] && tensors_overlap(sp, sp.tensors[t], sp.tensors[u])) return false;
+        }
+    }
     C.n_out = (unsigned)n_out;
     C.TR = 1;
     while ((long long)C.TR < chunks && C.TR < 64) C.TR <<= 1;

@@ -200,7 +200,26 @@ def _compile_executor():
             from concurrent.futures import ThreadPoolExecutor
             workers = max(1, min(4, (os.cpu_count() or 2) // 2))
             _executor = ThreadPoolExecutor(max_workers=workers, thread_name_prefix="ngh-jit")
+            _drop_pending_jobs_at_exit(_executor)
         return _executor
+
+
+def _drop_pending_jobs_at_exit(executor):
+    """Interpreter exit joins the workers, and a worker runs every job still queued before it
+    ends: a process that built many graphs would sit through their compilations for nothing.
+    The handler withdraws what has not started (a hipcc run in progress finishes, seconds).
+    It has to run before the thread pool's own exit hook, which `atexit` handlers do not."""
+    def drop():
+        executor.shutdown(wait=False, cancel_futures=True)
+    register = getattr(threading, "_register_atexit", None)
+    if register is not None:
+        try:
+            register(drop)
+            return
+        except RuntimeError:            # the interpreter is already shutting down
+            pass
+    import atexit
+    atexit.register(drop)
 
 
 class BackgroundPrograms(object):

@@ -4,7 +4,8 @@ Test infrastructure: registers a transformer named "cpu" that evaluates an op
 graph one op at a time with the NumPy call
 ngraph/transformers/cputransform.py:512-761 generates for it (table in
 oracle/numpy_ops.py), on float32 buffers (cputransform.py:998-1007), after the
-SimplePrune rewrite the CPU transformer also runs (cputransform.py:905-917).
+SimplePrune rewrite the CPU transformer also runs (cputransform.py:905-917; restated in
+oracle/prune.py).
 It shares the graph front (axes, views, ordering) with the product so the same
 graph can be run on both; what pins that shared front are the NumPy
 expressions written out in the tests themselves, as in the reference's own
@@ -17,10 +18,30 @@ import numpy as np
 from ngraph_hip.op_graph import op_graph as og
 from ngraph_hip.transformers.base import (ComputationGraphTransformer, DeviceBufferStorage,
                                           DeviceTensor)
-from ngraph_hip.transformers.passes.passes import SimplePrune
-from ngraph_hip.transformers.hiptransform import kernel_op_name
-
 from oracle import numpy_ops
+from oracle.prune import OraclePrune
+
+# Graph op class -> name of its NumPy call in oracle/numpy_ops.py, one row per `generate_op`
+# overload of ngraph/transformers/cputransform.py:512-761 (looked up along the op's class
+# hierarchy, so a subclass of a listed op takes its parent's row).
+NUMPY_CALL_OF = {
+    "AbsoluteOp": "abs", "CosOp": "cos", "ExpOp": "exp", "LogOp": "log", "NegativeOp": "neg",
+    "ReciprocalOp": "rcp", "SignOp": "sgn", "SinOp": "sin", "SqrtOp": "sqrt", "SquareOp": "sqr",
+    "TanhOp": "tanh", "SigmoidAtomicOp": "sig",
+    "Add": "add", "Subtract": "sub", "Multiply": "mul", "Divide": "div",
+    "FloorDivide": "int_div", "Mod": "mod", "Power": "pow", "Maximum": "maximum",
+    "Minimum": "minimum", "Equal": "eq", "NotEqual": "ne", "Less": "lt", "LessEqual": "le",
+    "Greater": "gt", "GreaterEqual": "ge",
+    "Sum": "sum", "Prod": "prod", "Max": "max", "Min": "min", "Argmax": "argmax",
+    "Argmin": "argmin",
+}
+
+
+def numpy_call_name(op):
+    for cls in type(op).__mro__:
+        if cls.__name__ in NUMPY_CALL_OF:
+            return NUMPY_CALL_OF[cls.__name__]
+    return None
 
 
 class NumpyDeviceBufferStorage(DeviceBufferStorage):
@@ -69,7 +90,7 @@ class NumpyTransformer(ComputationGraphTransformer):
 
     def __init__(self, **kwargs):
         super(NumpyTransformer, self).__init__(**kwargs)
-        self.graph_passes = [SimplePrune()]
+        self.graph_passes = [OraclePrune()]
 
     def device_buffer_storage(self, bytes, dtype, name):
         return NumpyDeviceBufferStorage(self, bytes, dtype, name="a_" + name)
@@ -105,7 +126,7 @@ class NumpyTransformer(ComputationGraphTransformer):
 
     def _step(self, op):
         view = self._view
-        name = kernel_op_name(op)
+        name = numpy_call_name(op)
         if isinstance(op, og.AssignOp):
             return lambda: view(op.args[0]).__setitem__((), view(op.args[1]))      # :723-725
         if isinstance(op, og.Fill):

@@ -173,11 +173,22 @@ def case_lookup_table():
     return [ng.lookuptable(lut, idx, ng.make_axes([N, F]), update=False) * w + 1.0], [lut, idx, w]
 
 
+def case_row_statistics_chain():
+    # mean and variance of every row feeding a consumer: one moments kernel (one-pass variance)
+    # plus a kernel for the consumer while interpreted, one row chain (sum, then the sum of
+    # squared differences) once compiled -- two ways to the same statistics
+    A, B = ng.make_axis(3000, name="A"), ng.make_axis(1000, name="B")
+    x, g = ng.placeholder([A, B]), ng.placeholder([B])
+    mean, var = ng.mean(x, out_axes=[A]), ng.variance(x, out_axes=[A])
+    return [ng.tanh((x - mean) * ng.reciprocal(ng.sqrt(var + 1e-3))) * g + mean], [x, g]
+
+
 FP32_CASES = [case_elementwise, case_column_reduction_with_store, case_row_reduction_with_store,
               case_transposed_operand, case_transposed_operands_large, case_softmax, case_mixed_storage_types, case_ragged,
               case_ragged_long_rows, case_ragged_many_rows, case_softmax_ragged_rows, case_softmax_long_rows, case_softmax_over_windows,
               case_softmax_forward_and_backward,
-              case_row_chain_with_stored_intermediate, case_misaligned_slices, case_short_rows, case_dropout, case_lookup_table]
+              case_row_chain_with_stored_intermediate, case_misaligned_slices, case_short_rows, case_dropout, case_lookup_table,
+              case_row_statistics_chain]
 
 
 def flex_case():

@@ -33,7 +33,7 @@ def _check(spec, asserts, tmp_path):
 def test_softmax_chain_keeps_the_row_the_results_and_the_exponentials_in_registers(tmp_path):
     # tensors: 0 x, 1 y, 2 row maximum, 3 row sum
     # stage 1: load x, load max, sub, exp, sum        stage 2: load x, load max, sub, exp, load sum, div, store
-    spec = chains._softmax_spec(4096, 8192, 12288, 16384, 1001, 300)
+    spec = chains._softmax_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 1001, 300)
     _check(spec, [
         "Info::n == 3",
         "Info::cache_slot(0) == 0",                          # x: read from memory by the first stage only
@@ -50,7 +50,7 @@ def test_softmax_chain_keeps_the_row_the_results_and_the_exponentials_in_registe
 
 def test_chain_results_that_cannot_stay_in_registers_wait_behind_a_fence(tmp_path):
     # tensors: 0 x, 1 position of the maximum (int32), 2 t (stored by stage 1, loaded by stage 2), 3 y, 4 sum of t*t
-    spec = chains._fenced_chain_spec(4096, 8192, 12288, 16384, 20480, 777, 3000)
+    spec = chains._fenced_chain_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 5 << 30, 777, 3000)
     _check(spec, [
         "Info::n == 3",
         "Info::forwarded(1, 1) < 0 && Info::needs_fence(1)",          # an int32 result is read back from memory
@@ -58,4 +58,26 @@ def test_chain_results_that_cannot_stay_in_registers_wait_behind_a_fence(tmp_pat
         "Info::from_memory(2, 2) && Info::needs_fence(2)",             # so is a tensor another stage stored
         "Info::forwarded(2, 4) >= 0",                                  # the fp32 sum is handed on
         "Info::cache_slot(0) == 0 && Info::last_loader(0) == 1",       # x: kept for the second stage, not needed by the third
+    ], tmp_path)
+
+
+def test_a_stage_that_overwrites_what_an_earlier_stage_read_waits_too(tmp_path):
+    # tensors: 0 x, 1 a per-row factor b (one value per row), 2 the row sum, 3 y
+    # stage 0: sum(x)      stage 1: y = x * b, b read from memory      stage 2: b = sum * 0.5, one store per row
+    R, rows = 5000, 300
+    sb = hiplib.FusedSpecBuilder([R, rows])
+    tx, tb = sb.tensor(1 << 30, [1, R]), sb.tensor(2 << 30, [0, 1])
+    ts, ty = sb.tensor(3 << 30, [0, 1]), sb.tensor(4 << 30, [1, R])
+    sb.reduce("sum", sb.load(tx), ts)
+    sb.end_stage()
+    sb.store(ty, sb.binary("mul", sb.load(tx), sb.load(tb)))
+    sb.end_stage()
+    sb.store(tb, sb.binary("mul", sb.load(ts), sb.constant(0.5)))
+    spec = sb.build()
+    assert hiplib.plan_chain(spec)["eligible"]
+    _check(spec, [
+        "Info::n == 3",
+        "Info::from_memory(1, 1) && !Info::needs_fence(1)",       # b: nobody wrote it before stage 1
+        "Info::stores(2, 1) && Info::needs_fence(2)",              # lanes of other wavefronts may still be reading b
+        "Info::forwarded(2, 2) >= 0",                              # the sum itself arrives in a register
     ], tmp_path)

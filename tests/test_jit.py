@@ -235,8 +235,11 @@ def test_compiled_programs_agree_with_the_interpreter(case):
         if case in (jit_cases.case_softmax, jit_cases.case_softmax_ragged_rows, jit_cases.case_short_rows,
                     jit_cases.case_softmax_long_rows, jit_cases.case_softmax_over_windows,
                     jit_cases.case_softmax_forward_and_backward,
-                    jit_cases.case_row_chain_with_stored_intermediate):
+                    jit_cases.case_row_chain_with_stored_intermediate, jit_cases.case_row_statistics_chain):
             assert any("/chain-of-" in n for n in names), names
+        if case is jit_cases.case_row_statistics_chain:
+            # (the other way to the statistics is what ran before the chain was there)
+            assert any("moments" in n for n in names_interp), names_interp
         if case is jit_cases.case_transposed_operands_large:
             assert any(n.endswith("/tiles64") for n in names), names
 
@@ -344,14 +347,19 @@ def test_which_specs_are_row_chains():
     if not default_kernel_choice():
         pytest.skip("a kernel-choice knob of the library is set")
     ok = lambda spec: hiplib.plan_chain(spec)["eligible"]
-    assert ok(_softmax_spec(4096, 8192, 12288, 16384, 1001, 300))
-    assert hiplib.plan_chain(_softmax_spec(4096, 8192, 12288, 16384, 1001, 300))["lanes_per_row"] == 64
-    assert hiplib.plan_chain(_softmax_spec(4096, 8192, 12288, 16384, 100, 300))["lanes_per_row"] == 32
-    assert hiplib.plan_chain(_softmax_spec(4096, 8192, 12288, 16384, 5000, 300))["lanes_per_row"] == 256
-    assert ok(_softmax_spec(4100, 8192, 12288, 16388, 1000, 300, row_stride=1003))      # any 4-byte-aligned start
-    assert not ok(_softmax_spec(4096, 8192, 12288, 16384, 7, 300))
-    assert not ok(_softmax_spec(4096, 8192, 12288, 16384, 8193, 300))
-    assert not ok(_softmax_spec(4096, 8192, 12288, 16384, 1000, 300, x_dtype=hiplib.NGH_FLEX16))
+    assert ok(_softmax_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 1001, 300))
+    assert hiplib.plan_chain(_softmax_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 1001, 300))["lanes_per_row"] == 64
+    assert hiplib.plan_chain(_softmax_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 100, 300))["lanes_per_row"] == 32
+    assert hiplib.plan_chain(_softmax_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 5000, 300))["lanes_per_row"] == 256
+    assert ok(_softmax_spec((1 << 30) + 4, 2 << 30, 3 << 30, (4 << 30) + 4, 1000, 300, row_stride=1003))      # any 4-byte-aligned start
+    assert not ok(_softmax_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 7, 300))
+    assert not ok(_softmax_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 8193, 300))
+    assert not ok(_softmax_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 1000, 300, x_dtype=hiplib.NGH_FLEX16))
+    # two operand slots over the same memory, one of them written: the stages must see each
+    # other's writes, which the chain's registers would hide
+    assert not ok(_softmax_spec(1 << 30, 2 << 30, 3 << 30, (1 << 30) + 4000, 1001, 300))
+    assert ok(_aliased_chain_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 1001, 300))
+    assert not ok(_aliased_chain_spec(1 << 30, 2 << 30, 3 << 30, 1 << 30, 1001, 300))
     # rows that are strided in memory
     sb = hiplib.FusedSpecBuilder([64, 300])
     tx, tm, ty = sb.tensor(4096, [300, 1]), sb.tensor(8192, [0, 1]), sb.tensor(16384, [300, 1])
@@ -387,10 +395,25 @@ def _fenced_chain_spec(px, pi, pt, py, pn, R, rows):
     return sb.build()
 
 
+def _aliased_chain_spec(px, pm, ps, pz, R, rows):
+    """m = max(x); z = x - m; s = sum(exp(x)) with x read through its own slot in every stage.
+    With z at x's address the third stage must see x - m."""
+    sb = hiplib.FusedSpecBuilder([R, rows])
+    tx, tz = sb.tensor(px, [1, R]), sb.tensor(pz, [1, R])
+    tm, ts = sb.tensor(pm, [0, 1]), sb.tensor(ps, [0, 1])
+    sb.reduce("max", sb.load(tx), tm)
+    sb.end_stage()
+    sb.store(tz, sb.binary("sub", sb.load(tx), sb.load(tm)))
+    sb.end_stage()
+    sb.reduce("sum", sb.unary("exp", sb.load(tx)), ts)
+    return sb.build()
+
+
 def test_row_chain_specs_compile_for_gfx950():
     """(also leaves their program libraries in the cache for the device tests below)"""
-    for spec in (_softmax_spec(4096, 8192, 12288, 16384, 1001, 300),
-                 _fenced_chain_spec(4096, 8192, 12288, 16384, 20480, 777, 3000)):
+    for spec in (_softmax_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 1001, 300),
+                 _fenced_chain_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 5 << 30, 777, 3000),
+                 _aliased_chain_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 500, 2000)):
         programs = jit.uncovered_programs([_SpecHolder(spec)], "chain", min_elements=1, include_covered=True)
         if default_kernel_choice():
             assert len(programs) == 1 and programs[0][8] == 4
@@ -468,6 +491,34 @@ def test_row_chain_with_results_that_go_through_memory(hip_runtime):
     np.testing.assert_allclose(n_d.get(), n_want, rtol=1e-5)
     np.testing.assert_allclose(y_d.get(), t_want / np.sqrt(n_want)[:, None], rtol=1e-5, atol=1e-7)
     for d in (x_d, i_d, t_d, y_d, n_d):
+        d.free()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("R", [500, 5000])
+def test_operand_slots_over_the_same_memory_never_run_as_a_chain(hip_runtime, R):
+    """A spec whose second stage writes, through a slot of its own, the memory its first and
+    third stages read: with the chain's program loaded the unaliased spec runs as one kernel,
+    the aliased one stage by stage, and the third stage sees what the second wrote."""
+    rt = hip_runtime
+    rows = 2000
+    x = np.random.RandomState(R).normal(0, 2, (rows, R)).astype(np.float32)
+    x_d, z_d, m_d, s_d = rt.array(x), rt.empty((rows, R)), rt.empty((rows,)), rt.empty((rows,))
+    apart = _aliased_chain_spec(x_d.ptr, m_d.ptr, s_d.ptr, z_d.ptr, R, rows)
+    jit.ensure_programs(rt, [_SpecHolder(apart)], "aliased_chain", min_elements=1)
+    if default_kernel_choice():
+        assert "/chain-of-3" in rt.describe_fused(apart, 0)
+    rt.launch_fused(apart)
+    m = x.max(axis=1)
+    np.testing.assert_array_equal(z_d.get(), x - m[:, None])
+    np.testing.assert_allclose(s_d.get(), np.exp(x.astype(np.float64)).sum(axis=1), rtol=1e-5)
+    aliased = _aliased_chain_spec(x_d.ptr, m_d.ptr, s_d.ptr, x_d.ptr, R, rows)
+    assert "chain" not in rt.describe_fused(aliased, 0)
+    rt.launch_fused(aliased)
+    shifted = x - m[:, None]
+    np.testing.assert_array_equal(x_d.get(), shifted)
+    np.testing.assert_allclose(s_d.get(), np.exp(shifted.astype(np.float64)).sum(axis=1), rtol=1e-5)
+    for d in (x_d, z_d, m_d, s_d):
         d.free()
 
 

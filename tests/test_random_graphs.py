@@ -9,6 +9,7 @@ import pytest
 import ngraph_hip as ng
 import ngraph_hip.transformers as ngt
 import oracle.cpu_transformer  # noqa: F401
+from oracle import error_bound
 from graph_generators import build, build_views, build_state  # noqa: F401
 
 
@@ -74,6 +75,38 @@ def test_graphs_lower_without_a_device(seed):
     _lower_without_a_device(results, inputs)
 
 
+def arbitrate(gen, seed, rtol=2e-5, atol=2e-5, **device_options):
+    """Device and oracle against float64 with a running error bound (oracle/error_bound.py).
+    Each of the three evaluations builds its own copy of the graph, so no rewrite one backend
+    makes is seen by another.  Both float32 results must lie within tolerance + bound of the
+    float64 value, element by element; an element where the oracle's own order of operations
+    overflowed float32 (a long product passing through inf) binds neither side.  Returns the
+    largest error of each side over the decided elements, for the record."""
+    want = run("cpu", *gen(seed))
+    got = run("hipgpu", *gen(seed), **device_options)
+    results, inputs, values = gen(seed)
+    t = ngt.make_transformer_factory("cpu_bound")()
+    try:
+        exact = [np.array(r) for r in t.computation(results, *inputs)(*values)]
+        bounds = [t.error_bound(r) for r in results]
+    finally:
+        t.close()
+    worst = [0.0, 0.0]
+    for g, w, v, b in zip(got, want, exact, bounds):
+        assert g.shape == w.shape == v.shape
+        overflowed = ~np.isfinite(w)
+        dev_ok = error_bound.within_bound(g, v, b, rtol, atol) | (overflowed & ~np.isfinite(g))
+        ora_ok = error_bound.within_bound(w, v, b, rtol, atol) | overflowed
+        assert ora_ok.all(), "oracle outside its own error bound at %s" % (np.argwhere(~ora_ok)[:3],)
+        assert dev_ok.all(), "device outside the error bound at %s: %s, float64 %s, bound %s" % (
+            np.argwhere(~dev_ok)[:3], g[~dev_ok][:3], v[~dev_ok][:3], b[~dev_ok][:3])
+        decided = np.isfinite(b) & np.isfinite(v) & ~overflowed & np.isfinite(g)
+        if decided.any():
+            worst[0] = max(worst[0], float(np.abs(g - v)[decided].max()))
+            worst[1] = max(worst[1], float(np.abs(w - v)[decided].max()))
+    return worst
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("seed", list(range(1000, 1100)) + [6789])
 def test_random_view_graph_matches_oracle(seed):
@@ -84,6 +117,84 @@ def test_random_view_graph_matches_oracle(seed):
         assert g.shape == w.shape
         ok = np.isfinite(w)
         np.testing.assert_allclose(g[ok], w[ok], rtol=1e-4, atol=1e-4)
+    arbitrate(build_views, seed)
+
+
+# Every seed of 50 000 swept on the device (generator `build` 200-24199, `build_views`
+# 1100-27099) whose result differs from the oracle's by more than rtol = atol = 2e-5 somewhere:
+# products of up to 100 factors, squares of exponentials and differences of nearly equal sums
+# (outputs of magnitude 1e7 to 1e32 whose last bits two float32 evaluations cannot share), and
+# comparisons / argmax positions that a last-bit difference of an operand flips (error "x25000"
+# = 0 against 1).  Arbitrated against float64: both sides are within the forward error bound of
+# the graph on every one, fused and one kernel per op.
+ILL_CONDITIONED_VIEW_SEEDS = [
+    1243, 1506, 1917, 2189, 2359, 2478, 2929, 3628, 3698, 3906, 4300, 4648, 4686, 5858, 6383, 6438,
+    6635, 8192, 8284, 8556, 9651, 9988, 11429, 11635, 12270, 12308, 12328, 12346, 12471, 12882,
+    12976, 13565, 14576, 14667, 14845, 15106, 15436, 15881, 16146, 16191, 16262, 17009, 17158,
+    17413, 17732, 18640, 19354, 19704, 20250, 20381, 20876, 21053, 21108, 21913, 21982, 22196,
+    22444, 22510, 22987, 23155, 23393, 23446, 23506, 23751, 23756, 24024, 24084, 24421, 24509,
+    25156, 25186, 25571, 25644, 26598]
+ILL_CONDITIONED_SEEDS = [19997]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fusion", [True, False], ids=["fused", "unfused"])
+@pytest.mark.parametrize("seed", ILL_CONDITIONED_VIEW_SEEDS)
+def test_ill_conditioned_view_graph_is_within_the_float64_error_bound(seed, fusion):
+    arbitrate(build_views, seed, fusion=fusion)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fusion", [True, False], ids=["fused", "unfused"])
+@pytest.mark.parametrize("seed", ILL_CONDITIONED_SEEDS + list(range(200, 260)))
+def test_graph_is_within_the_float64_error_bound(seed, fusion):
+    arbitrate(build, seed, fusion=fusion)
+
+
+def test_error_bound_is_not_vacuous_on_a_well_conditioned_graph():
+    """tanh(a*x + b) * sigmoid(x): the bound stays at a few dozen ulp of the result."""
+    H = ng.make_axis(512, name="vac_h")
+    x = ng.placeholder([H])
+    y = ng.tanh(x * 0.7 + 0.1) * ng.sigmoid(x)
+    xv = np.linspace(-4, 4, 512).astype(np.float32)
+    t = ngt.make_transformer_factory("cpu_bound")()
+    value = t.computation(y, x)(xv)
+    bound = t.error_bound(y)
+    want = run("cpu", [y], [x], [xv])[0]
+    assert (bound <= 64 * 2.0 ** -24 * np.maximum(np.abs(value), 1e-3)).all()
+    assert error_bound.within_bound(want, value, bound, 0, 0).all()
+
+
+def test_error_bound_sees_cancellation_and_undecided_comparisons():
+    """(x + 1e7) - 1e7 keeps one or two digits of x in float32: the bound must say so, and a
+    comparison of the result with x is undecided wherever the bound reaches the difference."""
+    H = ng.make_axis(64, name="canc_h")
+    x = ng.placeholder([H])
+    y = (x + 1e7) - 1e7
+    c = ng.greater(y, x)
+    xv = np.random.RandomState(5).uniform(1, 2, 64).astype(np.float32)
+    t = ngt.make_transformer_factory("cpu_bound")()
+    value, flag = t.computation([y, c], x)(xv)
+    bound, flag_bound = t.error_bound(y), t.error_bound(c)
+    np.testing.assert_array_equal(value, xv.astype(np.float64))
+    want = run("cpu", [y], [x], [xv])[0]
+    err = np.abs(want - value)
+    assert err.max() > 0.1 and (err <= bound).all() and (bound < 4.0).all()
+    assert np.isinf(flag_bound).all()
+
+
+@pytest.mark.parametrize("seed", range(150))
+def test_oracle_float32_lies_within_the_bound_of_the_float64_evaluation(seed):
+    """Pins the bound evaluator from the CPU side: with no tolerance added, the float32 oracle
+    result is inside the bound around the float64 value for both generators' graphs."""
+    for gen in (build, build_views):
+        want = run("cpu", *gen(seed))
+        results, inputs, values = gen(seed + 0)
+        t = ngt.make_transformer_factory("cpu_bound")()
+        exact = [np.array(r) for r in t.computation(results, *inputs)(*values)]
+        for w, v, r in zip(want, exact, results):
+            ok = error_bound.within_bound(w, v, t.error_bound(r), 0, 0) | ~np.isfinite(w)
+            assert ok.all()
 
 
 def run_state(backend, seed, **kwargs):
