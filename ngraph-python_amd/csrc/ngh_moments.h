@@ -5,7 +5,7 @@
 // (ngraph/op_graph/op_graph.py:4007-4009, 4252-4266), which reads x twice.
 // Here each workgroup accumulates sum(x - p) and sum((x - p)^2) around a pivot p
 // (the row's first element) over one segment of a row, and the last workgroup of the
-// row to finish merges the segments in a fixed order:  mean = p + S1/R,
+// row to finish (or a small second launch) merges the segments in a fixed order:  mean = p + S1/R,
 // var = S2/R - (S1/R)^2.  Optionally it also writes 1/sqrt(var + eps), the factor the
 // normalisation multiplies by (frontends/neon/layer.py:1255), which saves the graph a
 // kernel launch for a few hundred elements.
@@ -33,14 +33,53 @@ __device__ __forceinline__ float4 mom_load(const float4* p) {
     return make_float4(v.x, v.y, v.z, v.w);
 }
 
-// The workgroups of one row take a ticket when their partial sums are written; the one that
-// draws the last ticket merges the row (in segment order, so the result does not depend on
-// which workgroup that was) and resets the row's counter for the next launch.
+// Hand-over of the row's partial sums, `mode`:
+//  2  (the default) every workgroup stores its partial sum and the kernel ends; a second, small
+//     launch (moments_merge_kernel) merges each row.  The kernel boundary orders the two, so
+//     nothing here leans on more than the language's memory model promises.
+//  0, 1  one launch: the workgroups of a row take a ticket when their partial sums are written;
+//     the one that draws the last ticket merges the row and resets the row's counter for the
+//     next launch (0: relaxed atomics ordered by a data dependency, which relies on the
+//     hardware; 1: release tickets and an acquire fence).
+// All three merge in segment order with the same arithmetic (moments_merge_row): the result does
+// not depend on the mode, nor on which workgroup came last.
+__device__ __forceinline__ void moments_merge_row(const float* __restrict__ xr, float pivot, unsigned R, unsigned R4,
+                                                  unsigned n_seg, const float2* __restrict__ row_partial, unsigned lane,
+                                                  unsigned row, float* __restrict__ mean, float* __restrict__ var,
+                                                  float* __restrict__ rstd, float eps) {
+    float t1 = 0.0f, t2 = 0.0f;
+    for (unsigned g = lane; g < n_seg; g += 64) {
+        const unsigned long long p = __hip_atomic_load(
+            reinterpret_cast<const unsigned long long*>(row_partial) + g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        t1 += __uint_as_float((unsigned)p);
+        t2 += __uint_as_float((unsigned)(p >> 32));
+    }
+    // elements past the last whole float4 (R % 4) are added here
+    for (unsigned i = R4 * 4 + lane; i < R; i += 64) {
+        const float a = xr[i] - pivot;
+        t1 += a;
+        t2 += a * a;
+    }
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) {
+        t1 += __shfl_xor(t1, m, 64);
+        t2 += __shfl_xor(t2, m, 64);
+    }
+    if (lane == 0) {
+        const float inv = 1.0f / (float)R;
+        const float d = t1 * inv;
+        const float v = fmaxf(t2 * inv - d * d, 0.0f);
+        mean[row] = pivot + d;
+        var[row] = v;
+        if (rstd) rstd[row] = 1.0f / sqrtf(v + eps);
+    }
+}
+
 template <bool NT>
 __global__ __launch_bounds__(kMomBlock) void moments_kernel(
     const float* __restrict__ x, long long row_stride, unsigned R, unsigned R4, unsigned n_seg,
     unsigned seg_chunks, float2* __restrict__ partial, unsigned* __restrict__ row_tickets,
-    float* __restrict__ mean, float* __restrict__ var, float* __restrict__ rstd, float eps, int ordered) {
+    float* __restrict__ mean, float* __restrict__ var, float* __restrict__ rstd, float eps, int mode) {
     const unsigned row = blockIdx.x / n_seg;
     const unsigned seg = blockIdx.x - row * n_seg;
     const float* xr = x + (long long)row * row_stride;
@@ -85,7 +124,10 @@ __global__ __launch_bounds__(kMomBlock) void moments_kernel(
         for (int w = 1; w < kMomBlock / 64; ++w) { a.x += sh[w].x; a.y += sh[w].y; }
         const unsigned long long bits =
             (unsigned long long)__float_as_uint(a.x) | ((unsigned long long)__float_as_uint(a.y) << 32);
-        if (ordered) {
+        if (mode == 2) {
+            __hip_atomic_store(reinterpret_cast<unsigned long long*>(partial) + blockIdx.x, bits, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        } else if (mode == 1) {
             // By the memory model: the partial is stored, the ticket is a release read-modify-write
             // at device scope, and whoever draws the last ticket issues an acquire fence: it has
             // then acquired every earlier increment's release (a release sequence runs through
@@ -109,37 +151,24 @@ __global__ __launch_bounds__(kMomBlock) void moments_kernel(
             ticket = __hip_atomic_fetch_add(row_tickets + row, one, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
+    if (mode == 2) return;
     __syncthreads();
     if (ticket != n_seg - 1 || threadIdx.x >= 64) return;
     // last workgroup of the row, first wavefront
-    t1 = t2 = 0.0f;
-    for (unsigned g = threadIdx.x; g < n_seg; g += 64) {
-        const unsigned long long p = __hip_atomic_load(
-            reinterpret_cast<unsigned long long*>(partial) + row * n_seg + g, __ATOMIC_RELAXED,
-            __HIP_MEMORY_SCOPE_AGENT);
-        t1 += __uint_as_float((unsigned)p);
-        t2 += __uint_as_float((unsigned)(p >> 32));
-    }
-    // elements past the last whole float4 (R % 4) are added here
-    for (unsigned i = R4 * 4 + threadIdx.x; i < R; i += 64) {
-        const float a = xr[i] - pivot;
-        t1 += a;
-        t2 += a * a;
-    }
-#pragma unroll
-    for (int m = 32; m > 0; m >>= 1) {
-        t1 += __shfl_xor(t1, m, 64);
-        t2 += __shfl_xor(t2, m, 64);
-    }
-    if (threadIdx.x == 0) {
-        const float inv = 1.0f / (float)R;
-        const float d = t1 * inv;
-        const float v = fmaxf(t2 * inv - d * d, 0.0f);
-        mean[row] = pivot + d;
-        var[row] = v;
-        if (rstd) rstd[row] = 1.0f / sqrtf(v + eps);
+    moments_merge_row(xr, pivot, R, R4, n_seg, partial + (size_t)row * n_seg, threadIdx.x, row, mean, var, rstd, eps);
+    if (threadIdx.x == 0)
         __hip_atomic_store(row_tickets + row, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+}
+
+// The second launch of hand-over mode 2: a wavefront per row merges the row's partial sums.
+__global__ __launch_bounds__(kMomBlock) void moments_merge_kernel(
+    const float* __restrict__ x, long long row_stride, unsigned R, unsigned R4, unsigned rows, unsigned n_seg,
+    const float2* __restrict__ partial, float* __restrict__ mean, float* __restrict__ var, float* __restrict__ rstd,
+    float eps) {
+    const unsigned row = blockIdx.x * (kMomBlock / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float* xr = x + (long long)row * row_stride;
+    moments_merge_row(xr, xr[0], R, R4, n_seg, partial + (size_t)row * n_seg, threadIdx.x & 63, row, mean, var, rstd, eps);
 }
 
 // Many short rows (layer normalisation: tens of thousands of rows of a few thousand elements):

@@ -133,9 +133,12 @@ struct ngh_context {
                                      // loads, bit 1 = non-temporal stores in pre-built kernels
     long long   stream_bytes = 192ll << 20;  // hints act on stages touching at least this much memory
     int         moments_wgs_per_cu = 8;
-    int         ordered_arrival = 0; // last-arrival hand-offs: 1 = release tickets + acquire fence (what the memory
-                                     // model asks for; measured 2.6x slower on the moments kernel: a device-scope
-                                     // release per workgroup), 0 = relaxed tickets behind a data dependency
+    int         ordered_arrival = 2; // grid-wide hand-offs.  2 (default): the moments kernel ends after writing its
+                                     // partial sums and a second small launch merges them (ordered by the kernel
+                                     // boundary; +1 us on a 31 us kernel).  One launch with last-arrival tickets:
+                                     // 1 = release tickets + acquire fence (what the memory model asks for;
+                                     // measured 2.6x slower on the moments kernel: a device-scope release per
+                                     // workgroup), 0 = relaxed tickets behind a data dependency (relies on gfx950)
     int         flex_lazy_blocks_per_cu = 6;  // grid of a launch with deferred statistics
     char        name[256] = "";
     uint64_t    total_bytes = 0;
@@ -1115,9 +1118,10 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->cache_policy = env_int("NGH_CACHE_POLICY", -1);
     ctx->stream_bytes = (long long)env_int("NGH_STREAM_MIB", 192) << 20;
     ctx->moments_wgs_per_cu = std::max(1, env_int("NGH_MOMENTS_WGS_PER_CU", 8));
-    ctx->ordered_arrival = env_int("NGH_ORDERED_ARRIVAL", 0);
-    // the relaxed variant leans on what gfx950 does; on anything else only the ordered one runs
-    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) ctx->ordered_arrival = 1;
+    ctx->ordered_arrival = env_int("NGH_ORDERED_ARRIVAL", 2);
+    if (ctx->ordered_arrival < 0 || ctx->ordered_arrival > 2) ctx->ordered_arrival = 2;
+    // the relaxed variant leans on what gfx950 does; on anything else it never runs
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0 && ctx->ordered_arrival == 0) ctx->ordered_arrival = 1;
     hipError_t e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev0);
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev1);
@@ -1598,6 +1602,13 @@ int launch_moments(ngh_context* ctx, const MomentsPlan& m, const float* dev_x, i
                            (unsigned)R, m.R4, m.n_seg, m.seg_chunks, partial, tickets, dev_mean, dev_var, dev_rstd, eps,
                            ctx->ordered_arrival);
     HIP_TRY(hipGetLastError());
+    if (ctx->ordered_arrival == 2) {
+        const unsigned rows_per_wg = kMomBlock / 64;
+        hipLaunchKernelGGL(moments_merge_kernel, dim3((unsigned)((rows + rows_per_wg - 1) / rows_per_wg)),
+                           dim3(kMomBlock), 0, ctx->stream, dev_x, (long long)row_stride, (unsigned)R, m.R4,
+                           (unsigned)rows, m.n_seg, partial, dev_mean, dev_var, dev_rstd, eps);
+        HIP_TRY(hipGetLastError());
+    }
     return NGH_OK;
 }
 }  // namespace
@@ -1610,7 +1621,7 @@ int ngh_moments_f32(ngh_context* ctx, const float* dev_x, int64_t rows, int64_t 
     if (rows == 0) return NGH_OK;
     if (!m.per_wave) {
         NGH_TRY(ensure_ws(ctx, (size_t)rows * m.n_seg * sizeof(float2)));
-        NGH_TRY(ensure_tickets(ctx, (size_t)rows));
+        if (ctx->ordered_arrival != 2) NGH_TRY(ensure_tickets(ctx, (size_t)rows));
     }
     return launch_moments(ctx, m, dev_x, rows, R, row_stride, (float2*)ctx->ws, ctx->tickets, dev_mean, dev_var,
                           dev_rstd, eps, x_cache_hint);
@@ -1635,9 +1646,12 @@ int ngh_moments_f32_noalloc(ngh_context* ctx, const float* dev_x, int64_t rows, 
     // The array keeps what the last call left: the counters of the rows must start at zero (a fill
     // kernel rather than a memset, so that the call can be captured into a graph); the partial
     // sums need no clearing, every one that is read has been written by this launch.
-    const unsigned blocks = (unsigned)((rows + kBlock - 1) / kBlock);
-    hipLaunchKernelGGL(fill_kernel<uint32_t>, dim3(blocks), dim3(kBlock), 0, ctx->stream, tickets, 0u, (size_t)rows);
-    HIP_TRY(hipGetLastError());
+    // (only the one-launch hand-overs count arrivals)
+    if (ctx->ordered_arrival != 2) {
+        const unsigned blocks = (unsigned)((rows + kBlock - 1) / kBlock);
+        hipLaunchKernelGGL(fill_kernel<uint32_t>, dim3(blocks), dim3(kBlock), 0, ctx->stream, tickets, 0u, (size_t)rows);
+        HIP_TRY(hipGetLastError());
+    }
     return launch_moments(ctx, m, dev_x, rows, R, row_stride, partial, tickets, dev_mean, dev_var, dev_rstd, eps,
                           x_cache_hint);
 }
@@ -1922,7 +1936,7 @@ static int try_self_managed_launch(ngh_context* ctx, const ngh_fused_spec* spec,
         NGH_TRY(flex_settle_ids(ctx, dev, slot_id, P.k.n_stat_slots));
         NGH_TRY(ensure_tickets(ctx, (size_t)kFlexTicketWords + kFlexGroupMaxWords));
         P.k.flex_count = count;
-        P.k.ordered_arrival = ctx->ordered_arrival;
+        P.k.ordered_arrival = ctx->ordered_arrival == 1;
         P.k.tickets = ctx->tickets;
         P.k.group_max = (int*)(ctx->tickets + kFlexTicketWords);
     }

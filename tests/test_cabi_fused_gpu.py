@@ -670,17 +670,21 @@ def test_moments_of_rows_off_16_byte_boundaries(hip_runtime, rows, R, stride, fi
 
 
 def test_moments_hand_off_with_and_without_release_acquire_tickets(monkeypatch):
-    """The last workgroup of a row merges the row's segments.  By default the hand-off is a
-    relaxed ticket ordered behind the partial sums by a data dependency (what gfx950 honours);
-    NGH_ORDERED_ARRIVAL=1 selects release tickets and an acquire fence in the merger (what the
-    memory model asks for, at 2.6 times the kernel's duration).  Same sums in the same order:
-    identical results."""
+    """A row's segments are merged in segment order.  By default the moments kernel ends after
+    writing its partial sums and a second small launch merges them (the kernel boundary is the
+    hand-off).  NGH_ORDERED_ARRIVAL=0 / 1 merge inside the one launch, in the last workgroup of
+    the row to finish: 0 hands over with a relaxed ticket ordered behind the partial sums by a
+    data dependency (what gfx950 honours), 1 with release tickets and an acquire fence in the
+    merger (what the memory model asks of one launch, at 2.6 times the kernel's duration).  Same
+    sums in the same order: identical results."""
     from ngraph_hip.runtime.hiplib import HipRuntime
     rs = np.random.RandomState(21)
     x = rs.normal(3.0, 2.0, (300, 50000)).astype(f32)
     seen = []
-    for ordered in ("0", "1"):
-        monkeypatch.setenv("NGH_ORDERED_ARRIVAL", ordered)
+    for ordered in (None, "2", "0", "1"):
+        monkeypatch.delenv("NGH_ORDERED_ARRIVAL", raising=False)
+        if ordered is not None:
+            monkeypatch.setenv("NGH_ORDERED_ARRIVAL", ordered)
         rt = HipRuntime(0)
         try:
             x_d, out_d = rt.array(x), rt.empty((3, 300))

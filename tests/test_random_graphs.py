@@ -102,8 +102,8 @@ def arbitrate(gen, seed, rtol=2e-5, atol=2e-5, **device_options):
             np.argwhere(~dev_ok)[:3], g[~dev_ok][:3], v[~dev_ok][:3], b[~dev_ok][:3])
         decided = np.isfinite(b) & np.isfinite(v) & ~overflowed & np.isfinite(g)
         if decided.any():
-            worst[0] = max(worst[0], float(np.abs(g - v)[decided].max()))
-            worst[1] = max(worst[1], float(np.abs(w - v)[decided].max()))
+            worst[0] = max(worst[0], float(np.abs(g[decided] - v[decided]).max()))
+            worst[1] = max(worst[1], float(np.abs(w[decided] - v[decided]).max()))
     return worst
 
 
