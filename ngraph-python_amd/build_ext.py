@@ -37,7 +37,7 @@ def build_all(verbose=True):
     """Compile every HIP source into libngraph_hip.so; returns its path."""
     if not os.path.isdir(LIB_DIR):
         os.makedirs(LIB_DIR)
-    cmd = [find_hipcc()] + HIPCC_FLAGS + [
+    cmd = [find_hipcc()] + HIPCC_FLAGS + os.environ.get("NGH_EXTRA_HIPCC_FLAGS", "").split() + [
         "-I", INCLUDE, "-I", CSRC,
         os.path.join(CSRC, "ngraph_hip.hip"),
         "-o", LIB_PATH + ".tmp",

@@ -221,8 +221,17 @@ __device__ __forceinline__ int probe_bits(float v) {
 // ---------------------------------------------------------------------------
 // Element access by storage type.
 // ---------------------------------------------------------------------------
+// A word that is always there to be read.  A kernel's prologue fetches the scales of its flex
+// operands through pointers that may be NULL; "load if not NULL" is a branch, and a branch per
+// operand makes the fetches a chain of round trips, one after the other, ahead of the kernel's
+// first load of data.  Loading from this word instead of from NULL keeps them unconditional
+// and in flight together.
+static __device__ float ngh_safe_word = 1.0f;
+
 __device__ __forceinline__ float tensor_scale(const KTensor& t) {
-    return t.dscale ? *t.dscale : t.scale;
+    const float* p = t.dscale ? t.dscale : &ngh_safe_word;
+    const float v = *p;
+    return t.dscale ? v : t.scale;
 }
 
 __device__ __forceinline__ float load1(const KTensor& t, long long off, float scale) {

@@ -41,6 +41,9 @@ __device__ __forceinline__ int flex_fit_dec(double v) {
 
 __device__ __forceinline__ float flex_scale_of(int dec) { return ldexpf(1.0f, -dec); }
 
+// stand-in record for unconditional prologue loads (see ngh_safe_word)
+static __device__ ngh_flex_state ngh_safe_state = {};
+
 // The exponent a kernel writes a tensor with: the policy's choice once the tensor has been
 // written before, unless the kernel also reads it (an in-place update keeps its scale).
 __device__ __forceinline__ int flex_write_dec(const ngh_flex_state& s, int in_place) {
