@@ -2,8 +2,8 @@
 
 * The reference's flex known-answer vectors (tests/golden/flex_vectors.json) run through
   the `flexhip` transformer with fusion off, i.e. one kernel and one rounding per op as the
-  reference executes them, with the reference's own templates and tolerances
-  (ngraph/testing/flex_util.py:114-155).
+  reference executes them, under the reference's acceptance rule (exact for one step, the
+  flex tolerance for a sequence: tests/flex_known_answers.py).
 * The fused relu(x*w+b) kernel over 8 iterations against the NumPy flex model: mantissas,
   exponents and max|mantissa| bit-exact every iteration.
 """
@@ -18,8 +18,7 @@ import ngraph_hip as ng
 import ngraph_hip.transformers as ngt
 from ngraph_hip.frontends import neon
 from ngraph_hip.testing import executor
-from ngraph_hip.testing.flex_util import (template_one_placeholder, template_two_placeholders,
-                                          execute_calculation)
+from flex_known_answers import run_vector, check_steps
 from oracle import flex_model as fm
 from oracle import configs
 
@@ -62,11 +61,9 @@ def test_reference_flex_vector(flex_unfused, case):
         v, p = ng.variable(()), ng.placeholder(())
         vset = ng.sequential([ng.assign(v, p), v])
         with executor(vset, p) as ex:
-            execute_calculation(operands, operands[0][0], ex)
-    elif len(operands[0]) == 2:
-        template_one_placeholder(operands, NG_OPS[op])
+            check_steps(ex, operands)
     else:
-        template_two_placeholders(operands, NG_OPS[op])
+        run_vector(NG_OPS[op], operands)
 
 
 def _c5_graph(t, n):
