@@ -284,12 +284,41 @@ def bench_c2(ng, ngt, neon, workloads, args, want_cold, copy_calibration=0):
     assert np.abs(y.mean(axis=1) - b64).max() < 1e-4, "normalised output: per-channel mean is not beta"
     assert np.abs(y.var(axis=1) - g64 * g64 * var / (var + 1e-5)).max() < 1e-3, \
         "normalised output: per-channel variance is not gamma^2 var / (var + eps)"
+    boundary = call_boundary(t, f, x, x_np.reshape(dims))
     t.close()
     workload = ("C2 batch-norm forward: x fp32 [256,56,56,64] ~N(0.5,2), gamma, beta ~U(0.5,1.5), statistics over "
                 "H,W,N then normalise; algorithmic bytes 616562688 per step")
     blk = config_block("C2", workload, step_ms, nbytes, n_elems, warm, cold, cold_ms, n_elems, overhead=overhead,
                        dirty_ms=dirty_ms)
+    blk["call_boundary"] = boundary
     return blk, x_np, gamma_np, beta_np
+
+
+def call_boundary(t, f, x, x_host, repeats=5):
+    """What a caller of Computation.__call__ sees, with NumPy arrays in pageable host memory on
+    both sides (never `value`, which has its inputs resident): the whole call, and its two
+    transfers alone -- x written through its device tensor, y read back into a fresh array."""
+    x_view = t.get_op_tensor_view(x)
+    y_view = t.get_op_tensor_view(f.computation_op.values[0])
+    n = x_host.nbytes
+    call, put, get = [], [], []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        f(x_host)
+        call.append(time.perf_counter() - t0)
+        t0 = time.perf_counter()
+        x_view[...] = x_host
+        put.append(time.perf_counter() - t0)
+        t0 = time.perf_counter()
+        y = y_view.get(None)
+        get.append(time.perf_counter() - t0)
+        del y
+    med = lambda v: float(np.median(v))
+    return {"call_ms": round(med(call) * 1e3, 3), "host_to_device_ms": round(med(put) * 1e3, 3),
+            "host_to_device_GB/s": round(n / med(put) / 1e9, 1), "device_to_host_ms": round(med(get) * 1e3, 3),
+            "device_to_host_GB/s": round(n / med(get) / 1e9, 1), "bytes_each_way": n,
+            "what": "Computation.__call__ with x and y as NumPy arrays in pageable memory: x in, the step, y and "
+                    "the statistics out; large copies go through the context's pinned staging buffers"}
 
 
 def bench_c3(ng, ngt, neon, workloads, args, want_cold):

@@ -218,6 +218,16 @@ int  ngh_free(ngh_context* ctx, void* dev);
 int  ngh_memcpy_h2d(ngh_context* ctx, void* dev, const void* host, size_t bytes);
 int  ngh_memcpy_d2h(ngh_context* ctx, void* host, const void* dev, size_t bytes);
 int  ngh_memcpy_d2d(ngh_context* ctx, void* dev_dst, const void* dev_src, size_t bytes);
+/* The two host copies above block until the data has arrived, like GPUArray.set / .get.  From
+ * 4 MiB on they go through pinned staging buffers owned by the context (4 x 16 MiB from
+ * hipHostMalloc, allocated at the first such copy) with NGH_COPY_THREADS host threads (default
+ * 8; 0 leaves the staging to the runtime) moving the data between the caller's pageable array
+ * and the buffers while the copy engine works on the slot before.                            */
+/* Device scratch of at least `bytes`, owned by the context and reused from call to call: the
+ * contiguous intermediate of strided host reads and writes, which the reference allocates and
+ * frees per access (gputransform.py:873-909 through copy_transpose).  Valid until the next call
+ * that asks for more; the stream is drained before it is replaced.                           */
+int  ngh_io_scratch(ngh_context* ctx, size_t bytes, void** out_dev);
 int  ngh_memset32(ngh_context* ctx, void* dev, uint32_t value, size_t count);
 int  ngh_memset16(ngh_context* ctx, void* dev, uint16_t value, size_t count);
 

@@ -20,6 +20,7 @@
 #include "ngh_moments.h"
 #include "ngh_flex.h"
 #include "ngh_convert.h"
+#include "ngh_hostio.h"
 
 using namespace ngh;
 
@@ -110,6 +111,12 @@ struct ngh_context {
     void*       noalloc_scratch = nullptr;   // this device's copy of `scratch`
     hipStream_t stream = nullptr;
     hipEvent_t  ev0 = nullptr, ev1 = nullptr;
+    ngh::HostStaging staging;        // pinned ring + copy threads for large host <-> device copies
+    int         copy_threads = 8;    // 0: leave large copies to the runtime's own staging
+    size_t      staging_slot_bytes = 16u << 20;
+    size_t      staged_min_bytes = 4u << 20;   // smaller copies are not worth the threads
+    void*       io_tmp = nullptr;    // device scratch for strided host I/O (ngh_io_scratch)
+    size_t      io_tmp_bytes = 0;
     void*       ws = nullptr;        // partial results of split reductions
     size_t      ws_bytes = 0;
     unsigned*   tickets = nullptr;   // zero between launches: per-row / per-launch arrival counters
@@ -1118,6 +1125,8 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->cache_policy = env_int("NGH_CACHE_POLICY", -1);
     ctx->stream_bytes = (long long)env_int("NGH_STREAM_MIB", 192) << 20;
     ctx->moments_wgs_per_cu = std::max(1, env_int("NGH_MOMENTS_WGS_PER_CU", 8));
+    ctx->copy_threads = std::max(0, std::min(64, env_int("NGH_COPY_THREADS", 8)));
+    ctx->staging_slot_bytes = (size_t)std::max(1, env_int("NGH_STAGING_SLOT_MIB", 16)) << 20;
     ctx->ordered_arrival = env_int("NGH_ORDERED_ARRIVAL", 2);
     if (ctx->ordered_arrival < 0 || ctx->ordered_arrival > 2) ctx->ordered_arrival = 2;
     // the relaxed variant leans on what gfx950 does; on anything else it never runs
@@ -1152,6 +1161,8 @@ int ngh_shutdown(ngh_context* ctx) {
     if (!ctx) return NGH_OK;
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    ctx->staging.release();
+    if (ctx->io_tmp) (void)hipFree(ctx->io_tmp);
     if (ctx->ws) (void)hipFree(ctx->ws);
     if (ctx->stat_ws) (void)hipFree(ctx->stat_ws);
     if (ctx->tickets) (void)hipFree(ctx->tickets);
@@ -1205,9 +1216,25 @@ int ngh_free(ngh_context* ctx, void* dev) {
     return NGH_OK;
 }
 
+// Large copies go through the context's pinned ring (ngh_hostio.h); small ones, and all of them
+// with NGH_COPY_THREADS=0, are left to the runtime.
+static bool staged(ngh_context* ctx, size_t bytes) {
+    if (ctx->copy_threads <= 0 || bytes < ctx->staged_min_bytes) return false;
+    if (ctx->staging.ensure(ctx->staging_slot_bytes, ctx->copy_threads) != hipSuccess) {
+        (void)hipGetLastError();
+        ctx->copy_threads = 0;          // no pinned memory to be had: never try again
+        return false;
+    }
+    return true;
+}
+
 int ngh_memcpy_h2d(ngh_context* ctx, void* dev, const void* host, size_t bytes) {
     if (!ctx || (bytes && (!dev || !host))) return fail(NGH_E_INVALID, "ngh_memcpy_h2d: NULL argument");
     if (!bytes) return NGH_OK;
+    if (staged(ctx, bytes)) {
+        HIP_TRY(ctx->staging.to_device(dev, host, bytes, ctx->stream));
+        return NGH_OK;
+    }
     HIP_TRY(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, ctx->stream));
     HIP_TRY(hipStreamSynchronize(ctx->stream));
     return NGH_OK;
@@ -1216,8 +1243,28 @@ int ngh_memcpy_h2d(ngh_context* ctx, void* dev, const void* host, size_t bytes) 
 int ngh_memcpy_d2h(ngh_context* ctx, void* host, const void* dev, size_t bytes) {
     if (!ctx || (bytes && (!dev || !host))) return fail(NGH_E_INVALID, "ngh_memcpy_d2h: NULL argument");
     if (!bytes) return NGH_OK;
+    if (staged(ctx, bytes)) {
+        HIP_TRY(ctx->staging.to_host(host, dev, bytes, ctx->stream));
+        return NGH_OK;
+    }
     HIP_TRY(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
     HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return NGH_OK;
+}
+
+int ngh_io_scratch(ngh_context* ctx, size_t bytes, void** out_dev) {
+    if (!ctx || !out_dev) return fail(NGH_E_INVALID, "ngh_io_scratch: NULL argument");
+    if (bytes > ctx->io_tmp_bytes) {
+        HIP_TRY(hipSetDevice(ctx->device));
+        HIP_TRY(hipStreamSynchronize(ctx->stream));      // nothing may still be using the old one
+        if (ctx->io_tmp) (void)hipFree(ctx->io_tmp);
+        ctx->io_tmp = nullptr;
+        ctx->io_tmp_bytes = 0;
+        const size_t want = std::max<size_t>(bytes + bytes / 4, 1u << 20);
+        HIP_TRY(hipMalloc(&ctx->io_tmp, want));
+        ctx->io_tmp_bytes = want;
+    }
+    *out_dev = ctx->io_tmp;
     return NGH_OK;
 }
 

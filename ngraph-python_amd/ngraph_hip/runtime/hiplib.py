@@ -102,6 +102,7 @@ _SYMBOLS = {
     "ngh_memcpy_h2d": [_vp, _vp, _vp, ctypes.c_size_t],
     "ngh_memcpy_d2h": [_vp, _vp, _vp, ctypes.c_size_t],
     "ngh_memcpy_d2d": [_vp, _vp, _vp, ctypes.c_size_t],
+    "ngh_io_scratch": [_vp, ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p)],
     "ngh_memset32": [_vp, _vp, ctypes.c_uint32, ctypes.c_size_t],
     "ngh_memset16": [_vp, _vp, ctypes.c_uint16, ctypes.c_size_t],
     "ngh_copy_strided": [_vp, _vp, _vp, _i32, _i64p, _i64p, _i64p, _i32],
@@ -281,6 +282,12 @@ class HipRuntime(object):
     def memcpy_d2d(self, dst, src, nbytes):
         _check(self.lib, self.lib.ngh_memcpy_d2d(self.ctx, ctypes.c_void_p(dst), ctypes.c_void_p(src), int(nbytes)))
 
+    def io_scratch(self, nbytes):
+        """Context-owned device scratch of at least nbytes (valid until the next, larger request)."""
+        ptr = ctypes.c_void_p()
+        _check(self.lib, self.lib.ngh_io_scratch(self.ctx, int(nbytes), ctypes.byref(ptr)))
+        return ptr.value
+
     def memset32(self, dev, value, count):
         _check(self.lib, self.lib.ngh_memset32(self.ctx, ctypes.c_void_p(dev), int(value) & 0xffffffff, int(count)))
 
@@ -450,6 +457,9 @@ class DryRunRuntime(object):
 
     def memcpy_d2h(self, host, dev):
         raise HipLibraryError(-5, "dry-run runtime holds no data")
+
+    def io_scratch(self, nbytes):
+        return self.malloc(nbytes)
 
     def copy_strided(self, *args):
         pass

@@ -211,34 +211,41 @@ class HipDeviceTensor(DeviceTensor):
         if td.c_contiguous:
             rt.memcpy_d2h(out, self.ptr)
             return out
-        # strided or broadcast view: gather on the device, then one contiguous copy out
-        tmp = rt.malloc(out.nbytes)
-        try:
-            contiguous = [int(s) // out.itemsize for s in out.strides]
-            rt.copy_strided(tmp, self.ptr, td.shape, contiguous, td.full_strides, out.itemsize)
-            rt.memcpy_d2h(out, tmp)
-        finally:
-            rt.free(tmp)
+        # strided or broadcast view: gather on the device (into the context's scratch), then one
+        # contiguous copy out
+        tmp = rt.io_scratch(out.nbytes)
+        contiguous = [int(s) // out.itemsize for s in out.strides]
+        rt.copy_strided(tmp, self.ptr, td.shape, contiguous, td.full_strides, out.itemsize)
+        rt.memcpy_d2h(out, tmp)
         return out
 
-    def _write_raw(self, host):
-        td, rt = self.view, self.transformer.runtime
-        host = np.ascontiguousarray(np.broadcast_to(host, td.shape), dtype=self.np_dtype)
+    def _write_window(self, host, offset, shape, strides):
+        """host (broadcast to `shape`) into the window of the buffer that starts `offset` elements
+        into this view and has the given element strides."""
+        rt = self.transformer.runtime
+        host = np.ascontiguousarray(np.broadcast_to(host, shape), dtype=self.np_dtype)
         if host.size == 0:
             return
-        if td.c_contiguous:
-            rt.memcpy_h2d(self.ptr, host)
+        ptr = self.ptr + offset * self.itemsize
+        dense, run = True, 1
+        for n, s in zip(reversed(shape), reversed(strides)):
+            dense = dense and (n == 1 or s == run)
+            run *= n
+        if dense:
+            rt.memcpy_h2d(ptr, host)
             return
-        if any(s == 0 and n > 1 for s, n in zip(td.full_strides, td.shape)):
+        if any(s == 0 and n > 1 for s, n in zip(strides, shape)):
             raise ValueError("cannot write through a broadcast view")
-        tmp = rt.malloc(host.nbytes)
-        try:
-            rt.memcpy_h2d(tmp, host)
-            contiguous = [int(s) // host.itemsize for s in host.strides]
-            rt.copy_strided(self.ptr, tmp, td.shape, td.full_strides, contiguous, host.itemsize)
-            rt.sync()
-        finally:
-            rt.free(tmp)
+        # one contiguous copy in (the host copy returns when the data has arrived), then a
+        # scatter on the device, which later kernels on the stream are ordered behind
+        tmp = rt.io_scratch(host.nbytes)
+        rt.memcpy_h2d(tmp, host)
+        contiguous = [int(s) // host.itemsize for s in host.strides]
+        rt.copy_strided(ptr, tmp, shape, strides, contiguous, host.itemsize)
+
+    def _write_raw(self, host):
+        td = self.view
+        self._write_window(host, 0, td.shape, td.full_strides)
 
     def get(self, tensor):
         value = self._read_raw()
@@ -250,14 +257,49 @@ class HipDeviceTensor(DeviceTensor):
     def __getitem__(self, key):
         return self.get(None)[key]
 
+    def _window_of(self, key):
+        """(offset, shape, strides) in elements of view[key] for a key made of integers and
+        slices (what NumPy calls basic indexing); None for anything else."""
+        td = self.view
+        key = key if isinstance(key, tuple) else (key,)
+        if any(k is Ellipsis for k in key):
+            i = [k is Ellipsis for k in key].index(True)
+            if any(k is Ellipsis for k in key[i + 1:]):
+                return None
+            key = key[:i] + (slice(None),) * (len(td.shape) - (len(key) - 1)) + key[i + 1:]
+        if len(key) > len(td.shape):
+            return None
+        key = key + (slice(None),) * (len(td.shape) - len(key))
+        offset, shape, strides = 0, [], []
+        for k, n, s in zip(key, td.shape, td.full_strides):
+            if isinstance(k, (int, np.integer)):
+                k = int(k)
+                if not -n <= k < n:
+                    raise IndexError("index %d is out of bounds for an axis of length %d" % (k, n))
+                offset += (k % n) * s
+            elif isinstance(k, slice):
+                lo, hi, step = k.indices(n)
+                count = len(range(lo, hi, step))
+                offset += lo * s if count else 0
+                shape.append(count)
+                strides.append(s * step)
+            else:
+                return None
+        return offset, shape, strides
+
     def __setitem__(self, key, value):
         value = np.asarray(value)
-        if key is Ellipsis or key == () or key == slice(None, None, None):
+        if key is Ellipsis or key == () or (isinstance(key, slice) and key == slice(None, None, None)):
             self._write_raw(value.astype(self.np_dtype, copy=False))
-        else:
-            whole = self._read_raw()
-            whole[key] = value
-            self._write_raw(whole)
+            return
+        window = self._window_of(key)
+        if window is not None and all(s >= 0 for s in window[2]):
+            # only the addressed window travels: a contiguous copy in and a strided copy on the device
+            self._write_window(value.astype(self.np_dtype, copy=False), *window)
+            return
+        whole = self._read_raw()
+        whole[key] = value
+        self._write_raw(whole)
 
 
 # =============================================================================== kernels

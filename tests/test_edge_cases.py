@@ -271,6 +271,67 @@ def test_strided_host_io_through_views():
 
 
 @gpu
+@pytest.mark.parametrize("nbytes", [1, 4093, (4 << 20) - 4, 4 << 20, (16 << 20) + 1, (65 << 20) + 7, 136 << 20])
+def test_host_copies_of_every_size_arrive_intact(hip_runtime, nbytes):
+    """Copies below 4 MiB are left to the runtime; from there on they travel through the
+    context's ring of four 16 MiB pinned buffers, filled and drained by host threads: sizes
+    around the threshold, around a slot, ragged tails, and more chunks than the ring has
+    slots, into a destination array whose pages have never been touched."""
+    rt = hip_runtime
+    src = np.random.RandomState(nbytes % 1000).randint(0, 256, nbytes).astype(np.uint8)
+    dev = rt.malloc(nbytes)
+    try:
+        rt.memcpy_h2d(dev, src)
+        back = np.empty(nbytes, dtype=np.uint8)
+        rt.memcpy_d2h(back, dev)
+        np.testing.assert_array_equal(back, src)
+        # a second round through the same slots, other data, offset source and destination
+        src2 = (src[::-1].copy() ^ 0x5a)[1:]
+        rt.memcpy_h2d(dev + 1, src2) if nbytes > 1 else None
+        back2 = np.empty(nbytes, dtype=np.uint8)
+        rt.memcpy_d2h(back2, dev)
+        assert back2[0] == src[0]
+        np.testing.assert_array_equal(back2[1:], src2)
+    finally:
+        rt.free(dev)
+
+
+@gpu
+def test_keyed_host_writes_move_only_the_addressed_window():
+    """tensor[key] = value for keys of integers and slices is a copy of the window alone (a
+    contiguous copy in, a strided copy on the device); every other key reads the tensor back,
+    patches it and writes it again.  Both must give what NumPy gives (gputransform.py:807-871)."""
+    t = ngt.make_transformer_factory("hipgpu")()
+    try:
+        A, B, C = ng.make_axis(6, name="A"), ng.make_axis(10, name="B"), ng.make_axis(7, name="C")
+        x = ng.placeholder([A, B, C])
+        f = t.computation(x * 1.0, x)
+        rs = np.random.RandomState(3)
+        want = rs.uniform(-1, 1, (6, 10, 7)).astype(f32)
+        f(want)
+        view = t.get_op_tensor_view(x)
+        keys = [(slice(1, 4),), (2,), (-1, slice(None), 3), (slice(None), slice(2, 9, 3)), (Ellipsis, 5),
+                (slice(0, 6, 2), Ellipsis, slice(1, 7, 2)), (1, 2, 3), (slice(4, 2),),
+                (slice(None), [0, 3, 9]), (want[:, 0, 0] > 0,), (slice(5, None, -1),)]
+        reads_before = []
+        for i, key in enumerate(keys):
+            value = rs.uniform(-1, 1, want[key].shape).astype(f32) if i % 2 else f32(i + 0.5)
+            want[key] = value
+            view[key] = value
+            np.testing.assert_array_equal(view.get(None), want, err_msg=str(key))
+        assert view._window_of((slice(None), [0, 3, 9])) is None            # fancy keys take the long way
+        assert view._window_of((slice(1, 4),)) == (70, [3, 10, 7], [70, 7, 1])
+        # through a transposed view of the same buffer
+        xt = t.get_tensor_description_tensor_view(ng.axes_with_order(x, [C, A, B]).tensor_description())
+        patch = rs.uniform(-1, 1, (2, 6, 4)).astype(f32)
+        xt[1:3, :, 2:6] = patch
+        want.transpose(2, 0, 1)[1:3, :, 2:6] = patch
+        np.testing.assert_array_equal(view.get(None), want)
+    finally:
+        t.close()
+
+
+@gpu
 def test_library_rejects_bad_launches(hip_runtime):
     rt = hip_runtime
     x_d = rt.array(np.zeros(16, f32))
