@@ -555,6 +555,16 @@ def shape_survey_cases(ng):
         # kernels it is read three times)
         yield ("softmax of rows [%d,%d] (maximum, sum of exponentials, normalise)" % (rows, k),
                [e / ng.sum(e, out_axes=[R])], [w], {"chain": 2 * rows * k * 4, "kernels": 4 * rows * k * 4})
+    # classes x samples, the layout of the neon front end (op_graph.py:3849): the reduced axis is the
+    # strided one; as one column-chain kernel the operand is read once (few classes: kept in
+    # registers) or re-read from the caches by the later stages
+    for classes, samples in ((1000, 32768), (10, 4194304), (100, 327680)):
+        K, S = ax(classes, "KC%d" % classes), ax(samples, "SC%d" % classes)
+        w = ng.placeholder([K, S])
+        e = ng.exp(w - ng.max(w, out_axes=[S]))
+        yield ("softmax over classes [%d,%d] (classes x samples: the reduced axis strided)" % (classes, samples),
+               [e / ng.sum(e, out_axes=[S])], [w],
+               {"chain": 2 * classes * samples * 4, "kernels": 4 * classes * samples * 4})
     O1, O2 = ax(8191, "O1"), ax(8191, "O2")
     o, o2 = ng.placeholder([O1, O2]), ng.placeholder([O1, O2])
     odd = 8191 * 8191 * 4
@@ -563,12 +573,14 @@ def shape_survey_cases(ng):
     yield "sum across the contiguous axis [8191,8191]", [ng.sum(o, out_axes=[O2])], [o], odd
 
 
-def shape_survey(ng, ngt, steps, warmup):
+def shape_survey(ng, ngt, steps, warmup, only=""):
     """The graphs of shape_survey_cases with the transformer's default kernel choice (programs
     compiled at run time loaded before timing): ms per step, algorithmic GB/s, and each
     kernel's duration from HIP events."""
     out = {}
     for name, results, inputs, nbytes in shape_survey_cases(ng):
+        if only and only not in name:
+            continue
         t = ngt.make_transformer_factory("hipgpu")()
         try:
             f = t.computation(results, *inputs)
@@ -584,10 +596,10 @@ def shape_survey(ng, ngt, steps, warmup):
             kernels = [("+".join(sorted(set(d for ds in k.describe() for d in ds))), round(float(np.median(times)) * 1e3, 1))
                        for k, times in group.profile(repeats=3, inner=10)]
             if isinstance(nbytes, dict):
-                chained = any("/chain-of-" in d for d, _ in kernels)
+                chained = any("chain-of-" in d for d, _ in kernels)
                 passes = nbytes["kernels"] // (nbytes["chain"] // 2)
                 nbytes = nbytes["chain" if chained else "kernels"]
-                name += " (one row-chain kernel; 2 passes)" if chained else \
+                name += " (one chain kernel; 2 passes)" if chained else \
                     " (%d kernels; %d passes)" % (len(kernels), passes)
             out[name] = {"ms_per_step": round(ms, 5), "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
                          "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
@@ -665,6 +677,7 @@ def main():
     ap.add_argument("--compiled", action="store_true",
                     help="also time five user graphs: default kernel choice, interpreter only, compiled "
                          "(needs hipcc unless the program cache already holds them)")
+    ap.add_argument("--only", default="", help="with --shapes: only the cases whose name contains this text")
     ap.add_argument("--shapes", action="store_true",
                     help="also time a survey of everyday layouts and extents (broadcasts, transposed operands, "
                          "reductions over one and several axes, many short rows, odd extents)")
@@ -709,7 +722,7 @@ def main():
         out["configs"]["C5"] = bench_c5(ng, ngt, neon, workloads, args, not args.no_cold)
     out["configs"].update(small_configs(ng, ngt, neon, workloads, max(5, args.steps // 4), 2))
     if args.shapes:
-        out["shapes"] = shape_survey(ng, ngt, max(20, args.steps // 4), 2)
+        out["shapes"] = shape_survey(ng, ngt, max(20, args.steps // 4), 2, args.only)
     if args.compiled:
         out["compiled_at_run_time"] = compiled_vs_interpreted(ng, ngt, max(20, args.steps // 4), 2)
     if not args.no_cpu:

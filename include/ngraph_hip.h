@@ -315,8 +315,11 @@ int  ngh_plan_fused(const ngh_fused_spec* spec, int32_t stage, int32_t* out8);
  * reaching the next stage without a trip through a second launch (float_ew2.py:1135-1483,
  * stage loop :1268-1321)?  Possible for a "row chain": rows (spec axis 0, the reduced one) of up
  * to 8192 elements, fp32 operands with unit stride along the row or broadcast along it, at
- * least one reduction stage.  out4 = {1 if the spec qualifies, index of the compiled chain
- * program or -1 (without one the stages are launched one by one), lanes per row, stages}.
+ * least one reduction stage; and for a "column chain": the reduced axis (spec axis 0) strided,
+ * every operand contiguous along spec axis 2 in whole aligned groups of 4 floats (or broadcast
+ * along it), fp32, any number of rows.  out4 = {1 for a row chain, 2 for a column chain, 0 for
+ * neither; index of the compiled chain program or -1 (without one the stages are launched one
+ * by one); lanes per row / column chunks per workgroup; stages}.
  * A stage of a row chain may also STORE one value per row: a value that does not vary along
  * axis 0 (computed from operands with stride 0 there, such as earlier stages' results) into a
  * tensor with stride 0 on axis 0; ngh_launch_fused refuses such a spec (NGH_E_UNSUPPORTED)

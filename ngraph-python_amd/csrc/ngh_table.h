@@ -85,13 +85,18 @@ inline int match_special(int family, int V, const KArgs& k, long long /*tail*/) 
 // A chain (family 4) whose stages are the programs of `ks` (argument blocks of the spec's stages
 // in row order: kernel axis 2 = the reduced axis; families[i] = 1 for a stage with reductions,
 // 0 for an elementwise one), or -1.
-inline int match_chain(const KArgs* ks, const int* families, int n) {
+// `family` 5: a column chain (argument blocks in the spec's own axis order: kernel axis 0 = the
+// reduced, strided axis; families[i] = 2 for a stage with reductions); its entries mark the
+// operands that are the same for every row (stride 0 along kernel axis 0).
+inline int match_chain(const KArgs* ks, const int* families, int n, int family = 4) {
     auto matches = [&](const StaticEntry& e) {
-        if (e.family != 4 || e.chain_len != n) return false;
+        if (e.family != family || e.chain_len != n) return false;
         for (int i = 0; i < n; ++i) {
             if (!entry_matches(e.chain[i], families[i], 4, ks[i])) return false;
-            for (int t = 0; t < ks[i].n_tensors; ++t)
-                if ((e.chain[i].rowshared[t] != 0) != (ks[i].t[t].s[0] == 0 && ks[i].t[t].s[1] == 0)) return false;
+            for (int t = 0; t < ks[i].n_tensors; ++t) {
+                const bool shared = family == 5 ? ks[i].t[t].s[0] == 0 : (ks[i].t[t].s[0] == 0 && ks[i].t[t].s[1] == 0);
+                if ((e.chain[i].rowshared[t] != 0) != shared) return false;
+            }
         }
         return true;
     };
@@ -108,7 +113,7 @@ inline int match_chain(const KArgs* ks, const int* families, int n) {
 inline bool same_program(const StaticEntry& a, const StaticEntry& b) {
     if (a.family != b.family || a.V != b.V || a.n_ops != b.n_ops || a.n_tensors != b.n_tensors || a.n_red != b.n_red)
         return false;
-    if (a.family == 4) {
+    if (a.family == 4 || a.family == 5) {
         if (a.chain_len != b.chain_len) return false;
         for (int i = 0; i < a.chain_len; ++i) {
             if (!same_program(a.chain[i], b.chain[i])) return false;

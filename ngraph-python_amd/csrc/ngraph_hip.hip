@@ -1486,10 +1486,114 @@ bool plan_row_chain(const ngh_context* ctx, const ngh_fused_spec& sp, ChainPlan&
     return true;
 }
 
+// Could the spec run as a column chain: the reduced axis (spec axis 0) strided, every operand
+// contiguous (or broadcast) along spec axis 2 in whole aligned float4s, fp32 throughout (an
+// argmax may keep its position in int32)?  Fills C like plan_row_chain; C.TR is the number of
+// column chunks a workgroup is wide (TX), C.n_out the column blocks per index of spec axis 1.
+bool plan_col_chain(const ngh_context* ctx, const ngh_fused_spec& sp, ChainPlan& C) {
+    if (sp.flags & NGH_SPEC_PROBE) return false;
+    // (the columns are the spec's last axis that has an extent: kernel axis 2; the other one is kernel axis 1)
+    const int ca = sp.shape[2] > 1 ? 2 : 1, oa = 3 - ca;
+    const long long R = sp.shape[0], n1 = sp.shape[oa], n2 = sp.shape[ca];
+    if (R < 2 || n2 < 4 || n2 % 4 || n1 < 1 || R >= (1LL << 31) || n2 >= (1LL << 31)) return false;
+    bool any_red = false;
+    const int perm[3] = {0, oa, ca};
+    C.n = 0;
+    for (int s = 0; s < sp.n_stages; ++s) {
+        const ngh_stage& S = sp.stages[s];
+        if (S.op_end == S.op_begin) continue;
+        if (C.n == NGH_MAX_STAGES) return false;
+        KArgs& k = C.k[C.n];
+        fill_kargs(sp, S, perm, k);
+        if (k.n_stat_slots != 0 || k.probe) return false;
+        bool loads[NGH_MAX_TENSORS], stores[NGH_MAX_TENSORS];
+        stage_tensors(sp, S, loads, stores);
+        for (int r = 0; r < S.n_reductions; ++r) {
+            const ngh_tensor& T = sp.tensors[S.red_out[r]];
+            if (T.strides[0] != 0 || T.strides[ca] != 1 ||
+                (T.dtype != NGH_F32 && T.dtype != NGH_I32 && T.dtype != NGH_U32)) return false;
+            if ((uintptr_t)T.dev % 16 || T.strides[oa] % 4) return false;
+        }
+        for (int t = 0; t < sp.n_tensors; ++t) {
+            if (!loads[t] && !stores[t]) continue;
+            const ngh_tensor& T = sp.tensors[t];
+            // (integer results of an argmax are read back as they were written: one int per column)
+            const bool int_result = T.dtype == NGH_I32 || T.dtype == NGH_U32;
+            if (T.dtype != NGH_F32 && !(int_result && T.strides[0] == 0 && !stores[t])) return false;
+            if (T.strides[ca] == 1) {
+                if ((uintptr_t)T.dev % 16 || T.strides[0] % 4 || T.strides[oa] % 4) return false;
+            } else if (T.strides[ca] != 0 || stores[t]) {
+                return false;
+            }
+        }
+        for (int pc = S.op_begin; pc < S.op_end; ++pc) {
+            const int opc = sp.ops[pc].opcode;
+            if (opc == NGH_OP_TAKE || opc == NGH_OP_IOTA || opc == NGH_OP_RNG_UNIFORM || opc == NGH_OP_RNG_NORMAL ||
+                opc == NGH_OP_STORE_TRUNC)
+                return false;
+        }
+        any_red = any_red || S.n_reductions > 0;
+        C.stage_of[C.n] = s;
+        C.families[C.n] = S.n_reductions > 0 ? 2 : 0;
+        ++C.n;
+    }
+    if (C.n < 2 || !any_red) return false;
+    {
+        bool written[NGH_MAX_TENSORS] = {}, used[NGH_MAX_TENSORS] = {};
+        for (int i = 0; i < C.n; ++i) {
+            bool loads[NGH_MAX_TENSORS], stores[NGH_MAX_TENSORS];
+            const ngh_stage& S = sp.stages[C.stage_of[i]];
+            stage_tensors(sp, S, loads, stores);
+            for (int r = 0; r < S.n_reductions; ++r) stores[S.red_out[r]] = true;
+            for (int t = 0; t < sp.n_tensors; ++t) {
+                written[t] = written[t] || stores[t];
+                used[t] = used[t] || loads[t] || stores[t];
+            }
+        }
+        for (int t = 0; t < sp.n_tensors; ++t) {
+            if (!written[t]) continue;
+            for (int u = 0; u < sp.n_tensors; ++u)
+                if (u != t && used[u] && tensors_overlap(sp, sp.tensors[t], sp.tensors[u])) return false;
+        }
+    }
+    // Workgroup shape: as many column chunks wide as leaves every compute unit a few workgroups;
+    // the lanes that are not needed along the columns split the rows.
+    const long long chunks = n2 / 4;
+    const long long cus = ctx ? ctx->cus : 256;
+    unsigned TX = kBlock;
+    auto workgroups = [&](unsigned tx) { return n1 * ((chunks + tx - 1) / tx); };
+    if (workgroups(TX) < 2 * cus) TX = 64;
+    while (TX > 8 && workgroups(TX) < 2 * cus && R / (kBlock / (TX / 2)) >= 4) TX >>= 1;
+    // a lane that walks at most kColCached rows keeps them in registers and the operand is read
+    // once: worth narrower workgroups, down to 256-byte runs along the columns
+    auto rows_per_lane = [&](unsigned tx) { return tx == kBlock ? R : (R + kBlock / tx - 1) / (kBlock / tx); };
+    if (rows_per_lane(TX) > kColCached) {
+        for (unsigned tx = (TX == kBlock ? 64u : TX / 2); tx >= 16; tx >>= 1)
+            if (rows_per_lane(tx) <= kColCached) { TX = tx; break; }
+    }
+    C.TR = TX;
+    C.n_out = (unsigned)((chunks + TX - 1) / TX);
+    if (workgroups(TX) >= (1LL << 31)) return false;
+    return true;
+}
+
+// the grid of a column chain
+static unsigned col_chain_blocks(const ngh_fused_spec& sp, const ChainPlan& C) {
+    return (unsigned)(sp.shape[sp.shape[2] > 1 ? 1 : 2] * (long long)C.n_out);
+}
+
 int ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec) {
     if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
     NGH_TRY(validate(spec));
     NGH_TRY(flex_settle_spec(ctx, *spec));
+    if (spec->n_stages > 1 && !ctx->force_interp && !ctx->no_chain) {
+        ChainPlan C;
+        if (plan_col_chain(ctx, *spec, C) && (C.special = match_chain(C.k, C.families, C.n, 5)) >= 0) {
+            const int cp = stage_cache_policy(ctx, *spec, spec->stages[C.stage_of[C.n - 1]]) & kCpNtStore;
+            HIP_TRY(launch_special_chain(C.special, ctx->stream, col_chain_blocks(*spec, C), C.k[C.n - 1], C.n_out, C.TR, cp));
+            return NGH_OK;
+        }
+    }
     if (spec->n_stages > 1 && !ctx->force_interp && !ctx->no_chain && !ctx->no_ragged) {
         ChainPlan C;
         if (plan_row_chain(ctx, *spec, C) && (C.special = match_chain(C.k, C.families, C.n)) >= 0) {
@@ -1531,6 +1635,14 @@ int ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec, int32_t sta
     if (!ctx || !name128) return fail(NGH_E_INVALID, "NULL argument");
     NGH_TRY(validate(spec));
     if (stage < 0 || stage >= spec->n_stages) return fail(NGH_E_INVALID, "stage %d", stage);
+    if (spec->n_stages > 1 && !ctx->force_interp && !ctx->no_chain) {
+        ChainPlan C;
+        if (plan_col_chain(ctx, *spec, C) && (C.special = match_chain(C.k, C.families, C.n, 5)) >= 0) {
+            const int cp = stage_cache_policy(ctx, *spec, spec->stages[C.stage_of[C.n - 1]]) & kCpNtStore;
+            snprintf(name128, 128, "special:%s/column-chain-of-%d%s", special_name(C.special), C.n, cp ? "/nt-stores" : "");
+            return NGH_OK;
+        }
+    }
     if (spec->n_stages > 1 && !ctx->force_interp && !ctx->no_chain && !ctx->no_ragged) {
         ChainPlan C;
         if (plan_row_chain(ctx, *spec, C) && (C.special = match_chain(C.k, C.families, C.n)) >= 0) {
@@ -1764,10 +1876,20 @@ int ngh_plan_fused(const ngh_fused_spec* spec, int32_t stage, int32_t* out8) {
 int ngh_plan_chain(const ngh_fused_spec* spec, int32_t* out4) {
     if (!out4) return fail(NGH_E_INVALID, "out4 is NULL");
     NGH_TRY(validate(spec));
-    ChainPlan C;
     // (no context here: the knobs a context would carry are read from the environment, as it does)
-    const bool ok = spec->n_stages > 1 && !env_int("NGH_NO_CHAIN", 0) && !env_int("NGH_NO_RAGGED", 0) &&
-                    !env_int("NGH_FORCE_INTERP", 0) && env_int("NGH_ROW_WAVE_CHUNKS", kRowWaveChunks) > 0 &&
+    const bool chains = spec->n_stages > 1 && !env_int("NGH_NO_CHAIN", 0) && !env_int("NGH_FORCE_INTERP", 0);
+    {
+        ChainPlan C;
+        if (chains && plan_col_chain(nullptr, *spec, C)) {
+            out4[0] = 2;
+            out4[1] = match_chain(C.k, C.families, C.n, 5);
+            out4[2] = (int)C.TR;
+            out4[3] = C.n;
+            return NGH_OK;
+        }
+    }
+    ChainPlan C;
+    const bool ok = chains && !env_int("NGH_NO_RAGGED", 0) && env_int("NGH_ROW_WAVE_CHUNKS", kRowWaveChunks) > 0 &&
                     plan_row_chain(nullptr, *spec, C);
     out4[0] = ok ? 1 : 0;
     out4[1] = ok ? match_chain(C.k, C.families, C.n) : -1;

@@ -171,11 +171,15 @@ def plan_fused(spec, stage=0):
 
 
 def plan_chain(spec):
-    """Would the library run every stage of `spec` in one kernel (a row chain)?"""
+    """Would the library run every stage of `spec` in one kernel -- as a row chain (the reduced
+    axis contiguous) or a column chain (the reduced axis strided, outputs along the contiguous
+    one)?  lanes_per_row: lanes per row of a row chain, column chunks per workgroup of a column
+    chain."""
     lib = load_library()
     out = (ctypes.c_int32 * 4)()
     _check(lib, lib.ngh_plan_chain(ctypes.byref(spec), out))
-    return {"eligible": bool(out[0]), "special": out[1], "lanes_per_row": out[2], "stages": out[3]}
+    return {"eligible": bool(out[0]), "kind": {0: None, 1: "row", 2: "column"}[out[0]], "special": out[1],
+            "lanes_per_row": out[2], "stages": out[3]}
 
 
 def exported_symbols():

@@ -149,7 +149,7 @@ def uncovered_programs(kernels, name, min_elements=4096, include_covered=False):
     out = []
     for p in stage_programs(kernels, name, min_elements=min_elements):
         if p[-1] < 0 or include_covered:
-            if p[8] == 4:     # a chain: its stages are named by their place, not by the computation
+            if p[8] in (4, 5):     # a chain: its stages are named by their place, not by the computation
                 p = (p[0], [("stage%d" % j,) + tuple(m[1:]) for j, m in enumerate(p[1])]) + tuple(p[2:])
             # named by content: the same program gets the same library in every process,
             # whatever the computation it comes from is called there

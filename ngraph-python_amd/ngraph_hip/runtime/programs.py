@@ -91,10 +91,13 @@ def stage_programs(kernels, name, seen=None, min_elements=4096, vector_only=Fals
 
 
 def _chain_program(spec, name, seen, min_elements):
-    """The record of a spec whose stages run as one row-chain kernel (family 4: its second field
-    holds the records of the stages, which are programs over rows along spec axis 0, 4 elements
-    per lane); None when the spec is no chain, () when the chain is recorded already or too
-    small to be worth a kernel."""
+    """The record of a spec whose stages run as one chain kernel; None when the spec is no chain,
+    () when the chain is recorded already or too small to be worth a kernel.
+
+    Family 4, a row chain: the second field holds the records of the stages, which are programs
+    over rows along spec axis 0, 4 elements per lane.  Family 5, a column chain: the reduced
+    axis (spec axis 0) is the strided one, the stages are programs 4 columns (spec axis 2) wide;
+    their `rowshared` marks the operands that are the same for every row."""
     plan = hiplib.plan_chain(spec)
     if not plan["eligible"]:
         return None
@@ -102,11 +105,17 @@ def _chain_program(spec, name, seen, min_elements):
     # on the interpreter)
     if spec.shape[0] * spec.shape[1] * spec.shape[2] < min_elements // 16:
         return ()
+    columns = plan["kind"] == "column"
     dtypes = [spec.tensors[i].dtype for i in range(spec.n_tensors)]
-    bcast = [1 if spec.tensors[i].strides[0] == 0 else 0 for i in range(spec.n_tensors)]
-    # (the same for every row: a layer norm's gain and bias)
-    rowshared = [1 if spec.tensors[i].strides[1] == 0 and spec.tensors[i].strides[2] == 0 else 0
-                 for i in range(spec.n_tensors)]
+    if columns:
+        ca = 2 if spec.shape[2] > 1 else 1           # (the columns: the last axis that has an extent)
+        bcast = [1 if spec.tensors[i].strides[ca] == 0 else 0 for i in range(spec.n_tensors)]
+        rowshared = [1 if spec.tensors[i].strides[0] == 0 else 0 for i in range(spec.n_tensors)]
+    else:
+        bcast = [1 if spec.tensors[i].strides[0] == 0 else 0 for i in range(spec.n_tensors)]
+        # (the same for every row: a layer norm's gain and bias)
+        rowshared = [1 if spec.tensors[i].strides[1] == 0 and spec.tensors[i].strides[2] == 0 else 0
+                     for i in range(spec.n_tensors)]
     members = []
     for stage in range(spec.n_stages):
         st = spec.stages[stage]
@@ -117,14 +126,15 @@ def _chain_program(spec, name, seen, min_elements):
         stored = set(o[1] for o in ops if o[0] == hiplib.OPCODES["store"])
         loaded = set(o[2] for o in ops if o[0] == hiplib.OPCODES["load"])
         members.append(("%s_s%d" % (name, stage), ops, dtypes, bcast, [-1] * spec.n_tensors, 0, spec.n_regs, 4,
-                        1 if red_out else 0, red_out, [-1] * spec.n_tensors,
+                        ((2 if columns else 1) if red_out else 0), red_out, [-1] * spec.n_tensors,
                         [1 if i in loaded else 0 for i in range(spec.n_tensors)],
                         [1 if i in stored else 0 for i in range(spec.n_tensors)], -1, rowshared))
-    key = ("chain", tuple(rowshared)) + tuple((tuple(m[1]), tuple(m[2]), tuple(m[3]), m[8], tuple(m[9])) for m in members)
+    key = ("column chain" if columns else "chain", tuple(rowshared)) + \
+        tuple((tuple(m[1]), tuple(m[2]), tuple(m[3]), m[8], tuple(m[9])) for m in members)
     if key in seen:
         return ()
     seen.add(key)
-    return (name, members, dtypes, bcast, [], 0, spec.n_regs, 4, 4, [], [], [], [], plan["special"])
+    return (name, members, dtypes, bcast, [], 0, spec.n_regs, 4, 5 if columns else 4, [], [], [], [], plan["special"])
 
 
 def _render_struct(lines, struct, record):
@@ -157,7 +167,7 @@ def render(programs, header, prefix="SP", table="kStaticTable", count="kStaticCo
     """C++ text: one `struct <prefix>n` per record, the entry table and its length."""
     lines = list(header)
     for i, p in enumerate(programs):
-        if p[8] == 4:
+        if p[8] in (4, 5):
             # a chain: the structs of its stages and the array of their entries (no launchers)
             for j, member in enumerate(p[1]):
                 _render_struct(lines, "%s%d_%d" % (prefix, i, j), member)
@@ -171,10 +181,12 @@ def render(programs, header, prefix="SP", table="kStaticTable", count="kStaticCo
             _render_struct(lines, prefix + str(i), p)
     lines.append("static const StaticEntry %s[] = {" % table)
     for i, p in enumerate(programs):
-        if p[8] == 4:
+        if p[8] in (4, 5):
             stages = ", ".join("%s%d_%d" % (prefix, i, j) for j in range(len(p[1])))
-            lines.append('    {"%s", 4, 4, 0, nullptr, 0, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr, '
-                         '%d, %s%d_stages, nullptr, &launch_static_chain<%s>},' % (p[0], len(p[1]), prefix, i, stages))
+            lines.append('    {"%s", %d, 4, 0, nullptr, 0, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr, '
+                         '%d, %s%d_stages, nullptr, &%s<%s>},'
+                         % (p[0], p[8], len(p[1]), prefix, i,
+                            "launch_static_chain" if p[8] == 4 else "launch_static_col_chain", stages))
             continue
         if p[8] == 0:
             launch = "&launch_static<{0}>, nullptr, {0}::staged, nullptr".format(prefix + str(i))

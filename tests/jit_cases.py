@@ -173,6 +173,34 @@ def case_lookup_table():
     return [ng.lookuptable(lut, idx, ng.make_axes([N, F]), update=False) * w + 1.0], [lut, idx, w]
 
 
+def case_softmax_over_classes():
+    # classes x samples, the layout of the neon front end: the reduced axis is the strided one.
+    # Its three kernels become the stages of one column chain; 300 rows: row lanes share a
+    # column chunk and meet in LDS
+    A, B = ng.make_axis(300, name="A"), ng.make_axis(2048, name="B")
+    x = ng.placeholder([A, B])
+    e = ng.exp(x - ng.max(x, out_axes=[B]))
+    return [e / ng.sum(e, out_axes=[B])], [x]
+
+
+def case_softmax_over_few_classes():
+    # 10 classes: a lane walks all rows of its four columns and keeps them in registers
+    A, B = ng.make_axis(10, name="A"), ng.make_axis(65536, name="B")
+    x = ng.placeholder([A, B])
+    e = ng.exp(x - ng.max(x, out_axes=[B]))
+    return [e / ng.sum(e, out_axes=[B]), ng.argmax(x, out_axes=[B])], [x]
+
+
+def case_column_statistics_chain():
+    # batch statistics over the leading (strided) axis feeding a normalisation, with an outer axis
+    N, C, F = ng.make_axis(64, name="N"), ng.make_axis(6, name="C"), ng.make_axis(1024, name="F")
+    x, g = ng.placeholder([N, C, F]), ng.placeholder([C, F])
+    mean = ng.sum(x, out_axes=[C, F]) * (1.0 / 64)
+    d = x - mean
+    var = ng.sum(d * d, out_axes=[C, F]) * (1.0 / 64)
+    return [d * ng.reciprocal(ng.sqrt(var + 1e-3)) * g], [x, g]
+
+
 def case_row_statistics_chain():
     # mean and variance of every row feeding a consumer: one moments kernel (one-pass variance)
     # plus a kernel for the consumer while interpreted, one row chain (sum, then the sum of
@@ -188,7 +216,8 @@ FP32_CASES = [case_elementwise, case_column_reduction_with_store, case_row_reduc
               case_ragged_long_rows, case_ragged_many_rows, case_softmax_ragged_rows, case_softmax_long_rows, case_softmax_over_windows,
               case_softmax_forward_and_backward,
               case_row_chain_with_stored_intermediate, case_misaligned_slices, case_short_rows, case_dropout, case_lookup_table,
-              case_row_statistics_chain]
+              case_row_statistics_chain, case_softmax_over_classes, case_softmax_over_few_classes,
+              case_column_statistics_chain]
 
 
 def flex_case():

@@ -215,7 +215,7 @@ def test_compiled_programs_agree_with_the_interpreter(case):
     # Same bits as the interpreter -- except where the compiled program runs 4 elements per lane
     # over rows that are not whole aligned vectors (the interpreter takes those one element per
     # lane), or several stages as one row-chain kernel: a reduction then adds up in another order.
-    ragged = any("/ragged" in n or "/chain-of-" in n for n in names)
+    ragged = any("/ragged" in n or "chain-of-" in n for n in names)
     for a, b, w in zip(interp, compiled, want):
         if ragged:
             np.testing.assert_allclose(a, b, rtol=2e-6, atol=1e-6)
@@ -237,6 +237,9 @@ def test_compiled_programs_agree_with_the_interpreter(case):
                     jit_cases.case_softmax_forward_and_backward,
                     jit_cases.case_row_chain_with_stored_intermediate, jit_cases.case_row_statistics_chain):
             assert any("/chain-of-" in n for n in names), names
+        if case in (jit_cases.case_softmax_over_classes, jit_cases.case_softmax_over_few_classes,
+                    jit_cases.case_column_statistics_chain):
+            assert any("/column-chain-of-3" in n for n in names), names
         if case is jit_cases.case_row_statistics_chain:
             # (the other way to the statistics is what ran before the chain was there)
             assert any("moments" in n for n in names_interp), names_interp
@@ -258,7 +261,7 @@ def test_random_graphs_compiled_agree_with_the_interpreter(seed, views):
         finally:
             t.close()
     (interp, _), (compiled, names) = run(jit=False), run(jit=True, jit_min_elements=1)
-    ragged = any("/ragged" in n or "/chain-of-" in n for n in names)       # (see the test above)
+    ragged = any("/ragged" in n or "chain-of-" in n for n in names)       # (see the test above)
     for a, b in zip(interp, compiled):
         if ragged:
             np.testing.assert_allclose(a, b, rtol=1e-5, atol=1e-5)
