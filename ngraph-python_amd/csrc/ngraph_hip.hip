@@ -1567,7 +1567,7 @@ bool plan_col_chain(const ngh_context* ctx, const ngh_fused_spec& sp, ChainPlan&
     // a lane that walks at most kColCached rows keeps them in registers and the operand is read
     // once: worth narrower workgroups, down to 256-byte runs along the columns
     auto rows_per_lane = [&](unsigned tx) { return tx == kBlock ? R : (R + kBlock / tx - 1) / (kBlock / tx); };
-    if (rows_per_lane(TX) > kColCached) {
+    if (rows_per_lane(TX) > (TX == kBlock ? kColCachedWide : kColCached)) {
         for (unsigned tx = (TX == kBlock ? 64u : TX / 2); tx >= 16; tx >>= 1)
             if (rows_per_lane(tx) <= kColCached) { TX = tx; break; }
     }

@@ -176,7 +176,7 @@ def case_lookup_table():
 def case_softmax_over_classes():
     # classes x samples, the layout of the neon front end: the reduced axis is the strided one.
     # Its three kernels become the stages of one column chain; 300 rows: row lanes share a
-    # column chunk and meet in LDS
+    # column chunk and meet in LDS, and every stage streams x again
     A, B = ng.make_axis(300, name="A"), ng.make_axis(2048, name="B")
     x = ng.placeholder([A, B])
     e = ng.exp(x - ng.max(x, out_axes=[B]))
@@ -189,6 +189,15 @@ def case_softmax_over_few_classes():
     x = ng.placeholder([A, B])
     e = ng.exp(x - ng.max(x, out_axes=[B]))
     return [e / ng.sum(e, out_axes=[B]), ng.argmax(x, out_axes=[B])], [x]
+
+
+def case_softmax_over_ten_classes_of_many_samples():
+    # columns enough to fill the chip with workgroups 256 chunks wide: a lane owns its four
+    # columns outright, all ten rows in registers, no folds between lanes
+    A, B = ng.make_axis(10, name="A"), ng.make_axis(786432, name="B")
+    x = ng.placeholder([A, B])
+    e = ng.exp(x - ng.max(x, out_axes=[B]))
+    return [e / ng.sum(e, out_axes=[B])], [x]
 
 
 def case_column_statistics_chain():
@@ -217,7 +226,7 @@ FP32_CASES = [case_elementwise, case_column_reduction_with_store, case_row_reduc
               case_softmax_forward_and_backward,
               case_row_chain_with_stored_intermediate, case_misaligned_slices, case_short_rows, case_dropout, case_lookup_table,
               case_row_statistics_chain, case_softmax_over_classes, case_softmax_over_few_classes,
-              case_column_statistics_chain]
+              case_softmax_over_ten_classes_of_many_samples, case_column_statistics_chain]
 
 
 def flex_case():

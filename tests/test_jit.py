@@ -238,7 +238,7 @@ def test_compiled_programs_agree_with_the_interpreter(case):
                     jit_cases.case_row_chain_with_stored_intermediate, jit_cases.case_row_statistics_chain):
             assert any("/chain-of-" in n for n in names), names
         if case in (jit_cases.case_softmax_over_classes, jit_cases.case_softmax_over_few_classes,
-                    jit_cases.case_column_statistics_chain):
+                    jit_cases.case_softmax_over_ten_classes_of_many_samples, jit_cases.case_column_statistics_chain):
             assert any("/column-chain-of-3" in n for n in names), names
         if case is jit_cases.case_row_statistics_chain:
             # (the other way to the statistics is what ran before the chain was there)
