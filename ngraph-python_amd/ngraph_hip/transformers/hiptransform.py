@@ -649,10 +649,19 @@ class FusedKernel(HipKernel):
         shape = [d.length for d in inner] or [1]
         nd = len(inner)
         sb = FusedSpecBuilder(shape)
+        # Registers are fp32 (as in the reference's kernels wherever an integer meets a float:
+        # float_ew2.py:615-641), which is exact for integers up to 2**24 only.  A kernel that
+        # merely moves 32-bit integers declares them fp32: loads, register moves and stores pass
+        # the bits through untouched, so the move is exact over the whole range.
+        def is_dtype(td, numpy_type):
+            return isinstance(td.dtype, (np.dtype, type)) and np.dtype(td.dtype) == np.dtype(numpy_type)
+
+        moves_bits = (all(p[0] in ("load", "store", "assign") for p in program) and
+                      any(all(is_dtype(td, kind) for td in operands) for kind in (np.int32, np.uint32)))
         for s, td in enumerate(operands):
             view = t.get_tensor_description_tensor_view(td)
             strides = [d.strides[s] for d in inner] or [0]
-            dtype = t.ngh_dtype(td.dtype)
+            dtype = t.ngh_dtype(np.dtype(np.float32) if moves_bits else td.dtype)
             slot = sb.tensor(view.ptr + offsets[s] * view.itemsize, strides, dtype,
                              take_extent=self.take_extents.get(s, 0))
             assert slot == s

@@ -609,6 +609,20 @@ def test_variance_sqrt_inverse_forward(backend):
     np.testing.assert_allclose(got, want, atol=1e-4, rtol=1e-4)
 
 
+def test_moving_32_bit_integers_keeps_every_bit(backend):
+    """Kernel registers are fp32 (exact up to 2**24); a kernel that only moves int32 / uint32
+    values must not round them all the same."""
+    ax = axes(H=6)
+    for dtype, values in ((np.int32, [0, 16777217, -16777219, 2 ** 31 - 1, -2 ** 31, 123456789]),
+                          (np.uint32, [0, 16777217, 2 ** 32 - 1, 2 ** 31 + 1, 4000000001, 7])):
+        v = ng.variable(ax, dtype=dtype, initial_value=np.zeros(6, dtype=dtype))
+        x = ng.placeholder(ax, dtype=dtype)
+        with executor(ng.sequential([ng.assign(v, x), v]), x) as f:
+            got = np.array(f(np.array(values, dtype=dtype)))
+        assert got.dtype == dtype
+        np.testing.assert_array_equal(got, np.array(values, dtype=dtype))
+
+
 def test_multiply_uint32_scalar(backend):
     x = ng.placeholder((), dtype=np.uint32)
     with executor(0.5 * x * 0.5, x) as f:
