@@ -15,12 +15,13 @@ registry through its metaclass (base.py:265-279) and are made by its
 `make_transformer_factory` / `allocate_transformer` (base.py:834-847).  Nothing of the
 package is imported before `register` is called, so this module imports anywhere.
 
-How: the lowering (`ngraph_hip/transformers/hiptransform.py`, `flexhiptransform.py`,
+How: the lowering (`ngraph_hip/transformers/hiptransform.py` and the modules it is made of --
+`hipdevice`, `hiplowering`, `hipmoments`, `hipchains`, `hipplanner` --, `flexhiptransform.py`,
 `passes/hippasses.py`) reaches the graph package only through `import` statements naming
 `ngraph_hip.op_graph...`, `ngraph_hip.transformers.base` and
 `ngraph_hip.transformers.passes.passes` -- the modules this repository carries as stand-ins for
 `ngraph.op_graph...`, `ngraph.transformers.base` and `ngraph.transformers.passes.passes`, with
-the same names inside.  `bind(package)` executes those three source files a second time as
+the same names inside.  `bind(package)` executes those source files a second time as
 modules of their own in which these imports resolve to the package's modules instead: the op
 classes the lowering tests with isinstance, the base classes its own classes derive from and
 the pass driver are then the package's.  The kernels, the C ABI binding, the flex manager and
@@ -148,8 +149,10 @@ SUBSTITUTED = {
     "ngraph_hip.transformers.passes.passes": "transformers.passes.passes",
 }
 #: modules executed again per package, in dependency order
-REBOUND = ("ngraph_hip.transformers.passes.hippasses", "ngraph_hip.transformers.hiptransform",
-           "ngraph_hip.transformers.flexhiptransform")
+REBOUND = ("ngraph_hip.transformers.passes.hippasses", "ngraph_hip.transformers.hipdevice",
+           "ngraph_hip.transformers.hiplowering", "ngraph_hip.transformers.hipmoments",
+           "ngraph_hip.transformers.hipchains", "ngraph_hip.transformers.hipplanner",
+           "ngraph_hip.transformers.hiptransform", "ngraph_hip.transformers.flexhiptransform")
 
 _bound = {}
 
