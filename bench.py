@@ -510,8 +510,53 @@ def compiled_vs_interpreted(ng, ngt, steps, warmup, An=8192, Bn=8192):
                                                "frac_of_hbm_peak": round(nbytes / (cold * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
             finally:
                 t.close()
+        row["first_run"] = first_run_latency(name)
         out[name] = row
     return out
+
+
+def first_run_latency(name):
+    """What a machine pays once per program, measured in a child process (in this one the
+    programs are loaded already): seconds `initialize()` of a transformer with jit=True takes
+    with an empty program cache, hipcc compiling every stage's program."""
+    import subprocess
+    try:
+        out = subprocess.run([sys.executable, os.path.abspath(__file__), "--first-run-of", name],
+                             stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=600)
+        return json.loads(out.stdout.decode().strip().splitlines()[-1])
+    except Exception as e:
+        return {"error": str(e)[:200]}
+
+
+def first_run_child(name):
+    """The child of first_run_latency: one JSON line."""
+    import shutil
+    import tempfile
+    import ngraph_hip as ng
+    import ngraph_hip.transformers as ngt
+    tmp = tempfile.mkdtemp(prefix="ngh_programs_")
+    os.environ["NGH_PROGRAM_CACHE"] = tmp
+    try:
+        results, inputs = [(r, i) for n, r, i, _ in user_graphs(ng) if n == name][0]
+        seconds = {}
+        for label, mode in (("lowering_only_s", False), ("initialize_s_empty_cache", True)):
+            t = ngt.make_transformer_factory("hipgpu", jit=mode)()
+            try:
+                t.computation(results, *inputs)
+                t0 = time.perf_counter()
+                t.initialize()
+                seconds[label] = round(time.perf_counter() - t0, 3)
+            finally:
+                t.close()
+        n = len([f for f in os.listdir(tmp) if f.endswith(".so")])
+        seconds.update({"programs": n, "what": "jit=True: every stage's program compiled by hipcc at initialize(), "
+                        "the hipcc runs of one computation in parallel (up to 4); a later process finds them in "
+                        "the cache"})
+        print(json.dumps(seconds))
+    except Exception as e:                      # no hipcc on this machine
+        print(json.dumps({"error": str(e)[:200]}))
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
 
 
 # ------------------------------------------------------------------------------------- shapes
@@ -677,6 +722,7 @@ def main():
     ap.add_argument("--compiled", action="store_true",
                     help="also time five user graphs: default kernel choice, interpreter only, compiled "
                          "(needs hipcc unless the program cache already holds them)")
+    ap.add_argument("--first-run-of", default="", help=argparse.SUPPRESS)
     ap.add_argument("--only", default="", help="with --shapes: only the cases whose name contains this text")
     ap.add_argument("--shapes", action="store_true",
                     help="also time a survey of everyday layouts and extents (broadcasts, transposed operands, "
@@ -692,6 +738,9 @@ def main():
               file=sys.stderr)
         sys.exit(2)
     args.blocks = max(1, args.blocks)
+    if args.first_run_of:
+        first_run_child(args.first_run_of)
+        return
     which = set(s.strip().lower() for s in args.configs.split(","))
 
     import ngraph_hip as ng

@@ -14,11 +14,12 @@ kept, so a program is compiled once per machine, not once per process.
 Three modes (`make_transformer_factory("hipgpu", jit=...)`, default from NGH_JIT, else "auto"):
 
   "auto"  stages over large tensors (at least `jit_auto_min_elements` elements) that no compiled
-          kernel covers are compiled by worker threads once the computation runs for the second
-          time, while it goes on running on the interpreter; the kernel group loads the
+          kernel covers are handed to worker threads when the transformer is initialised
+          (`jit_after_calls=0`, the default; with n > 0 only once the computation has run n
+          times), while the computation starts on the interpreter; the kernel group loads the
           libraries when they are ready and the next launch finds them.  Program libraries
-          already in the cache are loaded when the computation is first run.  Without hipcc on
-          the machine the computation simply stays on the interpreter.
+          already in the cache are loaded when the kernels are bound.  Without hipcc on the
+          machine the computation simply stays on the interpreter.
   True    every stage of at least `jit_min_elements` elements is compiled before the first
           launch (the reference's behaviour: it compiles a computation's kernels when the
           transformer is initialised); a missing hipcc is an error.
@@ -226,9 +227,9 @@ class BackgroundPrograms(object):
     """The uncovered programs of a kernel group, compiled off the launch path.
 
     Libraries the cache already holds are loaded at once.  The others are handed to the
-    process-wide compile workers by `start` (the kernel group calls it once the computation has
-    run `after_calls` times: a computation that runs once never pays for a compiler run); the
-    workers run hipcc and touch no device.  `poll`, called from the thread that owns the
+    process-wide compile workers by `start`: at once with `after_calls` = 0, else once the
+    computation has run `after_calls` times (a computation that runs fewer times never pays for
+    a compiler run); the workers run hipcc and touch no device.  `poll`, called from the thread that owns the
     runtime, loads what has been compiled since the last call and returns True once nothing is
     outstanding.  A compiler that is missing or fails leaves the group on the interpreter; the
     message is kept in `error`.  `cancel` withdraws the jobs that have not started."""
@@ -248,6 +249,8 @@ class BackgroundPrograms(object):
                 self.loaded += runtime.programs_load(path)
             else:
                 self._todo.append(p)
+        if self.after_calls <= 0 and self._todo:
+            self.start()
 
     @property
     def started(self):

@@ -57,6 +57,8 @@ class HipKernelGroup(object):
     def bind(self):
         """Lower every kernel, then tell each operand what the rest of the computation does
         with its buffer (the cache hints of the C ABI)."""
+        if self._bound:
+            return
         for k in self.kernels:
             if not k.buffers_bound:
                 k.bind_buffers()
@@ -77,7 +79,8 @@ class HipKernelGroup(object):
             from ngraph_hip.runtime import jit
             self._programs = jit.start_background(self.transformer.runtime, self.kernels, self.name,
                                                   min_elements=self.transformer.jit_auto_min_elements,
-                                                  small_min_elements=self.transformer.jit_min_elements)
+                                                  small_min_elements=self.transformer.jit_min_elements,
+                                                  after_calls=self.transformer.jit_after_calls)
         self._bound = True
 
     _programs = None
@@ -179,7 +182,7 @@ class HipTransformer(ComputationGraphTransformer):
     chain_kernels = True                     # consecutive kernels over the same rows run as stages of one spec
 
     def __init__(self, device_id=0, fusion=True, dry_run=False, fuse_moments=None, rng_seed=0, jit=None,
-                 jit_min_elements=4096, jit_auto_min_elements=1 << 22, **kwargs):
+                 jit_min_elements=4096, jit_auto_min_elements=1 << 22, jit_after_calls=0, **kwargs):
         """dry_run=True lowers graphs to kernel specs without a device (no results can be
         read back); it exists so the host-side lowering can be inspected and tested.
         rng_seed keys the random fills (ng.uniform / ng.normal): same seed, same numbers.
@@ -193,6 +196,7 @@ class HipTransformer(ComputationGraphTransformer):
         self.jit = _jit.normalize_mode(jit)
         self.jit_min_elements = int(jit_min_elements)
         self.jit_auto_min_elements = int(jit_auto_min_elements)
+        self.jit_after_calls = int(jit_after_calls)
         try:
             self.runtime = DryRunRuntime() if dry_run else HipRuntime(device_id)
         except HipLibraryError as e:
@@ -312,6 +316,19 @@ class HipTransformer(ComputationGraphTransformer):
 
     def allocate_storage(self):
         pass
+
+    def allocate(self):
+        """Storage, initial values, and then -- where the reference compiles the kernels of every
+        computation (float_ew2.py:1553-1653, at `initialize()`) -- the kernels are lowered and
+        their programs asked for: compiled on the spot with jit=True, handed to the compile
+        workers with jit="auto" (the computations start on the interpreter and pick the
+        programs up when they are ready)."""
+        if self.allocated:
+            return
+        super(HipTransformer, self).allocate()
+        if self.jit is not False:
+            for group in self.kernel_groups.values():
+                group.bind()
 
     def close(self):
         for group in getattr(self, "kernel_groups", {}).values():

@@ -122,7 +122,8 @@ def test_background_programs_load_when_ready_and_only_for_large_stages(tmp_path,
     finally:
         t.close()
     for expect_thread in (True, False):
-        t = ngt.make_transformer_factory("hipgpu", dry_run=True, jit="auto", jit_auto_min_elements=1 << 18)()
+        t = ngt.make_transformer_factory("hipgpu", dry_run=True, jit="auto", jit_auto_min_elements=1 << 18,
+                                         jit_after_calls=2)()
         try:
             results, inputs = jit_cases.case_elementwise()
             f = t.computation(results, *inputs)
@@ -142,6 +143,23 @@ def test_background_programs_load_when_ready_and_only_for_large_stages(tmp_path,
             assert len(libs) == 1 and t.runtime.program_libraries == [os.path.join(str(tmp_path), libs[0])]
         finally:
             t.close()
+
+
+def test_by_default_compilation_starts_when_the_transformer_is_initialised(tmp_path, monkeypatch):
+    """The reference compiles a computation's kernels at initialize() (float_ew2.py:1553-1653);
+    the default mode hands the large stages to the compile workers at that point, before any run."""
+    monkeypatch.setenv("NGH_PROGRAM_CACHE", str(tmp_path))
+    t = ngt.make_transformer_factory("hipgpu", dry_run=True, jit="auto", jit_auto_min_elements=1 << 18)()
+    try:
+        results, inputs = jit_cases.case_elementwise()
+        f = t.computation(results, *inputs)
+        t.initialize()
+        group = t.kernel_groups[f]
+        assert group._bound and group._programs is not None and group._programs.started
+        assert group.wait_for_programs(timeout=300) is None
+        assert len([n for n in os.listdir(str(tmp_path)) if n.endswith(".so")]) == 1
+    finally:
+        t.close()
 
 
 def test_background_compilation_without_a_compiler_stays_on_the_interpreter(tmp_path, monkeypatch):
