@@ -24,14 +24,16 @@
 #ifndef NGRAPH_HIP_H
 #define NGRAPH_HIP_H
 
+#if !defined(__HIPCC_RTC__)     /* (in-process compilation of kernels has these types built in) */
 #include <stddef.h>
 #include <stdint.h>
+#endif
 
 #ifdef __cplusplus
 extern "C" {
 #endif
 
-#define NGH_ABI_VERSION 5
+#define NGH_ABI_VERSION 6
 
 /* ---- limits (float_ew2.py:285-286 MAX_AXES = 3) ------------------------ */
 #define NGH_MAX_AXES      3
@@ -270,6 +272,40 @@ int  ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec,
 int  ngh_programs_load(ngh_context* ctx, const char* path, int32_t* out_added);
 /* number of compiled programs the process knows: built in, loaded */
 int  ngh_programs_count(int32_t* built_in, int32_t* loaded);
+
+/* ---- the same without a compiler on the machine: the reference compiles inside the process
+ *      (NVRTC) and launches through the driver API (float_ew2.py:1626-1653
+ *      CudaSourceFile.compile -> SourceModule.get_function -> prepared_async_call).  The host
+ *      side compiles the generated source with hiprtc, device code only, into a code object and
+ *      hands it over with a description of every program in it.  A description restates what the
+ *      source's `struct <type_name>` holds, which is what ngh_launch_fused compares a stage
+ *      with; for a chain (family 4: stages over the same rows, 5: over the same columns) the
+ *      n_stages descriptions that follow it are its stages.                                   */
+typedef struct ngh_program_desc {
+    char     name[64];                        /* as shown by ngh_describe_fused            */
+    char     type_name[64];                   /* the C++ struct of the source, in namespace ngh */
+    int32_t  family, V, n_ops, n_tensors, n_red, n_stat_slots, n_stages;
+    ngh_op   ops[NGH_MAX_OPS];
+    int32_t  dtypes[NGH_MAX_TENSORS];
+    uint8_t  bcast[NGH_MAX_TENSORS];          /* constant along the lanes' axis            */
+    uint8_t  rowshared[NGH_MAX_TENSORS];      /* stages of a chain: the same for every row */
+    int8_t   staged[NGH_MAX_TENSORS];         /* family 3: LDS tile number or -1           */
+    int32_t  red_out[NGH_MAX_REDUCTIONS];
+} ngh_program_desc;
+#define NGH_PROGRAM_KERNEL_SLOTS 12
+/* The C++ name expressions of the kernels that program `index` of descs[0..n) may launch
+ * (cache-policy, ragged-row, deferred-statistics, tile-size and chunks-per-lane variants): what
+ * the host gives hiprtcAddNameExpression.  Written to `out` as NGH_PROGRAM_KERNEL_SLOTS lines
+ * ('\n'-terminated), an empty line for a slot the program has no kernel for.  `index` must be a
+ * program of its own or a chain, not a chain's stage.  Needs no context and no device.        */
+int  ngh_program_kernels(const ngh_program_desc* descs, int32_t n, int32_t index, char* out, size_t out_bytes);
+/* Loads the code object (hipModuleLoadData on the context's device; it stays loaded) and
+ * appends its programs to the table.  `lowered` holds, for every program of its own and every
+ * chain of descs in order, NGH_PROGRAM_KERNEL_SLOTS lines: the lowered (mangled) names of the
+ * kernels in the slots of ngh_program_kernels, empty where the slot is.  out_added as above.  */
+int  ngh_programs_load_code(ngh_context* ctx, const void* code, size_t code_bytes,
+                            const ngh_program_desc* descs, int32_t n, const char* lowered,
+                            int32_t* out_added);
 
 /* Per-row mean and (biased) variance of a [rows, R] fp32 matrix with contiguous rows in ONE
  * read of x (x_cache_hint: NGH_CACHE_* bits for x): fuses the reductions behind ng.mean + ng.variance

@@ -7,9 +7,23 @@
 // transformer dispatches (ngraph/transformers/gputransform.py:124-275,
 // templates in ngraph/transformers/gpu/float_ew2.py:31-108).
 #pragma once
+#if !defined(__HIPCC_RTC__)
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 #include <stdint.h>
+#else
+// Compiled in process (hiprtc): the HIP device headers are built in, host headers do not exist;
+// the fixed-width names the kernel headers use are spelled out here.
+typedef signed char int8_t;
+typedef unsigned char uint8_t;
+typedef short int16_t;
+typedef unsigned short uint16_t;
+typedef int int32_t;
+typedef unsigned int uint32_t;
+typedef long long int64_t;
+typedef unsigned long long uint64_t;
+typedef unsigned long uintptr_t;
+#endif
 #include "ngraph_hip.h"
 
 namespace ngh {

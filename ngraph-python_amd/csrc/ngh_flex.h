@@ -11,9 +11,6 @@
 // host mirror (ngraph_hip/flex/hipflex.py, _policy_step) executes the same steps in the same
 // order; the two must stay equivalent (the library is built with -ffp-contract=off).
 #pragma once
-#include <hip/hip_runtime.h>
-#include <stdint.h>
-#include "ngraph_hip.h"
 #include "ngh_device.h"
 
 namespace ngh {

@@ -162,28 +162,47 @@ inline unsigned streaming_blocks(int cus, int blocks_per_cu, unsigned n_chunks) 
     return blocks > cap ? cap : blocks;
 }
 
+// the launchers of programs whose kernels live in a code object loaded at run time (ngh_rtc.h)
+inline hipError_t rtc_launch_ew(const StaticEntry& e, hipStream_t stream, unsigned blocks, const KArgs& k,
+                                unsigned n_chunks, unsigned cpr, int cache_policy);
+inline hipError_t rtc_launch_red(const StaticEntry& e, hipStream_t stream, unsigned blocks, const KArgs& k,
+                                 unsigned n_first, unsigned n_seg, unsigned seg_len, unsigned TX, RedWs ws,
+                                 int cache_policy);
+inline hipError_t rtc_launch_tiled(const StaticEntry& e, hipStream_t stream, unsigned blocks, const KArgs& k,
+                                   unsigned tiles_a, unsigned tiles_b, unsigned n_tiles, int tile);
+inline hipError_t rtc_launch_chain(const StaticEntry& e, hipStream_t stream, unsigned blocks, const KArgs& k,
+                                   unsigned n_out, unsigned T, int cache_policy);
+
 inline hipError_t launch_special_tiled(int i, hipStream_t stream, unsigned blocks, const KArgs& k, unsigned tiles_a,
                                        unsigned tiles_b, unsigned n_tiles, int tile) {
-    special_entry(i).launch_tiled(stream, blocks, k, tiles_a, tiles_b, n_tiles, tile);
+    const StaticEntry& e = special_entry(i);
+    if (e.rtc) return rtc_launch_tiled(e, stream, blocks, k, tiles_a, tiles_b, n_tiles, tile);
+    e.launch_tiled(stream, blocks, k, tiles_a, tiles_b, n_tiles, tile);
     return hipGetLastError();
 }
 
 inline hipError_t launch_special_red(int i, hipStream_t stream, unsigned blocks, const KArgs& k, unsigned n_first,
                                      unsigned n_seg, unsigned seg_len, unsigned TX, RedWs ws, int cache_policy) {
-    special_entry(i).launch_red(stream, blocks, k, n_first, n_seg, seg_len, TX, ws, cache_policy);
+    const StaticEntry& e = special_entry(i);
+    if (e.rtc) return rtc_launch_red(e, stream, blocks, k, n_first, n_seg, seg_len, TX, ws, cache_policy);
+    e.launch_red(stream, blocks, k, n_first, n_seg, seg_len, TX, ws, cache_policy);
     return hipGetLastError();
 }
 
 inline hipError_t launch_special_chain(int i, hipStream_t stream, unsigned blocks, const KArgs& k, unsigned n_out,
                                        unsigned TR, int cache_policy) {
-    special_entry(i).launch_chain(stream, blocks, k, n_out, TR, cache_policy);
+    const StaticEntry& e = special_entry(i);
+    if (e.rtc) return rtc_launch_chain(e, stream, blocks, k, n_out, TR, cache_policy);
+    e.launch_chain(stream, blocks, k, n_out, TR, cache_policy);
     return hipGetLastError();
 }
 
 inline hipError_t launch_special(int i, hipStream_t stream, unsigned blocks, const KArgs& k,
                                  unsigned n_chunks, unsigned chunks_per_row, int cache_policy) {
     if (n_chunks == 0) return hipSuccess;
-    special_entry(i).launch(stream, blocks, k, n_chunks, chunks_per_row, cache_policy);
+    const StaticEntry& e = special_entry(i);
+    if (e.rtc) return rtc_launch_ew(e, stream, blocks, k, n_chunks, chunks_per_row, cache_policy);
+    e.launch(stream, blocks, k, n_chunks, chunks_per_row, cache_policy);
     return hipGetLastError();
 }
 

@@ -17,6 +17,7 @@
 #include "ngh_interp.h"
 #include "ngh_copy.h"
 #include "ngh_table.h"
+#include "ngh_rtc.h"
 #include "ngh_moments.h"
 #include "ngh_flex.h"
 #include "ngh_convert.h"
@@ -1689,6 +1690,85 @@ int ngh_programs_load(ngh_context* ctx, const char* path, int32_t* out_added) {
     // the handle is kept for the life of the process: table entries point into the library
     const int added = add_loaded_programs((const StaticEntry*)entries, n);
     if (added < 0) return fail(NGH_E_UNSUPPORTED, "the program table is full (%d loaded programs)", kMaxLoadedPrograms);
+    if (out_added) *out_added = added;
+    return NGH_OK;
+}
+
+int ngh_program_kernels(const ngh_program_desc* descs, int32_t n, int32_t index, char* out, size_t out_bytes) {
+    if (!descs || !out || n <= 0 || index < 0 || index >= n) return fail(NGH_E_INVALID, "descs / out / index");
+    for (int i = 0; i < n;) {
+        if (!desc_ok(descs[i]) || i + descs[i].n_stages >= n)
+            return fail(NGH_E_INVALID, "program description %d is malformed", i);
+        if (i == index) {
+            std::string text;
+            for (const std::string& name : rtc_kernel_names(descs[i], descs + i + 1)) text += name + "\n";
+            if (text.size() + 1 > out_bytes) return fail(NGH_E_INVALID, "out holds %zu bytes, %zu needed", out_bytes, text.size() + 1);
+            memcpy(out, text.c_str(), text.size() + 1);
+            return NGH_OK;
+        }
+        if (index > i && index <= i + descs[i].n_stages) return fail(NGH_E_INVALID, "description %d is a stage of chain %d", index, i);
+        i += 1 + descs[i].n_stages;
+    }
+    return fail(NGH_E_INVALID, "index %d", index);
+}
+
+int ngh_programs_load_code(ngh_context* ctx, const void* code, size_t code_bytes, const ngh_program_desc* descs,
+                           int32_t n, const char* lowered, int32_t* out_added) {
+    if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
+    if (!code || code_bytes < 64 || !descs || n <= 0 || !lowered) return fail(NGH_E_INVALID, "code / descs / lowered");
+    // the lowered names, line by line
+    std::vector<std::string> lines;
+    for (const char* p = lowered; *p;) {
+        const char* q = strchr(p, '\n');
+        if (!q) return fail(NGH_E_INVALID, "lowered: a line without its newline");
+        lines.emplace_back(p, q);
+        p = q + 1;
+    }
+    int n_top = 0;
+    for (int i = 0; i < n; i += 1 + descs[i].n_stages) {
+        if (!desc_ok(descs[i]) || i + descs[i].n_stages >= n)
+            return fail(NGH_E_INVALID, "program description %d is malformed", i);
+        if ((descs[i].family >= 4) != (descs[i].n_stages > 0)) return fail(NGH_E_INVALID, "description %d: family %d with %d stages", i, descs[i].family, descs[i].n_stages);
+        for (int j = 1; j <= descs[i].n_stages; ++j)
+            if (!desc_ok(descs[i + j]) || descs[i + j].n_stages != 0 || descs[i + j].family > 2)
+                return fail(NGH_E_INVALID, "stage description %d is malformed", i + j);
+        ++n_top;
+    }
+    if ((int)lines.size() != n_top * kRtcMaxKernels)
+        return fail(NGH_E_INVALID, "lowered holds %zu lines, %d programs x %d slots expected", lines.size(), n_top, kRtcMaxKernels);
+    HIP_TRY(hipSetDevice(ctx->device));
+    hipModule_t module = nullptr;
+    hipError_t me = hipModuleLoadData(&module, code);
+    if (me != hipSuccess) return fail(NGH_E_INVALID, "the code object does not load on this device: %s", hipGetErrorString(me));
+    int added = 0, top = 0;
+    for (int i = 0; i < n; i += 1 + descs[i].n_stages, ++top) {
+        const ngh_program_desc& d = descs[i];
+        // (kept for the life of the process, like a program library: the table points into it)
+        RtcProgram* r = new RtcProgram();
+        r->module = module;
+        r->ragged_ok = desc_ragged_ok(d);
+        r->stores = desc_stores(d);
+        r->quad_ok = program_quad_ok(d.ops, d.n_ops);
+        r->stat_slots = d.n_stat_slots > 0;
+        StaticEntry e;
+        rtc_fill_entry(e, *r, d);
+        for (int j = 0; j < d.n_stages; ++j) rtc_fill_entry(r->stages[j], *new RtcProgram(), descs[i + 1 + j]);
+        e.chain_len = d.n_stages;
+        e.chain = d.n_stages ? r->stages : nullptr;
+        e.rtc = r;
+        const std::vector<std::string> wanted = rtc_kernel_names(d, descs + i + 1);
+        for (int s = 0; s < kRtcMaxKernels; ++s) {
+            const std::string& name = lines[(size_t)top * kRtcMaxKernels + s];
+            if (name.empty() != wanted[s].empty())
+                return fail(NGH_E_INVALID, "program %s: kernel slot %d is %s in `lowered`", d.name, s, name.empty() ? "missing" : "not expected");
+            if (name.empty()) continue;
+            hipError_t fe = hipModuleGetFunction(&r->fn[s], module, name.c_str());
+            if (fe != hipSuccess) return fail(NGH_E_INVALID, "program %s: no kernel %s in the code object: %s", d.name, name.c_str(), hipGetErrorString(fe));
+        }
+        const int a = add_loaded_programs(&e, 1);
+        if (a < 0) return fail(NGH_E_UNSUPPORTED, "the program table is full (%d loaded programs)", kMaxLoadedPrograms);
+        added += a;
+    }
     if (out_added) *out_added = added;
     return NGH_OK;
 }

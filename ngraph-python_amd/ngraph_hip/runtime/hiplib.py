@@ -12,7 +12,7 @@ import os
 
 import numpy as np
 
-NGH_ABI_VERSION = 5
+NGH_ABI_VERSION = 6
 NGH_MAX_AXES = 3
 NGH_MAX_TENSORS = 12
 NGH_MAX_OPS = 96
@@ -129,9 +129,30 @@ _SYMBOLS = {
     "ngh_flex_unsettled": [_vp, ctypes.POINTER(ctypes.c_int32)],
     "ngh_programs_load": [_vp, ctypes.c_char_p, ctypes.POINTER(ctypes.c_int32)],
     "ngh_programs_count": [ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32)],
+    "ngh_program_kernels": [ctypes.c_void_p, _i32, _i32, ctypes.c_char_p, ctypes.c_size_t],
+    "ngh_programs_load_code": [_vp, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, _i32, ctypes.c_char_p,
+                               ctypes.POINTER(ctypes.c_int32)],
     "ngh_timer_begin": [_vp],
     "ngh_timer_end": [_vp, ctypes.POINTER(ctypes.c_float)],
 }
+
+NGH_PROGRAM_KERNEL_SLOTS = 12
+
+
+class ngh_program_desc(ctypes.Structure):
+    """What the library compares a stage with, restated for a program whose kernels arrive as a
+    code object (include/ngraph_hip.h)."""
+    _fields_ = [("name", ctypes.c_char * 64), ("type_name", ctypes.c_char * 64),
+                ("family", ctypes.c_int32), ("V", ctypes.c_int32), ("n_ops", ctypes.c_int32),
+                ("n_tensors", ctypes.c_int32), ("n_red", ctypes.c_int32), ("n_stat_slots", ctypes.c_int32),
+                ("n_stages", ctypes.c_int32),
+                ("ops", ngh_op * NGH_MAX_OPS),
+                ("dtypes", ctypes.c_int32 * NGH_MAX_TENSORS),
+                ("bcast", ctypes.c_uint8 * NGH_MAX_TENSORS),
+                ("rowshared", ctypes.c_uint8 * NGH_MAX_TENSORS),
+                ("staged", ctypes.c_int8 * NGH_MAX_TENSORS),
+                ("red_out", ctypes.c_int32 * NGH_MAX_REDUCTIONS)]
+
 
 _lib = None
 
@@ -182,6 +203,40 @@ def plan_chain(spec):
             "lanes_per_row": out[2], "stages": out[3]}
 
 
+def program_descs(dicts):
+    """An array of ngh_program_desc from plain dictionaries (a chain is followed by its stages)."""
+    flat = []
+    for d in dicts:
+        flat.append(d)
+        flat.extend(d.get("stages", []))
+    arr = (ngh_program_desc * len(flat))()
+    for rec, d in zip(arr, flat):
+        rec.name = d["name"].encode("utf-8")
+        rec.type_name = d["type_name"].encode("utf-8")
+        rec.family, rec.V, rec.n_stat_slots = d["family"], d["V"], d["n_stat_slots"]
+        rec.n_ops, rec.n_tensors, rec.n_red = len(d["ops"]), len(d["dtypes"]), len(d["red_out"])
+        rec.n_stages = len(d.get("stages", []))
+        for i, (opcode, dst, a, b) in enumerate(d["ops"]):
+            rec.ops[i] = ngh_op(opcode, dst, a, b)
+        for i in range(rec.n_tensors):
+            rec.dtypes[i], rec.bcast[i] = d["dtypes"][i], d["bcast"][i]
+            rec.rowshared[i], rec.staged[i] = d["rowshared"][i], d["staged"][i]
+        for i, r in enumerate(d["red_out"]):
+            rec.red_out[i] = r
+    return arr
+
+
+def program_kernels(descs, index):
+    """The C++ name expressions of the kernels program `index` of `descs` may launch, one per
+    slot ('' for an empty slot)."""
+    lib = load_library()
+    out = ctypes.create_string_buffer(NGH_PROGRAM_KERNEL_SLOTS * 1024)
+    _check(lib, lib.ngh_program_kernels(ctypes.cast(descs, ctypes.c_void_p), len(descs), int(index), out, len(out)))
+    names = out.value.decode("utf-8").split("\n")[:-1]
+    assert len(names) == NGH_PROGRAM_KERNEL_SLOTS, names
+    return names
+
+
 def exported_symbols():
     return sorted(_SYMBOLS)
 
@@ -190,6 +245,34 @@ def _check(lib, rc):
     if rc != 0:
         msg = lib.ngh_last_error()
         raise HipLibraryError(rc, msg.decode("utf-8", "replace") if msg else "")
+
+
+CODE_BUNDLE_SUFFIX = ".ngco"
+_BUNDLE_MAGIC = b"NGHCODE1"
+
+
+def write_code_bundle(path, dicts, lowered, code):
+    """One file per program library compiled in process: the descriptions of its programs, the
+    lowered names of their kernels (NGH_PROGRAM_KERNEL_SLOTS lines per program) and the code object."""
+    import json
+    import struct
+    head = json.dumps({"abi": NGH_ABI_VERSION, "programs": dicts, "lowered": lowered}).encode("utf-8")
+    with open(path, "wb") as fh:
+        fh.write(_BUNDLE_MAGIC + struct.pack("<I", len(head)) + head + code)
+
+
+def read_code_bundle(path):
+    import json
+    import struct
+    with open(path, "rb") as fh:
+        data = fh.read()
+    if data[:8] != _BUNDLE_MAGIC:
+        raise HipLibraryError(-1, "%s is not a code bundle of this library" % path)
+    n = struct.unpack("<I", data[8:12])[0]
+    head = json.loads(data[12:12 + n].decode("utf-8"))
+    if head.get("abi") != NGH_ABI_VERSION:
+        raise HipLibraryError(-1, "%s was made for ABI %s, this is %d" % (path, head.get("abi"), NGH_ABI_VERSION))
+    return head["programs"], head["lowered"], data[12 + n:]
 
 
 _NP_DTYPES = {NGH_F32: np.float32, NGH_FLEX16: np.int16, NGH_I32: np.int32, NGH_F16: np.float16,
@@ -235,6 +318,7 @@ class HipRuntime(object):
         _check(self.lib, self.lib.ngh_init(int(device_id), ctypes.byref(ctx)))
         self.ctx = ctx
         self._allocs = set()
+        self.program_libraries = []        # what this context asked the library to load
 
     # -- lifetime --------------------------------------------------------
     def close(self):
@@ -417,6 +501,16 @@ class HipRuntime(object):
         """Add the compiled programs of a program library (runtime/jit.py) to the library's
         table; returns how many were new."""
         n = ctypes.c_int32()
+        self.program_libraries.append(path)
+        if path.endswith(CODE_BUNDLE_SUFFIX):
+            # kernels compiled in process: a code object with the descriptions of its programs
+            dicts, lowered, code = read_code_bundle(path)
+            descs = program_descs(dicts)
+            buf = ctypes.create_string_buffer(code, len(code))
+            _check(self.lib, self.lib.ngh_programs_load_code(self.ctx, ctypes.cast(buf, ctypes.c_void_p), len(code),
+                                                             ctypes.cast(descs, ctypes.c_void_p), len(descs),
+                                                             lowered.encode("utf-8"), ctypes.byref(n)))
+            return n.value
         _check(self.lib, self.lib.ngh_programs_load(self.ctx, os.fsencode(path), ctypes.byref(n)))
         return n.value
 

@@ -6,10 +6,13 @@ NVRTC when the transformer is initialised (float_ew2.py:1135-1483 `_get_compound
 structural hash (:1486-1529).  The library here carries compiled kernels for the programs that
 dominate training graphs and an interpreter for everything else; this module closes the gap for
 a user's own graphs: the stage programs that no compiled kernel covers are written out as the
-same C++ tables the built-in ones are made from, compiled by hipcc into a *program library*
-(one shared object per program, named by a hash of its table, the kernel headers and the
-compiler flags) and handed to the library with `ngh_programs_load`.  The object files are
-kept, so a program is compiled once per machine, not once per process.
+same C++ tables the built-in ones are made from, compiled into a *program library* (one per program, named by a hash of its table, the kernel
+headers and the compiler flags) and handed to the library with `ngh_programs_load` or
+`ngh_programs_load_code`.  The libraries are kept, so a program is compiled once per machine,
+not once per process.  Two compilers (`compiler()`, NGH_JIT_COMPILER): hipcc, run as a
+subprocess, makes a shared object with host launchers; hiprtc compiles the same source inside
+this process, device code only, into a code object that the library launches through the module
+API -- the reference's way (NVRTC), and the one that works on a machine without hipcc.
 
 Three modes (`make_transformer_factory("hipgpu", jit=...)`, default from NGH_JIT, else "auto"):
 
@@ -108,9 +111,93 @@ def source_text(programs):
     return render(programs, header, prefix="LP_%s_" % tag, table="kLoadedTable", count="kLoadedCount") + _TRAILER
 
 
+def compiler():
+    """Which compiler builds program libraries: NGH_JIT_COMPILER = "hiprtc" (device code compiled
+    inside this process, launched through the module API: no hipcc needed, and about half the
+    time per program), "hipcc" (a shared object with host launchers, built by a hipcc
+    subprocess), or unset: hiprtc where the machine has libhiprtc, else hipcc."""
+    choice = os.environ.get("NGH_JIT_COMPILER", "").strip().lower()
+    if choice in ("hipcc", "hiprtc"):
+        return choice
+    from ngraph_hip.runtime import hiprtc
+    return "hiprtc" if hiprtc.available() else "hipcc"
+
+
+def _record_desc(record, type_name):
+    """A program record as the dictionary hiplib.program_descs takes."""
+    name, ops, dtypes, bcast, stat_slot, n_slots, n_regs, V, family, red_out, staged = record[:11]
+    rowshared = record[14] if len(record) > 14 else [0] * len(dtypes)
+    d = {"name": name, "type_name": type_name, "family": family, "V": V, "n_stat_slots": n_slots,
+         "dtypes": list(dtypes), "bcast": list(bcast), "rowshared": list(rowshared), "red_out": list(red_out)}
+    if family in (4, 5):
+        d.update(ops=[], staged=[-1] * len(dtypes),
+                 stages=[_record_desc(m, "%s_%d" % (type_name, j)) for j, m in enumerate(ops)])
+    else:
+        d.update(ops=[list(o) for o in ops], staged=list(staged) or [-1] * len(dtypes))
+    return d
+
+
+def device_source_text(programs):
+    """The structs of `programs` alone: what hiprtc compiles (kernels are instantiated by name
+    expression, there is no table and no host code)."""
+    text = source_text(programs)
+    lines, keep = [], True
+    for line in text.split("\n"):
+        if line.startswith("static const StaticEntry") or line.startswith("static const int kLoadedCount"):
+            keep = False
+        if line.startswith("}  // namespace ngh"):
+            lines.append(line)
+            break
+        if keep:
+            lines.append(line)
+        elif line == "};":
+            keep = True
+    return "\n".join(lines) + "\n"
+
+
+def _code_bundle(programs):
+    """(path in the cache, source, descriptions, compiler options) of the code bundle of `programs`."""
+    from ngraph_hip.runtime import hiprtc
+    flags, _ = _flags()
+    options = [f for f in flags if f not in ("-fPIC", "-shared")] + ["-I" + INCLUDE, "-I" + CSRC]
+    text = device_source_text(programs)
+    tag = "".join(c if c.isalnum() else "_" for c in programs[0][0])
+    dicts = [_record_desc(p, "LP_%s_%d" % (tag, i)) for i, p in enumerate(programs)]
+    key = hashlib.sha256((text + _sources_digest() + " ".join(flags) + "hiprtc " + hiprtc.version() +
+                          repr(dicts)).encode("utf-8")).hexdigest()[:20]
+    return os.path.join(cache_dir(), "ngh_programs_" + key + hiplib.CODE_BUNDLE_SUFFIX), text, dicts, options
+
+
+def compile_programs_in_process(programs, verbose=False):
+    """The path of a code bundle holding `programs`, compiled now with hiprtc unless the cache
+    has it."""
+    from ngraph_hip.runtime import hiprtc
+    path, text, dicts, options = _code_bundle(programs)
+    if os.path.exists(path):
+        return path
+    descs = hiplib.program_descs(dicts)
+    index, expressions, slots = 0, [], []
+    for d in dicts:
+        names = hiplib.program_kernels(descs, index)
+        slots.append(names)
+        expressions.extend(n for n in names if n)
+        index += 1 + len(d.get("stages", []))
+    if verbose:
+        print("hiprtc: %d kernels of %s" % (len(expressions), programs[0][0]))
+    code, lowered = hiprtc.compile_source(text, expressions, options, name=os.path.basename(path) + ".hip")
+    by_expression = dict(zip(expressions, lowered))
+    lines = "".join(by_expression.get(n, "") + "\n" for names in slots for n in names)
+    tmp = "%s.%d.%d.tmp" % (path, os.getpid(), threading.get_ident())
+    hiplib.write_code_bundle(tmp, dicts, lines, code)
+    os.replace(tmp, path)         # atomic: another process may be compiling the same programs
+    return path
+
+
 def compile_programs(programs, verbose=False):
     """The path of a program library holding `programs` (records of programs.stage_programs),
     compiled now unless the cache has it."""
+    if compiler() == "hiprtc":
+        return compile_programs_in_process(programs, verbose=verbose)
     flags, find_hipcc = _flags()
     text = source_text(programs)
     key = hashlib.sha256((text + _sources_digest() + " ".join(flags)).encode("utf-8")).hexdigest()[:20]
@@ -129,9 +216,9 @@ def compile_programs(programs, verbose=False):
     try:
         hipcc = find_hipcc()
     except RuntimeError:
-        raise RuntimeError("run-time compilation (jit=True / NGH_JIT=1) needs hipcc on this machine, or the "
-                           "program library %s in the cache; without jit the same stages run on the "
-                           "interpreter" % os.path.basename(lib))
+        raise RuntimeError("run-time compilation (jit=True / NGH_JIT=1) with NGH_JIT_COMPILER=hipcc, or on a "
+                           "machine without libhiprtc, needs hipcc, or the program library %s in the cache; "
+                           "without jit the same stages run on the interpreter" % os.path.basename(lib))
     cmd = [hipcc] + list(flags) + ["-I", INCLUDE, "-I", CSRC, src, "-o", tmp]
     if verbose:
         print(" ".join(cmd))
@@ -181,6 +268,8 @@ def ensure_programs(runtime, kernels, name, min_elements=4096, verbose=False):
 
 def library_path_of(programs):
     """Where the program library of `programs` lives in the cache (whether or not it exists)."""
+    if compiler() == "hiprtc":
+        return _code_bundle(programs)[0]
     flags, _ = _flags()
     text = source_text(programs)
     key = hashlib.sha256((text + _sources_digest() + " ".join(flags)).encode("utf-8")).hexdigest()[:20]
@@ -344,8 +433,20 @@ def precompile_graphs(builders, verbose=False):
             t.close()
     if not todo:
         return []
-    pool = ThreadPool(max(1, min(8, os.cpu_count() or 2)))      # the work is in hipcc subprocesses
+    workers = max(1, min(8, os.cpu_count() or 2))
+    if compiler() == "hiprtc":
+        # hiprtc compiles one program at a time per process: processes, not threads (started
+        # afresh, so that none inherits a device context)
+        import multiprocessing
+        from concurrent.futures import ProcessPoolExecutor
+        with ProcessPoolExecutor(max_workers=workers, mp_context=multiprocessing.get_context("spawn")) as ex:
+            return list(ex.map(_compile_one, list(todo.values())))
+    pool = ThreadPool(workers)      # the work is in hipcc subprocesses
     try:
         return pool.map(lambda p: compile_programs([p], verbose=verbose), list(todo.values()))
     finally:
         pool.close()
+
+
+def _compile_one(program):
+    return compile_programs([program])

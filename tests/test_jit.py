@@ -50,6 +50,7 @@ def test_program_library_compiles_and_checks_its_caller(tmp_path, monkeypatch):
     """hipcc cross-compiles a program library without a device; its entry point refuses a caller
     built from other sources (ABI number, structure sizes)."""
     monkeypatch.setenv("NGH_PROGRAM_CACHE", str(tmp_path))
+    monkeypatch.setenv("NGH_JIT_COMPILER", "hipcc")
     t, kernels = _dry_kernels(jit_cases.case_row_reduction_with_store)
     try:
         programs = jit.uncovered_programs(kernels, "case")
@@ -67,11 +68,53 @@ def test_program_library_compiles_and_checks_its_caller(tmp_path, monkeypatch):
         t.close()
 
 
-def test_every_case_compiles_for_gfx950():
-    """Every skeleton's generated source compiles (hipcc cross-compiles without a device).  The
+@pytest.mark.parametrize("compiler", ["hipcc", "hiprtc"])
+def test_every_case_compiles_for_gfx950(compiler, monkeypatch):
+    """Every skeleton's generated source compiles, with hipcc (which cross-compiles without a
+    device) into shared objects and with hiprtc, inside the process, into code bundles.  The
     libraries land in the program cache, where the GPU tests of this file find them."""
+    monkeypatch.setenv("NGH_JIT_COMPILER", compiler)
     paths = jit_cases.precompile()
     assert len(paths) >= 40 and all(os.path.exists(p) for p in paths)
+    assert all(p.endswith(".so" if compiler == "hipcc" else ".ngco") for p in paths)
+
+
+def test_without_hipcc_programs_are_compiled_in_process(tmp_path, monkeypatch):
+    """A machine without hipcc: the same program becomes a code bundle made by hiprtc -- the
+    descriptions of its programs, one lowered kernel name per slot the library asked for, and a
+    code object."""
+    import build_ext
+    from ngraph_hip.runtime import hiplib
+
+    def no_hipcc():
+        raise RuntimeError("hipcc not found")
+    from ngraph_hip.runtime import hiprtc
+    monkeypatch.setenv("NGH_PROGRAM_CACHE", str(tmp_path))
+    monkeypatch.delenv("NGH_JIT_COMPILER", raising=False)
+    monkeypatch.setattr(build_ext, "find_hipcc", no_hipcc)
+    assert jit.compiler() == "hiprtc"
+    with monkeypatch.context() as m:             # (no libhiprtc either: hipcc is what is asked for)
+        m.setattr(hiprtc, "available", lambda: False)
+        assert jit.compiler() == "hipcc"
+    for case, family in ((jit_cases.case_elementwise, 0), (jit_cases.case_softmax, 4),
+                         (jit_cases.case_softmax_over_classes, 5)):
+        t, kernels = _dry_kernels(case)
+        try:
+            programs = jit.uncovered_programs(kernels, "case")
+            path = jit.compile_programs(programs[:1])
+            assert path.endswith(hiplib.CODE_BUNDLE_SUFFIX) and path == jit.library_path_of(programs[:1])
+            dicts, lowered, code = hiplib.read_code_bundle(path)
+            assert len(dicts) == 1 and dicts[0]["family"] == family and dicts[0]["name"].startswith("jit_")
+            names = lowered.split("\n")[:-1]
+            assert len(names) == hiplib.NGH_PROGRAM_KERNEL_SLOTS
+            wanted = hiplib.program_kernels(hiplib.program_descs(dicts), 0)
+            assert [bool(n) for n in names] == [bool(w) for w in wanted] and any(names)
+            assert all(n.startswith("_Z") for n in names if n)
+            assert code[:4] == b"\x7fELF" and all(n.encode() in code for n in names if n)
+            if family >= 4:
+                assert len(dicts[0]["stages"]) == 3
+        finally:
+            t.close()
 
 
 def test_missing_compiler_is_reported_as_such(tmp_path, monkeypatch):
@@ -80,6 +123,7 @@ def test_missing_compiler_is_reported_as_such(tmp_path, monkeypatch):
     def no_hipcc():
         raise RuntimeError("hipcc not found")
     monkeypatch.setenv("NGH_PROGRAM_CACHE", str(tmp_path))
+    monkeypatch.setenv("NGH_JIT_COMPILER", "hipcc")          # (left to itself it would turn to hiprtc)
     monkeypatch.setattr(build_ext, "find_hipcc", no_hipcc)
     t, kernels = _dry_kernels(jit_cases.case_elementwise)
     try:
@@ -139,7 +183,7 @@ def test_background_programs_load_when_ready_and_only_for_large_stages(tmp_path,
                 assert group._programs.started
             assert group.wait_for_programs(timeout=300) is None
             assert group._programs is None
-            libs = [n for n in os.listdir(str(tmp_path)) if n.endswith(".so")]
+            libs = [n for n in os.listdir(str(tmp_path)) if n.endswith(".so") or n.endswith(".ngco")]
             assert len(libs) == 1 and t.runtime.program_libraries == [os.path.join(str(tmp_path), libs[0])]
         finally:
             t.close()
@@ -157,7 +201,7 @@ def test_by_default_compilation_starts_when_the_transformer_is_initialised(tmp_p
         group = t.kernel_groups[f]
         assert group._bound and group._programs is not None and group._programs.started
         assert group.wait_for_programs(timeout=300) is None
-        assert len([n for n in os.listdir(str(tmp_path)) if n.endswith(".so")]) == 1
+        assert len([n for n in os.listdir(str(tmp_path)) if n.endswith(".so") or n.endswith(".ngco")]) == 1
     finally:
         t.close()
 
@@ -168,6 +212,7 @@ def test_background_compilation_without_a_compiler_stays_on_the_interpreter(tmp_
     def no_hipcc():
         raise RuntimeError("hipcc not found")
     monkeypatch.setenv("NGH_PROGRAM_CACHE", str(tmp_path))
+    monkeypatch.setenv("NGH_JIT_COMPILER", "hipcc")          # (neither compiler: hiprtc is not asked)
     monkeypatch.setattr(build_ext, "find_hipcc", no_hipcc)
     t = ngt.make_transformer_factory("hipgpu", dry_run=True, jit="auto", jit_auto_min_elements=1 << 18)()
     try:
@@ -263,6 +308,29 @@ def test_compiled_programs_agree_with_the_interpreter(case):
             assert any("moments" in n for n in names_interp), names_interp
         if case is jit_cases.case_transposed_operands_large:
             assert any(n.endswith("/tiles64") for n in names), names
+
+
+@pytest.mark.gpu
+def test_programs_of_either_compiler_agree_with_the_interpreter():
+    """The same cases with each compiler named explicitly, one child process per compiler (a
+    program, once loaded, serves the whole process, whichever compiler made it): hiprtc -- kernels
+    compiled inside the process (here: found as code bundles in the cache, where the CPU suite
+    left them), loaded with hipModuleLoadData and launched with hipModuleLaunchKernel -- and
+    hipcc -- shared objects with host launchers."""
+    import json
+    import subprocess
+    import sys
+    child = os.path.join(os.path.dirname(os.path.abspath(__file__)), "rtc_child.py")
+    for compiler in ("hiprtc", "hipcc"):
+        proc = subprocess.run([sys.executable, child, compiler], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                              timeout=900)
+        assert proc.returncode == 0, proc.stderr.decode()[-2000:]
+        report = json.loads(proc.stdout.decode().strip().splitlines()[-1])
+        assert report["failures"] == [] and report["compiler"] == compiler, report
+        assert report["cases"] >= 26 and report["loaded"] >= 20 and report["compiled_kernels"] >= 40, report
+        mine, other = ("code_bundles_loaded", "shared_objects_loaded") if compiler == "hiprtc" else \
+            ("shared_objects_loaded", "code_bundles_loaded")
+        assert report[mine] >= 20 and report[other] == 0, report
 
 
 @pytest.mark.gpu
