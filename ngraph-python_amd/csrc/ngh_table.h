@@ -1,11 +1,12 @@
 // The table of compiled op programs: the ones built into the library (ngh_programs.inc) and the
-// ones loaded at run time from program libraries (ngh_programs_load).
+// ones loaded at run time (ngh_programs_load: a shared object hipcc built; ngh_programs_load_code:
+// a code object hiprtc built inside the process, ngh_rtc.h).
 //
 // Counterpart of the reference's kernel cache (ngraph/transformers/gpu/float_ew2.py:1486-1529
 // _ops_to_hash, :1560-1567 compiled-kernel lookup): there a structural hash of the op list finds
 // a kernel that NVRTC already compiled for this process, here a structural comparison finds a
-// kernel hipcc compiled -- with the library, or later into a program library by the host side
-// (ngraph_hip/runtime/jit.py).  Anything without an entry runs on the interpreter.
+// kernel compiled with the library, or later by the host side (ngraph_hip/runtime/jit.py).
+// Anything without an entry runs on the interpreter.
 #pragma once
 #include <atomic>
 #include <cstdint>
