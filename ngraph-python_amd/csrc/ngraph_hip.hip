@@ -128,6 +128,7 @@ struct ngh_context {
     int         force_interp = 0;    // never pick a specialised kernel
     int         red_wgs_per_cu = 8;  // workgroups per CU a split reduction along the contiguous axis aims for
     int         red_col_wgs_per_cu = 2;  // ... and one across it
+    int         col_chain_wgs_per_cu = 2; // workgroups per compute unit a column chain narrows its workgroups for
     int         row_wave_chunks = 0;     // rows of up to this many chunks are reduced by one wavefront each
     int         tile4 = 1;               // tiled elementwise programs may take 64 x 64 tiles with 16-byte accesses
     int         no_tiles = 0;        // never use the LDS-tiled elementwise skeleton
@@ -1121,6 +1122,7 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->wide_min_rows = std::max(1, env_int("NGH_WIDE_MIN_ROWS", 2));
     ctx->red_wgs_per_cu = std::max(1, env_int("NGH_RED_WGS_PER_CU", 8));
     ctx->red_col_wgs_per_cu = std::max(1, env_int("NGH_RED_COL_WGS_PER_CU", 2));
+    ctx->col_chain_wgs_per_cu = std::max(1, env_int("NGH_COL_CHAIN_WGS_PER_CU", 2));
     ctx->row_wave_chunks = std::max(0, env_int("NGH_ROW_WAVE_CHUNKS", kRowWaveChunks));
     ctx->tile4 = env_int("NGH_TILE4", 1);
     ctx->cache_policy = env_int("NGH_CACHE_POLICY", -1);
@@ -1561,10 +1563,13 @@ bool plan_col_chain(const ngh_context* ctx, const ngh_fused_spec& sp, ChainPlan&
     // the lanes that are not needed along the columns split the rows.
     const long long chunks = n2 / 4;
     const long long cus = ctx ? ctx->cus : 256;
+    const long long wanted = cus * (ctx ? ctx->col_chain_wgs_per_cu : 2);
     unsigned TX = kBlock;
     auto workgroups = [&](unsigned tx) { return n1 * ((chunks + tx - 1) / tx); };
-    if (workgroups(TX) < 2 * cus) TX = 64;
-    while (TX > 8 && workgroups(TX) < 2 * cus && R / (kBlock / (TX / 2)) >= 4) TX >>= 1;
+    if (workgroups(TX) < wanted) TX = 64;
+    // (not below 128-byte runs along the columns: 64-byte ones fetch every cache line twice,
+    // 137 against 81 us for a softmax over [1000, 32768])
+    while (TX > 8 && workgroups(TX) < wanted && R / (kBlock / (TX / 2)) >= 4) TX >>= 1;
     // a lane that walks at most kColCached rows keeps them in registers and the operand is read
     // once: worth narrower workgroups, down to 256-byte runs along the columns
     auto rows_per_lane = [&](unsigned tx) { return tx == kBlock ? R : (R + kBlock / tx - 1) / (kBlock / tx); };
