@@ -312,7 +312,36 @@ class HipFlexManager(FlexManager):
                 print("flex %s: maxabs %d -> next dec %s" % (entry.name, maxabs, entry.next_dec))
 
     def set_h5py_file(self, data_file):
+        """Where save_diagnostic_data writes (flexgputransform.py:105-114 hands autoflex an h5py
+        file for the same purpose): an object with h5py's `create_group` / `create_dataset`, or a
+        path, which gets a NumPy .npz archive."""
         self.data_file = data_file
 
+    def diagnostic_data(self):
+        """Per flex tensor, by name: the exponent in use and the one chosen for the next write,
+        the scale, the last max |mantissa|, whether it overflowed, and the recorded maxima."""
+        out = {}
+        for flex_id, entry in sorted(self.flex_entries.items()):
+            name = "%04d_%s" % (flex_id, entry.name or "tensor")
+            next_dec = entry.next_dec
+            out[name] = {"dec": entry.dec, "next_dec": -1 if next_dec is None else next_dec, "scale": entry.scale,
+                         "initialized": int(entry.initialized), "last_maxabs": entry.last_maxabs,
+                         "overflow": int(entry.last_maxabs >= entry.dtype.pclip),
+                         "history": np.asarray(entry.history, dtype=np.float64)}
+        return out
+
     def save_diagnostic_data(self):
-        pass
+        target = getattr(self, "data_file", None)
+        if target is None:
+            return
+        data = self.diagnostic_data()
+        if hasattr(target, "create_group"):
+            step = target.create_group("autoflex_count_%d" % self.autoflex_count)
+            for name, fields in data.items():
+                group = step.create_group(name)
+                for key, value in fields.items():
+                    group.create_dataset(key, data=value)
+            return
+        flat = {"%s/%s" % (name, key): np.asarray(value) for name, fields in data.items() for key, value in fields.items()}
+        flat["autoflex_count"] = np.asarray(self.autoflex_count)
+        np.savez(target, **flat)

@@ -375,3 +375,36 @@ def test_in_place_rule_iterated_on_the_device_agrees_across_policy_modes(monkeyp
     for name, (st, mant) in seen.items():
         assert st == seen["host"][0], (name, st, seen["host"][0])
         np.testing.assert_array_equal(mant, seen["host"][1], err_msg=name)
+
+
+@pytest.mark.gpu
+def test_flex_statistics_file_holds_the_exponent_state_of_every_tensor(tmp_path):
+    """set_output_statistics_file / save_output_statistics_file (base.py:407-417,
+    flexgputransform.py:105-114, called by the neon callbacks at callbacks.py:126-135): with
+    collect_flex_data the flex manager writes its per-tensor state."""
+    path = str(tmp_path / "flex_stats.npz")
+    t = ngt.make_transformer_factory("flexhip", collect_flex_data=True)()
+    try:
+        H = ng.make_axis(64, name="H")
+        x = ng.placeholder([H])
+        f = t.computation(x * 2.0 + 1.0, x)
+        t.set_output_statistics_file(path)
+        f(np.linspace(-3, 3, 64).astype(np.float32))
+        t.save_output_statistics_file()
+    finally:
+        t.close()
+    data = np.load(path)
+    assert int(data["autoflex_count"]) >= 1
+    decs = [k for k in data.files if k.endswith("/dec")]
+    assert decs and all(0 <= int(data[k]) <= 31 for k in decs)
+    # the result 2x + 1 reaches 7: 3 integer bits, so 15 - 3 - 1 fractional bits or fewer
+    assert any(int(data[k]) <= 12 and int(data[k.replace("/dec", "/last_maxabs")]) > 0 for k in decs)
+    # without collect_flex_data the calls are accepted and write nothing
+    other = str(tmp_path / "none.npz")
+    t = ngt.make_transformer_factory("flexhip")()
+    try:
+        t.set_output_statistics_file(other)
+        t.save_output_statistics_file()
+    finally:
+        t.close()
+    assert not os.path.exists(other)
