@@ -11,6 +11,7 @@
 // statistics, tile size, chunks or rows per lane) and launch with hipModuleLaunchKernel.
 // Host code only.
 #pragma once
+#include <atomic>
 #include <string>
 #include <vector>
 
@@ -32,7 +33,9 @@ constexpr int kRtcMaxKernels = 12;
 struct RtcProgram {
     hipModule_t   module = nullptr;
     hipFunction_t fn[kRtcMaxKernels] = {};
-    int           lazy_fit[kCachePolicies] = {0, 0, 0, 0};   // resident workgroups per compute unit, once asked
+    // resident workgroups per compute unit of the deferred-statistics kernels, 0 until asked
+    // (contexts on several threads may launch the same program)
+    std::atomic<int> lazy_fit[kCachePolicies];
     bool          ragged_ok = false, stores = false, quad_ok = false, stat_slots = false;
     // what the table entry points to
     char          name[64] = {};
@@ -42,10 +45,11 @@ struct RtcProgram {
     signed char   staged[NGH_MAX_TENSORS] = {};
     int           red_out[NGH_MAX_REDUCTIONS] = {};
     StaticEntry   stages[NGH_MAX_STAGES] = {};                // a chain's stages
+    RtcProgram() { for (auto& f : lazy_fit) f.store(0); }
 };
 
 inline bool desc_ok(const ngh_program_desc& d) {
-    return d.family >= 0 && d.family <= 5 && d.n_ops >= 0 && d.n_ops <= NGH_MAX_OPS && d.n_tensors >= 0 &&
+    return d.family >= 0 && d.family <= 5 && (d.V == 1 || d.V == 4 || d.V == 8) && d.n_ops >= 0 && d.n_ops <= NGH_MAX_OPS && d.n_tensors >= 0 &&
            d.n_tensors <= NGH_MAX_TENSORS && d.n_red >= 0 && d.n_red <= NGH_MAX_REDUCTIONS && d.n_stages >= 0 &&
            d.n_stages <= NGH_MAX_STAGES && d.type_name[sizeof(d.type_name) - 1] == 0 && d.name[sizeof(d.name) - 1] == 0;
 }
@@ -154,15 +158,15 @@ inline hipError_t rtc_launch_ew(const StaticEntry& e, hipStream_t stream, unsign
     void* args[] = {(void*)&k, &n_chunks, &cpr};
     if (r.stat_slots && k.flex_lazy) {
         hipFunction_t f = r.fn[8 + cp];
-        if (f && r.lazy_fit[cp] == 0) {
-            int n = 0;
-            if (hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&n, f, kBlock, 0) != hipSuccess || n < 1) {
+        int fit = r.lazy_fit[cp].load(std::memory_order_relaxed);
+        if (f && fit == 0) {
+            if (hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&fit, f, kBlock, 0) != hipSuccess || fit < 1) {
                 (void)hipGetLastError();
-                n = 1;
+                fit = 1;
             }
-            r.lazy_fit[cp] = n;
+            r.lazy_fit[cp].store(fit, std::memory_order_relaxed);
         }
-        const int fit = r.lazy_fit[cp] > 0 ? r.lazy_fit[cp] : 1;
+        if (fit < 1) fit = 1;
         const unsigned per_cu = k.lazy_blocks_per_cu < 0 ? (unsigned)(-k.lazy_blocks_per_cu)
                               : (unsigned)std::max(1, std::min(k.lazy_blocks_per_cu, fit > 6 ? fit - 2 : fit));
         blocks = std::min(blocks, (unsigned)k.flex_lazy * per_cu);

@@ -1744,12 +1744,26 @@ int ngh_programs_load_code(ngh_context* ctx, const void* code, size_t code_bytes
     HIP_TRY(hipSetDevice(ctx->device));
     hipModule_t module = nullptr;
     hipError_t me = hipModuleLoadData(&module, code);
-    if (me != hipSuccess) return fail(NGH_E_INVALID, "the code object does not load on this device: %s", hipGetErrorString(me));
-    int added = 0, top = 0;
+    if (me != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(NGH_E_INVALID, "the code object does not load on this device: %s", hipGetErrorString(me));
+    }
+    // Everything is resolved before anything is published: a bundle that does not fit its
+    // descriptions leaves no trace.
+    std::vector<RtcProgram*> owned;
+    std::vector<StaticEntry> entries;
+    auto refuse = [&](int code) {
+        for (RtcProgram* p : owned) delete p;
+        (void)hipModuleUnload(module);
+        (void)hipGetLastError();          // (a failed look-up must not surface in the next launch's check)
+        return code;
+    };
+    int top = 0;
     for (int i = 0; i < n; i += 1 + descs[i].n_stages, ++top) {
         const ngh_program_desc& d = descs[i];
         // (kept for the life of the process, like a program library: the table points into it)
         RtcProgram* r = new RtcProgram();
+        owned.push_back(r);
         r->module = module;
         r->ragged_ok = desc_ragged_ok(d);
         r->stores = desc_stores(d);
@@ -1757,7 +1771,11 @@ int ngh_programs_load_code(ngh_context* ctx, const void* code, size_t code_bytes
         r->stat_slots = d.n_stat_slots > 0;
         StaticEntry e;
         rtc_fill_entry(e, *r, d);
-        for (int j = 0; j < d.n_stages; ++j) rtc_fill_entry(r->stages[j], *new RtcProgram(), descs[i + 1 + j]);
+        for (int j = 0; j < d.n_stages; ++j) {
+            RtcProgram* stage = new RtcProgram();
+            owned.push_back(stage);
+            rtc_fill_entry(r->stages[j], *stage, descs[i + 1 + j]);
+        }
         e.chain_len = d.n_stages;
         e.chain = d.n_stages ? r->stages : nullptr;
         e.rtc = r;
@@ -1765,15 +1783,15 @@ int ngh_programs_load_code(ngh_context* ctx, const void* code, size_t code_bytes
         for (int s = 0; s < kRtcMaxKernels; ++s) {
             const std::string& name = lines[(size_t)top * kRtcMaxKernels + s];
             if (name.empty() != wanted[s].empty())
-                return fail(NGH_E_INVALID, "program %s: kernel slot %d is %s in `lowered`", d.name, s, name.empty() ? "missing" : "not expected");
+                return refuse(fail(NGH_E_INVALID, "program %s: kernel slot %d is %s in `lowered`", d.name, s, name.empty() ? "missing" : "not expected"));
             if (name.empty()) continue;
             hipError_t fe = hipModuleGetFunction(&r->fn[s], module, name.c_str());
-            if (fe != hipSuccess) return fail(NGH_E_INVALID, "program %s: no kernel %s in the code object: %s", d.name, name.c_str(), hipGetErrorString(fe));
+            if (fe != hipSuccess) return refuse(fail(NGH_E_INVALID, "program %s: no kernel %s in the code object: %s", d.name, name.c_str(), hipGetErrorString(fe)));
         }
-        const int a = add_loaded_programs(&e, 1);
-        if (a < 0) return fail(NGH_E_UNSUPPORTED, "the program table is full (%d loaded programs)", kMaxLoadedPrograms);
-        added += a;
+        entries.push_back(e);
     }
+    const int added = add_loaded_programs(entries.data(), (int)entries.size());
+    if (added < 0) return fail(NGH_E_UNSUPPORTED, "the program table is full (%d loaded programs)", kMaxLoadedPrograms);
     if (out_added) *out_added = added;
     return NGH_OK;
 }

@@ -79,6 +79,77 @@ def test_every_case_compiles_for_gfx950(compiler, monkeypatch):
     assert all(p.endswith(".so" if compiler == "hipcc" else ".ngco") for p in paths)
 
 
+def test_kernel_names_of_a_program_description():
+    """ngh_program_kernels: which kernels a program may launch follows from its description alone
+    (no device): cache-policy variants, ragged-row forms only where the program allows them,
+    non-temporal-store variants only where it stores, the stages of a chain in its kernels' names."""
+    from ngraph_hip.runtime import hiplib
+    load, store, add, rsum = (hiplib.OPCODES[n] for n in ("load", "store", "add", "sum"))
+    ew = {"name": "jit_a", "type_name": "LP_a_0", "family": 0, "V": 4, "n_stat_slots": 0,
+          "ops": [[load, 0, 0, 0], [load, 1, 1, 0], [add, 0, 0, 1], [store, 2, 0, 0]],
+          "dtypes": [0, 0, 0], "bcast": [0, 0, 0], "rowshared": [0, 0, 0], "staged": [-1, -1, -1], "red_out": []}
+    names = hiplib.program_kernels(hiplib.program_descs([ew]), 0)
+    assert names[0] == "ngh::ew_static_kernel<ngh::LP_a_0, 0>" and names[3].endswith(", 3>")
+    assert names[4] == "ngh::ew_ragged_static_kernel<ngh::LP_a_0, 0>" and not any(names[8:])
+    flex = dict(ew, dtypes=[1, 1, 1], n_stat_slots=1)          # flex16: no ragged rows, deferred statistics
+    names = hiplib.program_kernels(hiplib.program_descs([flex]), 0)
+    assert not any(names[4:8]) and names[8] == "ngh::ew_static_lazy_kernel<ngh::LP_a_0, 0>"
+    row_sum = {"name": "jit_b", "type_name": "LP_b_0", "family": 1, "V": 4, "n_stat_slots": 0,
+               "ops": [[load, 0, 0, 0], [rsum, 0, 0, 0]], "dtypes": [0, 0], "bcast": [0, 1], "rowshared": [0, 0],
+               "staged": [-1, -1], "red_out": [1]}
+    names = hiplib.program_kernels(hiplib.program_descs([row_sum]), 0)
+    assert names[0] and names[1] and not names[2] and not names[3]          # nothing stored elementwise
+    assert names[8] == "ngh::red_rows_small_static_kernel<ngh::LP_b_0, false>" and names[9]
+    chain = {"name": "jit_c", "type_name": "LP_c_0", "family": 4, "V": 4, "n_stat_slots": 0, "ops": [],
+             "dtypes": [0, 0], "bcast": [0, 1], "rowshared": [0, 0], "staged": [-1, -1], "red_out": [],
+             "stages": [dict(row_sum, type_name="LP_c_0_0"), dict(ew, type_name="LP_c_0_1", dtypes=[0, 0, 0])]}
+    descs = hiplib.program_descs([ew, chain])
+    names = hiplib.program_kernels(descs, 1)
+    assert names[0] == "ngh::row_chain_static_kernel<0, 4, ngh::LP_c_0_0, ngh::LP_c_0_1>"
+    assert names[3] == "ngh::row_chain_static_kernel<2, 8, ngh::LP_c_0_0, ngh::LP_c_0_1>" and not any(names[4:])
+    with pytest.raises(hiplib.HipLibraryError, match="stage of chain"):
+        hiplib.program_kernels(descs, 2)
+    with pytest.raises(hiplib.HipLibraryError):
+        hiplib.program_kernels(descs, 9)
+    bad = hiplib.program_descs([dict(ew, V=3)])
+    with pytest.raises(hiplib.HipLibraryError, match="malformed"):
+        hiplib.program_kernels(bad, 0)
+
+
+@pytest.mark.gpu
+def test_a_code_bundle_that_does_not_fit_its_descriptions_is_refused(hip_runtime, tmp_path, monkeypatch):
+    """ngh_programs_load_code checks what it is given before it publishes anything: the number
+    of lowered names, names the code object does not hold."""
+    import ctypes
+    from ngraph_hip.runtime import hiplib
+    monkeypatch.setenv("NGH_PROGRAM_CACHE", str(tmp_path))
+    monkeypatch.setenv("NGH_JIT_COMPILER", "hiprtc")
+    t, kernels = _dry_kernels(jit_cases.case_elementwise)
+    try:
+        path = jit.compile_programs(jit.uncovered_programs(kernels, "case")[:1])
+    finally:
+        t.close()
+    dicts, lowered, code = hiplib.read_code_bundle(path)
+    descs = hiplib.program_descs(dicts)
+    lib, n = hip_runtime.lib, ctypes.c_int32()
+    buf = ctypes.create_string_buffer(code, len(code))
+
+    def load(names):
+        return lib.ngh_programs_load_code(hip_runtime.ctx, ctypes.cast(buf, ctypes.c_void_p), len(code),
+                                          ctypes.cast(descs, ctypes.c_void_p), len(descs), names.encode(), ctypes.byref(n))
+    before = ctypes.c_int32()
+    lib.ngh_programs_count(None, ctypes.byref(before))
+    assert load(lowered + "\n") != 0 and b"lines" in lib.ngh_last_error()
+    wrong = "\n".join(("_Z9not_there" if line else "") for line in lowered.split("\n")[:-1]) + "\n"
+    assert load(wrong) != 0 and b"no kernel" in lib.ngh_last_error()
+    missing = "\n" * hiplib.NGH_PROGRAM_KERNEL_SLOTS
+    assert load(missing) != 0 and b"missing" in lib.ngh_last_error()
+    after = ctypes.c_int32()
+    lib.ngh_programs_count(None, ctypes.byref(after))
+    assert after.value == before.value                      # nothing was added by the refused calls
+    assert load(lowered) == 0                                # and the bundle as it was written loads
+
+
 def test_without_hipcc_programs_are_compiled_in_process(tmp_path, monkeypatch):
     """A machine without hipcc: the same program becomes a code bundle made by hiprtc -- the
     descriptions of its programs, one lowered kernel name per slot the library asked for, and a
