@@ -10,7 +10,7 @@ from that value when every op is computed from the float32 results before it and
 
 * once (unit roundoff u = 2^-24) for +, -, *, /, sqrt, reciprocal, square;
 * to within `TRANSCENDENTAL_ULPS` units in the last place for exp, log, tanh, sin, cos, pow,
-  sigmoid (BASELINE allows the device 2 ulp; NumPy's float32 loops are within 3);
+  sigmoid (the device is tested to stay within 2 ulp; NumPy's float32 loops are within 3);
 * a sum over n elements in any order: min(n, 8 sqrt(n)) u sum|x_i| -- the probabilistic bound
   of a serial sum, which is what NumPy does across a strided axis (the worst case n u says
   nothing at n ~ 10^5; trees are tighter than either);

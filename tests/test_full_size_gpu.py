@@ -147,3 +147,38 @@ def test_c5_flex_at_full_size_over_8_iterations(resident):
         t.close()
     if default_kernel_choice():
         assert names == ["special:flex_relu_fma_k0"], names
+
+
+@pytest.mark.parametrize("classes,samples,kept", [(10, 4194304, "12 rows in registers"), (1000, 32768, "streamed"),
+                                                  (100, 327680, "8 rows in registers")])
+def test_softmax_over_classes_at_full_size(classes, samples, kept):
+    """ng.softmax in the neon layout -- classes x samples, the reduced axis the strided one
+    (op_graph.py:3849, frontends/neon/activation.py:145-158) -- at the sizes the shape survey of
+    bench.py times: the three kernels of the graph as ONE column chain, against the NumPy
+    statements of the CPU transformer and against float64; every column sums to one."""
+    rs = np.random.RandomState(11)
+    x_np = rs.normal(0, 2, (classes, samples)).astype(np.float32)
+    t = ngt.make_transformer_factory("hipgpu")()
+    try:
+        A, B = ng.make_axis(classes, name="A"), ng.make_axis(samples, name="B")
+        x = ng.placeholder([A, B])
+        e = ng.exp(x - ng.max(x, out_axes=[B]))
+        f = t.computation(e / ng.sum(e, out_axes=[B]), x)
+        first = np.array(f(x_np)).copy()              # (may still run on the interpreter)
+        assert t.kernel_groups[f].wait_for_programs(timeout=600) is None
+        y = np.array(f(x_np)).copy()
+        names = _kernel_names(t, f)
+    finally:
+        t.close()
+    if default_kernel_choice():
+        assert len(names) >= 1 and all("/column-chain-of-3" in n for n in names), names
+    # the CPU transformer's statements, in float32
+    m = x_np.max(axis=0)
+    ew = np.exp(x_np - m)
+    want = ew / ew.sum(axis=0, dtype=np.float32)
+    np.testing.assert_allclose(y, want, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(first, want, rtol=RTOL, atol=ATOL)
+    x64 = x_np.astype(np.float64)
+    e64 = np.exp(x64 - x64.max(axis=0))
+    np.testing.assert_allclose(y, e64 / e64.sum(axis=0), rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(y.sum(axis=0, dtype=np.float64), 1.0, rtol=0, atol=1e-5)
