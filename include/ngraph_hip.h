@@ -86,7 +86,7 @@ extern "C" {
  * :70-77 (_redop_templates).  Arithmetic follows the NumPy float32 calls the
  * CPU transformer issues (cputransform.py:512-761) wherever the CUDA template
  * and NumPy disagree (floor_divide / mod on negative operands, sign of NaN).
- * All registers are fp32.                                                    */
+ * Registers are fp32 unless an op says otherwise (the integer ops at the end). */
 enum ngh_opcode {
     NGH_OP_NOP = 0,
     /* data movement: LOAD dst=reg a=tensor ; STORE dst=tensor a=reg ;
@@ -122,6 +122,21 @@ enum ngh_opcode {
      * (Box-Muller).  The streams differ from the reference's (curand / numpy), as those two
      * differ from each other; only the distributions can be compared.                      */
     NGH_OP_RNG_UNIFORM, NGH_OP_RNG_NORMAL,
+    /* 32-bit integer arithmetic.  The reference keeps int32 / uint32 operands in `int` /
+     * `unsigned int` registers (float_ew2.py:615-641 _get_register_type) and NumPy computes
+     * integer inputs with its integer loops before it casts to the output type
+     * (cputransform.py:512-761 hands the arrays to the ufuncs as they are): where every
+     * operand of an op is such an integer the arithmetic is integer arithmetic, exact over the
+     * whole range and wrapping at 2^32.  A register holds 32 bits either way; these ops read
+     * and write them as integers.  A tensor whose elements they produce or consume is bound as
+     * NGH_F32, so that LOAD and STORE move its bits untouched.
+     * unary: I2F / U2F = (float)int32 / (float)uint32, INEG, IABS (as int32)              */
+    NGH_OP_I2F, NGH_OP_U2F, NGH_OP_INEG, NGH_OP_IABS,
+    /* binary: IADD, ISUB, IMUL wrap (the same bits for int32 and uint32); IMIN / IMAX and
+     * UMIN / UMAX compare as int32 / uint32; the comparisons give 1.0f / 0.0f              */
+    NGH_OP_IADD, NGH_OP_ISUB, NGH_OP_IMUL, NGH_OP_IMIN, NGH_OP_IMAX, NGH_OP_UMIN, NGH_OP_UMAX,
+    NGH_OP_IEQ, NGH_OP_INE, NGH_OP_ILT, NGH_OP_ILE, NGH_OP_IGT, NGH_OP_IGE,
+    NGH_OP_ULT, NGH_OP_ULE, NGH_OP_UGT, NGH_OP_UGE,
     NGH_OP_COUNT_
 };
 

@@ -148,6 +148,14 @@ __device__ __forceinline__ float op_unary(int opc, float x) {
         case NGH_OP_SGN:     return np_sign(x);
         case NGH_OP_SIN:     return sinf(x);
         case NGH_OP_COS:     return cosf(x);
+        // integer ops: the register's bits read as int32 / uint32
+        case NGH_OP_I2F:     return (float)__float_as_int(x);
+        case NGH_OP_U2F:     return (float)__float_as_uint(x);
+        case NGH_OP_INEG:    return __uint_as_float(0u - __float_as_uint(x));
+        case NGH_OP_IABS: {
+            const int i = __float_as_int(x);
+            return __uint_as_float(i < 0 ? 0u - (unsigned)i : (unsigned)i);
+        }
         default:             return x;
     }
 }
@@ -169,13 +177,45 @@ __device__ __forceinline__ float op_binary(int opc, float x, float y) {
         case NGH_OP_POW: return powf(x, y);
         case NGH_OP_MINIMUM: return np_minimum(x, y);
         case NGH_OP_MAXIMUM: return np_maximum(x, y);
+        default: break;
+    }
+    // integer ops: both registers' bits read as int32 / uint32 (unsigned arithmetic wraps)
+    const unsigned ux = __float_as_uint(x), uy = __float_as_uint(y);
+    const int ix = (int)ux, iy = (int)uy;
+    switch (opc) {
+        case NGH_OP_IADD: return __uint_as_float(ux + uy);
+        case NGH_OP_ISUB: return __uint_as_float(ux - uy);
+        case NGH_OP_IMUL: return __uint_as_float(ux * uy);
+        case NGH_OP_IMIN: return __int_as_float(ix < iy ? ix : iy);
+        case NGH_OP_IMAX: return __int_as_float(ix > iy ? ix : iy);
+        case NGH_OP_UMIN: return __uint_as_float(ux < uy ? ux : uy);
+        case NGH_OP_UMAX: return __uint_as_float(ux > uy ? ux : uy);
+        case NGH_OP_IEQ: return (ix == iy) ? 1.0f : 0.0f;
+        case NGH_OP_INE: return (ix != iy) ? 1.0f : 0.0f;
+        case NGH_OP_ILT: return (ix <  iy) ? 1.0f : 0.0f;
+        case NGH_OP_ILE: return (ix <= iy) ? 1.0f : 0.0f;
+        case NGH_OP_IGT: return (ix >  iy) ? 1.0f : 0.0f;
+        case NGH_OP_IGE: return (ix >= iy) ? 1.0f : 0.0f;
+        case NGH_OP_ULT: return (ux <  uy) ? 1.0f : 0.0f;
+        case NGH_OP_ULE: return (ux <= uy) ? 1.0f : 0.0f;
+        case NGH_OP_UGT: return (ux >  uy) ? 1.0f : 0.0f;
+        case NGH_OP_UGE: return (ux >= uy) ? 1.0f : 0.0f;
         default: return x;
     }
 }
 
-__host__ __device__ __forceinline__ bool is_unary(int opc)  { return opc >= NGH_OP_ASSIGN && opc <= NGH_OP_COS; }
-__host__ __device__ __forceinline__ bool is_binary(int opc) { return opc >= NGH_OP_ADD && opc <= NGH_OP_MAXIMUM; }
-__host__ __device__ __forceinline__ bool is_reduce(int opc) { return opc >= NGH_OP_RED_SUM && opc <= NGH_OP_RED_ARGMIN; }
+__host__ __device__ constexpr bool is_unary(int opc) {
+    return (opc >= NGH_OP_ASSIGN && opc <= NGH_OP_COS) || (opc >= NGH_OP_I2F && opc <= NGH_OP_IABS);
+}
+__host__ __device__ constexpr bool is_binary(int opc) {
+    return (opc >= NGH_OP_ADD && opc <= NGH_OP_MAXIMUM) || (opc >= NGH_OP_IADD && opc <= NGH_OP_UGE);
+}
+__host__ __device__ constexpr bool is_reduce(int opc) { return opc >= NGH_OP_RED_SUM && opc <= NGH_OP_RED_ARGMIN; }
+// (ops that cost about as much as a handful of additions: transcendentals, division, power)
+__host__ __device__ constexpr bool is_slow_op(int opc) {
+    return (opc >= NGH_OP_EXP && opc <= NGH_OP_COS && opc != NGH_OP_RCP && opc != NGH_OP_SGN) || opc == NGH_OP_POW ||
+           opc == NGH_OP_DIV;
+}
 
 // ---------------------------------------------------------------------------
 // flex16 conversion (float_ew2.py:96-97, 261-277): load = scale * mantissa;

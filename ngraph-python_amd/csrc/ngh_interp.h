@@ -245,6 +245,7 @@ __device__ __forceinline__ void run_ops(const KArgs& k, LdsRegs<V>& rf, Extra& e
             NGH_UN(NGH_OP_SQR) NGH_UN(NGH_OP_EXP) NGH_UN(NGH_OP_LOG) NGH_UN(NGH_OP_RCP)
             NGH_UN(NGH_OP_EXP2) NGH_UN(NGH_OP_LOG2) NGH_UN(NGH_OP_SIG) NGH_UN(NGH_OP_TANH)
             NGH_UN(NGH_OP_SAFELOG) NGH_UN(NGH_OP_SGN) NGH_UN(NGH_OP_SIN) NGH_UN(NGH_OP_COS)
+            NGH_UN(NGH_OP_I2F) NGH_UN(NGH_OP_U2F) NGH_UN(NGH_OP_INEG) NGH_UN(NGH_OP_IABS)
 #undef NGH_UN
 #define NGH_BIN(OPC)                                                                  \
     case OPC: {                                                                       \
@@ -255,6 +256,11 @@ __device__ __forceinline__ void run_ops(const KArgs& k, LdsRegs<V>& rf, Extra& e
             NGH_BIN(NGH_OP_INT_DIV) NGH_BIN(NGH_OP_MOD) NGH_BIN(NGH_OP_EQ) NGH_BIN(NGH_OP_NE)
             NGH_BIN(NGH_OP_LT) NGH_BIN(NGH_OP_LE) NGH_BIN(NGH_OP_GT) NGH_BIN(NGH_OP_GE)
             NGH_BIN(NGH_OP_POW) NGH_BIN(NGH_OP_MINIMUM) NGH_BIN(NGH_OP_MAXIMUM)
+            NGH_BIN(NGH_OP_IADD) NGH_BIN(NGH_OP_ISUB) NGH_BIN(NGH_OP_IMUL) NGH_BIN(NGH_OP_IMIN)
+            NGH_BIN(NGH_OP_IMAX) NGH_BIN(NGH_OP_UMIN) NGH_BIN(NGH_OP_UMAX) NGH_BIN(NGH_OP_IEQ)
+            NGH_BIN(NGH_OP_INE) NGH_BIN(NGH_OP_ILT) NGH_BIN(NGH_OP_ILE) NGH_BIN(NGH_OP_IGT)
+            NGH_BIN(NGH_OP_IGE) NGH_BIN(NGH_OP_ULT) NGH_BIN(NGH_OP_ULE) NGH_BIN(NGH_OP_UGT)
+            NGH_BIN(NGH_OP_UGE)
 #undef NGH_BIN
             case NGH_OP_RED_SUM: case NGH_OP_RED_PROD: case NGH_OP_RED_MAX:
             case NGH_OP_RED_MIN: case NGH_OP_RED_ARGMAX: case NGH_OP_RED_ARGMIN: {

@@ -34,11 +34,15 @@ _OPCODE_NAMES = [
     "pow", "minimum", "maximum",
     "sum", "prod", "max", "min", "argmax", "argmin",
     "take", "store_trunc", "rng_uniform", "rng_normal",
+    # 32-bit integer arithmetic on the registers' bits (include/ngraph_hip.h)
+    "i2f", "u2f", "ineg", "iabs",
+    "iadd", "isub", "imul", "imin", "imax", "umin", "umax",
+    "ieq", "ine", "ilt", "ile", "igt", "ige", "ult", "ule", "ugt", "uge",
 ]
 #: op name (the reference's template names, float_ew2.py:31-77) -> opcode
 OPCODES = {name: i for i, name in enumerate(_OPCODE_NAMES)}
-UNARY_OPS = _OPCODE_NAMES[OPCODES["assign"]:OPCODES["cos"] + 1]
-BINARY_OPS = _OPCODE_NAMES[OPCODES["add"]:OPCODES["maximum"] + 1]
+UNARY_OPS = _OPCODE_NAMES[OPCODES["assign"]:OPCODES["cos"] + 1] + _OPCODE_NAMES[OPCODES["i2f"]:OPCODES["iabs"] + 1]
+BINARY_OPS = _OPCODE_NAMES[OPCODES["add"]:OPCODES["maximum"] + 1] + _OPCODE_NAMES[OPCODES["iadd"]:OPCODES["uge"] + 1]
 REDUCTION_OPS = _OPCODE_NAMES[OPCODES["sum"]:OPCODES["argmin"] + 1]
 
 

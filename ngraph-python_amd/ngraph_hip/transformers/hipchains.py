@@ -70,7 +70,9 @@ class ChainKernel(HipKernel):
             parts = None
         else:
             parts = [m._collect() for m in members]
-        return None if parts is None else cls._merge_parts(transformer, members, parts)
+        if parts is None or any(getattr(m, "raw_slots", None) for m in members):
+            return None      # (tensors bound for integer registers: a chain binds every operand by its own type)
+        return cls._merge_parts(transformer, members, parts)
 
     @staticmethod
     def _parts_after_moments(t, moments, rest):

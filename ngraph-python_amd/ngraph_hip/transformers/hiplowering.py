@@ -100,6 +100,32 @@ def _view_key(td):
     return (td.base, td.parameter_key)
 
 
+class _MixedIntegerUse(Exception):
+    """A kernel would move an integer tensor as bits and also write it through a conversion."""
+
+
+def _int_kind_of(dtype):
+    """"i" for int32, "u" for uint32, else None."""
+    if not isinstance(dtype, (np.dtype, type)):
+        return None
+    dtype = np.dtype(dtype)
+    return "i" if dtype == np.dtype(np.int32) else ("u" if dtype == np.dtype(np.uint32) else None)
+
+
+# Integer forms of the ops whose NumPy integer loop and whose C operator agree and wrap the same
+# way (cputransform.py:512-761 hands integer arrays to the ufuncs as they are; division and
+# remainder are not among them: NumPy divides integers in floating point and takes the floored
+# remainder, C truncates).
+_COMPARISONS = ("eq", "ne", "lt", "le", "gt", "ge")
+_INT_UNARY = {"neg": "ineg", "abs": "iabs"}
+_INT_BINARY = {
+    "i": {"add": "iadd", "sub": "isub", "mul": "imul", "minimum": "imin", "maximum": "imax",
+          "eq": "ieq", "ne": "ine", "lt": "ilt", "le": "ile", "gt": "igt", "ge": "ige"},
+    "u": {"add": "iadd", "sub": "isub", "mul": "imul", "minimum": "umin", "maximum": "umax",
+          "eq": "ieq", "ne": "ine", "lt": "ult", "le": "ule", "gt": "ugt", "ge": "uge"},
+}
+
+
 class HipKernel(object):
     """One launchable unit of a computation (gpu/kernel.py:18-87)."""
 
@@ -221,10 +247,21 @@ class FusedKernel(HipKernel):
             self._lower()
         super(FusedKernel, self).bind_buffers()
 
+    integer_registers = True     # (a flex kernel has none: every tensor of it is flex16)
+
     def _collect(self):
         """Pass 1 of the lowering: the operands (views) the group touches and its program over
         symbolic registers; returns (operands, program, it_axes, red_axes, onehot_axes,
-        take_axes, take_strides)."""
+        take_axes, take_strides).  Sets self.raw_slots."""
+        try:
+            return self._collect_once()
+        except _MixedIntegerUse:
+            # an integer tensor that this kernel both moves as bits and writes through a
+            # conversion: one binding cannot serve both, so the kernel keeps floats throughout
+            self.integer_registers = False
+            return self._collect_once()
+
+    def _collect_once(self):
         ops = self.ops
         reductions = [op for op in ops if isinstance(op, og.ReductionOp) and op.reduction_axes.size > 1]
         # (a kernel may carry a few ops over a subset of its axes, absorbed from a smaller kernel:
@@ -243,6 +280,13 @@ class FusedKernel(HipKernel):
         program = []             # tuples, see _emit below
         value_reg = {}           # producing op / view key -> symbolic register
         n_sym = [0]
+        # Registers that hold 32-bit integers as integers ("i": int32, "u": uint32) rather than
+        # as floats: what the reference declares `int` / `unsigned int` (float_ew2.py:615-641).
+        # Values loaded from int32 / uint32 tensors start out that way; an op all of whose
+        # operands do is integer arithmetic (NumPy's integer loops, C's integer operators),
+        # anything else converts them to float first.
+        int_kind = {}            # symbolic register -> "i" | "u"
+        self.raw_slots = set()   # operand slots whose 32-bit integers move as plain bits
 
         def new_reg():
             n_sym[0] += 1
@@ -271,9 +315,44 @@ class FusedKernel(HipKernel):
                 return value_reg[key]
             r = new_reg()
             program.append(("load", r, slot(td)))
+            kind = _int_kind_of(td.dtype)
+            if kind is not None and self.integer_registers and self.transformer.flex_entry_of(td) is None:
+                if slot(td) in converted_slots:
+                    raise _MixedIntegerUse()
+                int_kind[r] = kind
+                self.raw_slots.add(slot(td))
             value_reg[key] = r
             return r
 
+        def as_float(r):
+            """The register itself, or a float copy of the integer it holds."""
+            kind = int_kind.get(r)
+            if kind is None:
+                return r
+            f = new_reg()
+            program.append(("i2f" if kind == "i" else "u2f", f, r))
+            return f
+
+        def store(td, r):
+            """STORE of register r into the operand td: integers into an integer tensor of the
+            same kind go as they are, anything else through the store's own conversion."""
+            s_ = slot(td)
+            kind = int_kind.get(r)
+            if kind is not None and kind == _int_kind_of(td.dtype) and s_ not in converted_slots:
+                self.raw_slots.add(s_)
+                program.append(("store", s_, r))
+                return
+            converting(s_)
+            program.append(("store", s_, as_float(r)))
+
+        def converting(s_):
+            """Slot s_ is written through the library's own conversion (a float into an integer
+            tensor, a fill, a reduction's result)."""
+            if s_ in self.raw_slots:
+                raise _MixedIntegerUse()
+            converted_slots.add(s_)
+
+        converted_slots = set()  # integer tensors written through a conversion
         red_slots = []
         reductions_at_end = []
         for op in ops:
@@ -282,18 +361,19 @@ class FusedKernel(HipKernel):
                 target, val = op.args[0].forwarded, op.args[1].forwarded
                 r = operand_reg(val)
                 td = _td(target)
-                program.append(("store", slot(td), r))
+                store(td, r)
                 value_reg[_view_key(td)] = r
                 continue
             if isinstance(op, og.Fill):
                 td = _td(op.args[0].forwarded)
                 r = new_reg()
                 program.append(("const", r, float(op.scalar)))
+                converting(slot(td))
                 program.append((self.fill_store, slot(td), r))
                 value_reg[_view_key(td)] = r
                 continue
             if isinstance(op, og.OneHotOp):
-                x = operand_reg(op.args[0])
+                x = as_float(operand_reg(op.args[0]))
                 i = new_reg()
                 program.append(("iota", i, op.axis))
                 r = new_reg()
@@ -315,7 +395,7 @@ class FusedKernel(HipKernel):
             elif isinstance(op, og.LookupTableOp):
                 # gputransform.py:197-199: ("take", x=idx, y=lut, axis=lut_axis)
                 lut, idx = op.args[0].forwarded, op.args[1].forwarded
-                x = operand_reg(idx)
+                x = as_float(operand_reg(idx))
                 lut_td = _td(lut)
                 table = slot(lut_td)
                 out_axis = op.axes[op.lut_axis]
@@ -325,7 +405,7 @@ class FusedKernel(HipKernel):
                 r = new_reg()
                 program.append(("take", r, x, table, out_axis))
             elif isinstance(op, og.ReductionOp):
-                x = operand_reg(op.args[0])
+                x = as_float(operand_reg(op.args[0]))
                 if len(op.reduction_axes) == 0 or op.reduction_axes.size == 1:
                     # nothing to reduce: assign (gputransform.py:117-119, float_ew2.py:582-586)
                     r = new_reg()
@@ -335,20 +415,36 @@ class FusedKernel(HipKernel):
                         program.append(("assign", r, x))
                 else:
                     # reductions end the stage: collected here, emitted after every elementwise op
+                    converting(slot(_td(op)))
                     reductions_at_end.append(("reduce", name, x, slot(_td(op))))
                     red_slots.append(op)
                     continue
             elif name in og_unary_names:
                 x = operand_reg(op.args[0])
                 r = new_reg()
-                program.append((name, r, x))
+                kind = int_kind.get(x)
+                if kind == "i" and name in _INT_UNARY:
+                    program.append((_INT_UNARY[name], r, x))
+                    int_kind[r] = kind
+                else:
+                    program.append((name, r, as_float(x)))
             else:
                 x, y = operand_reg(op.args[0]), operand_reg(op.args[1])
                 r = new_reg()
-                program.append((name, r, x, y))
+                kind = int_kind.get(x)
+                if kind is not None and kind == int_kind.get(y) and name in _INT_BINARY[kind]:
+                    program.append((_INT_BINARY[kind][name], r, x, y))
+                    if name not in _COMPARISONS:          # (a comparison gives 1.0 / 0.0)
+                        int_kind[r] = kind
+                else:
+                    program.append((name, r, as_float(x), as_float(y)))
+            if r in int_kind and _int_kind_of(op.dtype) != int_kind[r]:
+                # the op's own type is not that integer type: its value is converted, as an
+                # assignment to a `float` register converts in C
+                r = as_float(r)
             value_reg[op] = r
             if op in self.store_ops:
-                program.append(("store", slot(_td(op)), r))
+                store(_td(op), r)
 
         program.extend(reductions_at_end)
         return operands, program, it_axes, red_axes, onehot_axes, take_axes, take_strides
@@ -446,19 +542,13 @@ class FusedKernel(HipKernel):
         shape = [d.length for d in inner] or [1]
         nd = len(inner)
         sb = FusedSpecBuilder(shape)
-        # Registers are fp32 (as in the reference's kernels wherever an integer meets a float:
-        # float_ew2.py:615-641), which is exact for integers up to 2**24 only.  A kernel that
-        # merely moves 32-bit integers declares them fp32: loads, register moves and stores pass
-        # the bits through untouched, so the move is exact over the whole range.
-        def is_dtype(td, numpy_type):
-            return isinstance(td.dtype, (np.dtype, type)) and np.dtype(td.dtype) == np.dtype(numpy_type)
-
-        moves_bits = (all(p[0] in ("load", "store", "assign") for p in program) and
-                      any(all(is_dtype(td, kind) for td in operands) for kind in (np.int32, np.uint32)))
+        # Integer tensors whose elements the program handles as integers (self.raw_slots: loaded
+        # into integer registers, stored from them) are bound as fp32: LOAD, register moves and
+        # STORE then pass their 32 bits through untouched; conversions are ops of the program.
         for s, td in enumerate(operands):
             view = t.get_tensor_description_tensor_view(td)
             strides = [d.strides[s] for d in inner] or [0]
-            dtype = t.ngh_dtype(np.dtype(np.float32) if moves_bits else td.dtype)
+            dtype = t.ngh_dtype(np.dtype(np.float32) if s in self.raw_slots else td.dtype)
             slot = sb.tensor(view.ptr + offsets[s] * view.itemsize, strides, dtype,
                              take_extent=self.take_extents.get(s, 0))
             assert slot == s

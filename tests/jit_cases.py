@@ -67,6 +67,16 @@ def case_mixed_storage_types():
     return [ng.minimum(x * h, 4.0) + i, ng.sum(h * x, out_axes=[B])], [x, h, i]
 
 
+def case_integer_arithmetic():
+    # int32 operands meeting each other: integer ops on the registers' bits, conversions as ops
+    # of the program, the integer tensors bound so that loads and stores move bits
+    A, B = _ab()
+    i, j = ng.placeholder([A, B], dtype=np.int32), ng.placeholder([A, B], dtype=np.int32)
+    x = ng.placeholder([A, B])
+    k = ng.add(ng.multiply(i, j, dtype=np.int32), j, dtype=np.int32)
+    return [k, ng.maximum(i, j) * x + ng.less(i, j), ng.sum(ng.subtract(i, j, dtype=np.int32), out_axes=[B])], [i, j, x]
+
+
 def case_ragged():
     # extents that leave a tail after the vector-wide part and rows that are not a multiple of 4
     A, B = ng.make_axis(301, name="A"), ng.make_axis(77, name="B")
@@ -221,7 +231,8 @@ def case_row_statistics_chain():
 
 
 FP32_CASES = [case_elementwise, case_column_reduction_with_store, case_row_reduction_with_store,
-              case_transposed_operand, case_transposed_operands_large, case_softmax, case_mixed_storage_types, case_ragged,
+              case_transposed_operand, case_transposed_operands_large, case_softmax, case_mixed_storage_types,
+              case_integer_arithmetic, case_ragged,
               case_ragged_long_rows, case_ragged_many_rows, case_softmax_ragged_rows, case_softmax_long_rows, case_softmax_over_windows,
               case_softmax_forward_and_backward,
               case_row_chain_with_stored_intermediate, case_misaligned_slices, case_short_rows, case_dropout, case_lookup_table,

@@ -623,6 +623,63 @@ def test_moving_32_bit_integers_keeps_every_bit(backend):
         np.testing.assert_array_equal(got, np.array(values, dtype=dtype))
 
 
+def test_integer_operands_meet_in_integer_arithmetic(backend):
+    """An op all of whose operands are int32 (or all uint32) computes as NumPy's integer loops
+    and C's integer operators do -- exactly, wrapping at 2**32 -- and only its result is
+    converted to the op's own type (float_ew2.py:615-641: `int` registers; cputransform.py hands
+    the integer arrays to the ufuncs as they are).  Where an integer meets a float the integer
+    is converted first."""
+    ax = axes(H=8)
+    a = np.array([16777217, 2 ** 31 - 1, -2 ** 31, 123456789, -16777219, 5, -7, 0], dtype=np.int32)
+    b = np.array([16777217, 1, -1, 987654321, 3, -5, 7, 0], dtype=np.int32)
+    x, y = ng.placeholder(ax, dtype=np.int32), ng.placeholder(ax, dtype=np.int32)
+    results = [x + y, x - y, x * y, ng.maximum(x, y), ng.minimum(x, y), -x, ng.absolute(x),
+               ng.equal(x, y), ng.less(x, y), ng.greater_equal(x, y),
+               ng.add(x, y, dtype=np.int32),                                   # stays an integer
+               (x + y) * 0.5,                                                   # converted, then float
+               ng.multiply(ng.add(x, y, dtype=np.int32), ng.subtract(x, y, dtype=np.int32))]
+    with np.errstate(over="ignore"):
+        s, d = a + b, a - b
+        want = [s.astype(np.float32), d.astype(np.float32), (a * b).astype(np.float32),
+                np.maximum(a, b).astype(np.float32), np.minimum(a, b).astype(np.float32),
+                (-a).astype(np.float32), np.abs(a).astype(np.float32),
+                (a == b).astype(np.float32), (a < b).astype(np.float32), (a >= b).astype(np.float32),
+                s, s.astype(np.float32) * np.float32(0.5), (s * d).astype(np.float32)]
+    with executor(results, x, y) as f:
+        got = f(a, b)
+    for i, (g, w) in enumerate(zip(got, want)):
+        g = np.array(g)
+        assert g.dtype == w.dtype, (i, g.dtype, w.dtype)
+        np.testing.assert_array_equal(g, w, err_msg="result %d" % i)
+    # unsigned: wraps modulo 2**32, compares as unsigned
+    ua = np.array([2 ** 32 - 1, 2 ** 31 + 5, 16777217, 7, 0, 4000000000, 1, 2 ** 31], dtype=np.uint32)
+    ub = np.array([1, 2 ** 31 + 5, 16777217, 9, 0, 300000000, 2 ** 32 - 1, 2 ** 31 - 1], dtype=np.uint32)
+    u, v = ng.placeholder(ax, dtype=np.uint32), ng.placeholder(ax, dtype=np.uint32)
+    with np.errstate(over="ignore"):
+        want = [(ua + ub).astype(np.float32), (ua * ub).astype(np.float32), np.maximum(ua, ub).astype(np.float32),
+                (ua < ub).astype(np.float32), (ua >= ub).astype(np.float32), ua + ub]
+    with executor([u + v, u * v, ng.maximum(u, v), ng.less(u, v), ng.greater_equal(u, v),
+                   ng.add(u, v, dtype=np.uint32)], u, v) as f:
+        got = f(ua, ub)
+    for i, (g, w) in enumerate(zip(got, want)):
+        g = np.array(g)
+        assert g.dtype == w.dtype, (i, g.dtype, w.dtype)
+        np.testing.assert_array_equal(g, w, err_msg="unsigned result %d" % i)
+
+
+def test_integer_tensor_moved_and_written_through_a_conversion_in_one_kernel(backend):
+    """The same int32 tensor read as integers and overwritten with a float result in one kernel:
+    one binding cannot serve both ways, so such a kernel keeps floats throughout (values below
+    2**24 are exact either way)."""
+    ax = axes(H=6)
+    v = ng.variable(ax, dtype=np.int32, initial_value=np.array([1, -2, 3, 70000, -5, 6], dtype=np.int32))
+    x = ng.placeholder(ax, dtype=np.int32)
+    step = ng.sequential([ng.assign(v, (v + x) * 0.5), v])
+    with executor(step, x) as f:
+        got = np.array(f(np.array([3, 4, -9, 10, 5, 1], dtype=np.int32)))
+    np.testing.assert_array_equal(got, np.array([2, 1, -3, 35005, 0, 3], dtype=np.int32))
+
+
 def test_multiply_uint32_scalar(backend):
     x = ng.placeholder((), dtype=np.uint32)
     with executor(0.5 * x * 0.5, x) as f:
