@@ -59,9 +59,10 @@ extern "C" {
 #define NGH_F16     3          /* IEEE half in memory, float in registers   */
 /* Integer storage: converted to float on load; a store converts toward zero and
  * saturates at the type's range (the device conversion the reference's generated
- * "(type)reg" assignment compiles to).  Registers are fp32, so integer values are exact up to
- * 2^24 (the reference keeps int32 / uint32 operands in integer registers, float_ew2.py:615-641).
- * Where an index could exceed that, the library keeps it an integer or refuses the spec with
+ * "(type)reg" assignment compiles to).  A value converted this way is exact up to 2^24; a caller
+ * that wants the reference's integer registers (float_ew2.py:615-641) binds the int32 / uint32
+ * tensor as NGH_F32, which moves its bits untouched, and uses the integer ops at the end of
+ * the opcode list.  Where an index could exceed 2^24, the library keeps it an integer or refuses the spec with
  * NGH_E_UNSUPPORTED instead of losing bits: argmax / argmin into NGH_I32 / NGH_U32 storage
  * store the integer index itself (over more than 2^24 elements any other result type is
  * refused); NGH_OP_TAKE from a table of more than 2^24 entries along the looked-up axis and

@@ -41,8 +41,13 @@ _OPCODE_NAMES = [
 ]
 #: op name (the reference's template names, float_ew2.py:31-77) -> opcode
 OPCODES = {name: i for i, name in enumerate(_OPCODE_NAMES)}
-UNARY_OPS = _OPCODE_NAMES[OPCODES["assign"]:OPCODES["cos"] + 1] + _OPCODE_NAMES[OPCODES["i2f"]:OPCODES["iabs"] + 1]
-BINARY_OPS = _OPCODE_NAMES[OPCODES["add"]:OPCODES["maximum"] + 1] + _OPCODE_NAMES[OPCODES["iadd"]:OPCODES["uge"] + 1]
+#: ops that read and write a register's 32 bits as an integer
+INTEGER_UNARY_OPS = _OPCODE_NAMES[OPCODES["i2f"]:OPCODES["iabs"] + 1]
+INTEGER_BINARY_OPS = _OPCODE_NAMES[OPCODES["iadd"]:OPCODES["uge"] + 1]
+FLOAT_UNARY_OPS = _OPCODE_NAMES[OPCODES["assign"]:OPCODES["cos"] + 1]
+FLOAT_BINARY_OPS = _OPCODE_NAMES[OPCODES["add"]:OPCODES["maximum"] + 1]
+UNARY_OPS = FLOAT_UNARY_OPS + INTEGER_UNARY_OPS
+BINARY_OPS = FLOAT_BINARY_OPS + INTEGER_BINARY_OPS
 REDUCTION_OPS = _OPCODE_NAMES[OPCODES["sum"]:OPCODES["argmin"] + 1]
 
 

@@ -11,7 +11,9 @@ Pinning status (what checks each restatement beyond itself):
   numpy_ops.py      closed forms: each entry IS the NumPy ufunc call the CPU
                     transformer emits; tests/test_cabi_fused_gpu.py and
                     tests/test_execution.py check them against float64 references
-                    and NumPy expressions written in each test.
+                    and NumPy expressions written in each test.  Its integer ops
+                    (int32 / uint32 operands) are pinned against arithmetic on
+                    Python integers modulo 2^32 in tests/test_oracle_integer_ops.py.
   configs.py        BatchNorm / Adam / LSTM pinned against independent float64
                     restatements of the reference's own test references
                     (neon/tests/test_batchnorm_layer.py:35-58,

@@ -96,6 +96,46 @@ def binary(name, x, y):
     return out
 
 
+# Integer operands: the CPU transformer hands int32 / uint32 arrays to the same ufuncs
+# (cputransform.py:512-761), and NumPy then runs its integer loop (exact, wrapping at 2^32)
+# and casts the result to `out`'s type; the GPU transformer keeps such operands in `int` /
+# `unsigned int` registers (float_ew2.py:615-641).  Names are the device library's: a
+# leading "i" reads int32, "u" uint32.
+INTEGER_UNARY = {
+    "i2f": (np.int32, lambda x: x.astype(f32)),
+    "u2f": (np.uint32, lambda x: x.astype(f32)),
+    "ineg": (np.int32, np.negative),           # :694-696
+    "iabs": (np.int32, np.abs),                # :512-514
+}
+
+INTEGER_BINARY = {
+    "iadd": (np.int32, np.add), "isub": (np.int32, np.subtract), "imul": (np.int32, np.multiply),
+    "imin": (np.int32, np.minimum), "imax": (np.int32, np.maximum),
+    "umin": (np.uint32, np.minimum), "umax": (np.uint32, np.maximum),
+    "ieq": (np.int32, np.equal), "ine": (np.int32, np.not_equal),
+    "ilt": (np.int32, np.less), "ile": (np.int32, np.less_equal),
+    "igt": (np.int32, np.greater), "ige": (np.int32, np.greater_equal),
+    "ult": (np.uint32, np.less), "ule": (np.uint32, np.less_equal),
+    "ugt": (np.uint32, np.greater), "uge": (np.uint32, np.greater_equal),
+}
+
+
+def integer_unary(name, x):
+    """`x` holds 32-bit patterns (any 4-byte dtype); the result has the integer type of the op,
+    float32 for the conversions."""
+    kind, fn = INTEGER_UNARY[name]
+    with np.errstate(all="ignore"):
+        return fn(np.asarray(x).view(kind))
+
+
+def integer_binary(name, x, y):
+    """As `integer_unary`; comparisons return 0.0 / 1.0 in float32 like `binary`."""
+    kind, fn = INTEGER_BINARY[name]
+    with np.errstate(all="ignore"):
+        r = fn(np.asarray(x).view(kind), np.asarray(y).view(kind))
+    return r.astype(f32) if r.dtype == np.bool_ else r
+
+
 def reduce(name, x, axis):
     x = np.asarray(x, dtype=f32)
     with np.errstate(all="ignore"):

@@ -10,7 +10,8 @@ import pytest
 
 from oracle import configs, numpy_ops
 from ngraph_hip.runtime import FusedSpecBuilder, NGH_F32, NGH_I32
-from ngraph_hip.runtime.hiplib import UNARY_OPS, BINARY_OPS
+from ngraph_hip.runtime.hiplib import (FLOAT_UNARY_OPS, FLOAT_BINARY_OPS, INTEGER_UNARY_OPS,
+                                       INTEGER_BINARY_OPS)
 from conftest import default_kernel_choice
 
 pytestmark = pytest.mark.gpu
@@ -241,7 +242,7 @@ def test_c4_lstm_cell_transposed(hip_runtime, H, N):
         d.free()
 
 
-@pytest.mark.parametrize("name", [n for n in UNARY_OPS])
+@pytest.mark.parametrize("name", FLOAT_UNARY_OPS)
 def test_every_unary_op(hip_runtime, name):
     rt = hip_runtime
     rs = np.random.RandomState(11)
@@ -344,7 +345,7 @@ def test_sigmoid_and_pow_within_ulps_of_the_oracle(hip_runtime):
         d.free()
 
 
-@pytest.mark.parametrize("name", [n for n in BINARY_OPS])
+@pytest.mark.parametrize("name", FLOAT_BINARY_OPS)
 def test_every_binary_op(hip_runtime, name):
     rt = hip_runtime
     rs = np.random.RandomState(12)
@@ -389,7 +390,7 @@ def _assert_same_special(got, want, what, zero_sign=True):
     np.testing.assert_allclose(got[fin], want[fin], rtol=RTOL, atol=0, err_msg=what)
 
 
-@pytest.mark.parametrize("name", [n for n in UNARY_OPS])
+@pytest.mark.parametrize("name", FLOAT_UNARY_OPS)
 def test_unary_ops_on_special_values(hip_runtime, name):
     """Zeros of both signs, denormals, values that overflow exp, infinities and NaN go through
     every unary op like through the oracle's NumPy call (cputransform.py:512-761)."""
@@ -407,7 +408,7 @@ def test_unary_ops_on_special_values(hip_runtime, name):
     _assert_same_special(got, want, name)
 
 
-@pytest.mark.parametrize("name", [n for n in BINARY_OPS])
+@pytest.mark.parametrize("name", FLOAT_BINARY_OPS)
 def test_binary_ops_on_special_values(hip_runtime, name):
     """Every pair of the special values through every binary op: division and remainder by zero,
     NaN in comparisons, minimum / maximum with NaN, powers of zero and of negative numbers."""
@@ -425,6 +426,52 @@ def test_binary_ops_on_special_values(hip_runtime, name):
     # maximum(+0, -0): NumPy's vector loop returns the second operand and its scalar loop (the
     # last few elements of an array) the first, so the sign of that zero is not compared
     _assert_same_special(got, want, name, zero_sign=name not in ("minimum", "maximum"))
+
+
+def _integer_patterns(seed, n):
+    """32-bit patterns over the whole range with the edges of both integer types in front."""
+    rs = np.random.RandomState(seed)
+    x = rs.randint(0, 1 << 32, n, dtype=np.uint64).astype(np.uint32)
+    edges = np.array([0, 1, 2, 0x7fffffff, 0x80000000, 0x80000001, 0xffffffff, 0xfffffffe, 1 << 24, (1 << 24) + 1,
+                      0x00ffffff, 0x7f800000, 0xff800000, 0x7fc00000], dtype=np.uint32)   # incl. the bits of inf / NaN
+    x[:len(edges)] = edges
+    return x
+
+
+@pytest.mark.parametrize("name", INTEGER_UNARY_OPS)
+def test_every_integer_unary_op(hip_runtime, name):
+    """The integer ops read a register's bits as int32 / uint32: compared bit for bit with
+    NumPy's integer loops over the whole 32-bit range (tensors bound as fp32 move their bits)."""
+    rt = hip_runtime
+    x = _integer_patterns(21, 4099)
+    want = numpy_ops.integer_unary(name, x)
+    x_d, y_d = rt.array(x.view(f32)), rt.empty(x.shape)
+    sb = FusedSpecBuilder(x.shape)
+    tx, ty = sb.tensor(x_d.ptr, [1]), sb.tensor(y_d.ptr, [1])
+    sb.store(ty, sb.unary(name, sb.load(tx)))
+    rt.launch_fused(sb.build())
+    got = y_d.get()
+    x_d.free()
+    y_d.free()
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("name", INTEGER_BINARY_OPS)
+def test_every_integer_binary_op(hip_runtime, name):
+    rt = hip_runtime
+    x = _integer_patterns(22, 37 * 129)
+    y = _integer_patterns(23, 37 * 129)[::-1].copy()
+    y[::5] = x[::5]                                        # equal operands for the comparisons
+    want = numpy_ops.integer_binary(name, x, y)
+    x_d, y_d, z_d = rt.array(x.view(f32)), rt.array(y.view(f32)), rt.empty(x.shape)
+    sb = FusedSpecBuilder(x.shape)
+    tx, ty, tz = sb.tensor(x_d.ptr, [1]), sb.tensor(y_d.ptr, [1]), sb.tensor(z_d.ptr, [1])
+    sb.store(tz, sb.binary(name, sb.load(tx), sb.load(ty)))
+    rt.launch_fused(sb.build())
+    got = z_d.get()
+    for d in (x_d, y_d, z_d):
+        d.free()
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
 @pytest.mark.parametrize("name", ["sum", "prod", "max", "min", "argmax", "argmin"])
