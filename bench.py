@@ -607,6 +607,15 @@ def shape_survey_cases(ng):
         # kernels it is read three times)
         yield ("softmax of rows [%d,%d] (maximum, sum of exponentials, normalise)" % (rows, k),
                [e / ng.sum(e, out_axes=[R])], [w], {"chain": 2 * rows * k * 4, "kernels": 4 * rows * k * 4})
+    # the same softmax with flex16 storage (the flexhip transformer): the maximum, the sum and the
+    # result are flex16 tensors with an exponent each; 2 bytes per element either way
+    for rows, k in ((32768, 1024), (32768, 1000)):
+        R, K = ax(rows, "FR%d" % k), ax(k, "FK%d" % k)
+        w = ng.placeholder([R, K])
+        e = ng.exp(w - ng.max(w, out_axes=[R]))
+        yield ("flex16 softmax of rows [%d,%d] (maximum, sum of exponentials, normalise)" % (rows, k),
+               [e / ng.sum(e, out_axes=[R])], [w],
+               {"chain": 2 * rows * k * 2, "kernels": 4 * rows * k * 2, "transformer": "flexhip"})
     # classes x samples, the layout of the neon front end (op_graph.py:3849): the reduced axis is the
     # strided one; as one column-chain kernel the operand is read once (few classes: kept in
     # registers) or re-read from the caches by the later stages
@@ -633,7 +642,7 @@ def shape_survey(ng, ngt, steps, warmup, only=""):
     for name, results, inputs, nbytes in shape_survey_cases(ng):
         if only and only not in name:
             continue
-        t = ngt.make_transformer_factory("hipgpu")()
+        t = ngt.make_transformer_factory(nbytes.get("transformer", "hipgpu") if isinstance(nbytes, dict) else "hipgpu")()
         try:
             f = t.computation(results, *inputs)
             values = [np.random.RandomState(i).uniform(0.5, 1.5, p.axes.lengths).astype(np.float32)

@@ -222,11 +222,18 @@ __host__ __device__ constexpr bool is_slow_op(int opc) {
 // store = cvt.rni.s16.f32(scale * value): round to nearest even, saturate to
 // [-32768, 32767], NaN -> 0; statistics = max |stored mantissa| as int32.
 // ---------------------------------------------------------------------------
+// The device's float -> int32 conversion as the instruction defines it: toward zero, values out
+// of range (infinities included) saturate, NaN gives 0.  A C cast leaves those cases undefined,
+// so code that relies on them asks for the instruction itself.
+__device__ __forceinline__ int cvt_i32_saturating(float v) {
+    int q;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(q) : "v"(v));
+    return q;
+}
+
 __device__ __forceinline__ int flex_quantize(float v) {
-    float r = rintf(v);                       // round-half-even in the default mode
-    r = fminf(fmaxf(r, -32768.0f), 32767.0f); // saturate (NaN -> -32768 by fmaxf, fixed below)
-    int q = (int)r;
-    return (v != v) ? 0 : q;
+    const int q = cvt_i32_saturating(rintf(v));   // round-half-even in the default mode; NaN -> 0
+    return min(max(q, -32768), 32767);
 }
 
 // ---------------------------------------------------------------------------
@@ -261,8 +268,7 @@ __device__ __forceinline__ float rng_normal(unsigned b0, unsigned b1) {
 
 // the fill rule: int(value / scale) cut toward zero, clipped (tensor_ops.py:690-707)
 __device__ __forceinline__ int flex_quantize_trunc(float v) {
-    const float r = fminf(fmaxf(truncf(v), -32768.0f), 32767.0f);   // (fmaxf drops a NaN: tested on v below)
-    return (v != v) ? 0 : (int)r;
+    return min(max(cvt_i32_saturating(v), -32768), 32767);          // (the conversion cuts toward zero; NaN -> 0)
 }
 
 __device__ __forceinline__ int iabs(int x) { return x < 0 ? -x : x; }

@@ -191,12 +191,40 @@ constexpr int kFlexPad = 32;            // ints between two counters: one 128-by
 constexpr int kFlexTicketWords = (kFlexGroups + 1) * kFlexPad;
 constexpr int kFlexGroupMaxWords = 4 * kFlexGroups * kFlexPad;
 
+// The last arrival's part: fold the group words of slots first, first + step, ... and apply the
+// policy to their records (one wavefront, all lanes).
 template <int NS>
-__device__ __forceinline__ void flex_epilogue(ngh_flex_state* const (&state)[4], const int (&in_place)[4],
-                                              int count, unsigned* tickets, int* group_max,
-                                              const int (&fmax)[4], int (*lds)[4] /* [NS][waves] */,
-                                              int ordered) {
+__device__ __forceinline__ void flex_epilogue_finish(ngh_flex_state* const (&state)[4], const int (&in_place)[4],
+                                                     int count, int* group_max, unsigned groups, int lane,
+                                                     int first, int step) {
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        if (s < first || (s - first) % step) continue;
+        int gm = 0;
+        if ((unsigned)lane < groups) {
+            int* w = group_max + (s * kFlexGroups + lane) * kFlexPad;
+            gm = __hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(w, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) gm = max(gm, __shfl_xor(gm, d, 64));
+        FlexInWave r = flex_wave_load(*state[s]);
+        const int dec = flex_write_dec(r.f, in_place[s]);
+        r.f.dec = dec;
+        r.f.scale = flex_scale_of(dec);
+        r.f.stats = gm;
+        flex_policy_step(r.f, r.h, gm, count);
+        flex_wave_store(*state[s], r);
+    }
+}
+
+// A workgroup's arrival (whole workgroup calls; what it returns is meaningful in the first
+// wavefront only: is this workgroup the grid's last arrival?)
+template <int NS>
+__device__ __forceinline__ int flex_epilogue_arrive(unsigned* tickets, int* group_max, const int (&fmax)[4],
+                                                    int (*lds)[4] /* [NS][waves] */, int ordered, unsigned& groups) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    groups = gridDim.x < (unsigned)kFlexGroups ? gridDim.x : (unsigned)kFlexGroups;
     int m[NS];
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
@@ -206,9 +234,8 @@ __device__ __forceinline__ void flex_epilogue(ngh_flex_state* const (&state)[4],
         if (lane == 0) lds[s][wave] = m[s];
     }
     __syncthreads();
-    if (wave != 0) return;
+    if (wave != 0) return 0;
     const unsigned g = blockIdx.x % kFlexGroups;
-    const unsigned groups = gridDim.x < (unsigned)kFlexGroups ? gridDim.x : (unsigned)kFlexGroups;
     int last = 0;
     if (lane == 0) {
         unsigned dep = 0;
@@ -243,28 +270,41 @@ __device__ __forceinline__ void flex_epilogue(ngh_flex_state* const (&state)[4],
             }
         }
     }
-    last = __shfl(last, 0, 64);
-    if (!last) return;
-    // the grid's last workgroup, first wavefront: lane g folds group g
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-        int gm = 0;
-        if ((unsigned)lane < groups) {
-            int* w = group_max + (s * kFlexGroups + lane) * kFlexPad;
-            gm = __hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(w, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-#pragma unroll
-        for (int d = 32; d > 0; d >>= 1) gm = max(gm, __shfl_xor(gm, d, 64));
-        FlexInWave r = flex_wave_load(*state[s]);
-        const int dec = flex_write_dec(r.f, in_place[s]);
-        r.f.dec = dec;
-        r.f.scale = flex_scale_of(dec);
-        r.f.stats = gm;
-        flex_policy_step(r.f, r.h, gm, count);
-        flex_wave_store(*state[s], r);
-    }
+    return __shfl(last, 0, 64);
 }
+
+template <int NS>
+__device__ __forceinline__ void flex_epilogue(ngh_flex_state* const (&state)[4], const int (&in_place)[4],
+                                              int count, unsigned* tickets, int* group_max,
+                                              const int (&fmax)[4], int (*lds)[4] /* [NS][waves] */,
+                                              int ordered) {
+    unsigned groups;
+    const int last = flex_epilogue_arrive<NS>(tickets, group_max, fmax, lds, ordered, groups);
+    if ((threadIdx.x >> 6) != 0 || !last) return;
+    // the grid's last workgroup, first wavefront: lane g folds group g
+    flex_epilogue_finish<NS>(state, in_place, count, group_max, groups, threadIdx.x & 63, 0, 1);
+}
+
+// The same with the last workgroup's wavefronts taking a record each (the policy step of a
+// record takes one wavefront a few microseconds, after everything else of the launch is done):
+// every wavefront waits to learn whether its workgroup came last.  For kernels that write
+// several flex tensors and whose workgroups are about to end anyway.
+template <int NS>
+__device__ __forceinline__ void flex_epilogue_wide(ngh_flex_state* const (&state)[4], const int (&in_place)[4],
+                                                   int count, unsigned* tickets, int* group_max,
+                                                   const int (&fmax)[4], int (*lds)[4] /* [NS][waves] */,
+                                                   int ordered) {
+    __shared__ int came_last;
+    unsigned groups;
+    const int last = flex_epilogue_arrive<NS>(tickets, group_max, fmax, lds, ordered, groups);
+    if (threadIdx.x == 0) came_last = last;
+    __syncthreads();
+    if (!came_last) return;
+    if (ordered) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    flex_epilogue_finish<NS>(state, in_place, count, group_max, groups, threadIdx.x & 63, (int)(threadIdx.x >> 6),
+                             (int)(blockDim.x >> 6));
+}
+
 
 // ---------------------------------------------------------------------------
 // Deferred statistics: no work at all after the last store.

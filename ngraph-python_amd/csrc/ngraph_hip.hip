@@ -407,7 +407,9 @@ bool vec4_ok(const KArgs& k, const bool* used) { return vec_ok(k, used, 4); }
 // Can the stage move 4 elements per lane along kernel axis 2 although vec_ok says no -- rows whose
 // length is not a multiple of 4, or that do not start on 16-byte boundaries?  The compiled
 // programs can (program_ragged_ok has the conditions on the program), given unit strides.
-bool ragged_rows_ok(const KArgs& k, const bool* used, bool row_stores = false) {
+// (chain: as a stage of a row chain, which also takes 16-bit operands whose every chunk of four
+// lies on a 4-byte boundary: an aligned start, rows an even number of elements apart)
+bool ragged_rows_ok(const KArgs& k, const bool* used, bool chain = false) {
     if (k.shape[2] < 8) return false;
     int dtypes[NGH_MAX_TENSORS];
     unsigned char bcast[NGH_MAX_TENSORS];
@@ -415,8 +417,14 @@ bool ragged_rows_ok(const KArgs& k, const bool* used, bool row_stores = false) {
         dtypes[t] = t < k.n_tensors ? k.t[t].dtype : NGH_F32;
         bcast[t] = (t < k.n_tensors && k.t[t].s[2] == 0) ? 1 : 0;
         if (t < k.n_tensors && used[t] && k.t[t].s[2] != 0 && k.t[t].s[2] != 1) return false;
+        if (t < k.n_tensors && used[t] && k.t[t].s[2] == 1 && itemsize_of(k.t[t].dtype) == 2) {
+            const KTensor& K = k.t[t];
+            if (((uintptr_t)K.p) % 4) return false;
+            for (int j = 0; j < 2; ++j)
+                if (k.shape[j] > 1 && K.s[j] % 2) return false;
+        }
     }
-    return program_ragged_ok(4, k.ops + k.op_begin, k.op_end - k.op_begin, dtypes, bcast, row_stores);
+    return program_ragged_ok(4, k.ops + k.op_begin, k.op_end - k.op_begin, dtypes, bcast, chain);
 }
 
 constexpr size_t kInterpLdsPreferred = 64 * 1024;   // keeps >= 2 workgroups per CU
@@ -1395,6 +1403,8 @@ static int stage_cache_policy(const ngh_context* ctx, const ngh_fused_spec& sp, 
 // of lanes of one wavefront each, and every stage can run over ragged rows (fp32 operands with
 // unit stride along the row, or broadcast along it).
 // ---------------------------------------------------------------------------
+constexpr int kChainManagedWgsPerCu = 8;    // grid of a chain launch that runs the exponent policy itself
+
 struct ChainPlan {
     int      n = 0;                       // stages (the spec's non-empty ones)
     int      stage_of[NGH_MAX_STAGES];
@@ -1402,6 +1412,7 @@ struct ChainPlan {
     KArgs    k[NGH_MAX_STAGES];
     unsigned n_out = 0, TR = 64;
     int      special = -1;
+    KArgs    launch;                      // what the chain's kernel is launched with (row chains)
 };
 
 // Do the byte ranges two operands span in the spec's iteration space intersect?
@@ -1443,12 +1454,14 @@ bool plan_row_chain(const ngh_context* ctx, const ngh_fused_spec& sp, ChainPlan&
         bool loads[NGH_MAX_TENSORS], stores[NGH_MAX_TENSORS], used[NGH_MAX_TENSORS];
         stage_tensors(sp, S, loads, stores);
         for (int t = 0; t < NGH_MAX_TENSORS; ++t) used[t] = loads[t] || stores[t];
-        if (k.n_stat_slots != 0 || k.probe || !ragged_rows_ok(k, used, true) ||
+        if (k.probe || !ragged_rows_ok(k, used, true) ||
             !program_loads_hoistable(k.ops + k.op_begin, k.op_end - k.op_begin))
             return false;
         for (int r = 0; r < S.n_reductions; ++r) {
             const ngh_tensor& T = sp.tensors[S.red_out[r]];
-            if (T.strides[0] != 0 || (T.dtype != NGH_F32 && T.dtype != NGH_I32 && T.dtype != NGH_U32)) return false;
+            if (T.strides[0] != 0 || (T.dtype != NGH_F32 && T.dtype != NGH_I32 && T.dtype != NGH_U32 &&
+                                      T.dtype != NGH_FLEX16 && T.dtype != NGH_F16))
+                return false;
         }
         any_red = any_red || S.n_reductions > 0;
         C.stage_of[C.n] = s;
@@ -1477,6 +1490,32 @@ bool plan_row_chain(const ngh_context* ctx, const ngh_fused_spec& sp, ChainPlan&
             for (int u = 0; u < sp.n_tensors; ++u)
                 if (u != t && used[u] && tensors_overlap(sp, sp.tensors[t], sp.tensors[u])) return false;
         }
+    }
+    // The kernel's arguments: the last stage's, with the statistics slots of the whole chain --
+    // one per flex16 tensor that a stage stores or reduces into, in operand order (the tables of
+    // a chain's compiled stages number them the same way).
+    C.launch = C.k[C.n - 1];
+    {
+        KArgs& L = C.launch;
+        L.n_stat_slots = L.n_store_stat_slots = 0;
+        for (int s = 0; s < 4; ++s) L.stat_ptr[s] = nullptr;
+        for (int t = 0; t < sp.n_tensors; ++t) {
+            L.t[t].stat_slot = -1;
+            if (sp.tensors[t].dtype != NGH_FLEX16) continue;
+            bool written = false;
+            for (int i = 0; i < C.n; ++i) {
+                bool loads[NGH_MAX_TENSORS], stores[NGH_MAX_TENSORS];
+                const ngh_stage& S = sp.stages[C.stage_of[i]];
+                stage_tensors(sp, S, loads, stores);
+                written = written || stores[t];
+                for (int r = 0; r < S.n_reductions; ++r) written = written || S.red_out[r] == t;
+            }
+            if (!written) continue;
+            if (L.n_stat_slots == 4) return false;
+            L.t[t].stat_slot = L.n_stat_slots;
+            L.stat_ptr[L.n_stat_slots++] = sp.tensors[t].dev_stats;
+        }
+        L.n_store_stat_slots = L.n_stat_slots;
     }
     C.n_out = (unsigned)n_out;
     C.TR = 1;
@@ -1606,8 +1645,9 @@ int ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec) {
             const unsigned rows_per_wg = kBlock / C.TR;
             const unsigned blocks = (C.n_out + rows_per_wg - 1) / rows_per_wg;
             const int cp = stage_cache_policy(ctx, *spec, spec->stages[C.stage_of[C.n - 1]]) & kCpNtStore;
-            HIP_TRY(launch_special_chain(C.special, ctx->stream, blocks, C.k[C.n - 1], C.n_out, C.TR, cp));
-            return NGH_OK;
+            NGH_TRY(stat_scratch(ctx, C.launch, blocks));
+            HIP_TRY(launch_special_chain(C.special, ctx->stream, blocks, C.launch, C.n_out, C.TR, cp));
+            return stat_fold(ctx, C.launch, blocks);
         }
     }
     for (int s = 0; s < spec->n_stages; ++s) {
@@ -2135,8 +2175,46 @@ static int try_self_managed_launch(ngh_context* ctx, const ngh_fused_spec* spec,
                                    const int32_t* ids, const int32_t* in_place, int32_t n_ids, int32_t count,
                                    bool* done) {
     *done = false;
-    if (ctx->force_interp || !ctx->flex_self_managed || spec->n_stages != 1 || (spec->flags & NGH_SPEC_PROBE))
+    if (ctx->force_interp || !ctx->flex_self_managed || (spec->flags & NGH_SPEC_PROBE)) return NGH_OK;
+    if (spec->n_stages > 1) {
+        // A row chain whose every statistics slot belongs to one of the managed tensors: each
+        // workgroup takes the write exponents from the records, the one that finishes last
+        // applies the policy (the end-of-kernel mode of the streaming kernels).
+        if (ctx->no_chain || ctx->no_ragged) return NGH_OK;
+        ChainPlan C;
+        if (!plan_row_chain(ctx, *spec, C) || (C.special = match_chain(C.k, C.families, C.n)) < 0) return NGH_OK;
+        KArgs& L = C.launch;
+        if (L.n_stat_slots != n_ids || n_ids < 1) return NGH_OK;
+        int32_t slot_id[4] = {0, 0, 0, 0};
+        for (int s = 0; s < L.n_stat_slots; ++s) {
+            const ptrdiff_t off = (const char*)L.stat_ptr[s] - (const char*)dev;
+            if (!L.stat_ptr[s] || off < 0 || off % (ptrdiff_t)sizeof(ngh_flex_state)) return NGH_OK;
+            const int32_t id = (int32_t)(off / (ptrdiff_t)sizeof(ngh_flex_state));
+            int j = 0;
+            while (j < n_ids && ids[j] != id) ++j;
+            if (j == n_ids) return NGH_OK;
+            for (int q = 0; q < s; ++q)
+                if (L.flex_state[q] == dev + id) return NGH_OK;      // two slots on one tensor
+            L.flex_state[s] = dev + id;
+            L.flex_in_place[s] = in_place ? in_place[j] : 0;
+            slot_id[s] = id;
+        }
+        NGH_TRY(flex_settle_spec(ctx, *spec));
+        NGH_TRY(flex_settle_ids(ctx, dev, slot_id, L.n_stat_slots));
+        NGH_TRY(ensure_tickets(ctx, (size_t)kFlexTicketWords + kFlexGroupMaxWords));
+        L.flex_count = count;
+        L.ordered_arrival = ctx->ordered_arrival == 1;
+        L.tickets = ctx->tickets;
+        L.group_max = (int*)(ctx->tickets + kFlexTicketWords);
+        // (every workgroup pays the hand-over at the end once: as many as keep the chip full, each
+        // taking several turns, not one per group of rows)
+        const unsigned rows_per_wg = kBlock / C.TR;
+        const unsigned blocks = std::min((C.n_out + rows_per_wg - 1) / rows_per_wg, (unsigned)(ctx->cus * kChainManagedWgsPerCu));
+        const int cp = stage_cache_policy(ctx, *spec, spec->stages[C.stage_of[C.n - 1]]) & kCpNtStore;
+        HIP_TRY(launch_special_chain(C.special, ctx->stream, blocks, L, C.n_out, C.TR, cp));
+        *done = true;
         return NGH_OK;
+    }
     if (spec->stages[0].op_end == spec->stages[0].op_begin) return NGH_OK;
     Plan P;
     NGH_TRY(plan_stage(ctx, *spec, 0, P));

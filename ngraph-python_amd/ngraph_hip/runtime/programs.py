@@ -116,6 +116,21 @@ def _chain_program(spec, name, seen, min_elements):
         # (the same for every row: a layer norm's gain and bias)
         rowshared = [1 if spec.tensors[i].strides[1] == 0 and spec.tensors[i].strides[2] == 0 else 0
                      for i in range(spec.n_tensors)]
+    # the statistics slots of a row chain's flex16 results are the chain's: one per flex16 tensor
+    # that a stage stores or reduces into, in operand order, the same in every stage's tables
+    # (plan_row_chain numbers the kernel's arguments the same way)
+    written = set()
+    for stage in range(spec.n_stages):
+        st = spec.stages[stage]
+        written |= set(o.dst for o in spec.ops[st.op_begin:st.op_end] if o.opcode == hiplib.OPCODES["store"])
+        written |= set(st.red_out[r] for r in range(st.n_reductions))
+    stat_slot, n_slots = [], 0
+    for i in range(spec.n_tensors):
+        if not columns and i in written and dtypes[i] == hiplib.NGH_FLEX16:
+            stat_slot.append(n_slots)
+            n_slots += 1
+        else:
+            stat_slot.append(-1)
     members = []
     for stage in range(spec.n_stages):
         st = spec.stages[stage]
@@ -125,7 +140,7 @@ def _chain_program(spec, name, seen, min_elements):
         red_out = [st.red_out[r] for r in range(st.n_reductions)]
         stored = set(o[1] for o in ops if o[0] == hiplib.OPCODES["store"])
         loaded = set(o[2] for o in ops if o[0] == hiplib.OPCODES["load"])
-        members.append(("%s_s%d" % (name, stage), ops, dtypes, bcast, [-1] * spec.n_tensors, 0, spec.n_regs, 4,
+        members.append(("%s_s%d" % (name, stage), ops, dtypes, bcast, stat_slot, n_slots, spec.n_regs, 4,
                         ((2 if columns else 1) if red_out else 0), red_out, [-1] * spec.n_tensors,
                         [1 if i in loaded else 0 for i in range(spec.n_tensors)],
                         [1 if i in stored else 0 for i in range(spec.n_tensors)], -1, rowshared))

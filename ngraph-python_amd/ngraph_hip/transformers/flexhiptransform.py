@@ -25,10 +25,10 @@ import numpy as np
 from ngraph_hip.flex import HipFlexManager, hipflex16, HipFlex
 from ngraph_hip.flex.base import flex_gpu_transformer_name
 from ngraph_hip.op_graph import op_graph as og
-from ngraph_hip.runtime.hiplib import NGH_FLEX16, NGH_SPEC_PROBE
+from ngraph_hip.runtime.hiplib import NGH_FLEX16, NGH_SPEC_PROBE, OPCODES
 from ngraph_hip.transformers.hiptransform import (HipTransformer, HipDeviceTensor,
                                                   HipDeviceBufferStorage, HipKernelGroup,
-                                                  FusedKernel, CopyKernel, _td)
+                                                  FusedKernel, CopyKernel, ChainKernel, _td)
 from ngraph_hip.transformers.passes.passes import PeepholeGraphPass
 
 
@@ -94,7 +94,54 @@ class FlexHipDeviceBufferStorage(HipDeviceBufferStorage):
                                    name="v_" + tensor_description.name)
 
 
-class FlexFusedKernel(FusedKernel):
+class FlexManaged(object):
+    """What the kernel group's flex management needs of a kernel that has `specs`,
+    `flex_bindings` [(spec index, operand slot, flex entry, is written)],
+    `output_flex_entries` and `in_place_flex_ids`."""
+
+    @property
+    def output_flex_ids(self):
+        return [e.flex_id for e in self.output_flex_entries]
+
+    def bind_flex_scales(self):
+        """Host-managed mode: the current scales travel as kernel arguments, rebound before
+        every launch (flexgputransform.py:56-61)."""
+        for index, slot, entry, is_output in self.flex_bindings:
+            t = self.specs[index].tensors[slot]
+            t.scale = entry.scale
+            t.dev_scale = None
+            t.dev_stats = entry.ptr if is_output else None
+
+    def bind_flex_state_pointers(self):
+        """Device-resident mode: kernels read scales from the state table; bound once."""
+        if getattr(self, "_state_bound", False):
+            return
+        for index, slot, entry, is_output in self.flex_bindings:
+            t = self.specs[index].tensors[slot]
+            t.dev_scale = entry.scale_ptr
+            t.dev_stats = entry.ptr if is_output else None
+        self._state_bound = True
+
+    def execute_managed(self, rt, dev_table, count):
+        self.bind_flex_state_pointers()
+        if not hasattr(self, "_id_arrays"):
+            ids = [e.flex_id for e in self.output_flex_entries]
+            in_place = [1 if i in self.in_place_flex_ids else 0 for i in ids]
+            self._id_lists = (ids, in_place)
+            self._id_arrays = rt.make_id_arrays(ids, in_place)
+        if len(self.specs) == 1:
+            rt.launch_fused_flex(self.specs[0], dev_table, self._id_arrays, count)
+            return
+        # several launches cover one set of tensors (an outer axis looped on the host): one
+        # exponent for all of them, statistics merged over all of them
+        ids, in_place = self._id_lists
+        rt.flex_prepare(dev_table, ids, in_place)
+        for spec in self.specs:
+            rt.launch_fused(spec)
+        rt.flex_update(dev_table, ids, count)
+
+
+class FlexFusedKernel(FlexManaged, FusedKernel):
     """Fused kernel whose operands carry flex scales and statistics words."""
 
     def __init__(self, *args, **kwargs):
@@ -125,46 +172,6 @@ class FlexFusedKernel(FusedKernel):
                 read_ids.add(entry.flex_id)
         self.output_flex_entries = entries
         self.in_place_flex_ids = set(e.flex_id for e in entries) & read_ids
-
-    @property
-    def output_flex_ids(self):
-        return [e.flex_id for e in self.output_flex_entries]
-
-    def bind_flex_scales(self):
-        """Host-managed mode: the current scales travel as kernel arguments, rebound before
-        every launch (flexgputransform.py:56-61)."""
-        for index, slot, entry, is_output in self.flex_bindings:
-            t = self.specs[index].tensors[slot]
-            t.scale = entry.scale
-            t.dev_scale = None
-            t.dev_stats = entry.ptr if is_output else None
-
-    def bind_flex_state_pointers(self):
-        """Device-resident mode: kernels read scales from the state table; bound once."""
-        if getattr(self, "_state_bound", False):
-            return
-        for index, slot, entry, is_output in self.flex_bindings:
-            t = self.specs[index].tensors[slot]
-            t.dev_scale = entry.scale_ptr
-            t.dev_stats = entry.ptr if is_output else None
-        self._state_bound = True
-
-    def execute_managed(self, rt, dev_table, count):
-        if not hasattr(self, "_id_arrays"):
-            ids = [e.flex_id for e in self.output_flex_entries]
-            in_place = [1 if i in self.in_place_flex_ids else 0 for i in ids]
-            self._id_lists = (ids, in_place)
-            self._id_arrays = rt.make_id_arrays(ids, in_place)
-        if len(self.specs) == 1:
-            rt.launch_fused_flex(self.specs[0], dev_table, self._id_arrays, count)
-            return
-        # several launches cover one set of tensors (an outer axis looped on the host): one
-        # exponent for all of them, statistics merged over all of them
-        ids, in_place = self._id_lists
-        rt.flex_prepare(dev_table, ids, in_place)
-        for spec in self.specs:
-            rt.launch_fused(spec)
-        rt.flex_update(dev_table, ids, count)
 
     def probe(self):
         """Measure max|fp32 result| of every not yet initialised output without storing."""
@@ -209,6 +216,68 @@ class FlexCopyKernel(CopyKernel):
         pass
 
 
+class FlexChainKernel(FlexManaged, ChainKernel):
+    """Consecutive flex kernels over the same rows as the stages of one spec, one launch when the
+    library has the chain's program: a softmax's maximum, sum of exponentials and result, each a
+    flex16 tensor with an exponent of its own.  One prepare / launch / update covers all of them.
+    A stage reads what an earlier stage wrote from memory, rounded as stored, so the chain leaves
+    the bits its members leave when they run one by one -- which they do until every output has
+    its first exponent (a member's probe needs its predecessors' results) and while the library
+    has no program for the chain."""
+
+    def __init__(self, transformer, members, spec, uses, operands=()):
+        super(FlexChainKernel, self).__init__(transformer, members, spec, uses, operands)
+        t = transformer
+        self.flex_bindings = []
+        for s, td in enumerate(self.operands):
+            entry = t.flex_entry_of(td)
+            if entry is not None:
+                self.flex_bindings.append((0, s, entry, uses[s][2]))
+        # an output holds data from before the launch that the chain reads when a stage loads it
+        # no later than the first stage that writes it
+        load, store = OPCODES["load"], OPCODES["store"]
+        first_load, first_write = {}, {}
+        for stage in range(spec.n_stages):
+            st = spec.stages[stage]
+            for o in spec.ops[st.op_begin:st.op_end]:
+                if o.opcode == load:
+                    first_load.setdefault(o.a, stage)
+                elif o.opcode == store:
+                    first_write.setdefault(o.dst, stage)
+            for r in range(st.n_reductions):
+                first_write.setdefault(st.red_out[r], stage)
+        seen, entries, in_place = set(), [], set()
+        for _, slot, entry, is_output in self.flex_bindings:
+            if not is_output:
+                continue
+            if entry.flex_id not in seen:
+                seen.add(entry.flex_id)
+                entries.append(entry)
+            if slot in first_load and first_load[slot] <= first_write.get(slot, spec.n_stages):
+                in_place.add(entry.flex_id)
+        self.output_flex_entries = entries
+        self.in_place_flex_ids = in_place
+
+    def active(self):
+        """One launch, managed as one kernel?  Else the members run, each managed by itself.
+        (Asked before every execution: once true it stays true, and looking at a record reads
+        the state table back from the device.)"""
+        if not getattr(self, "_active", False):
+            self._active = self.ready and all(e.initialized for e in self.output_flex_entries)
+        return self._active
+
+    @property
+    def _all_initialized(self):
+        return True            # (only asked of an active chain)
+
+    @_all_initialized.setter
+    def _all_initialized(self, value):
+        pass
+
+    def probe(self):
+        pass
+
+
 class FlexHipKernelGroup(HipKernelGroup):
     """Flex management around every kernel (flexgputransform.py:224-371)."""
 
@@ -236,15 +305,25 @@ class FlexHipKernelGroup(HipKernelGroup):
             # bound; one library call per kernel does prepare + launch + policy update
             manager.push()
             rt, count = self.transformer.runtime, manager.autoflex_count
-            for k in self.kernels:
+            for k in self.execution_units():
                 k.execute_managed(rt, manager.dev_table, count)
             manager.device_dirty = True
             return
         super(FlexHipKernelGroup, self).__call__()
         if manager.resident:
+            units = list(self.execution_units())
             self._steady = all(getattr(k, "_all_initialized", False) or not k.output_flex_entries
-                               for k in self.kernels) and \
-                all(isinstance(k, (FlexFusedKernel, FlexCopyKernel)) for k in self.kernels)
+                               for k in units) and \
+                all(isinstance(k, (FlexFusedKernel, FlexCopyKernel, FlexChainKernel)) for k in units)
+
+    def execution_units(self):
+        """A chain that is not one launch yet stands for its members."""
+        for k in self.kernels:
+            if isinstance(k, FlexChainKernel) and not k.active():
+                for m in k.members:
+                    yield m
+            else:
+                yield k
 
     @property
     def output_flex_ids(self):
@@ -262,6 +341,8 @@ class FlexHipTransformer(HipTransformer):
     default_rtol = 1e-02
     atol_precision_multiplier = 8
     kernel_group_class = FlexHipKernelGroup
+    chain_member_class = FlexFusedKernel
+    chain_kernel_class = FlexChainKernel
     max_written_views = 4        # a kernel merges max|mantissa| for at most 4 flex results
     split_reductions = False     # an intermediate result would be rounded to flex16 on its way
 

@@ -43,9 +43,10 @@ class ChainKernel(HipKernel):
     have alone, with the programs they match by themselves.
     """
 
-    def __init__(self, transformer, members, spec, uses):
+    def __init__(self, transformer, members, spec, uses, operands=()):
         super(ChainKernel, self).__init__(transformer)
         self.members = list(members)
+        self.operands = list(operands)        # tensor descriptions (or scratch rows) of the spec's operand slots
         self.name = self.members[0].name
         self.ops = [op for m in self.members for op in getattr(m, "ops", None) or [m.op]]
         self.specs = [spec]
@@ -251,7 +252,7 @@ class ChainKernel(HipKernel):
         if not hiplib.plan_chain(spec)["eligible"]:
             return None
         t.runtime.validate_fused(spec)
-        return cls(t, members, spec, [(td.base, s in read, s in written) for s, td in enumerate(union)])
+        return cls(t, members, spec, [(td.base, s in read, s in written) for s, td in enumerate(union)], union)
 
     def buffer_uses(self):
         return list(self.spec_uses[0])
@@ -313,7 +314,7 @@ class KernelRun(HipKernel):
             while a < n:
                 merged = None
                 for b in range(min(n, a + self.max_stages), a + 1, -1):
-                    merged = ChainKernel.merged(self.transformer, self.members[a:b])
+                    merged = self.transformer.chain_kernel_class.merged(self.transformer, self.members[a:b])
                     if merged is not None:
                         break
                 if merged is None:

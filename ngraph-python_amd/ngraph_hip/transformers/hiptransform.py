@@ -141,10 +141,14 @@ class HipKernelGroup(object):
         if self._programs is not None and self._programs.poll():
             self._programs = None
             self.programs_changed()
-        for k in self.kernels:
+        for k in self.execution_units():
             self.setup_kernel_execute(k)
             k.execute()
             self.after_kernel_execute(k)
+
+    def execution_units(self):
+        """The kernels in the order they are launched."""
+        return self.kernels
 
     def profile(self, repeats=1, inner=1):
         """Per-kernel durations from HIP events on the launch stream.
@@ -157,16 +161,17 @@ class HipKernelGroup(object):
         rt = self.transformer.runtime
         if not self._bound:
             self.bind()
-        times = [[] for _ in self.kernels]
+        units = list(self.execution_units())
+        times = [[] for _ in units]
         for _ in range(repeats):
-            for i, k in enumerate(self.kernels):
+            for i, k in enumerate(units):
                 self.setup_kernel_execute(k)
                 rt.timer_begin()
                 for _ in range(inner):
                     k.execute()
                 times[i].append(rt.timer_end() / inner)
                 self.after_kernel_execute(k)
-        return list(zip(self.kernels, times))
+        return list(zip(units, times))
 
 
 class HipTransformer(ComputationGraphTransformer):
@@ -180,6 +185,8 @@ class HipTransformer(ComputationGraphTransformer):
     max_written_views = NGH_MAX_TENSORS      # results one fused kernel may write
     split_reductions = True                  # ReductionLayoutPass: reduce group by group of axes, no copy
     chain_kernels = True                     # consecutive kernels over the same rows run as stages of one spec
+    chain_member_class = FusedKernel         # (the kernels that may merge, and what they merge into)
+    chain_kernel_class = ChainKernel
 
     def __init__(self, device_id=0, fusion=True, dry_run=False, fuse_moments=None, rng_seed=0, jit=None,
                  jit_min_elements=4096, jit_auto_min_elements=1 << 22, jit_after_calls=0, **kwargs):
@@ -293,7 +300,7 @@ class HipTransformer(ComputationGraphTransformer):
             del run[:]
 
         for k in kernels:
-            if type(k) is FusedKernel:
+            if type(k) is self.chain_member_class:
                 run.append(k)
             elif type(k) is MomentsKernel:
                 # (the statistics of rows and the kernels that use them may merge as well)

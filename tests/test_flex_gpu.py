@@ -408,3 +408,158 @@ def test_flex_statistics_file_holds_the_exponent_state_of_every_tensor(tmp_path)
     finally:
         t.close()
     assert not os.path.exists(other)
+
+
+# ---- row chains of flex kernels: one launch for the maximum, the sum of exponentials and the
+# normalised result of a softmax, each a flex16 tensor with an exponent of its own -------------
+def _rows_graph(t, rows, k, shift_only):
+    R, K = ng.make_axis(rows, name="R"), ng.make_axis(k, name="K")
+    x = ng.placeholder([R, K])
+    m = ng.max(x, out_axes=[R])
+    if shift_only:
+        out = x - m
+    else:
+        e = ng.exp(x - m)
+        out = e / ng.sum(e, out_axes=[R])
+    return t.computation(out, x)
+
+
+def _model_rows(xs, shift_only):
+    """The fused kernels in the NumPy flex model: every stored tensor (the maximum, the sum, the
+    result) rounds to its own exponent, what a later kernel loads is what was stored, and the
+    values in between are float32 (op by op as the CPU transformer computes them)."""
+    from oracle import numpy_ops as ops
+    rows = xs[0].shape[0]
+    tx, tm, ts, ty = fm._SimTensor(xs[0].shape), fm._SimTensor((rows,)), fm._SimTensor((rows,)), \
+        fm._SimTensor(xs[0].shape)
+    out = []
+    for x in xs:
+        tx.host_write(x)
+        tm.kernel_write(lambda: ops.reduce("max", tx.load(), 1))
+        shifted = lambda: ops.binary("sub", tx.load(), tm.load()[:, None])
+        if shift_only:
+            ty.kernel_write(shifted)
+            sums = None
+        else:
+            ts.kernel_write(lambda: ops.reduce("sum", ops.unary("exp", shifted()), 1))
+            ty.kernel_write(lambda: ops.binary("div", ops.unary("exp", shifted()), ts.load()[:, None]))
+            sums = (ts.mantissa.copy(), ts.stored_dec, ts.policy.dec)
+        out.append({"max": (tm.mantissa.copy(), tm.stored_dec, tm.policy.dec), "sum": sums,
+                    "out": (ty.mantissa.copy(), ty.stored_dec, ty.policy.dec)})
+    return out
+
+
+def _run_rows(xs, shift_only, resident):
+    """Per input: the result's mantissas, and (exponent in use, next exponent, last max
+    |mantissa|) of every flex tensor the computation writes, in the order they are written."""
+    rows, k = xs[0].shape
+    t = ngt.make_transformer_factory("flexhip", resident=resident, jit=True)()
+    try:
+        f = _rows_graph(t, rows, k, shift_only)
+        seen = []
+        for x in xs:
+            f(x)
+            group = t.kernel_groups[f]
+            view = t.get_op_tensor_view(f.computation_op.values[0])
+            t.flex_manager.pull()
+            entries = []
+            for kernel in group.kernels:
+                for e in kernel.output_flex_entries:
+                    entries.append((e.dec, e.next_dec, e.last_maxabs))
+            seen.append((view._read_raw().copy(), entries))
+        names = [d for kernel in group.execution_units() for ds in kernel.describe() for d in ds]
+        return seen, names
+    finally:
+        t.close()
+
+
+@pytest.mark.parametrize("resident", [False, True], ids=["host-policy", "device-policy"])
+@pytest.mark.parametrize("rows,k", [(512, 1024), (300, 1000), (64, 4098)])
+def test_flex_row_chain_of_a_maximum_and_its_consumer_is_bit_exact(rows, k, resident, monkeypatch):
+    """x - max(x) along rows: as one chain kernel, as two kernels, and in the NumPy flex model
+    -- the same mantissas and exponents after every one of several inputs whose range moves."""
+    rs = np.random.RandomState(21)
+    x0 = rs.uniform(-2, 2, (rows, k)).astype(np.float32)
+    xs = [(x0 * g).astype(np.float32) for g in (1.0, 1.0, 5.0, 40.0, 0.3, 0.01, 1.0)]
+    want = _model_rows(xs, True)
+    monkeypatch.delenv("NGH_NO_CHAIN", raising=False)
+    chained, names = _run_rows(xs, True, resident)
+    if default_kernel_choice():
+        assert any("chain-of-2" in nm for nm in names), names
+    monkeypatch.setenv("NGH_NO_CHAIN", "1")
+    apart, names = _run_rows(xs, True, resident)
+    assert not any("chain-of" in nm for nm in names), names
+    for i, ((mant, entries), (mant2, entries2)) in enumerate(zip(chained, apart)):
+        np.testing.assert_array_equal(mant, want[i]["out"][0], err_msg="input %d" % i)
+        np.testing.assert_array_equal(mant2, want[i]["out"][0], err_msg="input %d, kernel by kernel" % i)
+        assert entries == entries2, (i, entries, entries2)
+        for (dec, next_dec, last), which in zip(entries, ("max", "out")):
+            m_want, dec_want, next_want = want[i][which]
+            assert (dec, next_dec, last) == (dec_want, next_want, fm.maxabs(m_want)), (i, which)
+
+
+@pytest.mark.parametrize("resident", [False, True], ids=["host-policy", "device-policy"])
+@pytest.mark.parametrize("rows,k", [(512, 1024), (300, 1000)])
+def test_flex_softmax_of_rows_as_one_chain(rows, k, resident, monkeypatch):
+    """A flex16 softmax of rows as one chain kernel against the same kernels launched one by one
+    and against the NumPy flex model.  The sum of exponentials is added up in another order by
+    each of the three and the device's exp differs from NumPy's in the last place, so a sum's
+    mantissa may land on the neighbouring 16-bit value, which moves that row's results by the
+    fraction 1 / (the sum's mantissa): the results agree to that plus one unit of rounding, most
+    of them exactly, and the exponents are the same."""
+    rs = np.random.RandomState(22)
+    x0 = rs.uniform(-2, 2, (rows, k)).astype(np.float32)
+    xs = [(x0 * g).astype(np.float32) for g in (1.0, 1.0, 4.0, 0.1, 1.0)]
+    want = _model_rows(xs, False)
+    monkeypatch.delenv("NGH_NO_CHAIN", raising=False)
+    chained, names = _run_rows(xs, False, resident)
+    if default_kernel_choice():
+        assert any("chain-of-3" in nm for nm in names), names
+    monkeypatch.setenv("NGH_NO_CHAIN", "1")
+    apart, names = _run_rows(xs, False, resident)
+    assert not any("chain-of" in nm for nm in names), names
+    for i, ((mant, entries), (mant2, entries2)) in enumerate(zip(chained, apart)):
+        for got, what in ((mant, "chain"), (mant2, "kernel by kernel")):
+            m_out, m_sum = want[i]["out"][0].astype(np.float64), want[i]["sum"][0].astype(np.float64)
+            diff = np.abs(got.astype(np.float64) - m_out)
+            allowed = 1.0 + np.abs(m_out) / m_sum[:, None]
+            assert (diff <= allowed).all(), (i, what, diff.max(), (diff - allowed).max())
+            assert (diff != 0).mean() < 0.05, (i, what, (diff != 0).mean())
+        for (dec, next_dec, last), (dec2, next2, last2), which in zip(entries, entries2, ("max", "sum", "out")):
+            m_want, dec_want, next_want = want[i][which]
+            assert (dec, next_dec) == (dec2, next2) == (dec_want, next_want), (i, which)
+            assert abs(last - fm.maxabs(m_want)) <= 1 and abs(last2 - fm.maxabs(m_want)) <= 1, (i, which)
+
+
+def test_flex_row_chain_agrees_across_policy_modes(monkeypatch):
+    """The chain launched with nobody looking in between, under every way the library has of
+    running the exponent policy (on the host, as three launches, at the end of the kernel):
+    the same records and mantissas."""
+    rows, k = 384, 1024
+    rs = np.random.RandomState(23)
+    x0 = rs.uniform(-2, 2, (rows, k)).astype(np.float32)
+    seen = {}
+    for name, mode, grid, ordered, stream_mib in _POLICY_MODES:
+        _with_policy_mode(monkeypatch, mode, grid, ordered, stream_mib)
+        t = ngt.make_transformer_factory("flexhip", resident=name != "host", jit=True)()
+        try:
+            f = _rows_graph(t, rows, k, True)
+            states = []
+            for gain in (1.0, 30.0, 30.0, 0.02):
+                f((x0 * gain).astype(np.float32))
+                group = t.kernel_groups[f]
+                for it in range(3):
+                    group()
+                view = t.get_op_tensor_view(f.computation_op.values[0])
+                t.flex_manager.pull()
+                entries = [_entry_state(e) for kernel in group.kernels for e in kernel.output_flex_entries]
+                states.append((entries, view._read_raw().copy()))
+            seen[name] = states
+        finally:
+            t.close()
+    ref = seen["host"]
+    assert ref[0][0] != ref[1][0]
+    for name, states in seen.items():
+        for (st, mant), (st_ref, mant_ref) in zip(states, ref):
+            assert st == st_ref, (name, st, st_ref)
+            np.testing.assert_array_equal(mant, mant_ref, err_msg=name)

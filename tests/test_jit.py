@@ -510,8 +510,8 @@ def _softmax_spec(px, pm, ps, py, R, rows, row_stride=None, x_dtype=hiplib.NGH_F
 
 
 def test_which_specs_are_row_chains():
-    """ngh_plan_chain without a device: rows of 8 to 8192 fp32 elements with unit stride, at least
-    one reduction stage, more than one stage."""
+    """ngh_plan_chain without a device: rows of 8 to 8192 fp32 (or flex16 / fp16) elements with unit
+    stride, at least one reduction stage, more than one stage."""
     if not default_kernel_choice():
         pytest.skip("a kernel-choice knob of the library is set")
     ok = lambda spec: hiplib.plan_chain(spec)["eligible"]
@@ -522,7 +522,13 @@ def test_which_specs_are_row_chains():
     assert ok(_softmax_spec((1 << 30) + 4, 2 << 30, 3 << 30, (4 << 30) + 4, 1000, 300, row_stride=1003))      # any 4-byte-aligned start
     assert not ok(_softmax_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 7, 300))
     assert not ok(_softmax_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 8193, 300))
-    assert not ok(_softmax_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 1000, 300, x_dtype=hiplib.NGH_FLEX16))
+    # 16-bit operands: every chunk of four on a 4-byte boundary (an aligned start, rows an even
+    # number of elements apart); other integer storage stays out
+    assert ok(_softmax_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 1000, 300, x_dtype=hiplib.NGH_FLEX16))
+    assert ok(_softmax_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 1001, 300, row_stride=1002, x_dtype=hiplib.NGH_F16))
+    assert not ok(_softmax_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 1001, 300, x_dtype=hiplib.NGH_FLEX16))
+    assert not ok(_softmax_spec((1 << 30) + 2, 2 << 30, 3 << 30, 4 << 30, 1000, 300, x_dtype=hiplib.NGH_FLEX16))
+    assert not ok(_softmax_spec(1 << 30, 2 << 30, 3 << 30, 4 << 30, 1000, 300, x_dtype=hiplib.NGH_I16))
     # two operand slots over the same memory, one of them written: the stages must see each
     # other's writes, which the chain's registers would hide
     assert not ok(_softmax_spec(1 << 30, 2 << 30, 3 << 30, (1 << 30) + 4000, 1001, 300))
