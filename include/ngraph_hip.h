@@ -425,7 +425,10 @@ int  ngh_flex_update(ngh_context* ctx, ngh_flex_state* dev, const int32_t* ids, 
  * in its first instructions, and every other entry point that reads or writes a record, or
  * launches a kernel whose operands point into one, first brings it up to date.  A record read
  * through ngh_flex_states_read is therefore always current; device memory of a table must not
- * be copied out by other means while ngh_flex_unsettled reports a non-zero count.          */
+ * be copied out by other means while ngh_flex_unsettled reports a non-zero count.
+ * A spec of several stages that runs as a row chain, every flex16 tensor it writes among `ids`,
+ * is one launch as well: the chain takes the write exponents from the records and its last
+ * workgroup applies the policy.                                                             */
 int  ngh_launch_fused_flex(ngh_context* ctx, const ngh_fused_spec* spec, ngh_flex_state* dev,
                            const int32_t* ids, const int32_t* in_place, int32_t n_ids, int32_t count);
 /* number of records whose statistics are still unfolded (no counterpart in the reference,

@@ -182,3 +182,68 @@ def test_softmax_over_classes_at_full_size(classes, samples, kept):
     e64 = np.exp(x64 - x64.max(axis=0))
     np.testing.assert_allclose(y, e64 / e64.sum(axis=0), rtol=RTOL, atol=ATOL)
     np.testing.assert_allclose(y.sum(axis=0, dtype=np.float64), 1.0, rtol=0, atol=1e-5)
+
+
+@pytest.mark.parametrize("rows,k", [(32768, 1024), (32768, 1000)])
+def test_flex16_softmax_of_rows_at_full_size(rows, k):
+    """The flex16 softmax of rows that bench.py --shapes times, as ONE chain kernel with the
+    exponent policy inside the launch, over three inputs whose range moves: against the NumPy flex
+    model of the fused kernels (oracle/flex_model.py: every stored tensor rounds to its own
+    exponent) within what the order of a row's sum can move a result -- one unit of the sum's
+    mantissa, i.e. the fraction 1 / mantissa of a row's results, plus one unit of rounding -- with
+    the same exponents chosen, and against float64 under the reference's flex acceptance rule
+    (rtol 1e-2, atol 8 x scale: flexgputransform.py:80-103)."""
+    from oracle import flex_model as fm
+    from oracle import numpy_ops as ops
+    rs = np.random.RandomState(31)
+    x0 = rs.uniform(-2, 2, (rows, k)).astype(np.float32)
+    xs = [x0, (x0 * 3).astype(np.float32), (x0 * 0.2).astype(np.float32)]
+    compared = 0
+    tx, tm, ts, ty = fm._SimTensor(x0.shape), fm._SimTensor((rows,)), fm._SimTensor((rows,)), fm._SimTensor(x0.shape)
+    t = ngt.make_transformer_factory("flexhip")()
+    try:
+        R, K = ng.make_axis(rows, name="R"), ng.make_axis(k, name="K")
+        x = ng.placeholder([R, K])
+        e = ng.exp(x - ng.max(x, out_axes=[R]))
+        f = t.computation(e / ng.sum(e, out_axes=[R]), x)
+        f(xs[0])
+        group = t.kernel_groups[f]
+        assert group.wait_for_programs(timeout=600) is None
+        f(xs[0])
+        names = [d for kernel in group.execution_units() for ds in kernel.describe() for d in ds]
+        if default_kernel_choice():
+            assert len(names) == 3 and all("/chain-of-3" in n for n in names), names
+        # the model: two calls with the first input (as above), then the others
+        for step, xi in enumerate([xs[0], xs[0], xs[1], xs[2], xs[2]]):
+            tx.host_write(xi)
+            tm.kernel_write(lambda: ops.reduce("max", tx.load(), 1))
+            shifted = lambda: ops.binary("sub", tx.load(), tm.load()[:, None])
+            ts.kernel_write(lambda: ops.reduce("sum", ops.unary("exp", shifted()), 1))
+            ty.kernel_write(lambda: ops.binary("div", ops.unary("exp", shifted()), ts.load()[:, None]))
+            if step == 0:
+                continue
+            got = np.array(f(xi)).copy() if step > 1 else np.array(f(xs[0])).copy()
+            view = t.get_op_tensor_view(f.computation_op.values[0])
+            mant = view._read_raw().astype(np.float64)
+            # (the next exponent is predicted from the recorded maxima, which may differ by the
+            # unit the sum's order moves: next to a boundary the prediction can fall on either side)
+            entries = [en for kernel in group.kernels for en in kernel.output_flex_entries]      # maximum, sum, result
+            assert len(entries) == 3 and entries[2] is view.flex_entry
+            for model, entry in zip((tm, ts, ty), entries):
+                assert entry.dec == model.stored_dec and abs(entry.next_dec - model.policy.dec) <= 1, step
+            m_out, m_sum = ty.mantissa.astype(np.float64), ts.mantissa.astype(np.float64)
+            diff = np.abs(mant - m_out)
+            assert (diff <= 1.0 + np.abs(m_out) / m_sum[:, None]).all(), (step, diff.max())
+            for model, entry in zip((tm, ts, ty), entries):
+                model.policy.dec = entry.next_dec             # (the model follows the device's choice from here)
+            if max(fm.maxabs(tt.mantissa) for tt in (tm, ts, ty)) >= 32767:
+                continue          # (a range that jumped saturates a tensor once, in the model as on the device; the policy then moves its exponent)
+            x64 = fm.dequantize(tx.mantissa, tx.stored_dec).astype(np.float64)
+            e64 = np.exp(x64 - x64.max(axis=1, keepdims=True))
+            want = e64 / e64.sum(axis=1, keepdims=True)
+            atol, rtol = t.get_default_tolerance(want)
+            np.testing.assert_allclose(got, want, rtol=rtol, atol=atol)
+            compared += 1
+        assert compared >= 2
+    finally:
+        t.close()
