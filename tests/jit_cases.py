@@ -108,6 +108,17 @@ def case_softmax_ragged_rows():
     return [e / ng.sum(e, out_axes=[N])], [x]
 
 
+def case_softmax_of_half_rows():
+    # 16-bit storage in a row chain: fp16 operand and result, the row's maximum an fp16 tensor
+    # too (rounded for its tensor and handed on in a register as a load would return it), the
+    # sum fp32; rows of 1002 elements (a row starts on a 4-byte boundary, not on an 8-byte one)
+    C, N = ng.make_axis(1002, name="C"), ng.make_axis(1200, name="N")
+    x = ng.placeholder([N, C], dtype=np.float16)
+    m = ng.max(x * 3.3, out_axes=[N], dtype=np.float16)
+    e = ng.exp(x * 3.3 - m)
+    return [ng.divide(e, ng.sum(e, out_axes=[N]), dtype=np.float16), m], [x]
+
+
 def case_softmax_long_rows():
     # rows of 4099 and of 8192 elements: a workgroup per row in the chain kernel
     C, N, C2 = ng.make_axis(4099, name="C"), ng.make_axis(300, name="N"), ng.make_axis(8192, name="C2")
@@ -233,7 +244,7 @@ def case_row_statistics_chain():
 FP32_CASES = [case_elementwise, case_column_reduction_with_store, case_row_reduction_with_store,
               case_transposed_operand, case_transposed_operands_large, case_softmax, case_mixed_storage_types,
               case_integer_arithmetic, case_ragged,
-              case_ragged_long_rows, case_ragged_many_rows, case_softmax_ragged_rows, case_softmax_long_rows, case_softmax_over_windows,
+              case_ragged_long_rows, case_ragged_many_rows, case_softmax_ragged_rows, case_softmax_of_half_rows, case_softmax_long_rows, case_softmax_over_windows,
               case_softmax_forward_and_backward,
               case_row_chain_with_stored_intermediate, case_misaligned_slices, case_short_rows, case_dropout, case_lookup_table,
               case_row_statistics_chain, case_softmax_over_classes, case_softmax_over_few_classes,

@@ -49,12 +49,13 @@ def main():
             reordered = any("/ragged" in n or "chain-of-" in n for n in names) or "over_classes" in case.__name__ \
                 or "over_few_classes" in case.__name__ or "ten_classes" in case.__name__ or "column_statistics" in case.__name__
             for a, b, w in zip(interp, compiled, want):
+                half = np.asarray(b).dtype == np.float16       # (an fp16 result may land on the neighbouring value)
                 if reordered:
-                    np.testing.assert_allclose(a, b, rtol=2e-6, atol=1e-6)
+                    np.testing.assert_allclose(a, b, rtol=1e-3 if half else 2e-6, atol=1e-6)
                 else:
                     np.testing.assert_array_equal(a, b)
                 if case is not jit_cases.case_dropout:
-                    np.testing.assert_allclose(b, w, rtol=1e-5, atol=1e-5)
+                    np.testing.assert_allclose(b, w, rtol=1e-3 if half else 1e-5, atol=1e-5)
             if default_kernel_choice() and any("interp" in n for n in names if "tail" not in n):
                 raise AssertionError("still interpreted: %s" % names)
             compiled_names += sum(1 for n in names if n.startswith("special:jit_"))

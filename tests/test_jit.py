@@ -357,7 +357,12 @@ def test_compiled_programs_agree_with_the_interpreter(case):
     # longer segments than the interpreted one: the softmax over classes when its stages run apart)
     ragged = any("/ragged" in n or "chain-of-" in n for n in names) or case in COLUMN_SOFTMAX_CASES
     for a, b, w in zip(interp, compiled, want):
-        if ragged:
+        half = np.asarray(b).dtype == np.float16
+        if ragged and half:
+            # (a sum added up in another order can put a result on the neighbouring fp16 value)
+            np.testing.assert_allclose(a, b, rtol=1e-3, atol=1e-6)
+            assert (np.asarray(a) != np.asarray(b)).mean() < 1e-3
+        elif ragged:
             np.testing.assert_allclose(a, b, rtol=2e-6, atol=1e-6)
         else:
             np.testing.assert_array_equal(a, b)
@@ -365,7 +370,7 @@ def test_compiled_programs_agree_with_the_interpreter(case):
             # the oracle draws from NumPy's generator: only the distribution is comparable
             assert abs(np.count_nonzero(compiled[0]) / compiled[0].size - 0.75) < 0.01
         else:
-            np.testing.assert_allclose(b, w, rtol=1e-5, atol=1e-5)
+            np.testing.assert_allclose(b, w, rtol=1e-3 if half else 1e-5, atol=1e-5)
     if default_kernel_choice():
         # every stage large enough to be worth a compiled kernel has one now
         assert not any("interp" in n for n in names if "tail" not in n), names
@@ -373,6 +378,7 @@ def test_compiled_programs_agree_with_the_interpreter(case):
                     jit_cases.case_misaligned_slices):
             assert any(n.endswith("/ragged") for n in names), names
         if case in (jit_cases.case_softmax, jit_cases.case_softmax_ragged_rows, jit_cases.case_short_rows,
+                    jit_cases.case_softmax_of_half_rows,
                     jit_cases.case_softmax_long_rows, jit_cases.case_softmax_over_windows,
                     jit_cases.case_softmax_forward_and_backward,
                     jit_cases.case_row_chain_with_stored_intermediate, jit_cases.case_row_statistics_chain):
