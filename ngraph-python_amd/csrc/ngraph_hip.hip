@@ -128,6 +128,7 @@ struct ngh_context {
     int         force_interp = 0;    // never pick a specialised kernel
     int         red_wgs_per_cu = 8;  // workgroups per CU a split reduction along the contiguous axis aims for
     int         red_col_wgs_per_cu = 2;  // ... and one across it
+    int         chain_wgs_per_cu = 8;     // row chains: workgroups per compute unit, each taking several turns (0: one workgroup per group of rows)
     int         col_chain_wgs_per_cu = 2; // workgroups per compute unit a column chain narrows its workgroups for
     int         row_wave_chunks = 0;     // rows of up to this many chunks are reduced by one wavefront each
     int         tile4 = 1;               // tiled elementwise programs may take 64 x 64 tiles with 16-byte accesses
@@ -1131,6 +1132,7 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->red_wgs_per_cu = std::max(1, env_int("NGH_RED_WGS_PER_CU", 8));
     ctx->red_col_wgs_per_cu = std::max(1, env_int("NGH_RED_COL_WGS_PER_CU", 2));
     ctx->col_chain_wgs_per_cu = std::max(1, env_int("NGH_COL_CHAIN_WGS_PER_CU", 2));
+    ctx->chain_wgs_per_cu = std::max(0, env_int("NGH_CHAIN_WGS_PER_CU", 8));
     ctx->row_wave_chunks = std::max(0, env_int("NGH_ROW_WAVE_CHUNKS", kRowWaveChunks));
     ctx->tile4 = env_int("NGH_TILE4", 1);
     ctx->cache_policy = env_int("NGH_CACHE_POLICY", -1);
@@ -1643,7 +1645,8 @@ int ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec) {
         ChainPlan C;
         if (plan_row_chain(ctx, *spec, C) && (C.special = match_chain(C.k, C.families, C.n)) >= 0) {
             const unsigned rows_per_wg = kBlock / C.TR;
-            const unsigned blocks = (C.n_out + rows_per_wg - 1) / rows_per_wg;
+            unsigned blocks = (C.n_out + rows_per_wg - 1) / rows_per_wg;
+            if (ctx->chain_wgs_per_cu > 0) blocks = std::min(blocks, (unsigned)(ctx->cus * ctx->chain_wgs_per_cu));
             const int cp = stage_cache_policy(ctx, *spec, spec->stages[C.stage_of[C.n - 1]]) & kCpNtStore;
             NGH_TRY(stat_scratch(ctx, C.launch, blocks));
             HIP_TRY(launch_special_chain(C.special, ctx->stream, blocks, C.launch, C.n_out, C.TR, cp));
@@ -2209,7 +2212,8 @@ static int try_self_managed_launch(ngh_context* ctx, const ngh_fused_spec* spec,
         // (every workgroup pays the hand-over at the end once: as many as keep the chip full, each
         // taking several turns, not one per group of rows)
         const unsigned rows_per_wg = kBlock / C.TR;
-        const unsigned blocks = std::min((C.n_out + rows_per_wg - 1) / rows_per_wg, (unsigned)(ctx->cus * kChainManagedWgsPerCu));
+        const unsigned blocks = std::min((C.n_out + rows_per_wg - 1) / rows_per_wg,
+                                         (unsigned)(ctx->cus * (ctx->chain_wgs_per_cu > 0 ? ctx->chain_wgs_per_cu : kChainManagedWgsPerCu)));
         const int cp = stage_cache_policy(ctx, *spec, spec->stages[C.stage_of[C.n - 1]]) & kCpNtStore;
         HIP_TRY(launch_special_chain(C.special, ctx->stream, blocks, L, C.n_out, C.TR, cp));
         *done = true;
