@@ -366,8 +366,10 @@ int  ngh_plan_fused(const ngh_fused_spec* spec, int32_t stage, int32_t* out8);
  * compound kernels run their stages one after the other inside one launch, a reduction's result
  * reaching the next stage without a trip through a second launch (float_ew2.py:1135-1483,
  * stage loop :1268-1321)?  Possible for a "row chain": rows (spec axis 0, the reduced one) of up
- * to 8192 elements, fp32 operands with unit stride along the row or broadcast along it, at
- * least one reduction stage; and for a "column chain": the reduced axis (spec axis 0) strided,
+ * to 8192 elements, fp32 operands with unit stride along the row or broadcast along it (flex16
+ * and fp16 operands too, when every row starts an even number of elements from a 4-byte-aligned
+ * address; at most four flex16 tensors written), at least one reduction stage; and for a
+ * "column chain": the reduced axis (spec axis 0) strided,
  * every operand contiguous along spec axis 2 in whole aligned groups of 4 floats (or broadcast
  * along it), fp32, any number of rows.  out4 = {1 for a row chain, 2 for a column chain, 0 for
  * neither; index of the compiled chain program or -1 (without one the stages are launched one

@@ -49,8 +49,8 @@ def stage_programs(kernels, name, seen=None, min_elements=4096, vector_only=Fals
                 if total < min_elements and not scalar:
                     continue          # small stages are launch-bound; the interpreter is fine
                 codes = set(o.opcode for o in spec.ops[st.op_begin:st.op_end])
-                if hiplib.OPCODES["store_trunc"] in codes:
-                    continue          # the truncating store of a flex fill only runs in the interpreter
+                if hiplib.OPCODES["store_trunc"] in codes and (family == 3 or vector_only):
+                    continue          # the truncating store of a flex fill: not through the tiles, no built-in entries
                 if codes & {hiplib.OPCODES["take"], hiplib.OPCODES["rng_uniform"], hiplib.OPCODES["rng_normal"]} \
                         and (family == 3 or vector_only):
                     continue          # lookups, random fills: not through the tiles, no built-in entries
@@ -59,7 +59,7 @@ def stage_programs(kernels, name, seen=None, min_elements=4096, vector_only=Fals
                 red_out = [st.red_out[r] for r in range(st.n_reductions)]
                 dtypes = [spec.tensors[i].dtype for i in range(spec.n_tensors)]
                 bcast = [1 if spec.tensors[i].strides[fast] == 0 else 0 for i in range(spec.n_tensors)]
-                stored = set(o[1] for o in ops if o[0] == hiplib.OPCODES["store"])
+                stored = set(o[1] for o in ops if o[0] in (hiplib.OPCODES["store"], hiplib.OPCODES["store_trunc"]))
                 loaded = set(o[2] for o in ops if o[0] == hiplib.OPCODES["load"])
                 staged, n_staged = [], 0
                 for i in range(spec.n_tensors):

@@ -852,3 +852,36 @@ def test_normalisations_over_short_rows_run_as_built_in_chains():
                                rtol=1e-5, atol=2e-6)
     e = np.exp(w64 - w64.max(axis=1, keepdims=True))
     np.testing.assert_allclose(sm_, e / e.sum(axis=1, keepdims=True), rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.gpu
+def test_compiled_flex_fill_truncates_like_the_interpreter():
+    """A fill of a flex16 tensor stores int(value / scale) cut toward zero (the reference's
+    FlexFillKernel, tensor_ops.py:690-707): compiled at run time and interpreted give the same
+    mantissas and exponent, for values that round differently from how they are cut."""
+    def run(use_jit):
+        t = ngt.make_transformer_factory("flexhip", jit=use_jit, jit_min_elements=1)()
+        try:
+            P = ng.make_axis(1 << 16, name="P")
+            v = ng.variable([P], initial_value=0)
+            out, names = [], []
+            fills = [t.computation(ng.sequential([ng.fill(v, value), v * 1.0])) for value in (1.2, -1.7, 0.99999, 3.0)]
+            for f in fills:
+                f()
+                view = t.get_op_tensor_view(v)
+                out.append((view._read_raw().copy(), view.flex_entry.dec))
+                names += [d for k in t.kernel_groups[f].kernels for ds in k.describe() for d in ds]
+            return out, names
+        finally:
+            t.close()
+    a, names_interp = run(False)
+    b, names = run(True)
+    for (ma, da), (mb, db) in zip(a, b):
+        assert da == db
+        np.testing.assert_array_equal(ma, mb)
+    # cut toward zero: 1.2 at the exponent of the variable's first use
+    first, dec = b[0]
+    assert (first == int(np.trunc(np.float32(1.2) * np.float32(2.0 ** dec)))).all()
+    if default_kernel_choice():
+        assert any(n.startswith("special:jit_") for n in names), names
+        assert not any(n.startswith("special:") for n in names_interp), names_interp
