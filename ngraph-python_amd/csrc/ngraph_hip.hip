@@ -128,7 +128,7 @@ struct ngh_context {
     int         force_interp = 0;    // never pick a specialised kernel
     int         red_wgs_per_cu = 8;  // workgroups per CU a split reduction along the contiguous axis aims for
     int         red_col_wgs_per_cu = 2;  // ... and one across it
-    int         chain_wgs_per_cu = 8;     // row chains: workgroups per compute unit, each taking several turns (0: one workgroup per group of rows)
+    int         chain_wgs_per_cu = 0;     // row chains: at most this many workgroups per compute unit, each taking several turns (0: one workgroup per group of rows)
     int         col_chain_wgs_per_cu = 2; // workgroups per compute unit a column chain narrows its workgroups for
     int         row_wave_chunks = 0;     // rows of up to this many chunks are reduced by one wavefront each
     int         tile4 = 1;               // tiled elementwise programs may take 64 x 64 tiles with 16-byte accesses
@@ -1132,7 +1132,7 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->red_wgs_per_cu = std::max(1, env_int("NGH_RED_WGS_PER_CU", 8));
     ctx->red_col_wgs_per_cu = std::max(1, env_int("NGH_RED_COL_WGS_PER_CU", 2));
     ctx->col_chain_wgs_per_cu = std::max(1, env_int("NGH_COL_CHAIN_WGS_PER_CU", 2));
-    ctx->chain_wgs_per_cu = std::max(0, env_int("NGH_CHAIN_WGS_PER_CU", 8));
+    ctx->chain_wgs_per_cu = std::max(0, env_int("NGH_CHAIN_WGS_PER_CU", 0));
     ctx->row_wave_chunks = std::max(0, env_int("NGH_ROW_WAVE_CHUNKS", kRowWaveChunks));
     ctx->tile4 = env_int("NGH_TILE4", 1);
     ctx->cache_policy = env_int("NGH_CACHE_POLICY", -1);
