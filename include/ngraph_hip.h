@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define NGH_ABI_VERSION 6
+#define NGH_ABI_VERSION 7
 
 /* ---- limits (float_ew2.py:285-286 MAX_AXES = 3) ------------------------ */
 #define NGH_MAX_AXES      3
@@ -436,6 +436,33 @@ int  ngh_launch_fused_flex(ngh_context* ctx, const ngh_fused_spec* spec, ngh_fle
 /* number of records whose statistics are still unfolded (no counterpart in the reference,
  * whose policy runs on the host after every kernel)                                        */
 int  ngh_flex_unsettled(ngh_context* ctx, int32_t* out_count);
+
+/* ---- the launches of a computation as one HIP graph -----------------------
+ * No counterpart in the reference, which launches kernel by kernel through pycuda
+ * (gputransform.py:343-345, float_ew2.py:1553-1653): for computations of a few small kernels,
+ * whose time is launches rather than work.  Between ngh_graph_begin and ngh_graph_end the
+ * context's launches (ngh_launch_fused, ngh_copy_strided) are recorded instead of run;
+ * ngh_graph_launch replays them, in the order of the context's other work.  Launches that do
+ * not depend on each other may be recorded side by side so that the device may run them
+ * together: ngh_graph_fork marks the point both sides start from, ngh_graph_side(1 / 0) says
+ * which side the next launches belong to, ngh_graph_join (implied by fork and end) makes what
+ * follows wait for both.  Whether two launches are independent is the caller's knowledge.
+ * What a recorded launch was given -- addresses, constants, random-number counters -- is what
+ * every replay uses: record only launches whose arguments do not change from call to call, and
+ * none that allocates (a launch that ran once before with the same shapes allocates nothing) or
+ * waits for the device.  ngh_graph_end with out == NULL gives a capture up.
+ * (Measured on an MI355X with ROCm 7.2: two 4 us kernels take 10.6 us as two launches, 18.3 us
+ * as a graph of two nodes in a row, 31.4 us as two nodes side by side; the transformers record
+ * graphs only when asked to.)                                                                  */
+typedef struct ngh_graph ngh_graph;
+int  ngh_graph_begin(ngh_context* ctx);
+int  ngh_graph_fork(ngh_context* ctx);
+int  ngh_graph_side(ngh_context* ctx, int32_t on);
+int  ngh_graph_join(ngh_context* ctx);
+int  ngh_graph_end(ngh_context* ctx, ngh_graph** out);
+int  ngh_graph_launch(ngh_context* ctx, ngh_graph* graph);
+int  ngh_graph_nodes(const ngh_graph* graph, int32_t* out_nodes);
+int  ngh_graph_free(ngh_context* ctx, ngh_graph* graph);
 
 /* ---- timing (HIP events on the context's stream; used by the bench) ----- */
 int  ngh_timer_begin(ngh_context* ctx);

@@ -128,6 +128,11 @@ struct ngh_context {
     int         force_interp = 0;    // never pick a specialised kernel
     int         red_wgs_per_cu = 8;  // workgroups per CU a split reduction along the contiguous axis aims for
     int         red_col_wgs_per_cu = 2;  // ... and one across it
+    // launches captured into a HIP graph (ngh_graph_*)
+    hipStream_t main_stream = nullptr;    // the context's stream while a capture redirects ctx->stream
+    hipStream_t side_stream = nullptr;    // carries the launches of a side branch during a capture
+    hipEvent_t  fork_ev = nullptr, join_ev = nullptr;
+    bool        capturing = false, side_open = false;
     int         chain_wgs_per_cu = 0;     // row chains: at most this many workgroups per compute unit, each taking several turns (0: one workgroup per group of rows)
     int         col_chain_wgs_per_cu = 2; // workgroups per compute unit a column chain narrows its workgroups for
     int         row_wave_chunks = 0;     // rows of up to this many chunks are reduced by one wavefront each
@@ -1185,6 +1190,9 @@ int ngh_shutdown(ngh_context* ctx) {
     }
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
     if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
+    if (ctx->fork_ev) (void)hipEventDestroy(ctx->fork_ev);
+    if (ctx->join_ev) (void)hipEventDestroy(ctx->join_ev);
+    if (ctx->side_stream) (void)hipStreamDestroy(ctx->side_stream);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return NGH_OK;
@@ -2315,6 +2323,116 @@ int ngh_launch_fused_flex(ngh_context* ctx, const ngh_fused_spec* spec, ngh_flex
     NGH_TRY(ngh_flex_prepare(ctx, dev, ids, in_place, n_ids));
     NGH_TRY(ngh_launch_fused(ctx, spec));
     return ngh_flex_update(ctx, dev, ids, n_ids, count);
+}
+
+// ---------------------------------------------------------------------------
+// The launches of a computation as one HIP graph: what the caller launches between
+// ngh_graph_begin and ngh_graph_end is recorded, not run; ngh_graph_launch replays it with one
+// call.  Two launches that do not depend on each other may be recorded side by side
+// (ngh_graph_fork / ngh_graph_side / ngh_graph_join), so that the device may run them
+// together: worth it for computations of a few small kernels, whose time is launches, not work.
+// ---------------------------------------------------------------------------
+struct ngh_graph {
+    hipGraph_t     graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    int            nodes = 0;
+};
+
+static int graph_join(ngh_context* ctx) {
+    if (ctx->side_open) {
+        HIP_TRY(hipEventRecord(ctx->join_ev, ctx->side_stream));
+        HIP_TRY(hipStreamWaitEvent(ctx->main_stream, ctx->join_ev, 0));
+        ctx->side_open = false;
+    }
+    ctx->stream = ctx->main_stream;
+    return NGH_OK;
+}
+
+int ngh_graph_begin(ngh_context* ctx) {
+    if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
+    if (ctx->capturing) return fail(NGH_E_INVALID, "ngh_graph_begin: a capture is open already");
+    if (!ctx->side_stream) {
+        HIP_TRY(hipStreamCreateWithFlags(&ctx->side_stream, hipStreamNonBlocking));
+        HIP_TRY(hipEventCreateWithFlags(&ctx->fork_ev, hipEventDisableTiming));
+        HIP_TRY(hipEventCreateWithFlags(&ctx->join_ev, hipEventDisableTiming));
+    }
+    HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
+    ctx->main_stream = ctx->stream;
+    ctx->capturing = true;
+    ctx->side_open = false;
+    return NGH_OK;
+}
+
+int ngh_graph_fork(ngh_context* ctx) {
+    if (!ctx || !ctx->capturing) return fail(NGH_E_INVALID, "ngh_graph_fork: no capture is open");
+    NGH_TRY(graph_join(ctx));
+    HIP_TRY(hipEventRecord(ctx->fork_ev, ctx->main_stream));
+    HIP_TRY(hipStreamWaitEvent(ctx->side_stream, ctx->fork_ev, 0));
+    ctx->side_open = true;
+    return NGH_OK;
+}
+
+int ngh_graph_side(ngh_context* ctx, int32_t on) {
+    if (!ctx || !ctx->capturing) return fail(NGH_E_INVALID, "ngh_graph_side: no capture is open");
+    if (on && !ctx->side_open) return fail(NGH_E_INVALID, "ngh_graph_side: no fork is open");
+    ctx->stream = on ? ctx->side_stream : ctx->main_stream;
+    return NGH_OK;
+}
+
+int ngh_graph_join(ngh_context* ctx) {
+    if (!ctx || !ctx->capturing) return fail(NGH_E_INVALID, "ngh_graph_join: no capture is open");
+    return graph_join(ctx);
+}
+
+int ngh_graph_end(ngh_context* ctx, ngh_graph** out) {
+    if (!ctx || !ctx->capturing) return fail(NGH_E_INVALID, "ngh_graph_end: no capture is open");
+    const int joined = graph_join(ctx);
+    ctx->stream = ctx->main_stream;
+    ctx->capturing = false;
+    ctx->side_open = false;
+    hipGraph_t g = nullptr;
+    const hipError_t e = hipStreamEndCapture(ctx->main_stream, &g);
+    if (e != hipSuccess || !g || joined != NGH_OK || !out) {
+        (void)hipGetLastError();
+        if (g) (void)hipGraphDestroy(g);
+        if (!out && e == hipSuccess) return NGH_OK;          // (the caller gave the capture up)
+        return fail(NGH_E_RUNTIME, "ngh_graph_end: %s", e != hipSuccess ? hipGetErrorString(e) : "nothing was captured");
+    }
+    ngh_graph* G = new ngh_graph();
+    G->graph = g;
+    size_t n = 0;
+    if (hipGraphGetNodes(g, nullptr, &n) == hipSuccess) G->nodes = (int)n;
+    const hipError_t ei = hipGraphInstantiate(&G->exec, g, nullptr, nullptr, 0);
+    if (ei != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipGraphDestroy(g);
+        delete G;
+        return fail(NGH_E_RUNTIME, "hipGraphInstantiate: %s", hipGetErrorString(ei));
+    }
+    *out = G;
+    return NGH_OK;
+}
+
+int ngh_graph_launch(ngh_context* ctx, ngh_graph* graph) {
+    if (!ctx || !graph || !graph->exec) return fail(NGH_E_INVALID, "ngh_graph_launch: NULL argument");
+    if (ctx->capturing) return fail(NGH_E_INVALID, "ngh_graph_launch: a capture is open");
+    HIP_TRY(hipGraphLaunch(graph->exec, ctx->stream));
+    return NGH_OK;
+}
+
+int ngh_graph_nodes(const ngh_graph* graph, int32_t* out_nodes) {
+    if (!graph || !out_nodes) return fail(NGH_E_INVALID, "ngh_graph_nodes: NULL argument");
+    *out_nodes = graph->nodes;
+    return NGH_OK;
+}
+
+int ngh_graph_free(ngh_context* ctx, ngh_graph* graph) {
+    if (!graph) return NGH_OK;
+    if (ctx && ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
+    if (graph->graph) (void)hipGraphDestroy(graph->graph);
+    delete graph;
+    return NGH_OK;
 }
 
 int ngh_timer_begin(ngh_context* ctx) {

@@ -12,7 +12,7 @@ import os
 
 import numpy as np
 
-NGH_ABI_VERSION = 6
+NGH_ABI_VERSION = 7
 NGH_MAX_AXES = 3
 NGH_MAX_TENSORS = 12
 NGH_MAX_OPS = 96
@@ -141,6 +141,14 @@ _SYMBOLS = {
     "ngh_program_kernels": [ctypes.c_void_p, _i32, _i32, ctypes.c_char_p, ctypes.c_size_t],
     "ngh_programs_load_code": [_vp, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, _i32, ctypes.c_char_p,
                                ctypes.POINTER(ctypes.c_int32)],
+    "ngh_graph_begin": [_vp],
+    "ngh_graph_fork": [_vp],
+    "ngh_graph_side": [_vp, _i32],
+    "ngh_graph_join": [_vp],
+    "ngh_graph_end": [_vp, ctypes.POINTER(_vp)],
+    "ngh_graph_launch": [_vp, _vp],
+    "ngh_graph_nodes": [_vp, ctypes.POINTER(ctypes.c_int32)],
+    "ngh_graph_free": [_vp, _vp],
     "ngh_timer_begin": [_vp],
     "ngh_timer_end": [_vp, ctypes.POINTER(ctypes.c_float)],
 }
@@ -522,6 +530,41 @@ class HipRuntime(object):
             return n.value
         _check(self.lib, self.lib.ngh_programs_load(self.ctx, os.fsencode(path), ctypes.byref(n)))
         return n.value
+
+    # -- launches recorded as one HIP graph ---------------------------------
+    graphs = True
+
+    def graph_begin(self):
+        _check(self.lib, self.lib.ngh_graph_begin(self.ctx))
+
+    def graph_fork(self):
+        _check(self.lib, self.lib.ngh_graph_fork(self.ctx))
+
+    def graph_side(self, on):
+        _check(self.lib, self.lib.ngh_graph_side(self.ctx, 1 if on else 0))
+
+    def graph_join(self):
+        _check(self.lib, self.lib.ngh_graph_join(self.ctx))
+
+    def graph_end(self):
+        """The graph of what was launched since graph_begin (a handle for graph_launch)."""
+        g = _vp()
+        _check(self.lib, self.lib.ngh_graph_end(self.ctx, ctypes.byref(g)))
+        return g
+
+    def graph_abandon(self):
+        self.lib.ngh_graph_end(self.ctx, None)
+
+    def graph_launch(self, graph):
+        _check(self.lib, self.lib.ngh_graph_launch(self.ctx, graph))
+
+    def graph_nodes(self, graph):
+        n = ctypes.c_int32()
+        _check(self.lib, self.lib.ngh_graph_nodes(graph, ctypes.byref(n)))
+        return n.value
+
+    def graph_free(self, graph):
+        _check(self.lib, self.lib.ngh_graph_free(self.ctx, graph))
 
     # -- timing ------------------------------------------------------------
     def timer_begin(self):

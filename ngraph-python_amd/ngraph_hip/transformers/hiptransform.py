@@ -26,6 +26,8 @@ All arithmetic runs in libngraph_hip.so; if the library or a GPU is missing,
 constructing the transformer raises.
 """
 from __future__ import division
+
+import os
 from collections import OrderedDict
 
 import numpy as np
@@ -89,6 +91,77 @@ class HipKernelGroup(object):
         for k in self.kernels:
             if hasattr(k, "programs_changed"):
                 k.programs_changed()
+        self.drop_graph()            # (recorded launches name the kernels of before)
+
+    # -- the launches as one HIP graph (off unless the transformer is given graphs=True) -------
+    # A computation of a few small kernels spends its time on launches.  With graphs=True its
+    # launches are recorded once, after `graph_after_calls` ordinary executions (ngh_graph_begin /
+    # _end), and replayed with one call from then on; two consecutive kernels that touch no common
+    # buffer one of them writes are recorded side by side, so the device may run them together (an
+    # LSTM cell and the column sum for its bias gradient).  Only kernels whose arguments are the
+    # same in every execution are recorded (no random fills, no flex exponents), and only small
+    # ones.  Off by default because it measured slower here: the LSTM step of two 4 us kernels
+    # takes 10.6 us as two launches, 18.3 us as a graph of two nodes in a row and 31.4 us with the
+    # nodes side by side.
+    graph_after_calls = 2
+    graph_max_elements = 1 << 21            # per kernel
+    _graph = None
+    _graph_calls = 0
+    _graph_refused = False
+
+    def drop_graph(self):
+        graph, self._graph = self._graph, None
+        self._graph_calls = 0
+        if graph is not None and self.transformer.runtime is not None:
+            self.transformer.runtime.graph_free(graph)
+
+    def _graph_eligible(self):
+        t = self.transformer
+        if self._graph_refused or self._programs is not None:
+            return False             # (while kernels are being compiled the launches may still change)
+        if not t.graphs or type(self) is not HipKernelGroup or not getattr(t.runtime, "graphs", False) or \
+                len(self.kernels) < 2:
+            self._graph_refused = True
+            return False
+        for k in self.kernels:
+            recordable = type(k) in (FusedKernel, ChainKernel) and not getattr(k, "n_rng_streams", 0) and \
+                not any(getattr(m, "n_rng_streams", 0) for m in getattr(k, "members", ())) and \
+                all(spec.shape[0] * spec.shape[1] * spec.shape[2] <= self.graph_max_elements for spec in k.specs)
+            if not recordable:
+                self._graph_refused = True
+                return False
+        return True
+
+    @staticmethod
+    def _independent(a, b):
+        """Neither kernel writes a buffer the other touches."""
+        def sets(k):
+            uses = k.buffer_uses()
+            return set(base for base, _, w in uses if w), set(base for base, _, _ in uses)
+        wa, ua = sets(a)
+        wb, ub = sets(b)
+        return not (wa & ub) and not (wb & ua)
+
+    def _record_graph(self):
+        rt = self.transformer.runtime
+        rt.graph_begin()
+        try:
+            ks, i = self.kernels, 0
+            while i < len(ks):
+                if i + 1 < len(ks) and self._independent(ks[i], ks[i + 1]):
+                    rt.graph_fork()
+                    ks[i].execute()
+                    rt.graph_side(True)
+                    ks[i + 1].execute()
+                    rt.graph_join()
+                    i += 2
+                else:
+                    ks[i].execute()
+                    i += 1
+            self._graph = rt.graph_end()
+        except Exception:
+            rt.graph_abandon()
+            self._graph_refused = True          # (this computation stays with ordinary launches)
 
     def wait_for_programs(self, timeout=None):
         """Block until the kernels being compiled for this computation (jit="auto") are loaded;
@@ -141,10 +214,16 @@ class HipKernelGroup(object):
         if self._programs is not None and self._programs.poll():
             self._programs = None
             self.programs_changed()
+        if self._graph is not None:
+            self.transformer.runtime.graph_launch(self._graph)
+            return
         for k in self.execution_units():
             self.setup_kernel_execute(k)
             k.execute()
             self.after_kernel_execute(k)
+        self._graph_calls += 1
+        if self._graph_calls >= self.graph_after_calls and not self._graph_refused and self._graph_eligible():
+            self._record_graph()
 
     def execution_units(self):
         """The kernels in the order they are launched."""
@@ -189,7 +268,7 @@ class HipTransformer(ComputationGraphTransformer):
     chain_kernel_class = ChainKernel
 
     def __init__(self, device_id=0, fusion=True, dry_run=False, fuse_moments=None, rng_seed=0, jit=None,
-                 jit_min_elements=4096, jit_auto_min_elements=1 << 22, jit_after_calls=0, **kwargs):
+                 jit_min_elements=4096, jit_auto_min_elements=1 << 22, jit_after_calls=0, graphs=None, **kwargs):
         """dry_run=True lowers graphs to kernel specs without a device (no results can be
         read back); it exists so the host-side lowering can be inspected and tested.
         rng_seed keys the random fills (ng.uniform / ng.normal): same seed, same numbers.
@@ -198,7 +277,11 @@ class HipTransformer(ComputationGraphTransformer):
         "auto" (the default unless NGH_JIT says otherwise): stages of at least
         jit_auto_min_elements elements are compiled in the background and swapped in when
         ready; True: every stage of at least jit_min_elements elements is compiled before the
-        first launch; False: never."""
+        first launch; False: never.
+        graphs: record the launches of computations of a few small kernels as one HIP graph
+        after their first executions (default: off unless NGH_GRAPHS=1; replaying a graph of two
+        small kernels measured slower than launching them)."""
+        self.graphs = (os.environ.get("NGH_GRAPHS", "0") == "1") if graphs is None else bool(graphs)
         from ngraph_hip.runtime import jit as _jit
         self.jit = _jit.normalize_mode(jit)
         self.jit_min_elements = int(jit_min_elements)
@@ -341,6 +424,8 @@ class HipTransformer(ComputationGraphTransformer):
         for group in getattr(self, "kernel_groups", {}).values():
             if hasattr(group, "cancel_programs"):
                 group.cancel_programs()
+            if hasattr(group, "drop_graph") and getattr(self, "runtime", None) is not None:
+                group.drop_graph()
         rt = getattr(self, "runtime", None)
         if rt is not None:
             try:
