@@ -300,6 +300,10 @@ class FlexHipKernelGroup(HipKernelGroup):
     def __call__(self):
         manager = self.transformer.flex_manager
         manager.autoflex_count += 1
+        if self._programs is not None and self._programs.poll():
+            # (kernels compiled in the background are loaded by the thread that owns the runtime)
+            self._programs = None
+            self.programs_changed()
         if manager.resident and getattr(self, "_steady", False):
             # steady state of the device-resident mode: every tensor initialised, pointers
             # bound; one library call per kernel does prepare + launch + policy update

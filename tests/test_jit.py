@@ -885,3 +885,33 @@ def test_compiled_flex_fill_truncates_like_the_interpreter():
     if default_kernel_choice():
         assert any(n.startswith("special:jit_") for n in names), names
         assert not any(n.startswith("special:") for n in names_interp), names_interp
+
+
+@pytest.mark.gpu
+def test_flex_computation_picks_up_programs_compiled_in_the_background():
+    """jit="auto" with the flex transformer: once every exponent is initialised the kernel group
+    makes one library call per kernel and nothing else; it still has to load what the compile
+    workers finish, or the computation would stay on the interpreter for good."""
+    import time
+    t = ngt.make_transformer_factory("flexhip", jit="auto", jit_auto_min_elements=1, jit_min_elements=1)()
+    try:
+        P = ng.make_axis(1 << 16, name="P")
+        x, w = ng.placeholder([P]), ng.placeholder([P])
+        f = t.computation(ng.tanh(x * w + 0.25) * 1.5 - x, x, w)      # (a program no other test compiles)
+        vals = jit_cases.inputs_for([x, w], 21)
+        f(*vals)
+        group = t.kernel_groups[f]
+        names = []
+        for _ in range(400):
+            out = np.array(f(*vals)).copy()
+            names = [d for k in group.kernels for ds in k.describe() for d in ds]
+            if default_kernel_choice() and any(n.startswith("special:jit_") for n in names):
+                break
+            time.sleep(0.05)
+        want = np.tanh(vals[0].astype(np.float64) * vals[1] + 0.25) * 1.5 - vals[0]
+        atol, rtol = t.get_default_tolerance(want)
+        np.testing.assert_allclose(out, want, rtol=rtol, atol=atol)
+        if default_kernel_choice():
+            assert any(n.startswith("special:jit_") for n in names), names
+    finally:
+        t.close()
