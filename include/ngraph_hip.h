@@ -437,6 +437,16 @@ int  ngh_launch_fused_flex(ngh_context* ctx, const ngh_fused_spec* spec, ngh_fle
  * whose policy runs on the host after every kernel)                                        */
 int  ngh_flex_unsettled(ngh_context* ctx, int32_t* out_count);
 
+/* Two specs that do not depend on each other -- neither writes what the other touches; the
+ * caller's knowledge -- in one call, and in ONE launch when the library has their programs built
+ * as a pair: a single tiled elementwise stage and a single reduction across the contiguous axis,
+ * the LSTM cell and the column sum for its bias gradient, which the reference's compound kernel
+ * also has in one launch (layer.py:1630-1647, float_ew2.py:553-612).  The first workgroups of the
+ * launch run one program, the rest the other.  Otherwise the same as ngh_launch_fused(a)
+ * followed by ngh_launch_fused(b).  *out_one_launch (may be NULL) says which it was.         */
+int  ngh_launch_fused_pair(ngh_context* ctx, const ngh_fused_spec* a, const ngh_fused_spec* b,
+                           int32_t* out_one_launch);
+
 /* ---- the launches of a computation as one HIP graph -----------------------
  * No counterpart in the reference, which launches kernel by kernel through pycuda
  * (gputransform.py:343-345, float_ew2.py:1553-1653): for computations of a few small kernels,

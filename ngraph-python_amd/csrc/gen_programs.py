@@ -209,12 +209,15 @@ def collect():
     return programs
 
 
+# programs that one launch runs side by side: the LSTM cell and the column sum for its bias gradient
+PAIRS = [("lstm_cell_k0", "sum_across_small_k0")]
+
 HEADER = ["// GENERATED by gen_programs.py from the host lowering -- do not edit.",
           "// One entry per streaming elementwise op program that gets a pre-built kernel."]
 
 
 if __name__ == "__main__":
-    text = render(collect(), HEADER)
+    text = render(collect(), HEADER, pairs=PAIRS)
     if "--check" in sys.argv:
         sys.exit(0 if open(OUT).read() == text else 1)
     with open(OUT, "w") as fh:

@@ -138,6 +138,7 @@ struct ngh_context {
     int         row_wave_chunks = 0;     // rows of up to this many chunks are reduced by one wavefront each
     int         tile4 = 1;               // tiled elementwise programs may take 64 x 64 tiles with 16-byte accesses
     int         no_tiles = 0;        // never use the LDS-tiled elementwise skeleton
+    int         no_pairs = 0;        // never run two independent specs as one launch
     int         no_chain = 0;        // never run the stages of a spec as one row-chain kernel
     int         wide_min_rows = 2;   // column reductions: rows from which a whole workgroup lies along the columns
     int         no_ragged = 0;       // never run compiled programs 4-wide over rows that are not whole aligned vectors
@@ -1133,6 +1134,7 @@ int ngh_init(int device_id, ngh_context** out_ctx) {
     ctx->no_tiles = env_int("NGH_NO_TILES", 0);
     ctx->no_ragged = env_int("NGH_NO_RAGGED", 0);
     ctx->no_chain = env_int("NGH_NO_CHAIN", 0);
+    ctx->no_pairs = env_int("NGH_NO_PAIRS", 0);
     ctx->wide_min_rows = std::max(1, env_int("NGH_WIDE_MIN_ROWS", 2));
     ctx->red_wgs_per_cu = std::max(1, env_int("NGH_RED_WGS_PER_CU", 8));
     ctx->red_col_wgs_per_cu = std::max(1, env_int("NGH_RED_COL_WGS_PER_CU", 2));
@@ -1686,6 +1688,64 @@ int ngh_launch_fused(ngh_context* ctx, const ngh_fused_spec* spec) {
         NGH_TRY(launch_interp(ctx, P));
     }
     return NGH_OK;
+}
+
+// Two specs that do not depend on each other as ONE launch, when one of them is a single tiled
+// elementwise stage and the other a single unsplit reduction across the contiguous axis and the
+// library has their programs built as a pair (kPairTable); `dry` only says whether.
+static int try_pair_launch(ngh_context* ctx, const ngh_fused_spec& A, const ngh_fused_spec& B, bool dry, bool* done) {
+    *done = false;
+    if (ctx->force_interp || ctx->no_pairs || ((A.flags | B.flags) & NGH_SPEC_PROBE)) return NGH_OK;
+    auto only_stage = [](const ngh_fused_spec& sp) {
+        int found = -1;
+        for (int s = 0; s < sp.n_stages; ++s) {
+            if (sp.stages[s].op_end == sp.stages[s].op_begin) continue;
+            if (found >= 0) return -1;
+            found = s;
+        }
+        return found;
+    };
+    const int sa = only_stage(A), sb = only_stage(B);
+    if (sa < 0 || sb < 0) return NGH_OK;
+    Plan PA, PB;
+    NGH_TRY(plan_stage(ctx, A, sa, PA));
+    NGH_TRY(plan_stage(ctx, B, sb, PB));
+    if (PA.family != F_EW_TILED || PB.family != F_RED_COL) return NGH_OK;
+    PA.special = match_special(PA.family, PA.V, PA.k, 0);
+    PB.special = match_special(PB.family, PB.V, PB.k, 0);
+    if (PA.special < 0 || PB.special < 0 || PA.special >= kStaticCount || PB.special >= kStaticCount) return NGH_OK;
+    const PairEntry* pair = nullptr;
+    for (int i = 0; i < kPairCount && !pair; ++i)
+        if (!strcmp(kPairTable[i].first, special_name(PA.special)) && !strcmp(kPairTable[i].second, special_name(PB.special)))
+            pair = &kPairTable[i];
+    long long ta4, tb4, n4;
+    if (!pair || PA.tile != 16 || wants_tile4(ctx, PA, ta4, tb4, n4) || PA.n_tiles == 0 || PB.n_out == 0 || PB.n_seg != 1 ||
+        PA.k.n_stat_slots != 0 || PB.k.n_stat_slots != 0)
+        return NGH_OK;
+    const unsigned blocks_a = std::min<unsigned>(PA.n_tiles, (unsigned)(ctx->cus * ctx->ew_blocks_per_cu));
+    const unsigned long long blocks_b = (unsigned long long)PB.n_bx * (unsigned)PB.k.shape[1] * PB.n_seg;
+    if (blocks_b == 0 || blocks_a + blocks_b >= (1ULL << 31)) return NGH_OK;
+    *done = true;
+    if (dry) return NGH_OK;
+    pair->launch(ctx->stream, blocks_a, PA.k, PA.tiles_a, PA.tiles_b, PA.n_tiles, (unsigned)blocks_b, PB.k, PB.n_bx, PB.n_seg,
+                 PB.seg_len, PB.tx, RedWs{nullptr, nullptr});
+    HIP_TRY(hipGetLastError());
+    return NGH_OK;
+}
+
+int ngh_launch_fused_pair(ngh_context* ctx, const ngh_fused_spec* a, const ngh_fused_spec* b, int32_t* out_one_launch) {
+    if (!ctx) return fail(NGH_E_INVALID, "ctx is NULL");
+    NGH_TRY(validate(a));
+    NGH_TRY(validate(b));
+    NGH_TRY(flex_settle_spec(ctx, *a));
+    NGH_TRY(flex_settle_spec(ctx, *b));
+    bool done = false;
+    NGH_TRY(try_pair_launch(ctx, *a, *b, false, &done));
+    if (!done) NGH_TRY(try_pair_launch(ctx, *b, *a, false, &done));
+    if (out_one_launch) *out_one_launch = done ? 1 : 0;
+    if (done) return NGH_OK;
+    NGH_TRY(ngh_launch_fused(ctx, a));
+    return ngh_launch_fused(ctx, b);
 }
 
 int ngh_describe_fused(ngh_context* ctx, const ngh_fused_spec* spec, int32_t stage, char* name128) {

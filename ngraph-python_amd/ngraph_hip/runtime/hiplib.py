@@ -141,6 +141,8 @@ _SYMBOLS = {
     "ngh_program_kernels": [ctypes.c_void_p, _i32, _i32, ctypes.c_char_p, ctypes.c_size_t],
     "ngh_programs_load_code": [_vp, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, _i32, ctypes.c_char_p,
                                ctypes.POINTER(ctypes.c_int32)],
+    "ngh_launch_fused_pair": [_vp, ctypes.POINTER(ngh_fused_spec), ctypes.POINTER(ngh_fused_spec),
+                              ctypes.POINTER(ctypes.c_int32)],
     "ngh_graph_begin": [_vp],
     "ngh_graph_fork": [_vp],
     "ngh_graph_side": [_vp, _i32],
@@ -530,6 +532,12 @@ class HipRuntime(object):
             return n.value
         _check(self.lib, self.lib.ngh_programs_load(self.ctx, os.fsencode(path), ctypes.byref(n)))
         return n.value
+
+    def launch_fused_pair(self, a, b):
+        """Two specs that do not depend on each other; True when they ran as one launch."""
+        one = ctypes.c_int32()
+        _check(self.lib, self.lib.ngh_launch_fused_pair(self.ctx, ctypes.byref(a), ctypes.byref(b), ctypes.byref(one)))
+        return bool(one.value)
 
     # -- launches recorded as one HIP graph ---------------------------------
     graphs = True

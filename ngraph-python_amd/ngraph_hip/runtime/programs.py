@@ -178,8 +178,10 @@ _ENTRY = ('{{"{1}", {0}::family, {0}::V, {0}::n_ops, {0}::ops, {0}::n_tensors, {
           '{0}::bcast, {0}::n_red, {0}::red_out, {2}}},')
 
 
-def render(programs, header, prefix="SP", table="kStaticTable", count="kStaticCount"):
-    """C++ text: one `struct <prefix>n` per record, the entry table and its length."""
+def render(programs, header, prefix="SP", table="kStaticTable", count="kStaticCount", pairs=None):
+    """C++ text: one `struct <prefix>n` per record, the entry table and its length; with `pairs`
+    [(name of a tiled elementwise program, name of a column reduction)] also the table of programs
+    that one launch runs side by side (kPairTable / kPairCount)."""
     lines = list(header)
     for i, p in enumerate(programs):
         if p[8] in (4, 5):
@@ -214,4 +216,15 @@ def render(programs, header, prefix="SP", table="kStaticTable", count="kStaticCo
         lines.append('    {"none", 0, 4, 0, nullptr, 0, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr},')
     lines.append("};")
     lines.append("static const int %s = %d;" % (count, len(programs)))
+    if pairs is not None:
+        index = {p[0]: i for i, p in enumerate(programs)}
+        lines.append("static const PairEntry kPairTable[] = {")
+        for first, second in pairs:
+            a, b = programs[index[first]], programs[index[second]]
+            assert a[8] == 3 and b[8] == 2 and a[5] == 0 and b[5] == 0, (first, second)
+            lines.append('    {"%s", "%s", &launch_static_pair<%s%d, %s%d>},' % (first, second, prefix, index[first], prefix, index[second]))
+        if not pairs:
+            lines.append('    {nullptr, nullptr, nullptr},')
+        lines.append("};")
+        lines.append("static const int kPairCount = %d;" % len(pairs))
     return "\n".join(lines) + "\n"

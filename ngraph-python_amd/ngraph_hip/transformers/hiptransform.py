@@ -92,6 +92,7 @@ class HipKernelGroup(object):
             if hasattr(k, "programs_changed"):
                 k.programs_changed()
         self.drop_graph()            # (recorded launches name the kernels of before)
+        self._pairs = None
 
     # -- the launches as one HIP graph (off unless the transformer is given graphs=True) -------
     # A computation of a few small kernels spends its time on launches.  With graphs=True its
@@ -217,10 +218,15 @@ class HipKernelGroup(object):
         if self._graph is not None:
             self.transformer.runtime.graph_launch(self._graph)
             return
-        for k in self.execution_units():
-            self.setup_kernel_execute(k)
-            k.execute()
-            self.after_kernel_execute(k)
+        if self._pairs is None:
+            self._pairs = self._find_pairs()
+        if self._pairs:
+            self._execute_with_pairs()
+        else:
+            for k in self.execution_units():
+                self.setup_kernel_execute(k)
+                k.execute()
+                self.after_kernel_execute(k)
         self._graph_calls += 1
         if self._graph_calls >= self.graph_after_calls and not self._graph_refused and self._graph_eligible():
             self._record_graph()
@@ -228,6 +234,38 @@ class HipKernelGroup(object):
     def execution_units(self):
         """The kernels in the order they are launched."""
         return self.kernels
+
+    # -- two independent kernels in one launch -------------------------------------------------
+    # Consecutive fused kernels that touch no common buffer one of them writes go to the library
+    # in one call (ngh_launch_fused_pair), which runs them as ONE launch when it has their programs
+    # built as a pair (an LSTM cell and the column sum for its bias gradient).  A pair the library
+    # launches one by one anyway is not tried again.
+    _pairs = None                # {index of the first kernel of a pair}
+
+    def _find_pairs(self):
+        pairs = set()
+        if type(self) is not HipKernelGroup or not hasattr(self.transformer.runtime, "launch_fused_pair"):
+            return pairs
+        ks, i = self.kernels, 0
+        plain = lambda k: type(k) is FusedKernel and len(k.specs) == 1 and not k.n_rng_streams
+        while i + 1 < len(ks):
+            if plain(ks[i]) and plain(ks[i + 1]) and self._independent(ks[i], ks[i + 1]):
+                pairs.add(i)
+                i += 2
+            else:
+                i += 1
+        return pairs
+
+    def _execute_with_pairs(self):
+        rt, ks, i = self.transformer.runtime, self.kernels, 0
+        while i < len(ks):
+            if i in self._pairs:
+                if not rt.launch_fused_pair(ks[i].specs[0], ks[i + 1].specs[0]):
+                    self._pairs.discard(i)
+                i += 2
+            else:
+                ks[i].execute()
+                i += 1
 
     def profile(self, repeats=1, inner=1):
         """Per-kernel durations from HIP events on the launch stream.

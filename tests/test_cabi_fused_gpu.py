@@ -242,6 +242,52 @@ def test_c4_lstm_cell_transposed(hip_runtime, H, N):
         d.free()
 
 
+@pytest.mark.parametrize("H,N", [(1024, 64), (96, 7), (64, 64)])
+def test_c4_cell_and_bias_gradient_as_one_launch(hip_runtime, H, N):
+    """The LSTM cell and the column sum for its bias gradient depend on nothing of each other:
+    ngh_launch_fused_pair takes them in one call, whichever spec comes first, and gives the
+    results of the two launches.  (ONE launch needs the library's own pair of programs, which
+    the cell as the transformer lowers it matches -- tests/test_configs.py::test_c4_graph
+    checks that path -- and this hand-written cell does not: the call reports which it was.)"""
+    rt = hip_runtime
+    gates, cprev = configs.c4_inputs(H, N, seed=5)
+    c_w, h_w, db_w = configs.c4_cpu(gates, cprev)
+    gates_d, cprev_d = rt.array(gates), rt.array(cprev)
+    for swap in (False, True):
+        c_d, h_d, db_d = rt.empty((H, N)), rt.empty((H, N)), rt.empty((4 * H,))
+        for d in (c_d, h_d, db_d):
+            d.set(np.full(d.shape, np.nan, f32))
+        cell, bias = lstm_specs(rt, gates_d, cprev_d, c_d, h_d, db_d, H, N)
+        paired = rt.describe_fused(cell, 0) == "special:lstm_cell_k0" and \
+            rt.describe_fused(bias, 0) == "special:sum_across_small_k0"
+        one = rt.launch_fused_pair(bias, cell) if swap else rt.launch_fused_pair(cell, bias)
+        assert one == paired
+        np.testing.assert_allclose(c_d.get(), c_w, rtol=RTOL, atol=ATOL)
+        np.testing.assert_allclose(h_d.get(), h_w, rtol=RTOL, atol=ATOL)
+        np.testing.assert_allclose(db_d.get(), db_w, rtol=RTOL, atol=1e-5)
+        for d in (c_d, h_d, db_d):
+            d.free()
+    gates_d.free()
+    cprev_d.free()
+
+
+def test_a_pair_the_library_has_no_kernel_for_is_two_launches(hip_runtime):
+    rt = hip_runtime
+    n = 4099
+    x = np.random.RandomState(2).normal(0, 1, n).astype(f32)
+    x_d, y_d, z_d = rt.array(x), rt.empty((n,)), rt.empty((n,))
+    specs = []
+    for out, name in ((y_d, "tanh"), (z_d, "exp")):
+        sb = FusedSpecBuilder([n])
+        sb.store(sb.tensor(out.ptr, [1]), sb.unary(name, sb.load(sb.tensor(x_d.ptr, [1]))))
+        specs.append(sb.build())
+    assert not rt.launch_fused_pair(specs[0], specs[1])
+    np.testing.assert_allclose(y_d.get(), numpy_ops.unary("tanh", x), rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(z_d.get(), numpy_ops.unary("exp", x), rtol=RTOL, atol=ATOL)
+    for d in (x_d, y_d, z_d):
+        d.free()
+
+
 @pytest.mark.parametrize("name", FLOAT_UNARY_OPS)
 def test_every_unary_op(hip_runtime, name):
     rt = hip_runtime

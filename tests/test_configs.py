@@ -153,6 +153,10 @@ def test_c4_graph(transformer, Hn, Nn):
     np.testing.assert_allclose(c_g, c_w, rtol=RTOL, atol=ATOL)
     np.testing.assert_allclose(h_g, h_w, rtol=RTOL, atol=ATOL)
     np.testing.assert_allclose(db_g, db_w, rtol=RTOL, atol=1e-5)
+    group = getattr(transformer, "kernel_groups", {}).get(f)
+    if group is not None and getattr(transformer, "fusion", False) and default_kernel_choice() and Hn * Nn >= 4096:
+        # the cell and the bias gradient's column sum went to the device as ONE launch
+        assert group._pairs == {0}, (group._pairs, [type(k).__name__ for k in group.kernels])
 
 
 @pytest.mark.gpu
