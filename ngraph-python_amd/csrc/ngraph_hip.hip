@@ -1412,8 +1412,9 @@ static int stage_cache_policy(const ngh_context* ctx, const ngh_fused_spec& sp, 
 // ---------------------------------------------------------------------------
 // Row chains: every stage of a spec in one kernel (row_chain_static_kernel).  Possible when the
 // spec's rows -- spec axis 0, the axis its reduction stages reduce -- are short enough for a group
-// of lanes of one wavefront each, and every stage can run over ragged rows (fp32 operands with
-// unit stride along the row, or broadcast along it).
+// of lanes of one wavefront each, and every stage can run over ragged rows (operands with unit
+// stride along the row -- fp32, or flex16 / fp16 whose every chunk of four lies on a 4-byte
+// boundary -- or broadcast along it).
 // ---------------------------------------------------------------------------
 constexpr int kChainManagedWgsPerCu = 8;    // grid of a chain launch that runs the exponent policy itself
 
