@@ -247,3 +247,32 @@ def test_flex16_softmax_of_rows_at_full_size(rows, k):
         assert compared >= 2
     finally:
         t.close()
+
+
+def test_integer_arithmetic_over_the_whole_32_bit_range_at_full_size():
+    """25.6 M int32 operands drawn from the whole range: sums, products and comparisons of integers
+    are integer arithmetic (exact, wrapping at 2**32) as NumPy's integer loops and the reference's
+    `int` registers compute them (float_ew2.py:615-641, cputransform.py:512-761); every element is
+    compared for equality."""
+    n = 25600000
+    rs = np.random.RandomState(41)
+    a = rs.randint(-2 ** 31, 2 ** 31, n, dtype=np.int64).astype(np.int32)
+    b = rs.randint(-2 ** 31, 2 ** 31, n, dtype=np.int64).astype(np.int32)
+    b[::7] = a[::7]
+    t = ngt.make_transformer_factory("hipgpu")()
+    try:
+        P = ng.make_axis(n, name="P")
+        x, y = ng.placeholder([P], dtype=np.int32), ng.placeholder([P], dtype=np.int32)
+        k = ng.add(ng.multiply(x, y, dtype=np.int32), y, dtype=np.int32)
+        f = t.computation([k, ng.maximum(x, y), ng.equal(x, y), ng.less(x, y)], x, y)
+        first = [np.array(r).copy() for r in f(a, b)]
+        assert t.kernel_groups[f].wait_for_programs(timeout=600) is None
+        got = [np.array(r).copy() for r in f(a, b)]
+    finally:
+        t.close()
+    with np.errstate(over="ignore"):
+        want = [a * b + b, np.maximum(a, b).astype(np.float32), (a == b).astype(np.float32), (a < b).astype(np.float32)]
+    for i, (g0, g, w) in enumerate(zip(first, got, want)):
+        assert g.dtype == w.dtype, (i, g.dtype, w.dtype)
+        np.testing.assert_array_equal(g, w, err_msg="result %d" % i)
+        np.testing.assert_array_equal(g0, w, err_msg="result %d, first call" % i)
