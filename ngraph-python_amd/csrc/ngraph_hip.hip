@@ -1007,9 +1007,11 @@ int launch_interp(ngh_context* ctx, Plan& P) {
         ws.idx = (int*)ctx->ws + n;
     }
     // the merge kernel of a split reduction: few outputs with many segments each take a wavefront
-    // per output; else 64 outputs a workgroup.  It emits the results, so the statistics of flex
-    // results come from its workgroups (the partial arrays hold the larger of the two grids).
-    const bool finish_by_wave = P.n_seg >= 32 && P.n_out < 1024;
+    // per output (with 256 segments or more also a thousand or two outputs: 64 of them a
+    // workgroup would be a handful of workgroups walking a long chain of round trips); else 64
+    // outputs a workgroup.  It emits the results, so the statistics of flex results come from
+    // its workgroups (the partial arrays hold the larger of the two grids).
+    const bool finish_by_wave = P.n_seg >= 32 && (P.n_out < 1024 || P.n_seg >= 256);
     const unsigned finish_blocks = P.n_seg > 1 ? (finish_by_wave ? (P.n_out + kWaves - 1) / kWaves : (P.n_out + 63) / 64) : 0;
     unsigned red_blocks = 0;
     if (P.special >= 0 && !k.probe) {
