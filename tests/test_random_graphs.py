@@ -133,7 +133,11 @@ ILL_CONDITIONED_VIEW_SEEDS = [
     12976, 13565, 14576, 14667, 14845, 15106, 15436, 15881, 16146, 16191, 16262, 17009, 17158,
     17413, 17732, 18640, 19354, 19704, 20250, 20381, 20876, 21053, 21108, 21913, 21982, 22196,
     22444, 22510, 22987, 23155, 23393, 23446, 23506, 23751, 23756, 24024, 24084, 24421, 24509,
-    25156, 25186, 25571, 25644, 26598]
+    25156, 25186, 25571, 25644, 26598,
+    # a later sweep (`build` 30000-34050: none; `build_views` 30000-35367, and 40000-42999 with one
+    # kernel per op) with the chain kernels, ragged rows and the pair launch in place
+    30183, 30373, 30846, 32106, 32127, 32138, 32209, 32934, 33034, 33217, 33252, 33455, 33936,
+    34690, 34699, 35129, 40648, 41076, 41229, 41651, 41933, 41952, 42104, 42334]
 ILL_CONDITIONED_SEEDS = [19997]
 
 
