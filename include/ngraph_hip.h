@@ -459,8 +459,9 @@ int  ngh_launch_fused_pair(ngh_context* ctx, const ngh_fused_spec* a, const ngh_
  * follows wait for both.  Whether two launches are independent is the caller's knowledge.
  * What a recorded launch was given -- addresses, constants, random-number counters -- is what
  * every replay uses: record only launches whose arguments do not change from call to call, and
- * none that allocates (a launch that ran once before with the same shapes allocates nothing) or
- * waits for the device.  ngh_graph_end with out == NULL gives a capture up.
+ * none that allocates (a launch that ran once before with the same shapes allocates nothing; one
+ * that would have to grow a buffer of the context while recording fails with NGH_E_INVALID and
+ * records nothing) or waits for the device.  ngh_graph_end with out == NULL gives a capture up.
  * (Measured on an MI355X with ROCm 7.2: two 4 us kernels take 10.6 us as two launches, 18.3 us
  * as a graph of two nodes in a row, 31.4 us as two nodes side by side; the transformers record
  * graphs only when asked to.)                                                                  */

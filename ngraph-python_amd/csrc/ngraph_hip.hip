@@ -730,8 +730,17 @@ int plan_stage_impl(const ngh_context* ctx, const ngh_fused_spec& sp, int stage,
     return NGH_OK;
 }
 
+// (While launches are being recorded into a graph, the context's buffers may not grow: growing
+// synchronises the stream, and a recorded launch would keep the old buffer's address.)
+static int no_growth_while_recording(const ngh_context* ctx, const char* what) {
+    if (!ctx->capturing) return NGH_OK;
+    return fail(NGH_E_INVALID, "%s would have to grow while a graph is being recorded: run the launches once "
+                "before ngh_graph_begin", what);
+}
+
 int ensure_ws(ngh_context* ctx, size_t bytes) {
     if (bytes <= ctx->ws_bytes) return NGH_OK;
+    NGH_TRY(no_growth_while_recording(ctx, "the workspace of split reductions"));
     if (ctx->ws) {
         HIP_TRY(hipStreamSynchronize(ctx->stream));
         HIP_TRY(hipFree(ctx->ws));
@@ -836,6 +845,7 @@ int flex_settle_spec(ngh_context* ctx, const ngh_fused_spec& sp, const KArgs* wr
 
 int ensure_tickets(ngh_context* ctx, size_t n) {
     if (n <= ctx->n_tickets) return NGH_OK;
+    NGH_TRY(no_growth_while_recording(ctx, "the arrival counters"));
     if (ctx->tickets) {
         HIP_TRY(hipStreamSynchronize(ctx->stream));
         HIP_TRY(hipFree(ctx->tickets));
@@ -854,6 +864,7 @@ int ensure_tickets(ngh_context* ctx, size_t n) {
 // workgroups, and, after the launch, fold the scratch into each tensor's statistics word.
 int ensure_stat_ws(ngh_context* ctx, unsigned blocks) {
     if (blocks > ctx->stat_ws_blocks) {
+        NGH_TRY(no_growth_while_recording(ctx, "the per-workgroup statistics buffer"));
         if (ctx->stat_ws) {
             HIP_TRY(hipStreamSynchronize(ctx->stream));
             HIP_TRY(hipFree(ctx->stat_ws));
@@ -2135,6 +2146,7 @@ int ngh_stats_read(ngh_context* ctx, const int32_t* dev, int32_t n, int32_t* hos
 
 int ngh_flex_states_alloc(ngh_context* ctx, int32_t n, ngh_flex_state** out_dev) {
     if (!ctx || !out_dev || n <= 0) return fail(NGH_E_INVALID, "ngh_flex_states_alloc: bad argument");
+    NGH_TRY(no_growth_while_recording(ctx, "ngh_flex_states_alloc: the table of flex records"));
     void* p = nullptr;
     NGH_TRY(ngh_malloc(ctx, (size_t)n * sizeof(ngh_flex_state), &p));
     std::vector<ngh_flex_state> init((size_t)n);

@@ -86,6 +86,41 @@ def test_recording_needs_an_open_capture(hip_runtime):
     rt.sync()                                  # the context works as before
 
 
+def test_a_launch_whose_buffers_would_have_to_grow_is_refused_while_recording():
+    """A split reduction takes a workspace the context allocates at its first such launch; in a
+    fresh context that first launch cannot be a recorded one (growing would synchronise the
+    stream, and the graph would keep an address).  The refusal leaves the context usable: the
+    same launch made once outside a recording can then be recorded."""
+    from ngraph_hip.runtime import HipRuntime
+    rt = HipRuntime(0)
+    try:
+        R, A = 1 << 20, 4
+        x = np.random.RandomState(2).uniform(0.5, 1.5, (R, A)).astype(f32)
+        x_d, out_d = rt.array(x), rt.empty((A,))
+        sb = FusedSpecBuilder([R, A])
+        sb.reduce("sum", sb.load(sb.tensor(x_d.ptr, [A, 1])), sb.tensor(out_d.ptr, [0, 1]))
+        spec = sb.build()
+        rt.graph_begin()
+        with pytest.raises(HipLibraryError, match="while a graph is being recorded"):
+            rt.launch_fused(spec)
+        rt.graph_abandon()
+        rt.launch_fused(spec)
+        want = numpy_ops.reduce("sum", x, 0)
+        np.testing.assert_allclose(out_d.get(), want, rtol=1e-5)
+        rt.graph_begin()
+        rt.launch_fused(spec)
+        graph = rt.graph_end()
+        for i in range(3):
+            out_d.set(np.full(A, np.nan, f32))
+            rt.graph_launch(graph)
+            np.testing.assert_allclose(out_d.get(), want, rtol=1e-5, err_msg="replay %d" % i)
+        rt.graph_free(graph)
+        x_d.free()
+        out_d.free()
+    finally:
+        rt.close()
+
+
 def _lstm_computation(t, Hn, Nn):
     H, N, G = ng.make_axis(Hn, name="H"), ng.make_axis(Nn, name="N"), ng.make_axis(4 * Hn, name="G")
     gates_st, cprev_st = ng.placeholder([N, G]), ng.placeholder([N, H])
