@@ -708,7 +708,8 @@ __device__ __forceinline__ void red_stats_flush(const KArgs& k, const RedStats& 
 // Second pass of a split reduction: merges an output's segments (in a fixed order) and
 // stores through the output's storage type.  `row_mode` tells how an output number maps to
 // kernel coordinates.  With few segments a thread takes an output; with many, a wavefront
-// does: lanes stride over the segments and a butterfly folds them.
+// does: lanes stride over the segments and a butterfly folds them; a handful of outputs with
+// hundreds of segments each take a workgroup per output.
 __device__ __forceinline__ void red_finish_coords(const KArgs& k, unsigned out, int row_mode, long long& o0,
                                                   long long& o1, long long& o2) {
     if (row_mode) {
@@ -769,6 +770,30 @@ __global__ __launch_bounds__(kBlock) void red_finish_kernel(const KArgs k, unsig
     red_stats_flush(k, emitted);
 }
 
+// The partial results of output `out` that lanes first, first + step, ... of a group own, merged:
+// four of them are asked for before the first is merged (independent loads, dependent merges).
+__device__ __forceinline__ Acc red_finish_strided(const RedWs& ws, int opc, int s, unsigned n_seg, unsigned n_out,
+                                                  unsigned out, unsigned first, unsigned step) {
+    constexpr int kBatch = 4;
+    const bool with_index = opc >= NGH_OP_RED_ARGMAX;
+    Acc a = acc_init(opc);
+    for (unsigned g0 = first; g0 < n_seg; g0 += step * kBatch) {
+        Acc b[kBatch];
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j) {
+            const unsigned g = min(g0 + j * step, n_seg - 1);          // (a repeated load, merged only once)
+            const size_t w = ((size_t)s * n_seg + g) * n_out + out;
+            b[j].v = ws.val[w];
+            b[j].i = with_index ? ws.idx[w] : 0;
+        }
+#pragma unroll
+        for (int j = 0; j < kBatch; ++j)
+            if (g0 + j * step < n_seg) a = acc_merge(opc, a, b[j]);
+    }
+    return a;
+}
+
+// A wavefront per output: for fewer outputs than would fill workgroups of 64, with many segments each.
 __global__ __launch_bounds__(kBlock) void red_finish_wave_kernel(const KArgs k, unsigned n_out,
                                                                  unsigned n_seg, int row_mode, RedWs ws) {
     const unsigned lane = threadIdx.x & 63;
@@ -778,19 +803,41 @@ __global__ __launch_bounds__(kBlock) void red_finish_wave_kernel(const KArgs k, 
     if (out < n_out) red_finish_coords(k, out, row_mode, o0, o1, o2);
     for (int s = 0; s < k.n_red && out < n_out; ++s) {
         const int opc = red_opcode(k, s);
-        Acc a = acc_init(opc);
-        const bool with_index = opc >= NGH_OP_RED_ARGMAX;
-        for (unsigned g = lane; g < n_seg; g += 64) {
-            const size_t w = ((size_t)s * n_seg + g) * n_out + out;
-            Acc b; b.v = ws.val[w]; b.i = with_index ? ws.idx[w] : 0;
-            a = acc_merge(opc, a, b);
-        }
+        Acc a = red_finish_strided(ws, opc, s, n_seg, n_out, out, lane, 64);
 #pragma unroll
         for (int m = 32; m > 0; m >>= 1) a = acc_merge(opc, a, acc_shfl_xor(a, m));
         if (lane == 0) {
             RedWs none{nullptr, nullptr};
             red_emit(k, s, a, o0, o1, o2, out, n_out, 0, 1, none, emitted);
         }
+    }
+    red_stats_flush(k, emitted);
+}
+
+// A workgroup per output: a handful of outputs with hundreds of segments each (a sum of a whole
+// tensor into one number), where a wavefront per output would be one or two wavefronts walking a
+// long chain of round trips.
+__global__ __launch_bounds__(kBlock) void red_finish_block_kernel(const KArgs k, unsigned n_out,
+                                                                  unsigned n_seg, int row_mode, RedWs ws) {
+    __shared__ Acc sh[kWaves];
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned out = blockIdx.x;                 // (the grid has n_out workgroups)
+    RedStats emitted;
+    long long o0 = 0, o1 = 0, o2 = 0;
+    red_finish_coords(k, out, row_mode, o0, o1, o2);
+    for (int s = 0; s < k.n_red; ++s) {
+        const int opc = red_opcode(k, s);
+        Acc a = red_finish_strided(ws, opc, s, n_seg, n_out, out, threadIdx.x, kBlock);
+#pragma unroll
+        for (int m = 32; m > 0; m >>= 1) a = acc_merge(opc, a, acc_shfl_xor(a, m));
+        if (lane == 0) sh[wave] = a;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            for (int w = 1; w < kWaves; ++w) a = acc_merge(opc, a, sh[w]);
+            RedWs none{nullptr, nullptr};
+            red_emit(k, s, a, o0, o1, o2, out, n_out, 0, 1, none, emitted);
+        }
+        __syncthreads();                             // (sh is written again for the next reduction)
     }
     red_stats_flush(k, emitted);
 }

@@ -1022,8 +1022,11 @@ int launch_interp(ngh_context* ctx, Plan& P) {
     // workgroup would be a handful of workgroups walking a long chain of round trips); else 64
     // outputs a workgroup.  It emits the results, so the statistics of flex results come from
     // its workgroups (the partial arrays hold the larger of the two grids).
-    const bool finish_by_wave = P.n_seg >= 32 && (P.n_out < 1024 || P.n_seg >= 256);
-    const unsigned finish_blocks = P.n_seg > 1 ? (finish_by_wave ? (P.n_out + kWaves - 1) / kWaves : (P.n_out + 63) / 64) : 0;
+    // A handful of outputs with 256 segments or more each take a workgroup per output.
+    const bool finish_by_block = P.n_seg >= 256 && P.n_out <= 64;
+    const bool finish_by_wave = !finish_by_block && P.n_seg >= 32 && (P.n_out < 1024 || P.n_seg >= 256);
+    const unsigned finish_blocks = P.n_seg <= 1 ? 0 : finish_by_block ? P.n_out
+                                 : finish_by_wave ? (P.n_out + kWaves - 1) / kWaves : (P.n_out + 63) / 64;
     unsigned red_blocks = 0;
     if (P.special >= 0 && !k.probe) {
         // a pre-built reduction: same grid and workspace as the interpreter's kernel
@@ -1064,7 +1067,10 @@ int launch_interp(ngh_context* ctx, Plan& P) {
     HIP_TRY(hipGetLastError());
     if (k.n_stat_slots) NGH_TRY(stat_fold(ctx, k, red_blocks, 0, P.n_seg > 1 ? k.n_store_stat_slots : 4));
     if (P.n_seg > 1) {
-        if (finish_by_wave)
+        if (finish_by_block)
+            hipLaunchKernelGGL(red_finish_block_kernel, dim3(finish_blocks), dim3(kBlock), 0, ctx->stream,
+                               k, P.n_out, P.n_seg, P.family == F_RED_ROW ? 1 : 0, ws);
+        else if (finish_by_wave)
             hipLaunchKernelGGL(red_finish_wave_kernel, dim3(finish_blocks), dim3(kBlock), 0, ctx->stream,
                                k, P.n_out, P.n_seg, P.family == F_RED_ROW ? 1 : 0, ws);
         else

@@ -617,6 +617,55 @@ def test_reductions_over_nan_and_infinities(hip_runtime, name, layout):
         np.testing.assert_allclose(got[~np.isnan(want)], want[~np.isnan(want)], rtol=1e-4)
 
 
+@pytest.mark.parametrize("name", ["sum", "max", "min", "argmax", "argmin"])
+@pytest.mark.parametrize("shape,layout", [((1 << 20, 3), "row"), ((1 << 20, 4), "col"), ((1 << 21, 1), "row")])
+def test_reductions_into_a_handful_of_outputs_with_hundreds_of_segments(hip_runtime, name, shape, layout):
+    """A few outputs, each split into 256 segments or more: the merge takes a workgroup per
+    output.  Ties across segments (the lowest index wins) and a NaN in one segment included."""
+    from ngraph_hip.runtime.hiplib import plan_fused
+    rt = hip_runtime
+    R, A = shape
+    rs = np.random.RandomState(15)
+    logical = (rs.uniform(0.5, 1.5, (R, A)) if name == "sum" else rs.normal(0, 1, (R, A))).astype(f32)
+    if name != "sum":
+        extreme = f32(9.0 if name in ("max", "argmax") else -9.0)
+        logical[R // 3, :] = extreme                   # the same extreme value in two far-apart segments
+        logical[R // 3 * 2, :] = extreme
+        if name in ("max", "min"):
+            logical[R // 2, A - 1] = np.nan            # ... and a NaN in the last output's rows
+    want = numpy_ops.reduce(name, logical, 0)
+    if layout == "row":
+        store, strides = np.ascontiguousarray(logical.T), [1, R]
+    else:
+        store, strides = logical, [A, 1]
+    x_d = rt.array(store)
+    is_arg = name.startswith("arg")
+    out_d = rt.empty((A,), NGH_I32 if is_arg else NGH_F32)
+    sb = FusedSpecBuilder([R, A])
+    sb.reduce(name, sb.load(sb.tensor(x_d.ptr, strides)), sb.tensor(out_d.ptr, [0, 1], NGH_I32 if is_arg else NGH_F32))
+    spec = sb.build()
+    if default_kernel_choice():
+        assert plan_fused(spec)["segments"] >= 256
+    rt.launch_fused(spec)
+    got = out_d.get()
+    if is_arg:
+        np.testing.assert_array_equal(got, want)
+    else:
+        np.testing.assert_array_equal(np.isnan(got), np.isnan(want))
+        ok = ~np.isnan(want)
+        if name == "sum":
+            # a million same-sign terms: the oracle's ufunc adds the rows of a C-ordered operand one
+            # after the other in float32 and drifts by up to 2e-5 of the result; float64 decides,
+            # and the device's segments and tree are the closer side
+            truth = logical.astype(np.float64).sum(axis=0)
+            np.testing.assert_allclose(got, truth, rtol=2e-6)
+            np.testing.assert_allclose(want, truth, rtol=1e-4)
+        else:
+            np.testing.assert_allclose(got[ok], want[ok], rtol=1e-5)
+    x_d.free()
+    out_d.free()
+
+
 @pytest.mark.parametrize("name", ["argmax", "argmin"])
 def test_arg_reduction_index_beyond_2_to_24_is_exact(hip_runtime, name):
     """An index above 2^24 reaches int32 storage as the integer it is (no trip through an fp32
