@@ -721,16 +721,18 @@ __device__ __forceinline__ void red_finish_coords(const KArgs& k, unsigned out, 
     }
 }
 
-// A workgroup takes 64 outputs (one per lane: partial results of consecutive outputs are
-// consecutive in the workspace) and its four wavefronts a quarter of the segments each, in
-// segment order; the quarters meet in shared memory and are merged in wavefront order.
-__global__ __launch_bounds__(kBlock) void red_finish_kernel(const KArgs k, unsigned n_out,
-                                                            unsigned n_seg, int row_mode, RedWs ws) {
-    __shared__ Acc sh[kWaves][64];
-    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const unsigned out = blockIdx.x * 64 + lane;
-    const unsigned per_wave = (n_seg + kWaves - 1) / kWaves;
-    const unsigned g_begin = min(n_seg, wave * per_wave), g_end = min(n_seg, g_begin + per_wave);
+// A workgroup takes `outs` outputs (64, 32 or 16: partial results of consecutive outputs are
+// consecutive in the workspace) and its 256 / outs groups of lanes an equal share of the segments
+// each, in segment order; the shares meet in shared memory and are merged in group order.  Fewer
+// outputs a workgroup are more workgroups with shorter chains of round trips, which is what a
+// merge of a few thousand outputs consists of.
+__global__ __launch_bounds__(kBlock) void red_finish_kernel(const KArgs k, unsigned n_out, unsigned n_seg,
+                                                            int row_mode, RedWs ws, unsigned outs) {
+    __shared__ Acc sh[kBlock];
+    const unsigned mine = threadIdx.x & (outs - 1), group = threadIdx.x / outs, groups = kBlock / outs;
+    const unsigned out = blockIdx.x * outs + mine;
+    const unsigned per_group = (n_seg + groups - 1) / groups;
+    const unsigned g_begin = min(n_seg, group * per_group), g_end = min(n_seg, g_begin + per_group);
     long long o0 = 0, o1 = 0, o2 = 0;
     if (out < n_out) red_finish_coords(k, out, row_mode, o0, o1, o2);
     RedStats emitted;
@@ -757,11 +759,11 @@ __global__ __launch_bounds__(kBlock) void red_finish_kernel(const KArgs k, unsig
                     if (g0 + j < g_end) a = acc_merge(opc, a, b[j]);
             }
         }
-        sh[wave][lane] = a;
+        sh[threadIdx.x] = a;
         __syncthreads();
-        if (wave == 0 && out < n_out) {
-            // (a wavefront that had no segments holds the reduction's identity)
-            for (int w = 1; w < kWaves; ++w) a = acc_merge(opc, a, sh[w][lane]);
+        if (group == 0 && out < n_out) {
+            // (a group that had no segments holds the reduction's identity)
+            for (unsigned g = 1; g < groups; ++g) a = acc_merge(opc, a, sh[g * outs + mine]);
             RedWs none{nullptr, nullptr};
             red_emit(k, s, a, o0, o1, o2, out, n_out, 0, 1, none, emitted);
         }

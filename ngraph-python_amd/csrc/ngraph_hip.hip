@@ -1025,8 +1025,15 @@ int launch_interp(ngh_context* ctx, Plan& P) {
     // A handful of outputs with 256 segments or more each take a workgroup per output.
     const bool finish_by_block = P.n_seg >= 256 && P.n_out <= 64;
     const bool finish_by_wave = !finish_by_block && P.n_seg >= 32 && (P.n_out < 1024 || P.n_seg >= 256);
+    // Else 64 outputs a workgroup, or 32 or 16 while that leaves compute units without a workgroup
+    // and every group of lanes more than one batch of segments.
+    unsigned finish_outs = 64;
+    while (finish_outs > 16 && (P.n_out + finish_outs - 1) / finish_outs < (unsigned)ctx->cus &&
+           P.n_seg / (kBlock / finish_outs) > 8)
+        finish_outs >>= 1;
     const unsigned finish_blocks = P.n_seg <= 1 ? 0 : finish_by_block ? P.n_out
-                                 : finish_by_wave ? (P.n_out + kWaves - 1) / kWaves : (P.n_out + 63) / 64;
+                                 : finish_by_wave ? (P.n_out + kWaves - 1) / kWaves
+                                                  : (P.n_out + finish_outs - 1) / finish_outs;
     unsigned red_blocks = 0;
     if (P.special >= 0 && !k.probe) {
         // a pre-built reduction: same grid and workspace as the interpreter's kernel
@@ -1075,7 +1082,7 @@ int launch_interp(ngh_context* ctx, Plan& P) {
                                k, P.n_out, P.n_seg, P.family == F_RED_ROW ? 1 : 0, ws);
         else
             hipLaunchKernelGGL(red_finish_kernel, dim3(finish_blocks), dim3(kBlock), 0, ctx->stream,
-                               k, P.n_out, P.n_seg, P.family == F_RED_ROW ? 1 : 0, ws);
+                               k, P.n_out, P.n_seg, P.family == F_RED_ROW ? 1 : 0, ws, finish_outs);
         HIP_TRY(hipGetLastError());
         if (k.n_stat_slots > k.n_store_stat_slots) NGH_TRY(stat_fold(ctx, k, finish_blocks, k.n_store_stat_slots, 4));
     }
